@@ -1,0 +1,253 @@
+/*
+ * ucm_hip.h — C ABI of the MI355X (gfx950) sparse-retrieval and KV-transfer library.
+ *
+ * Every entry point takes plain pointers and sizes, returns an int status and never
+ * throws.  Device pointers are ordinary HIP device addresses; `stream` arguments are a
+ * `hipStream_t` passed as `void*` (NULL = the null stream).  Unless a function says
+ * "sync" it only enqueues work on the given stream.
+ *
+ * Status codes follow the reference's UC::Status convention
+ * (ucm/shared/infra/status/status.h:40-53): 0 = OK, -1 = generic error,
+ * -50000-i = typed errors.  ucm_last_error() returns the message of the last failure
+ * on the calling thread.
+ */
+#ifndef UCM_HIP_H
+#define UCM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define UCM_OK            0
+#define UCM_ERROR        (-1)
+#define UCM_EPARAM       (-50000)
+#define UCM_EOOM         (-50001)
+#define UCM_EOSERROR     (-50002)
+#define UCM_EUNSUPPORTED (-50008)
+#define UCM_ETIMEOUT     (-50010)
+
+/* element types of encoder inputs */
+#define UCM_DT_BF16 0
+#define UCM_DT_F16  1
+#define UCM_DT_F32  2
+
+typedef void* ucm_stream_t;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int ucm_version(void);
+/* Message of the last failing call on this thread ("" if none). */
+const char* ucm_last_error(void);
+
+/* ------------------------------------------------------------------------------------
+ * 1. Hash encoder: codes = pack_lsb_first( x · W > 0 )
+ * ------------------------------------------------------------------------------------ */
+
+/*
+ * Replaces HashEncoder.compute_hash (ucm/sparse/gsa_on_device/hash_encoder.py:450-507)
+ * and its Triton kernel (hash_encoder.py:37-134).
+ *
+ * x        [T, H, K] of x_dtype, K contiguous; strides in elements.
+ * w        [n_w, K, N_bits] row-major of w_dtype.  Head h uses matrix
+ *          min(h / heads_per_w, n_w - 1); n_w = 1 shares one matrix (the reference's case).
+ * out      uint32 [T, H, N_bits/32]; strides in 32-bit words.  Hash bit n of a row is bit
+ *          n%32 of word n/32, i.e. byte n/8, bit n%8 (LSB first), little endian — the byte
+ *          order torch_hash_code produces (hash_encoder.py:359-370).
+ * A projection that is 0, -0 or NaN gives bit 0.  Requires K % 16 == 0, N_bits % 32 == 0.
+ */
+int ucm_hash_encode(const void* x, int x_dtype, int64_t T, int32_t H, int32_t K,
+                    int64_t x_stride_t, int64_t x_stride_h,
+                    const void* w, int w_dtype, int32_t n_w, int32_t heads_per_w,
+                    int32_t N_bits,
+                    uint32_t* out, int64_t out_stride_t, int64_t out_stride_h,
+                    ucm_stream_t stream);
+
+/*
+ * Replaces HashEncoder.compute_hash_and_cache (hash_encoder.py:548-662) and
+ * fused_hash_and_cache_kernel (hash_encoder.py:263-356): encode x[t,h,:] and store the
+ * code at cache[slot/BS, slot%BS, h, :].  Rows whose slot is < 0 or >= NB*BS are
+ * skipped (hash_encoder.py:338-344).
+ *
+ * slot_mapping  [T] int32 (slot_is_i64 = 0) or int64 (slot_is_i64 = 1), device memory.
+ * cache         uint32 words; strides (block, token, head) in 32-bit words, the N_bits/32
+ *               words of a code are contiguous.
+ */
+int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int32_t K,
+                          int64_t x_stride_t, int64_t x_stride_h,
+                          const void* w, int w_dtype, int32_t n_w, int32_t heads_per_w,
+                          int32_t N_bits,
+                          const void* slot_mapping, int slot_is_i64,
+                          uint32_t* cache, int64_t NB, int32_t BS,
+                          int64_t cs_block, int64_t cs_token, int64_t cs_head,
+                          ucm_stream_t stream);
+
+/*
+ * Replaces reshape_and_cache_khash_triton (hash_encoder.py:136-261): scatter already
+ * computed codes [T, H, Wd] into the paged code cache by slot.
+ */
+int ucm_code_scatter(const uint32_t* codes, int64_t T, int32_t H, int32_t Wd,
+                     int64_t in_stride_t, int64_t in_stride_h,
+                     const void* slot_mapping, int slot_is_i64,
+                     uint32_t* cache, int64_t NB, int32_t BS,
+                     int64_t cs_block, int64_t cs_token, int64_t cs_head,
+                     ucm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * 2. Hamming scorer + deterministic block top-k
+ * ------------------------------------------------------------------------------------ */
+
+/* flags of ucm_hamming_topk */
+#define UCM_TOPK_REDUCE_HEADS    1u  /* one list per request: block score = max over KV heads
+                                        (= the min over heads of paged_ham_dist_mla.cu:203-211) */
+#define UCM_TOPK_RETURN_PHYSICAL 2u  /* out_idx holds block_table[b, j] instead of logical j
+                                        (hamming_topk.py:54) */
+#define UCM_TOPK_SCORE_ORDER     4u  /* order the k results by (score desc, index asc) instead
+                                        of ascending index (hash_retrieval_backend.cpp:396-406) */
+#define UCM_TOPK_DISTANCE        8u  /* out_score holds Hamming distance G*bits - s */
+
+/* Bytes of device workspace ucm_hamming_topk needs for these sizes. */
+size_t ucm_hamming_topk_workspace_bytes(int32_t B, int32_t Hkv, int32_t max_blocks);
+
+/*
+ * Replaces hamming.hamming_score + the torch min/topk/sort/gather chain of
+ * cuda_hamming_topk (ucm/sparse/gsa_on_device/hamming_topk.py:15-54,
+ * csrc/cuda/ham_dist/paged_ham_dist_mla.cu:111-248,332-443), with the per-KV-head,
+ * similarity-score output contract of npu_hamming_dist_top_k
+ * (csrc/ascend/torch_binding.cpp:39-57).
+ *
+ * q_codes     uint32 [B, Hq, Wd], strides in words (Wd contiguous).
+ * k_cache     uint32 paged codes, logical shape [NB, BS, Hkv, Wd]; strides (block, token,
+ *             head) in words, Wd contiguous.  Token-major [NB,BS,Hkv,Wd] and head-major
+ *             [NB,Hkv,BS,Wd] caches are both expressed through the strides.
+ * block_table int32 [B, table_stride], logical block j of request b is block_table[b, j].
+ *             NULL = request b owns blocks b*max_blocks ... (contiguous cache).
+ * seq_lens    int32 [B] valid tokens per request.
+ * G = Hq / Hkv query heads are summed per KV head:
+ *   s[b,h,j] = max over valid tokens t of block j of
+ *              sum_g ( 32*Wd - popcount(q[b,h*G+g] xor k[table[b,j], t, h]) )      (int32)
+ * A block holding a position < sink_tok or >= len - recent_tok gets s = G*32*Wd
+ * (paged_ham_dist_mla.cu:194-197).  A table entry outside [0, NB) scores -1.
+ * Per (b, h) [or per b with UCM_TOPK_REDUCE_HEADS] the min(k, nblk) blocks with the
+ * largest s are selected, ties to the lower logical index, and written in ascending
+ * logical index order; unused output slots get index -1 and score 0.
+ *
+ * out_idx, out_score  int32 [B, Hkv or 1, k]; out_score may be NULL.
+ * workspace   device memory of at least ucm_hamming_topk_workspace_bytes(...) bytes,
+ *             16-byte aligned; contents need no initialisation.
+ */
+int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                     const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
+                     int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                     const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                     const int32_t* seq_lens,
+                     int32_t B, int32_t Hq, int32_t k,
+                     int32_t sink_tok, int32_t recent_tok, uint32_t flags,
+                     int32_t* out_idx, int32_t* out_score,
+                     void* workspace, size_t workspace_bytes,
+                     ucm_stream_t stream);
+
+/*
+ * Replaces kvlib::HammingScoreContiCUDA (csrc/cuda/ham_dist/operator.h:10-13,
+ * paged_ham_dist_mla.cu:332-443) for callers that want its per-token output:
+ * out[b, h, p] for p < max_seq_len is the group-summed Hamming distance of position p,
+ * 0 for sink/recent positions and "infinity" for p >= seq_lens[b].
+ * out_is_f16 = 1 writes IEEE half exactly as the reference (inf = 0x7C00);
+ * out_is_f16 = 0 writes int32 with infinity = INT32_MAX.
+ * reduce_heads = 1 writes the min over KV heads, shape [B, 1, max_seq_len].
+ */
+int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                      const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
+                      int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                      const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                      const int32_t* seq_lens,
+                      int32_t B, int32_t Hq, int32_t max_seq_len,
+                      int32_t sink_tok, int32_t recent_tok, int reduce_heads,
+                      void* out, int out_is_f16,
+                      ucm_stream_t stream);
+
+/* Replaces update_seq_lens (hamming_topk.py:7-12):
+ * out[b] = len[b] - ceil(max(len[b] - topk_tok, 0) / BS) * BS. */
+int ucm_update_seq_lens(const int32_t* seq_lens, int32_t B, int32_t topk_tok, int32_t BS,
+                        int32_t* out, ucm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * 3. KV block gather / scatter ("trans")
+ * ------------------------------------------------------------------------------------ */
+
+typedef struct ucm_trans_stream ucm_trans_stream_t;
+
+/* Replaces UC::Trans::Device::Setup (ucm/shared/trans/cuda/cuda_device.cc:32-73):
+ * make device_id current for the calling thread.  A negative or absent id fails. */
+int ucm_trans_setup(int32_t device_id);
+
+/* Stream kinds: copy-engine (Device::MakeStream, cuda_stream.cc:28-33) and
+ * compute-unit kernel copies (Device::MakeSMStream, cuda_sm_stream.cc:29-55). */
+#define UCM_TRANS_CE 0
+#define UCM_TRANS_SM 1
+int ucm_trans_stream_create(int kind, ucm_trans_stream_t** out);
+int ucm_trans_stream_destroy(ucm_trans_stream_t* s);
+/* the underlying hipStream_t */
+void* ucm_trans_stream_handle(ucm_trans_stream_t* s);
+/* Stream::Synchronized (cuda_stream.cc:151-156) */
+int ucm_trans_stream_sync(ucm_trans_stream_t* s);
+/* Stream::WaitEvent (cuda_stream.cc:158-164); event is a hipEvent_t, NULL is a no-op */
+int ucm_trans_stream_wait_event(ucm_trans_stream_t* s, void* event);
+/* Stream::AppendCallback (cuda_stream.cc:131-149): cb(ok, user) runs on a runtime thread
+ * once all work enqueued so far has finished. */
+int ucm_trans_stream_append_callback(ucm_trans_stream_t* s, void (*cb)(int ok, void* user),
+                                     void* user);
+
+/* Single copies, Stream::DeviceToHost[Async] / HostToDevice[Async] (cuda_stream.cc:35-40,
+ * 56-61,82-87,103-108).  `sync` != 0 waits for completion. */
+int ucm_trans_d2h(ucm_trans_stream_t* s, const void* device, void* host, size_t size, int sync);
+int ucm_trans_h2d(ucm_trans_stream_t* s, const void* host, void* device, size_t size, int sync);
+
+/*
+ * Pointer-table copies of `number` chunks of `size` bytes
+ * (cuda_stream.cc:63-80,110-127; cuda_sm_kernel.cu:52-114).
+ *   gather : dst + i*size  <- src[i]
+ *   scatter: dst[i]        <- src + i*size
+ *   batch  : dst[i]        <- src[i]
+ * table_on_device = 0: the pointer arrays are host arrays (read before the call returns);
+ * table_on_device = 1: they already live in device-readable memory
+ * (the SM-stream convention, ucm/shared/test/case/trans/trans_test.cc:84-89).
+ * On an SM stream one kernel moves all chunks; the flat side may be device memory or
+ * pinned/registered host memory.  On a CE stream one hipMemcpyAsync is issued per chunk.
+ * Unlike the reference's kernel (cuda_sm_kernel.cu:56) a tail shorter than the copy unit
+ * is copied, not dropped.
+ */
+int ucm_trans_gather(ucm_trans_stream_t* s, const void* const* src, int table_on_device,
+                     void* dst, size_t size, size_t number, int sync);
+int ucm_trans_scatter(ucm_trans_stream_t* s, const void* src, void* const* dst,
+                      int table_on_device, size_t size, size_t number, int sync);
+int ucm_trans_batch(ucm_trans_stream_t* s, const void* const* src, void* const* dst,
+                    int table_on_device, size_t size, size_t number, int sync);
+
+/*
+ * Table-free form for a paged KV cache whose address rule is
+ *   addr(block, col) = base[col] + block_id * col_bytes[col]
+ * (KVCacheLayout.extract_block_addrs, ucm/integration/vllm/ucm_connector.py:91-148).
+ * The flat buffer is laid out (block, col) row-major, column c of a block at the running
+ * sum of col_bytes (dump_queue.cc:145-161).  base / col_bytes are host arrays of n_cols
+ * entries; block_ids is a host array of n_blocks entries.  to_cache = 0 gathers cache ->
+ * flat, 1 scatters flat -> cache.  SM streams only.
+ */
+int ucm_trans_paged_copy(ucm_trans_stream_t* s, const uint64_t* base, const uint64_t* col_bytes,
+                         int32_t n_cols, const int32_t* block_ids, int64_t n_blocks,
+                         void* flat, int to_cache, int sync);
+
+/* Buffer::MakeHostBuffer / MakeDeviceBuffer / RegisterHostBuffer
+ * (ucm/shared/trans/buffer.h:32-47, cuda/cuda_buffer.cc:29-56). */
+int ucm_trans_host_alloc(size_t size, void** out);
+int ucm_trans_host_free(void* p);
+int ucm_trans_device_alloc(size_t size, void** out);
+int ucm_trans_device_free(void* p);
+int ucm_trans_host_register(void* host, size_t size, void** device_alias);
+int ucm_trans_host_unregister(void* host);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UCM_HIP_H */

@@ -1,0 +1,457 @@
+/*
+ * ucm_oracle.c — CPU restatement of the reference's sparse-retrieval / KV-transfer
+ * arithmetic.  TEST INFRASTRUCTURE ONLY: it is the checker that the HIP library is
+ * compared against (tests, the smoke check, and the CPU-baseline leg of the benchmark).
+ * Nothing in the shipped library calls into this file.
+ *
+ * Each function names the reference lines it restates (paths relative to the reference
+ * checkout).  Plain C, scalar loops; the *_mt entry uses pthreads with one thread per
+ * request, which is the reference CPU backend's execution model
+ * (ucm/sparse/gsa_on_device/csrc/cuda/hash_retrieval/cpy/hash_retrieval_backend.cpp:180-199,338).
+ */
+#include <limits.h>
+#include <math.h>
+#include <pthread.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORACLE_INF INT32_MAX
+
+static inline int popc32(uint32_t v) { return __builtin_popcount(v); }
+
+/* ------------------------------------------------------------------------------------
+ * Encoder.  ucm/sparse/gsa_on_device/hash_encoder.py:359-370 (torch_hash_code):
+ *   p = x @ W ; bit = p > 0 ; byte j = sum_i bit[8j+i] << i.
+ * x [M,K] fp32 (callers widen bf16/fp16 exactly), W [K,N] fp32.
+ * acc_f64 = 0: fp32 accumulation in ascending k; 1: fp64 accumulation.
+ * margin (optional, [M,N]) = |p| / ||x_row||_2, used by tests for the tolerance rule.
+ * ------------------------------------------------------------------------------------ */
+void oracle_hash_encode(const float* x, int64_t M, int32_t K, const float* W, int32_t N,
+                        int acc_f64, uint32_t* codes, float* margin)
+{
+    const int32_t Wd = N / 32;
+    for (int64_t m = 0; m < M; ++m) {
+        const float* xr = x + m * K;
+        double nrm2 = 0.0;
+        for (int32_t k = 0; k < K; ++k) nrm2 += (double)xr[k] * (double)xr[k];
+        const double nrm = sqrt(nrm2);
+        for (int32_t w = 0; w < Wd; ++w) codes[m * Wd + w] = 0u;
+        for (int32_t n = 0; n < N; ++n) {
+            double p;
+            if (acc_f64) {
+                double a = 0.0;
+                for (int32_t k = 0; k < K; ++k) a += (double)xr[k] * (double)W[(int64_t)k * N + n];
+                p = a;
+            } else {
+                float a = 0.0f;
+                for (int32_t k = 0; k < K; ++k) a += xr[k] * W[(int64_t)k * N + n];
+                p = (double)a;
+            }
+            if (p > 0.0) codes[m * Wd + (n >> 5)] |= 1u << (n & 31);
+            if (margin) margin[m * N + n] = nrm > 0.0 ? (float)(fabs(p) / nrm) : 0.0f;
+        }
+    }
+}
+
+/*
+ * Fused encode + paged store.  hash_encoder.py:263-356 (fused_hash_and_cache_kernel):
+ * row (t,h) is encoded with W[min(h / heads_per_w, n_w-1)] and stored at
+ * cache[slot/BS, slot%BS, h, :]; slots < 0 or >= NB*BS are skipped (:338-344).
+ * x [T,H,K] fp32 contiguous, W [n_w,K,N]; cache strides in 32-bit words.
+ */
+void oracle_hash_encode_cache(const float* x, int64_t T, int32_t H, int32_t K, const float* W,
+                              int32_t n_w, int32_t heads_per_w, int32_t N, const int64_t* slot,
+                              uint32_t* cache, int64_t NB, int32_t BS, int64_t cs_block,
+                              int64_t cs_token, int64_t cs_head)
+{
+    const int32_t Wd = N / 32;
+    uint32_t* tmp = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)Wd);
+    for (int64_t t = 0; t < T; ++t) {
+        const int64_t s = slot[t];
+        if (s < 0 || s >= NB * (int64_t)BS) continue;
+        for (int32_t h = 0; h < H; ++h) {
+            int32_t wi = heads_per_w > 0 ? h / heads_per_w : 0;
+            if (wi > n_w - 1) wi = n_w - 1;
+            oracle_hash_encode(x + (t * H + h) * (int64_t)K, 1, K, W + (int64_t)wi * K * N, N, 0,
+                               tmp, NULL);
+            uint32_t* dst = cache + (s / BS) * cs_block + (s % BS) * cs_token + h * cs_head;
+            memcpy(dst, tmp, sizeof(uint32_t) * (size_t)Wd);
+        }
+    }
+    free(tmp);
+}
+
+/* Scatter of precomputed codes.  hash_encoder.py:136-195 (_reshape_and_cache_khash_kernel). */
+void oracle_code_scatter(const uint32_t* codes, int64_t T, int32_t H, int32_t Wd,
+                         const int64_t* slot, uint32_t* cache, int64_t NB, int32_t BS,
+                         int64_t cs_block, int64_t cs_token, int64_t cs_head)
+{
+    for (int64_t t = 0; t < T; ++t) {
+        const int64_t s = slot[t];
+        if (s < 0 || s >= NB * (int64_t)BS) continue;
+        for (int32_t h = 0; h < H; ++h)
+            memcpy(cache + (s / BS) * cs_block + (s % BS) * cs_token + h * cs_head,
+                   codes + (t * H + h) * (int64_t)Wd, sizeof(uint32_t) * (size_t)Wd);
+    }
+}
+
+/* ------------------------------------------------------------------------------------
+ * Scorer.
+ * ------------------------------------------------------------------------------------ */
+
+/* Group-summed Hamming distance of one cached token against the G query heads of KV head
+ * h.  csrc/cuda/ham_dist/paged_ham_dist_mla.cu:172-178 (the KVGroup loop). */
+static int32_t group_distance(const uint32_t* q_bh, int64_t q_stride_h, int32_t G,
+                              const uint32_t* kcode, int32_t Wd)
+{
+    int32_t d = 0;
+    for (int32_t g = 0; g < G; ++g)
+        for (int32_t w = 0; w < Wd; ++w) d += popc32(q_bh[g * q_stride_h + w] ^ kcode[w]);
+    return d;
+}
+
+/*
+ * Per-token distances in the reference scorer's output shape.
+ * paged_ham_dist_mla.cu:148-247: out[b,h,p] = distance; 0 if p < sink or
+ * len-recent <= p < len; INF if p >= len (:194-197,213-214,243-244); with reduce_heads the
+ * min over KV heads is written to out[b,0,p] (:203-211).
+ * The cache is addressed [block, token, head] through explicit strides.
+ * out int32 [B, (reduce ? 1 : Hkv), max_seq_len].
+ */
+void oracle_hamming_score(const uint32_t* q, int64_t q_stride_b, int64_t q_stride_h,
+                          const uint32_t* kc, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
+                          int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                          const int32_t* table, int32_t table_stride, int32_t max_blocks,
+                          const int32_t* lens, int32_t B, int32_t Hq, int32_t max_seq_len,
+                          int32_t sink, int32_t recent, int reduce_heads, int32_t* out)
+{
+    const int32_t G = Hq / Hkv;
+    const int32_t Ho = reduce_heads ? 1 : Hkv;
+    for (int32_t b = 0; b < B; ++b) {
+        const int32_t len = lens[b];
+        for (int32_t p = 0; p < max_seq_len; ++p) {
+            const int32_t j = p / BS, t = p % BS;
+            const int is_inf = p >= len;
+            const int keep = (p < sink) || (p >= len - recent && p < len);
+            int32_t red = ORACLE_INF;
+            for (int32_t h = 0; h < Hkv; ++h) {
+                int32_t v;
+                if (is_inf) {
+                    v = ORACLE_INF;
+                } else if (keep) {
+                    v = 0;
+                } else {
+                    const int64_t pb = table ? table[(int64_t)b * table_stride + j]
+                                             : (int64_t)b * max_blocks + j;
+                    if (pb < 0 || pb >= NB) {
+                        v = ORACLE_INF;
+                    } else {
+                        v = group_distance(q + b * q_stride_b + (int64_t)h * G * q_stride_h,
+                                           q_stride_h, G,
+                                           kc + pb * ks_block + t * ks_token + h * ks_head, Wd);
+                    }
+                }
+                if (reduce_heads) {
+                    if (v < red) red = v;
+                } else {
+                    out[((int64_t)b * Ho + h) * max_seq_len + p] = v;
+                }
+            }
+            if (reduce_heads) out[(int64_t)b * max_seq_len + p] = red;
+        }
+    }
+}
+
+/* flag bits, same values as the library's UCM_TOPK_* */
+#define F_REDUCE_HEADS 1u
+#define F_PHYSICAL 2u
+#define F_SCORE_ORDER 4u
+#define F_DISTANCE 8u
+
+typedef struct {
+    int32_t score;
+    int32_t idx;
+} cand_t;
+
+/* (score desc, index asc): the deterministic order that fixes the reference's unspecified
+ * ties (torch.topk in hamming_topk.py:49-51; std::partial_sort on .first only in
+ * hash_retrieval_backend.cpp:396-400). */
+static int cand_cmp(const void* a, const void* b)
+{
+    const cand_t* x = (const cand_t*)a;
+    const cand_t* y = (const cand_t*)b;
+    if (x->score != y->score) return x->score > y->score ? -1 : 1;
+    return x->idx < y->idx ? -1 : (x->idx > y->idx ? 1 : 0);
+}
+static int idx_cmp(const void* a, const void* b)
+{
+    const cand_t* x = (const cand_t*)a;
+    const cand_t* y = (const cand_t*)b;
+    return x->idx < y->idx ? -1 : (x->idx > y->idx ? 1 : 0);
+}
+
+/*
+ * Block scores of one request: s[h][j], j < nblk.
+ * Block reduction = min distance over the block's valid tokens (hamming_topk.py:45-47)
+ * restated as max similarity G*bits - d (the NPU op's form,
+ * csrc/ascend/hamming_dist_top_k/op_kernel/hamming_dist_top_k_base.h:150-289).
+ * Sink/recent positions have distance 0 (paged_ham_dist_mla.cu:194-197) so any block that
+ * holds one scores G*bits.
+ */
+static void block_scores_one(const uint32_t* q_b, int64_t q_stride_h, const uint32_t* kc,
+                             int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd, int64_t ks_block,
+                             int64_t ks_token, int64_t ks_head, const int32_t* table_b,
+                             int64_t contiguous_base, int32_t len, int32_t G, int32_t sink,
+                             int32_t recent, int32_t nblk, int32_t* s /* [Hkv][nblk] */)
+{
+    const int32_t full = G * 32 * Wd;
+    for (int32_t j = 0; j < nblk; ++j) {
+        const int64_t pb = table_b ? table_b[j] : contiguous_base + j;
+        const int32_t p0 = j * BS;
+        const int32_t p1 = (p0 + BS < len) ? p0 + BS : len; /* valid positions [p0,p1) */
+        const int forced = (p0 < sink) || (p1 > len - recent);
+        for (int32_t h = 0; h < Hkv; ++h) {
+            int32_t best;
+            if (pb < 0 || pb >= NB) {
+                best = -1;
+            } else if (forced) {
+                best = full;
+            } else {
+                int32_t dmin = ORACLE_INF;
+                for (int32_t p = p0; p < p1; ++p) {
+                    const int32_t d =
+                        group_distance(q_b + (int64_t)h * G * q_stride_h, q_stride_h, G,
+                                       kc + pb * ks_block + (p - p0) * ks_token + h * ks_head, Wd);
+                    if (d < dmin) dmin = d;
+                }
+                best = full - dmin;
+            }
+            s[(int64_t)h * nblk + j] = best;
+        }
+    }
+}
+
+static void topk_one(const uint32_t* q_b, int64_t q_stride_h, const uint32_t* kc, int64_t NB,
+                     int32_t BS, int32_t Hkv, int32_t Wd, int64_t ks_block, int64_t ks_token,
+                     int64_t ks_head, const int32_t* table_b, int64_t contiguous_base,
+                     int32_t len, int32_t max_blocks, int32_t Hq, int32_t k, int32_t sink,
+                     int32_t recent, uint32_t flags, int32_t* out_idx_b, int32_t* out_score_b)
+{
+    const int32_t G = Hq / Hkv;
+    const int32_t full = G * 32 * Wd;
+    const int32_t Ho = (flags & F_REDUCE_HEADS) ? 1 : Hkv;
+    int32_t nblk = len > 0 ? (len + BS - 1) / BS : 0;
+    if (nblk > max_blocks) nblk = max_blocks;
+    for (int32_t i = 0; i < Ho * k; ++i) {
+        out_idx_b[i] = -1;
+        if (out_score_b) out_score_b[i] = 0;
+    }
+    if (nblk == 0) return;
+    int32_t* s = (int32_t*)malloc(sizeof(int32_t) * (size_t)Hkv * (size_t)nblk);
+    cand_t* c = (cand_t*)malloc(sizeof(cand_t) * (size_t)nblk);
+    block_scores_one(q_b, q_stride_h, kc, NB, BS, Hkv, Wd, ks_block, ks_token, ks_head, table_b,
+                     contiguous_base, len, G, sink, recent, nblk, s);
+    for (int32_t ho = 0; ho < Ho; ++ho) {
+        for (int32_t j = 0; j < nblk; ++j) {
+            int32_t v;
+            if (flags & F_REDUCE_HEADS) {
+                v = s[j];
+                for (int32_t h = 1; h < Hkv; ++h)
+                    if (s[(int64_t)h * nblk + j] > v) v = s[(int64_t)h * nblk + j];
+            } else {
+                v = s[(int64_t)ho * nblk + j];
+            }
+            c[j].score = v;
+            c[j].idx = j;
+        }
+        const int32_t kk = k < nblk ? k : nblk;
+        qsort(c, (size_t)nblk, sizeof(cand_t), cand_cmp);
+        if (!(flags & F_SCORE_ORDER)) qsort(c, (size_t)kk, sizeof(cand_t), idx_cmp);
+        for (int32_t i = 0; i < kk; ++i) {
+            const int32_t j = c[i].idx;
+            out_idx_b[ho * k + i] =
+                (flags & F_PHYSICAL) ? (table_b ? table_b[j] : (int32_t)(contiguous_base + j)) : j;
+            if (out_score_b)
+                out_score_b[ho * k + i] = (flags & F_DISTANCE) ? full - c[i].score : c[i].score;
+        }
+    }
+    free(c);
+    free(s);
+}
+
+typedef struct {
+    const uint32_t* q;
+    int64_t q_stride_b, q_stride_h;
+    const uint32_t* kc;
+    int64_t NB;
+    int32_t BS, Hkv, Wd;
+    int64_t ks_block, ks_token, ks_head;
+    const int32_t* table;
+    int32_t table_stride, max_blocks;
+    const int32_t* lens;
+    int32_t B, Hq, k, sink, recent;
+    uint32_t flags;
+    int32_t* out_idx;
+    int32_t* out_score;
+    int32_t b0, b1;
+} topk_job_t;
+
+static void* topk_range(void* arg)
+{
+    topk_job_t* a = (topk_job_t*)arg;
+    const int32_t Ho = (a->flags & F_REDUCE_HEADS) ? 1 : a->Hkv;
+    for (int32_t b = a->b0; b < a->b1; ++b)
+        topk_one(a->q + b * a->q_stride_b, a->q_stride_h, a->kc, a->NB, a->BS, a->Hkv, a->Wd,
+                 a->ks_block, a->ks_token, a->ks_head,
+                 a->table ? a->table + (int64_t)b * a->table_stride : NULL,
+                 (int64_t)b * a->max_blocks, a->lens[b], a->max_blocks, a->Hq, a->k, a->sink,
+                 a->recent, a->flags, a->out_idx + (int64_t)b * Ho * a->k,
+                 a->out_score ? a->out_score + (int64_t)b * Ho * a->k : NULL);
+    return NULL;
+}
+
+/*
+ * Block top-k.  Follows hamming_topk.py:15-54 (block min, top-k, ascending sort, block
+ * table gather), paged_ham_dist_mla.cu:148-247 (group sum, masking, sink/recent, head
+ * reduce) and the ascending-index + table-map output of the NPU op
+ * (hamming_dist_top_k_base.h:307-347).  nthreads > 1 splits requests over pthreads
+ * (one request per thread at nthreads == B).
+ * out_idx / out_score: int32 [B, (reduce ? 1 : Hkv), k]; unused slots -1 / 0.
+ */
+void oracle_hamming_topk(const uint32_t* q, int64_t q_stride_b, int64_t q_stride_h,
+                         const uint32_t* kc, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
+                         int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                         const int32_t* table, int32_t table_stride, int32_t max_blocks,
+                         const int32_t* lens, int32_t B, int32_t Hq, int32_t k, int32_t sink,
+                         int32_t recent, uint32_t flags, int32_t* out_idx, int32_t* out_score,
+                         int32_t nthreads)
+{
+    topk_job_t base = {q,  q_stride_b, q_stride_h, kc,     NB,        BS,    Hkv,
+                       Wd, ks_block,   ks_token,   ks_head, table,     table_stride,
+                       max_blocks, lens, B, Hq, k, sink, recent, flags, out_idx, out_score, 0, B};
+    if (nthreads <= 1 || B <= 1) {
+        topk_range(&base);
+        return;
+    }
+    if (nthreads > B) nthreads = B;
+    pthread_t* th = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)nthreads);
+    topk_job_t* jobs = (topk_job_t*)malloc(sizeof(topk_job_t) * (size_t)nthreads);
+    for (int32_t i = 0; i < nthreads; ++i) {
+        jobs[i] = base;
+        jobs[i].b0 = (int32_t)((int64_t)B * i / nthreads);
+        jobs[i].b1 = (int32_t)((int64_t)B * (i + 1) / nthreads);
+        pthread_create(&th[i], NULL, topk_range, &jobs[i]);
+    }
+    for (int32_t i = 0; i < nthreads; ++i) pthread_join(th[i], NULL);
+    free(jobs);
+    free(th);
+}
+
+/*
+ * The CPU retrieval backend's form.  hash_retrieval_backend.cpp:321-407: for every row b
+ * and every allowed block index (entries == -1 removed, :241-246) the score is the min
+ * over ALL block_size tokens of popcount(q xor k) over dim bytes, starting from
+ * UINT16_MAX (:357-388, no masking); the top min(k, n_allowed) smallest scores are
+ * returned in ascending score order (:396-406).  Ties are broken here by position in the
+ * allowed list (the reference leaves them unspecified).
+ * data u8 [NB,BS,dim]; query u8 [B,dim]; indexes i32 [B,max_idx];
+ * out_idx/out_score i32 [B,k], unused slots -1 / 0.  out_n[b] = number of results.
+ */
+void oracle_hash_retrieval(const uint8_t* data, int64_t NB, int32_t BS, int32_t dim,
+                           const uint8_t* query, int32_t B, const int32_t* indexes,
+                           int32_t max_idx, int32_t k, int32_t* out_idx, int32_t* out_score,
+                           int32_t* out_n)
+{
+    (void)NB;
+    cand_t* c = (cand_t*)malloc(sizeof(cand_t) * (size_t)(max_idx > 0 ? max_idx : 1));
+    int32_t* blk = (int32_t*)malloc(sizeof(int32_t) * (size_t)(max_idx > 0 ? max_idx : 1));
+    for (int32_t b = 0; b < B; ++b) {
+        const uint8_t* qp = query + (int64_t)b * dim;
+        int32_t n = 0;
+        for (int32_t i = 0; i < max_idx; ++i) {
+            const int32_t idx = indexes[(int64_t)b * max_idx + i];
+            if (idx == -1) continue;
+            const uint8_t* base = data + (int64_t)idx * BS * dim;
+            int32_t score = 65535;
+            for (int32_t t = 0; t < BS; ++t) {
+                int32_t sum = 0;
+                for (int32_t d = 0; d < dim; ++d)
+                    sum += __builtin_popcount((unsigned)(qp[d] ^ base[(int64_t)t * dim + d]));
+                if (sum < score) {
+                    score = sum;
+                    if (score == 0) break;
+                }
+            }
+            /* cand_cmp sorts by score desc: store the negated distance, position as idx */
+            c[n].score = -score;
+            c[n].idx = n;
+            blk[n] = idx;
+            ++n;
+        }
+        const int32_t kk = k < n ? k : n;
+        qsort(c, (size_t)n, sizeof(cand_t), cand_cmp);
+        for (int32_t i = 0; i < k; ++i) {
+            out_idx[(int64_t)b * k + i] = i < kk ? blk[c[i].idx] : -1;
+            out_score[(int64_t)b * k + i] = i < kk ? -c[i].score : 0;
+        }
+        if (out_n) out_n[b] = kk;
+    }
+    free(blk);
+    free(c);
+}
+
+/* hamming_topk.py:7-12 (update_seq_lens). */
+void oracle_update_seq_lens(const int32_t* lens, int32_t B, int32_t topk_tok, int32_t BS,
+                            int32_t* out)
+{
+    for (int32_t b = 0; b < B; ++b) {
+        int32_t over = lens[b] - topk_tok;
+        if (over < 0) over = 0;
+        out[b] = lens[b] - ((over + BS - 1) / BS) * BS;
+    }
+}
+
+/* ------------------------------------------------------------------------------------
+ * Transfer.  ucm/shared/trans/cuda/cuda_stream.cc:63-80,110-127 and
+ * ucm/shared/trans/simu/simu_stream.cc:81-90,125-134: chunk i of `size` bytes.
+ * ------------------------------------------------------------------------------------ */
+void oracle_gather(const void* const* src, void* dst, size_t size, size_t number)
+{
+    for (size_t i = 0; i < number; ++i) memcpy((char*)dst + i * size, src[i], size);
+}
+void oracle_scatter(const void* src, void* const* dst, size_t size, size_t number)
+{
+    for (size_t i = 0; i < number; ++i) memcpy(dst[i], (const char*)src + i * size, size);
+}
+void oracle_batch(const void* const* src, void* const* dst, size_t size, size_t number)
+{
+    for (size_t i = 0; i < number; ++i) memcpy(dst[i], src[i], size);
+}
+
+/* ucm/integration/vllm/ucm_connector.py:135-148 (extract_block_addrs, block-first):
+ * out[blk, col] = base[col] + block_id[blk] * col_bytes[col]. */
+void oracle_block_addrs(const uint64_t* base, const uint64_t* col_bytes, int32_t n_cols,
+                        const int32_t* block_ids, int64_t n_blocks, uint64_t* out)
+{
+    for (int64_t i = 0; i < n_blocks; ++i)
+        for (int32_t c = 0; c < n_cols; ++c)
+            out[i * n_cols + c] = base[c] + (uint64_t)block_ids[i] * col_bytes[c];
+}
+
+/* Paged copy with per-column sizes: the flat buffer holds (block, col) row-major, column
+ * offsets accumulate (ucm/store/cache/cc/dump_queue.cc:145-161, load_queue.cc:178-194). */
+void oracle_paged_copy(const uint64_t* base, const uint64_t* col_bytes, int32_t n_cols,
+                       const int32_t* block_ids, int64_t n_blocks, void* flat, int to_cache)
+{
+    size_t off = 0;
+    for (int64_t i = 0; i < n_blocks; ++i)
+        for (int32_t c = 0; c < n_cols; ++c) {
+            void* p = (void*)(uintptr_t)(base[c] + (uint64_t)block_ids[i] * col_bytes[c]);
+            if (to_cache)
+                memcpy(p, (char*)flat + off, (size_t)col_bytes[c]);
+            else
+                memcpy((char*)flat + off, p, (size_t)col_bytes[c]);
+            off += (size_t)col_bytes[c];
+        }
+}
