@@ -1,0 +1,202 @@
+"""GPU parity: the HIP sign-hash encoder against the CPU oracle.
+
+Tolerance rule (the only floating-point tolerance in the suite): a hash bit may differ from
+the oracle only where |projection| < 1e-2 * ||x||; everywhere else it must be identical.
+The oracle used for the comparison accumulates in float64.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import rng_for
+from oracle import brute, c_api
+
+pytestmark = pytest.mark.gpu
+
+MARGIN_TOL = 1e-2
+
+
+def bf16_round(a):
+    return torch.from_numpy(np.asarray(a, np.float32)).to(torch.bfloat16)
+
+
+def assert_codes_match(codes_u8, x32, W32):
+    """codes_u8 [M, N/8] from the GPU; x32 [M,K], W32 [K,N] the exact values the GPU saw."""
+    ref = brute.hash_encode(x32, W32).view(np.uint8)
+    got = np.ascontiguousarray(codes_u8)
+    if np.array_equal(got, ref):
+        return 0
+    diff_bits = np.unpackbits(got ^ ref, axis=-1, bitorder="little").astype(bool)
+    marg = brute.margins(x32, W32)
+    assert not np.any(diff_bits & (marg >= MARGIN_TOL)), "bit flipped outside the margin"
+    return int(diff_bits.sum())
+
+
+def make_encoder(K, N, dtype, W, n_w=1, hpw=1):
+    from ucm_amd.sparse import HashEncoder
+
+    enc = HashEncoder(K, N, dtype, torch.device("cuda:0"), num_weights=n_w, heads_per_weight=hpw)
+    enc.set_hash_weight(W.to(dtype).cuda())
+    return enc
+
+
+def test_bit_and_byte_order_with_identity_weights():
+    K = N = 128
+    enc = make_encoder(K, N, torch.bfloat16, torch.eye(K))
+    x = torch.zeros(5, K)
+    x[0, 0] = 1.0
+    x[1, 9] = 2.0
+    x[2, 37] = 0.5
+    x[2, 3] = -1.0
+    x[3, 127] = 3.0
+    x[4, :] = -1.0
+    codes = enc.compute_hash(x.to(torch.bfloat16).cuda()).cpu().numpy()
+    words = np.ascontiguousarray(codes).view("<u4")
+    assert words[0].tolist() == [1, 0, 0, 0]
+    assert words[1].tolist() == [1 << 9, 0, 0, 0]
+    assert words[2].tolist() == [0, 1 << 5, 0, 0]
+    assert words[3].tolist() == [0, 0, 0, 1 << 31]
+    assert words[4].tolist() == [0, 0, 0, 0]
+    assert codes[1, 1] == 2  # byte 1, bit 1
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K,N", [(1, 128, 128), (33, 128, 128), (300, 128, 128),
+                                   (70, 64, 64), (40, 256, 128), (50, 512, 256), (17, 128, 96)])
+def test_compute_hash_matches_oracle(dtype, M, K, N):
+    rng = rng_for(1000 + M + K + N)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    W = torch.from_numpy(rng.standard_normal((K, N)).astype(np.float32)).to(dtype)
+    enc = make_encoder(K, N, dtype, W)
+    codes = enc.compute_hash(x.cuda())
+    assert codes.dtype == torch.uint8 and tuple(codes.shape) == (M, N // 8)
+    assert_codes_match(codes.cpu().numpy(), x.float().numpy(), W.float().numpy())
+
+
+def test_leading_dims_and_negation():
+    rng = rng_for(7)
+    x = bf16_round(rng.standard_normal((3, 5, 128)))
+    W = bf16_round(rng.standard_normal((128, 128)))
+    enc = make_encoder(128, 128, torch.bfloat16, W)
+    c = enc.compute_hash(x.cuda())
+    assert tuple(c.shape) == (3, 5, 16)
+    cn = enc.compute_hash((-x).cuda())
+    assert torch.equal(cn, ~c)  # no projection is exactly zero for Gaussian data
+
+
+def test_zero_and_nan_rows_give_zero_bits():
+    enc = make_encoder(128, 128, torch.bfloat16, torch.eye(128))
+    x = torch.zeros(2, 128)
+    x[1, 2] = float("nan")
+    x[1, 5] = 1.0
+    c = enc.compute_hash(x.to(torch.bfloat16).cuda()).cpu().numpy()
+    assert not c.any()
+
+
+def test_per_head_weights_gqa_queries():
+    """BASELINE config 2 query side: 32 q heads, one projection per KV head (group of 4)."""
+    rng = rng_for(8)
+    B, Hq, Hkv, K, N = 6, 32, 8, 128, 128
+    x = bf16_round(rng.standard_normal((B, Hq, K)))
+    W = bf16_round(rng.standard_normal((Hkv, K, N)))
+    enc = make_encoder(K, N, torch.bfloat16, W, n_w=Hkv, hpw=Hq // Hkv)
+    c = enc.compute_hash(x.cuda(), per_head=True).cpu().numpy()
+    assert c.shape == (B, Hq, N // 8)
+    for h in range(Hq):
+        assert_codes_match(c[:, h], x[:, h].float().numpy(), W[h // 4].float().numpy())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("slot_dtype", [torch.int32, torch.int64])
+def test_compute_hash_and_cache(dtype, slot_dtype):
+    rng = rng_for(9)
+    T, H, K, N, NB, BS = 200, 8, 128, 128, 6, 128
+    x = torch.from_numpy(rng.standard_normal((T, H, K)).astype(np.float32)).to(dtype)
+    W = torch.from_numpy(rng.standard_normal((H, K, N)).astype(np.float32)).to(dtype)
+    slots = rng.permutation(NB * BS)[:T].astype(np.int64)
+    slots[5] = -1
+    slots[17] = NB * BS          # first slot past the cache
+    slots[40] = NB * BS + 1000
+    enc = make_encoder(K, N, dtype, W, n_w=H, hpw=1)
+    cache = torch.full((NB, BS, H, N // 8), 0xAB, dtype=torch.uint8, device="cuda")
+    out = enc.compute_hash_and_cache(x.cuda(), torch.from_numpy(slots).to(slot_dtype).cuda(),
+                                     cache, block_size=BS)
+    assert out is cache
+    got = cache.cpu().numpy()
+    # fused write == separate encode + the oracle's scatter (hash_encoder.py:136-195)
+    codes = enc.compute_hash(x.cuda(), per_head=True).cpu().numpy()  # [T,H,16]
+    expect = np.full((NB, BS, H, N // 32), 0xABABABAB, np.uint32)
+    c_api.code_scatter(np.ascontiguousarray(codes).view(np.uint32), slots, expect, BS)
+    assert np.array_equal(got.view(np.uint32), expect)
+    for h in range(H):
+        assert_codes_match(codes[:, h], x[:, h].float().numpy(), W[h].float().numpy())
+
+
+def test_cache_as_bf16_view_and_shared_weight():
+    """The plugin allocates the code cache as bfloat16 [NB,BS,H,hash_numbers/2]
+    (hash_encoder.py:509-546) and uses one projection for all heads."""
+    rng = rng_for(10)
+    T, H, K, N, NB, BS = 64, 4, 128, 128, 2, 64
+    x = bf16_round(rng.standard_normal((T, H, K)))
+    W = bf16_round(rng.standard_normal((K, N)))
+    enc = make_encoder(K, N, torch.bfloat16, W)
+    cache = torch.zeros((NB, BS, H, N // 16), dtype=torch.bfloat16, device="cuda")
+    slots = torch.arange(T, dtype=torch.int64, device="cuda") + 10
+    enc.compute_hash_and_cache(x.cuda(), slots, cache, block_size=BS)
+    got = cache.view(torch.uint8).cpu().numpy().reshape(NB * BS, H, N // 8)
+    for h in range(H):
+        assert_codes_match(got[10:10 + T, h], x[:, h].float().numpy(), W.float().numpy())
+    assert not got[:10].any() and not got[10 + T:].any()
+
+
+def test_reshape_and_cache_head_major_shape_of_the_reference_fixture():
+    """Shapes of ucm/sparse/test/gsa/pt/npu_reshape_and_cache_bnsd_tensor.pt (that file holds
+    inputs only): 1 token, 2 heads, 16-byte codes, slot 22552, head-major cache
+    [402, 2, 128, 16].  Data here is synthetic."""
+    from ucm_amd.sparse.hash_encoder import reshape_and_cache_khash
+
+    rng = rng_for(11)
+    codes = torch.from_numpy(rng.integers(0, 256, size=(1, 2, 16), dtype=np.uint8)).cuda()
+    cache_hm = torch.zeros((402, 2, 128, 16), dtype=torch.uint8, device="cuda")
+    slot = torch.tensor([22552], dtype=torch.int32, device="cuda")
+    # token-major view [NB, BS, H, W] of the head-major storage
+    reshape_and_cache_khash(codes, slot, cache_hm.permute(0, 2, 1, 3), block_size=128)
+    got = cache_hm.cpu().numpy()
+    assert np.array_equal(got[176, :, 24, :], codes[0].cpu().numpy())
+    got[176, :, 24, :] = 0
+    assert not got.any()
+
+
+def test_argument_errors_match_the_reference_behaviour():
+    from ucm_amd.sparse import HashEncoder
+
+    with pytest.raises(ValueError):
+        HashEncoder(128, 100, torch.bfloat16, torch.device("cuda:0"))
+    enc = HashEncoder(128, 128, torch.bfloat16, torch.device("cuda:0"))
+    with pytest.raises(ValueError):
+        enc.compute_hash(torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        enc.compute_hash(torch.zeros(4, 128, dtype=torch.bfloat16))  # wrong device
+    with pytest.raises(ValueError):
+        enc.set_hash_weight(torch.zeros(128, 64, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        enc.set_hash_weight(torch.zeros(128, 128, dtype=torch.float32, device="cuda"))
+    cache = torch.zeros((2, 64, 4, 16), dtype=torch.uint8, device="cuda")
+    x = torch.zeros(3, 4, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        enc.compute_hash_and_cache(x, torch.zeros(2, dtype=torch.int64, device="cuda"), cache, 64)
+    with pytest.raises(ValueError):
+        enc.compute_hash_and_cache(x, torch.zeros(3, dtype=torch.int64, device="cuda"), cache, 128)
+    # Haar-orthogonal default weights: W^T W = I
+    w = enc.hash_weights.float()
+    assert torch.allclose(w.T @ w, torch.eye(128, device="cuda"), atol=5e-2)
+
+
+def test_unpack_hash_roundtrip():
+    enc = make_encoder(128, 128, torch.bfloat16, torch.eye(128))
+    x = torch.zeros(2, 128)
+    x[0, 3] = 1.0
+    x[1, 100] = 1.0
+    c = enc.compute_hash(x.to(torch.bfloat16).cuda())
+    pm = enc._unpack_hash(c).cpu()
+    assert pm[0, 3] == 1 and pm[1, 100] == 1 and pm.sum() == 2 - (256 - 2)

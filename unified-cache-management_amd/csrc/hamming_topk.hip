@@ -1,0 +1,775 @@
+// Hamming scorer + deterministic block top-k for gfx950.
+//
+// Three kernels per call:
+//   1. (group size > 4 only) plane_kernel: the G query codes of one KV head are reduced to
+//      per-bit counts c_b, stored as binary bit planes, so that the group-summed distance of
+//      a cached code k is   sum_b c_b + G*popc(k) - 2 * sum_p 2^p * popc(k & plane_p)
+//      — exact integer arithmetic, 2*P+1 ops per word instead of 2*G.
+//   2. block_score_*: every 16-byte piece of the paged code cache is read exactly once with
+//      128-bit loads (one wave = 1 KiB contiguous), XOR+popcount in registers, summed across
+//      the lanes that share a token, min-reduced per (block, KV head) with wave shuffles and
+//      LDS atomics.  Result: one int32 similarity per (request, KV head, logical block).
+//   3. select_kernel: per (request, KV head) an LDS radix search finds the k-th largest
+//      score, ties are resolved towards the lower block index by an ordered prefix sum, and
+//      the winners are compacted in ascending index order — no sort is needed for the
+//      default output order.
+//
+// Semantics follow ucm/sparse/gsa_on_device/hamming_topk.py:15-54 and
+// csrc/cuda/ham_dist/paged_ham_dist_mla.cu:148-247 of the reference (block min of the
+// group-summed distance, sink/recent keep, +inf past seq_len), in the similarity form of
+// its NPU op (csrc/ascend/hamming_dist_top_k/op_kernel/hamming_dist_top_k_base.h:150-347).
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWave = 64;
+constexpr int kInf = 0x7fffffff;
+constexpr int kMaxTileHeads = 1024;  // TB * Hkv bound of the LDS min table
+constexpr int kSelLdsCap = 8192;     // block scores kept in LDS by select_kernel
+constexpr int kSelSortCap = 2048;    // largest k for score-ordered output
+
+struct ScoreArgs {
+    const uint32_t* q;
+    int64_t q_stride_b, q_stride_h;
+    const uint32_t* kc;
+    int64_t NB;
+    int BS, Hkv, Wd;
+    int64_t ks_block, ks_token, ks_head;
+    const int32_t* table;
+    int table_stride, max_blocks;
+    const int32_t* lens;
+    int B, Hq, G, sink, recent;
+    int TB;                  // logical blocks per workgroup
+    const uint32_t* planes;  // [B][Hkv][PMAX][Wd], planes mode only
+    int32_t* scores;         // [B][Hkv][max_blocks]
+};
+
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int popc4(u32x4 v)
+{
+    return __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+}
+
+// Physical block of logical block j of request b, or -1 when the entry is unusable.
+__device__ __forceinline__ int64_t physical_block(const ScoreArgs& a, int b, int j)
+{
+    int64_t pb = a.table ? (int64_t)a.table[(int64_t)b * a.table_stride + j]
+                         : (int64_t)b * a.max_blocks + j;
+    return (pb < 0 || pb >= a.NB) ? -1 : pb;
+}
+
+__device__ __forceinline__ int num_blocks_of(const ScoreArgs& a, int len)
+{
+    int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
+    return n < a.max_blocks ? n : a.max_blocks;
+}
+
+// Writes the similarity of every (block, head) of the tile from the LDS min table.
+__device__ __forceinline__ void write_tile_scores(const ScoreArgs& a, int b, int j0, int nb_tile,
+                                                  int len, const int* smin)
+{
+    const int full = a.G * 32 * a.Wd;
+    for (int i = threadIdx.x; i < nb_tile * a.Hkv; i += kThreads) {
+        const int blk = i / a.Hkv, h = i % a.Hkv, j = j0 + blk;
+        const int p0 = j * a.BS;
+        const int p1 = (p0 + a.BS < len) ? p0 + a.BS : len;
+        const bool forced = (p0 < a.sink) || (p1 > len - a.recent);
+        int s;
+        if (physical_block(a, b, j) < 0) s = -1;
+        else if (forced) s = full;
+        else s = full - smin[i];
+        a.scores[((int64_t)b * a.Hkv + h) * a.max_blocks + j] = s;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Bit planes of the per-bit query counts (group size > 4).
+// planes[b][h][p][w] bit i  =  bit p of  #{ g : q[b, h*G+g, w] has bit i set }.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void plane_kernel(const uint32_t* __restrict__ q,
+                                                         int64_t q_stride_b, int64_t q_stride_h,
+                                                         int Hkv, int G, int Wd, int PMAX,
+                                                         uint32_t* __restrict__ planes)
+{
+    const int b = blockIdx.x / Hkv, h = blockIdx.x % Hkv;
+    const uint32_t* qb = q + b * q_stride_b + (int64_t)h * G * q_stride_h;
+    uint32_t* out = planes + ((int64_t)b * Hkv + h) * PMAX * Wd;
+    const int nbits = 32 * Wd;
+    for (int i0 = wave_id() * kWave; i0 < nbits; i0 += kThreads) {
+        const int i = i0 + lane_id();
+        int cnt = 0;
+        if (i < nbits) {
+            const int w = i >> 5, sh = i & 31;
+            for (int g = 0; g < G; ++g) cnt += (qb[g * q_stride_h + w] >> sh) & 1u;
+        }
+        for (int p = 0; p < PMAX; ++p) {
+            const unsigned long long m = __ballot((cnt >> p) & 1);
+            const int w0 = i0 >> 5;
+            if (lane_id() == 0 && w0 < Wd) out[p * Wd + w0] = (uint32_t)m;
+            if (lane_id() == 32 && w0 + 1 < Wd) out[p * Wd + w0 + 1] = (uint32_t)(m >> 32);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Fast block scorer.  Requirements (checked by the host): the [BS][Hkv][Wd] codes of a block
+// are contiguous, Wd = 4*CPU, Hkv*CPU divides 64, BS*Hkv*CPU is a multiple of 64, all
+// addresses 16-byte aligned.
+//   CPU   : 16-byte pieces per code (1, 2 or 4)
+//   DIRECT: true  -> G = GP query codes kept in registers, xor+popcount per query head
+//           false -> GP = PMAX bit planes in registers
+// A workgroup owns TB consecutive logical blocks of one request; lane l of the wave that
+// handles 64-piece run r reads piece r*64+l, so each load instruction covers 1 KiB of
+// contiguous memory.  (head, piece-in-code) of a lane never changes, so its query material
+// lives in registers for the whole kernel.
+// ---------------------------------------------------------------------------------------
+template <int CPU, bool DIRECT, int GP, int UNROLL>
+__global__ __launch_bounds__(kThreads) void block_score_fast(ScoreArgs a)
+{
+    __shared__ int smin[kMaxTileHeads];
+    const int b = blockIdx.y;
+    const int len = a.lens[b];
+    const int nblk = num_blocks_of(a, len);
+    const int j0 = blockIdx.x * a.TB;
+    if (j0 >= nblk) return;
+    const int nb_tile = (a.TB < nblk - j0) ? a.TB : nblk - j0;
+
+    for (int i = threadIdx.x; i < nb_tile * a.Hkv; i += kThreads) smin[i] = kInf;
+
+    const int period = a.Hkv * CPU;  // pieces per token
+    const int lane = lane_id();
+    const int lane_c = lane % period;
+    const int h = lane_c / CPU, part = lane_c % CPU;
+    const int period_shift = __builtin_ctz(period);
+
+    uint32_t qr[GP][4];
+    int ctot = 0;
+    if (DIRECT) {
+        const uint32_t* qp = a.q + b * a.q_stride_b + (int64_t)h * GP * a.q_stride_h + part * 4;
+#pragma unroll
+        for (int g = 0; g < GP; ++g)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[g][w] = qp[g * a.q_stride_h + w];
+    } else {
+        const uint32_t* pp = a.planes + ((int64_t)b * a.Hkv + h) * GP * a.Wd + part * 4;
+#pragma unroll
+        for (int p = 0; p < GP; ++p)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                qr[p][w] = pp[p * a.Wd + w];
+                ctot += __popc(qr[p][w]) << p;
+            }
+    }
+    __syncthreads();
+
+    const int CPB = a.BS * period;          // pieces per block, multiple of 64
+    const int runs = nb_tile * (CPB >> 6);  // 64-piece runs in the tile
+    const int runs_per_block = CPB >> 6;
+    const int wid = wave_id();
+
+    int cur_blk = -1;
+    int m = kInf;
+
+    auto flush = [&](int blk, int mm) {
+        for (int s = period; s < kWave; s <<= 1) {
+            const int o = __shfl_xor(mm, s);
+            mm = o < mm ? o : mm;
+        }
+        if (lane < period && part == 0) atomicMin(&smin[blk * a.Hkv + h], mm);
+    };
+
+    for (int r0 = wid; r0 < runs; r0 += 4 * UNROLL) {
+        u32x4 kv[UNROLL];
+        int blk_u[UNROLL];
+        int cc_u[UNROLL];
+        bool ok_u[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int r = r0 + 4 * u;
+            ok_u[u] = false;
+            blk_u[u] = 0;
+            cc_u[u] = 0;
+            kv[u] = (u32x4)(0u);
+            if (r < runs) {
+                const int blk = r / runs_per_block;
+                const int cc = (r - blk * runs_per_block) * 64 + lane;
+                const int64_t pb = physical_block(a, b, j0 + blk);
+                blk_u[u] = blk;
+                cc_u[u] = cc;
+                if (pb >= 0) {
+                    ok_u[u] = true;
+                    const u32x4* src =
+                        reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + cc;
+                    kv[u] = __builtin_nontemporal_load(src);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int r = r0 + 4 * u;
+            if (r >= runs) break;
+            if (blk_u[u] != cur_blk) {
+                if (cur_blk >= 0) flush(cur_blk, m);
+                cur_blk = blk_u[u];
+                m = kInf;
+            }
+            if (!ok_u[u]) continue;
+            int d;
+            if (DIRECT) {
+                d = 0;
+#pragma unroll
+                for (int g = 0; g < GP; ++g)
+                    d += __popc(kv[u].x ^ qr[g][0]) + __popc(kv[u].y ^ qr[g][1]) +
+                         __popc(kv[u].z ^ qr[g][2]) + __popc(kv[u].w ^ qr[g][3]);
+            } else {
+                int acc = 0;
+#pragma unroll
+                for (int p = 0; p < GP; ++p)
+                    acc += (__popc(kv[u].x & qr[p][0]) + __popc(kv[u].y & qr[p][1]) +
+                            __popc(kv[u].z & qr[p][2]) + __popc(kv[u].w & qr[p][3]))
+                           << p;
+                d = ctot + a.G * popc4(kv[u]) - 2 * acc;
+            }
+            if (CPU >= 2) d += __shfl_xor(d, 1);
+            if (CPU >= 4) d += __shfl_xor(d, 2);
+            const int t = cc_u[u] >> period_shift;
+            const int pos = (j0 + blk_u[u]) * a.BS + t;
+            if (pos < len && d < m) m = d;
+        }
+    }
+    if (cur_blk >= 0) flush(cur_blk, m);
+    __syncthreads();
+    write_tile_scores(a, b, j0, nb_tile, len, smin);
+}
+
+// ---------------------------------------------------------------------------------------
+// Generic block scorer: any strides, code width, head count and group size.  One thread per
+// (token, head) code, word-by-word loads; query codes staged in LDS.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void block_score_generic(ScoreArgs a)
+{
+    extern __shared__ uint32_t dyn[];
+    __shared__ int smin[kMaxTileHeads];
+    uint32_t* qs = dyn;  // [Hq][Wd]
+    const int b = blockIdx.y;
+    const int len = a.lens[b];
+    const int nblk = num_blocks_of(a, len);
+    const int j0 = blockIdx.x * a.TB;
+    if (j0 >= nblk) return;
+    const int nb_tile = (a.TB < nblk - j0) ? a.TB : nblk - j0;
+
+    for (int i = threadIdx.x; i < nb_tile * a.Hkv; i += kThreads) smin[i] = kInf;
+    for (int i = threadIdx.x; i < a.Hq * a.Wd; i += kThreads)
+        qs[i] = a.q[b * a.q_stride_b + (int64_t)(i / a.Wd) * a.q_stride_h + (i % a.Wd)];
+    __syncthreads();
+
+    const int units = a.BS * a.Hkv;
+    for (int blk = 0; blk < nb_tile; ++blk) {
+        const int64_t pb = physical_block(a, b, j0 + blk);
+        if (pb < 0) continue;
+        const uint32_t* base = a.kc + pb * a.ks_block;
+        for (int u = threadIdx.x; u < units; u += kThreads) {
+            const int t = u / a.Hkv, h = u % a.Hkv;
+            if ((j0 + blk) * a.BS + t >= len) continue;
+            const uint32_t* kp = base + t * a.ks_token + h * a.ks_head;
+            int d = 0;
+            for (int w = 0; w < a.Wd; ++w) {
+                const uint32_t kw = kp[w];
+                for (int g = 0; g < a.G; ++g) d += __popc(kw ^ qs[(h * a.G + g) * a.Wd + w]);
+            }
+            atomicMin(&smin[blk * a.Hkv + h], d);
+        }
+    }
+    __syncthreads();
+    write_tile_scores(a, b, j0, nb_tile, len, smin);
+}
+
+// ---------------------------------------------------------------------------------------
+// Selection.
+// ---------------------------------------------------------------------------------------
+struct SelectArgs {
+    const int32_t* scores;  // [B][Hkv][max_blocks]
+    int32_t* reduced;       // [B][max_blocks] scratch for head-reduced rows beyond the LDS cap
+    const int32_t* table;
+    int table_stride, max_blocks;
+    const int32_t* lens;
+    int BS, Hkv, Ho, k, full, key_bits;
+    uint32_t flags;
+    int32_t* out_idx;    // [B][Ho][k]
+    int32_t* out_score;  // may be null
+};
+
+// Exclusive prefix sum of one int per thread over the 256-thread workgroup; *total gets the
+// sum.  `wsum` is a 4-entry LDS array.
+__device__ __forceinline__ int block_exclusive_scan(int v, int* wsum, int* total)
+{
+    int inc = v;
+#pragma unroll
+    for (int s = 1; s < kWave; s <<= 1) {
+        const int o = __shfl_up(inc, s);
+        if (lane_id() >= s) inc += o;
+    }
+    __syncthreads();  // protects wsum from the previous use
+    if (lane_id() == kWave - 1) wsum[threadIdx.x >> 6] = inc;
+    __syncthreads();
+    int base = 0;
+    const int w = threadIdx.x >> 6;
+    for (int i = 0; i < w; ++i) base += wsum[i];
+    *total = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+    return base + inc - v;
+}
+
+__global__ __launch_bounds__(kThreads) void select_kernel(SelectArgs a)
+{
+    __shared__ int sbuf[kSelLdsCap];
+    __shared__ int hist[256];
+    __shared__ int wsum[4];
+    __shared__ int sh_digit, sh_need;
+    __shared__ int sel_idx[kSelSortCap];
+    __shared__ int sel_key[kSelSortCap];
+
+    const int b = blockIdx.x / a.Ho, ho = blockIdx.x % a.Ho;
+    const int tid = threadIdx.x;
+    const int len = a.lens[b];
+    int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
+    if (n > a.max_blocks) n = a.max_blocks;
+    int32_t* oi = a.out_idx + ((int64_t)b * a.Ho + ho) * a.k;
+    int32_t* os = a.out_score ? a.out_score + ((int64_t)b * a.Ho + ho) * a.k : nullptr;
+    const int kk = a.k < n ? a.k : n;
+
+    for (int i = kk + tid; i < a.k; i += kThreads) {
+        oi[i] = -1;
+        if (os) os[i] = 0;
+    }
+    if (n == 0) return;
+
+    // stage the row (reduced over heads when asked) where every pass can re-read it
+    const bool reduce = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
+    const int32_t* row = a.scores + ((int64_t)b * a.Hkv + (reduce ? 0 : ho)) * a.max_blocks;
+    const int* s;
+    if (n <= kSelLdsCap) {
+        for (int j = tid; j < n; j += kThreads) {
+            int v = row[j];
+            if (reduce)
+                for (int h = 1; h < a.Hkv; ++h) {
+                    const int o = row[(int64_t)h * a.max_blocks + j];
+                    v = o > v ? o : v;
+                }
+            sbuf[j] = v;
+        }
+        s = sbuf;
+    } else if (reduce) {
+        int32_t* red = a.reduced + (int64_t)b * a.max_blocks;
+        for (int j = tid; j < n; j += kThreads) {
+            int v = row[j];
+            for (int h = 1; h < a.Hkv; ++h) {
+                const int o = row[(int64_t)h * a.max_blocks + j];
+                v = o > v ? o : v;
+            }
+            red[j] = v;
+        }
+        __threadfence_block();
+        s = red;
+    } else {
+        s = row;
+    }
+    __syncthreads();
+
+    // ---- radix search for the kk-th largest key (key = score + 1 >= 0) ----
+    uint32_t prefix = 0;  // decided high digits
+    int need = kk;        // how many still to take among keys matching the prefix
+    int shift = ((a.key_bits + 7) / 8) * 8;
+    while (shift > 0) {
+        shift -= 8;
+        hist[tid] = 0;
+        __syncthreads();
+        for (int j = tid; j < n; j += kThreads) {
+            const uint32_t key = (uint32_t)(s[j] + 1);
+            if ((key >> (shift + 8)) == prefix) atomicAdd(&hist[(key >> shift) & 255], 1);
+        }
+        __syncthreads();
+        if (tid < kWave) {
+            // lane l owns digits 255-4l .. 252-4l (descending), so an inclusive scan over
+            // lanes walks the digits from the largest down
+            const int d0 = 255 - 4 * tid;
+            const int c0 = hist[d0], c1 = hist[d0 - 1], c2 = hist[d0 - 2], c3 = hist[d0 - 3];
+            const int mine = c0 + c1 + c2 + c3;
+            int inc = mine;
+#pragma unroll
+            for (int st = 1; st < kWave; st <<= 1) {
+                const int o = __shfl_up(inc, st);
+                if (tid >= st) inc += o;
+            }
+            const int above = inc - mine;  // keys with a larger digit than any of mine
+            if (above < need && need <= inc) {
+                int acc = above, digit = d0, cnt = c0;
+                if (acc + cnt < need) { acc += cnt; digit = d0 - 1; cnt = c1; }
+                if (acc + cnt < need) { acc += cnt; digit = d0 - 2; cnt = c2; }
+                if (acc + cnt < need) { acc += cnt; digit = d0 - 3; cnt = c3; }
+                sh_digit = digit;
+                sh_need = need - acc;
+            }
+        }
+        __syncthreads();
+        prefix = (prefix << 8) | (uint32_t)sh_digit;
+        need = sh_need;
+        __syncthreads();
+    }
+    const int thr = (int)prefix - 1;  // threshold score; `need` ties at thr are taken
+
+    // ---- ordered compaction: thread t owns indices [t*E, (t+1)*E) ----
+    const int E = (n + kThreads - 1) / kThreads;
+    const int jb = tid * E;
+    const int je = (jb + E < n) ? jb + E : n;
+    int eq = 0, gt = 0;
+    for (int j = jb; j < je; ++j) {
+        const int v = s[j];
+        eq += (v == thr);
+        gt += (v > thr);
+    }
+    int tot;
+    const int eq_before = block_exclusive_scan(eq, wsum, &tot);
+    int eq_take = need - eq_before;
+    eq_take = eq_take < 0 ? 0 : (eq_take > eq ? eq : eq_take);
+    int pos = block_exclusive_scan(gt + eq_take, wsum, &tot);
+
+    const bool score_order = (a.flags & UCM_TOPK_SCORE_ORDER) != 0;
+    int eq_seen = 0;
+    for (int j = jb; j < je; ++j) {
+        const int v = s[j];
+        bool take = v > thr;
+        if (v == thr) {
+            take = eq_seen < eq_take;
+            ++eq_seen;
+        }
+        if (!take || pos >= a.k) continue;
+        if (score_order) {
+            sel_idx[pos] = j;
+            sel_key[pos] = v;
+        } else {
+            oi[pos] = (a.flags & UCM_TOPK_RETURN_PHYSICAL)
+                          ? (a.table ? a.table[(int64_t)b * a.table_stride + j]
+                                     : b * a.max_blocks + j)
+                          : j;
+            if (os) os[pos] = (a.flags & UCM_TOPK_DISTANCE) ? a.full - v : v;
+        }
+        ++pos;
+    }
+    if (!score_order) return;
+
+    // ---- score order: rank by counting among the kk winners (index order breaks ties;
+    // sel_idx is ascending, so "earlier position" == "lower index") ----
+    __syncthreads();
+    for (int i = tid; i < kk; i += kThreads) {
+        const int v = sel_key[i];
+        int rank = 0;
+        for (int m = 0; m < kk; ++m) {
+            const int o = sel_key[m];
+            rank += (o > v) || (o == v && m < i);
+        }
+        const int j = sel_idx[i];
+        oi[rank] = (a.flags & UCM_TOPK_RETURN_PHYSICAL)
+                       ? (a.table ? a.table[(int64_t)b * a.table_stride + j] : b * a.max_blocks + j)
+                       : j;
+        if (os) os[rank] = (a.flags & UCM_TOPK_DISTANCE) ? a.full - v : v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Per-token scores in the reference scorer's output shape.
+// ---------------------------------------------------------------------------------------
+struct TokenArgs {
+    ScoreArgs s;
+    int max_seq_len, reduce_heads, out_is_f16;
+    void* out;
+};
+
+// fp16 accumulation exactly as paged_ham_dist_mla.cu:204-210,235-241: the code is cut into
+// 64-bit pieces when Wd is even (:384-387) and 32-bit pieces otherwise; each piece's
+// group-summed popcount is converted to half and added in half precision, piece 0 first.
+__global__ __launch_bounds__(kThreads) void token_score_kernel(TokenArgs t)
+{
+    extern __shared__ uint32_t dyn[];
+    const ScoreArgs& a = t.s;
+    uint32_t* qs = dyn;
+    const int b = blockIdx.y;
+    for (int i = threadIdx.x; i < a.Hq * a.Wd; i += kThreads)
+        qs[i] = a.q[b * a.q_stride_b + (int64_t)(i / a.Wd) * a.q_stride_h + (i % a.Wd)];
+    __syncthreads();
+    const int p = blockIdx.x * kThreads + threadIdx.x;
+    if (p >= t.max_seq_len) return;
+    const int len = a.lens[b];
+    const bool is_inf = p >= len;
+    const bool keep = (p < a.sink) || (p >= len - a.recent && p < len);
+    const int j = p / a.BS, tok = p % a.BS;
+    const int Ho = t.reduce_heads ? 1 : a.Hkv;
+    const int piece = (a.Wd % 2 == 0) ? 2 : 1;  // words per fp16 accumulation step
+
+    int red_i = kInf;
+    _Float16 red_h = (_Float16)__builtin_inff();
+    for (int h = 0; h < a.Hkv; ++h) {
+        int di = kInf;
+        _Float16 dh = (_Float16)__builtin_inff();
+        if (!is_inf) {
+            if (keep) {
+                di = 0;
+                dh = (_Float16)0.0f;
+            } else {
+                const int64_t pb = (j < a.max_blocks) ? physical_block(a, b, j) : -1;
+                if (pb >= 0) {
+                    const uint32_t* kp = a.kc + pb * a.ks_block + tok * a.ks_token + h * a.ks_head;
+                    di = 0;
+                    dh = (_Float16)0.0f;
+                    for (int w0 = 0; w0 < a.Wd; w0 += piece) {
+                        int part = 0;
+                        for (int w = w0; w < w0 + piece; ++w) {
+                            const uint32_t kw = kp[w];
+                            for (int g = 0; g < a.G; ++g)
+                                part += __popc(kw ^ qs[(h * a.G + g) * a.Wd + w]);
+                        }
+                        di += part;
+                        dh = dh + (_Float16)(float)part;
+                    }
+                }
+            }
+        }
+        if (t.reduce_heads) {
+            red_i = di < red_i ? di : red_i;
+            red_h = dh < red_h ? dh : red_h;
+        } else {
+            const int64_t o = ((int64_t)b * Ho + h) * t.max_seq_len + p;
+            if (t.out_is_f16) {
+                uint16_t u;
+                __builtin_memcpy(&u, &dh, 2);
+                ((uint16_t*)t.out)[o] = u;
+            } else {
+                ((int32_t*)t.out)[o] = di;
+            }
+        }
+    }
+    if (t.reduce_heads) {
+        const int64_t o = (int64_t)b * t.max_seq_len + p;
+        if (t.out_is_f16) {
+            uint16_t u;
+            __builtin_memcpy(&u, &red_h, 2);
+            ((uint16_t*)t.out)[o] = u;
+        } else {
+            ((int32_t*)t.out)[o] = red_i;
+        }
+    }
+}
+
+__global__ void update_seq_lens_kernel(const int32_t* lens, int B, int topk_tok, int BS,
+                                       int32_t* out)
+{
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    int over = lens[b] - topk_tok;
+    over = over < 0 ? 0 : over;
+    out[b] = lens[b] - ((over + BS - 1) / BS) * BS;
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+int planes_for_group(int G)
+{
+    int p = 0;
+    while ((1 << p) <= G) ++p;  // bit width of G
+    return p <= 4 ? 4 : 8;
+}
+
+struct Workspace {
+    int32_t* scores;
+    int32_t* reduced;
+    uint32_t* planes;
+    size_t bytes;
+};
+
+Workspace carve(void* base, int B, int Hkv, int max_blocks)
+{
+    Workspace w;
+    size_t off = 0;
+    w.scores = (int32_t*)((char*)base + off);
+    off += align_up((size_t)B * Hkv * max_blocks * 4, 256);
+    w.reduced = (int32_t*)((char*)base + off);
+    off += align_up((size_t)B * max_blocks * 4, 256);
+    w.planes = (uint32_t*)((char*)base + off);
+    // worst case: 8 planes, widest code handled by the plane path (16 words)
+    off += align_up((size_t)B * Hkv * 8 * 16 * 4, 256);
+    w.bytes = off;
+    return w;
+}
+
+template <int CPU, bool DIRECT, int GP>
+void launch_fast(const ScoreArgs& a, dim3 grid, hipStream_t st)
+{
+    hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 4>), grid, dim3(kThreads), 0, st, a);
+}
+
+template <int CPU>
+bool dispatch_fast(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+{
+    if (a.G == 1) launch_fast<CPU, true, 1>(a, grid, st);
+    else if (a.G == 2) launch_fast<CPU, true, 2>(a, grid, st);
+    else if (a.G == 4) launch_fast<CPU, true, 4>(a, grid, st);
+    else if (pmax == 4) launch_fast<CPU, false, 4>(a, grid, st);
+    else launch_fast<CPU, false, 8>(a, grid, st);
+    return true;
+}
+
+bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+int common_checks(const uint32_t* q, const uint32_t* kc, const int32_t* lens, int64_t NB, int BS,
+                  int Hkv, int Wd, int B, int Hq, int max_blocks)
+{
+    UCM_REQUIRE(q && kc && lens, "null input pointer");
+    UCM_REQUIRE(B >= 0 && B <= 65535, "batch %d out of range [0, 65535]", B);
+    UCM_REQUIRE(NB > 0 && BS > 0 && Hkv > 0 && Wd > 0 && Hq > 0, "non-positive shape");
+    UCM_REQUIRE(Hq % Hkv == 0, "query heads %d not a multiple of KV heads %d", Hq, Hkv);
+    UCM_REQUIRE(Hq / Hkv <= 255, "group size %d above 255", Hq / Hkv);
+    UCM_REQUIRE(max_blocks > 0, "max_blocks must be positive");
+    UCM_REQUIRE((int64_t)max_blocks * BS <= INT32_MAX, "max_blocks * BS overflows int32");
+    UCM_REQUIRE((int64_t)Hq * Wd * 4 <= 48 * 1024, "query codes of one request exceed 48 KiB");
+    return UCM_OK;
+}
+
+}  // namespace
+
+extern "C" size_t ucm_hamming_topk_workspace_bytes(int32_t B, int32_t Hkv, int32_t max_blocks)
+{
+    if (B <= 0 || Hkv <= 0 || max_blocks <= 0) return 256;
+    return carve(nullptr, B, Hkv, max_blocks).bytes;
+}
+
+extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                                const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
+                                int32_t Wd, int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                                const int32_t* block_table, int32_t table_stride,
+                                int32_t max_blocks, const int32_t* seq_lens, int32_t B,
+                                int32_t Hq, int32_t k, int32_t sink_tok, int32_t recent_tok,
+                                uint32_t flags, int32_t* out_idx, int32_t* out_score,
+                                void* workspace, size_t workspace_bytes, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    int rc = common_checks(q_codes, k_cache, seq_lens, NB, BS, Hkv, Wd, B, Hq, max_blocks);
+    if (rc != UCM_OK) return rc;
+    UCM_REQUIRE(out_idx, "out_idx is null");
+    UCM_REQUIRE(k > 0, "k must be positive");
+    UCM_REQUIRE(!block_table || table_stride >= max_blocks, "table_stride %d < max_blocks %d",
+                table_stride, max_blocks);
+    UCM_REQUIRE(sink_tok >= 0 && recent_tok >= 0, "negative sink/recent");
+    UCM_REQUIRE(Hkv <= kMaxTileHeads, "more than %d KV heads", kMaxTileHeads);
+    if ((flags & UCM_TOPK_SCORE_ORDER) && k > kSelSortCap)
+        return ucm::fail(UCM_EUNSUPPORTED, "score-ordered output supports k <= %d", kSelSortCap);
+    if (B == 0) return UCM_OK;
+    const Workspace ws = carve(workspace, B, Hkv, max_blocks);
+    UCM_REQUIRE(workspace && workspace_bytes >= ws.bytes, "workspace too small: %zu < %zu",
+                workspace_bytes, ws.bytes);
+    UCM_REQUIRE(((uintptr_t)workspace & 15) == 0, "workspace not 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+
+    ScoreArgs a;
+    a.q = q_codes; a.q_stride_b = q_stride_b; a.q_stride_h = q_stride_h;
+    a.kc = k_cache; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.Wd = Wd;
+    a.ks_block = ks_block; a.ks_token = ks_token; a.ks_head = ks_head;
+    a.table = block_table; a.table_stride = table_stride; a.max_blocks = max_blocks;
+    a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
+    a.recent = recent_tok; a.planes = ws.planes; a.scores = ws.scores;
+
+    // fast path eligibility
+    const int cpu = Wd / 4;
+    const bool fast = (Wd % 4 == 0) && (cpu == 1 || cpu == 2 || cpu == 4) && ks_head == Wd &&
+                      ks_token == (int64_t)Hkv * Wd && (ks_block % 4 == 0) &&
+                      (((uintptr_t)k_cache & 15) == 0) && is_pow2(Hkv * cpu) &&
+                      Hkv * cpu <= 64 && ((int64_t)BS * Hkv * cpu) % 64 == 0;
+    const int64_t block_bytes = (int64_t)BS * Hkv * Wd * 4;
+    int TB = (int)(16384 / block_bytes);
+    if (TB < 1) TB = 1;
+    while (TB > 1 && TB * Hkv > kMaxTileHeads) TB >>= 1;
+    // keep at least ~8 workgroups per CU in flight when the problem allows it
+    while (TB > 1 && (int64_t)B * ucm::ceil_div(max_blocks, TB) < 2048) TB >>= 1;
+    a.TB = TB;
+    const dim3 grid((unsigned)ucm::ceil_div(max_blocks, TB), (unsigned)B);
+
+    if (fast) {
+        const int pmax = planes_for_group(a.G);
+        const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
+        if (!direct) {
+            hipLaunchKernelGGL(plane_kernel, dim3(B * Hkv), dim3(kThreads), 0, st, q_codes,
+                               q_stride_b, q_stride_h, Hkv, a.G, Wd, pmax, ws.planes);
+            rc = ucm::launch_status("plane_kernel");
+            if (rc != UCM_OK) return rc;
+        }
+        if (cpu == 1) dispatch_fast<1>(a, pmax, grid, st);
+        else if (cpu == 2) dispatch_fast<2>(a, pmax, grid, st);
+        else dispatch_fast<4>(a, pmax, grid, st);
+    } else {
+        hipLaunchKernelGGL(block_score_generic, grid, dim3(kThreads), (size_t)Hq * Wd * 4, st, a);
+    }
+    rc = ucm::launch_status("block_score");
+    if (rc != UCM_OK) return rc;
+
+    SelectArgs s;
+    s.scores = ws.scores; s.reduced = ws.reduced; s.table = block_table;
+    s.table_stride = table_stride; s.max_blocks = max_blocks; s.lens = seq_lens; s.BS = BS;
+    s.Hkv = Hkv; s.Ho = (flags & UCM_TOPK_REDUCE_HEADS) ? 1 : Hkv; s.k = k;
+    s.full = a.G * 32 * Wd;
+    s.key_bits = 1;
+    while ((1ll << s.key_bits) <= (int64_t)s.full + 1) ++s.key_bits;
+    s.flags = flags; s.out_idx = out_idx; s.out_score = out_score;
+    hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
+    return ucm::launch_status("select_kernel");
+}
+
+extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                                 const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
+                                 int32_t Wd, int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                                 const int32_t* block_table, int32_t table_stride,
+                                 int32_t max_blocks, const int32_t* seq_lens, int32_t B,
+                                 int32_t Hq, int32_t max_seq_len, int32_t sink_tok,
+                                 int32_t recent_tok, int reduce_heads, void* out, int out_is_f16,
+                                 ucm_stream_t stream)
+{
+    ucm::clear_error();
+    int rc = common_checks(q_codes, k_cache, seq_lens, NB, BS, Hkv, Wd, B, Hq, max_blocks);
+    if (rc != UCM_OK) return rc;
+    UCM_REQUIRE(out, "out is null");
+    UCM_REQUIRE(max_seq_len > 0, "max_seq_len must be positive");
+    UCM_REQUIRE(!block_table || table_stride >= max_blocks, "table_stride %d < max_blocks %d",
+                table_stride, max_blocks);
+    if (B == 0) return UCM_OK;
+    TokenArgs t;
+    ScoreArgs& a = t.s;
+    a.q = q_codes; a.q_stride_b = q_stride_b; a.q_stride_h = q_stride_h;
+    a.kc = k_cache; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.Wd = Wd;
+    a.ks_block = ks_block; a.ks_token = ks_token; a.ks_head = ks_head;
+    a.table = block_table; a.table_stride = table_stride; a.max_blocks = max_blocks;
+    a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
+    a.recent = recent_tok; a.TB = 1; a.planes = nullptr; a.scores = nullptr;
+    t.max_seq_len = max_seq_len; t.reduce_heads = reduce_heads; t.out_is_f16 = out_is_f16;
+    t.out = out;
+    const dim3 grid((unsigned)ucm::ceil_div(max_seq_len, kThreads), (unsigned)B);
+    hipLaunchKernelGGL(token_score_kernel, grid, dim3(kThreads), (size_t)Hq * Wd * 4,
+                       (hipStream_t)stream, t);
+    return ucm::launch_status("token_score_kernel");
+}
+
+extern "C" int ucm_update_seq_lens(const int32_t* seq_lens, int32_t B, int32_t topk_tok,
+                                   int32_t BS, int32_t* out, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(seq_lens && out, "null pointer");
+    UCM_REQUIRE(BS > 0 && B >= 0, "bad sizes");
+    if (B == 0) return UCM_OK;
+    hipLaunchKernelGGL(update_seq_lens_kernel, dim3((unsigned)ucm::ceil_div(B, 256)), dim3(256), 0,
+                       (hipStream_t)stream, seq_lens, B, topk_tok, BS, out);
+    return ucm::launch_status("update_seq_lens_kernel");
+}

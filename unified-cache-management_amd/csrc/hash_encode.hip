@@ -1,0 +1,376 @@
+// Sign-hash encoder for gfx950: codes = pack_lsb_first(x . W > 0), optionally scattered into
+// the paged code cache.
+//
+// Follows the reference's HashEncoder (ucm/sparse/gsa_on_device/hash_encoder.py:359-370 for
+// the arithmetic and bit order, :263-356 for the fused cache write, :136-195 for the code
+// scatter).  Design for MI355X:
+//   * bf16 / fp16 inputs go through v_mfma_f32_32x32x16_{bf16,f16}: a wave owns 32 rows, keeps
+//     their K values in registers (A operand, one 16-byte load per lane and k-step) and walks
+//     the hash columns 32 at a time; the projection matrix slice lives in LDS, transposed so a
+//     B operand is one 16-byte LDS read;
+//   * the sign of an accumulator register is a v_cmp whose 64-bit lane mask already IS two
+//     packed output words (32 columns of two rows), so packing costs no shuffles;
+//   * the row's words are written with one store, either to a dense [T,H,Wd] tensor or to
+//     cache[slot/BS, slot%BS, h, :].
+// Everything else (fp32 operands, odd shapes, unaligned rows) takes a plain FMA kernel.
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kRowsPerWave = 32;
+constexpr int kRowsPerWg = 128;
+constexpr int kPad = 8;  // elements of padding per LDS row (16 bytes)
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+struct EncArgs {
+    const void* x;
+    int64_t T;
+    int H, K;
+    int64_t x_stride_t, x_stride_h;
+    const void* w;
+    int n_w, heads_per_w, N;
+    // dense output
+    uint32_t* out;
+    int64_t out_stride_t, out_stride_h;
+    // paged output (cache != null)
+    const void* slot;
+    int slot_is_i64;
+    uint32_t* cache;
+    int64_t NB;
+    int BS;
+    int64_t cs_block, cs_token, cs_head;
+    int BN;  // hash columns per workgroup slice
+};
+
+__device__ __forceinline__ int weight_index(const EncArgs& a, int h)
+{
+    int wi = a.heads_per_w > 0 ? h / a.heads_per_w : 0;
+    return wi < a.n_w ? wi : a.n_w - 1;
+}
+
+// Destination of the code words of row (t, h), or null when the row must be skipped.
+__device__ __forceinline__ uint32_t* row_dst(const EncArgs& a, int64_t t, int h)
+{
+    if (!a.cache) return a.out + t * a.out_stride_t + (int64_t)h * a.out_stride_h;
+    const int64_t s = a.slot_is_i64 ? ((const int64_t*)a.slot)[t] : (int64_t)((const int32_t*)a.slot)[t];
+    if (s < 0 || s >= a.NB * (int64_t)a.BS) return nullptr;
+    return a.cache + (s / a.BS) * a.cs_block + (s % a.BS) * a.cs_token + (int64_t)h * a.cs_head;
+}
+
+template <typename V>
+struct Mfma;
+template <>
+struct Mfma<bf16x8> {
+    static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma<f16x8> {
+    static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// V: 8-element vector type of the 16-bit input format.  KS = K / 16.
+// grid = (row-tile workers, column slices, heads); a workgroup loads its W slice into LDS once
+// and then walks row tiles of 128 rows (32 per wave) with a grid stride.
+template <typename V, int KS>
+__global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
+{
+    extern __shared__ uint16_t wt[];  // [BN][K + kPad], k contiguous
+    constexpr int K = KS * 16;
+    constexpr int KP = K + kPad;
+    const int h = blockIdx.z;
+    const int n0 = blockIdx.y * a.BN;
+    const int bn = (a.N - n0 < a.BN) ? a.N - n0 : a.BN;  // columns in this slice
+    const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N;
+
+    // W[k][n0 + 8j .. +8] -> wt[8j + i][k]
+    for (int idx = threadIdx.x; idx < K * (bn / 8); idx += kThreads) {
+        const int k = idx / (bn / 8), j = idx % (bn / 8);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(wsrc + (int64_t)k * a.N + n0 + 8 * j);
+        const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            wt[(8 * j + 2 * i) * KP + k] = (uint16_t)(wv[i] & 0xffffu);
+            wt[(8 * j + 2 * i + 1) * KP + k] = (uint16_t)(wv[i] >> 16);
+        }
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 31, kb = lane >> 5;
+    const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)h * a.x_stride_h;
+    const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
+    const int nt_count = bn / 32;
+    const int word0 = n0 / 32;
+
+    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const int64_t row0 = tile * kRowsPerWg + wave * kRowsPerWave;
+        if (row0 >= a.T) continue;
+        int64_t t = row0 + r;
+        const bool row_ok = t < a.T;
+        if (!row_ok) t = a.T - 1;  // read a valid row, discard its result
+        const uint16_t* xr = xbase + t * a.x_stride_t + kb * 8;
+        V av[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
+
+        uint32_t* dst = (row_ok && lane < 32) ? row_dst(a, t, h) : nullptr;
+
+        for (int nt0 = 0; nt0 < nt_count; nt0 += 4) {
+            uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nt = nt0 + q;
+                if (nt >= nt_count) break;
+                f32x16 acc = {0};
+                const uint16_t* bp = wt + (nt * 32 + r) * KP + kb * 8;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const V bv = *reinterpret_cast<const V*>(bp + ks * 16);
+                    acc = Mfma<V>::run(av[ks], bv, acc);
+                }
+                // accumulator v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
+                uint32_t word = 0;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const unsigned long long m = __ballot(acc[v] > 0.0f);
+                    const int r0 = 8 * (v / 4) + (v % 4);
+                    if (lane == r0) word = (uint32_t)m;
+                    if (lane == r0 + 4) word = (uint32_t)(m >> 32);
+                }
+                words[q] = word;
+            }
+            if (dst) {
+                const int nq = (nt_count - nt0 < 4) ? nt_count - nt0 : 4;
+                uint32_t* d = dst + word0 + nt0;
+                if (nq == 4 && (((uintptr_t)d) & 15) == 0) {
+                    u32x4 v = {words[0], words[1], words[2], words[3]};
+                    *reinterpret_cast<u32x4*>(d) = v;
+                } else {
+                    for (int q = 0; q < nq; ++q) d[q] = words[q];
+                }
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ float load_as_float(const void* p, int dtype, int64_t i)
+{
+    if (dtype == UCM_DT_F32) return ((const float*)p)[i];
+    if (dtype == UCM_DT_F16) return __half2float(((const __half*)p)[i]);
+    const uint32_t u = (uint32_t)((const uint16_t*)p)[i] << 16;
+    return __uint_as_float(u);
+}
+
+// Plain FMA path: one thread per (row, head, output word); fp32 accumulation in ascending k.
+__global__ __launch_bounds__(kThreads) void encode_fma_kernel(EncArgs a, int x_dtype, int w_dtype)
+{
+    const int Wd = a.N / 32;
+    const int64_t total = a.T * a.H * Wd;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * kThreads) {
+        const int w = (int)(i % Wd);
+        const int h = (int)((i / Wd) % a.H);
+        const int64_t t = i / ((int64_t)Wd * a.H);
+        uint32_t* dst = row_dst(a, t, h);
+        if (!dst) continue;
+        const int64_t xo = t * a.x_stride_t + (int64_t)h * a.x_stride_h;
+        const int64_t wo = (int64_t)weight_index(a, h) * a.K * a.N + w * 32;
+        float acc[32];
+#pragma unroll
+        for (int j = 0; j < 32; ++j) acc[j] = 0.0f;
+        for (int k = 0; k < a.K; ++k) {
+            const float xv = load_as_float(a.x, x_dtype, xo + k);
+#pragma unroll
+            for (int j = 0; j < 32; ++j)
+                acc[j] = __builtin_fmaf(xv, load_as_float(a.w, w_dtype, wo + (int64_t)k * a.N + j), acc[j]);
+        }
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) word |= (acc[j] > 0.0f ? 1u : 0u) << j;
+        dst[w] = word;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void code_scatter_kernel(const uint32_t* __restrict__ codes,
+                                                                int64_t T, int H, int Wd,
+                                                                int64_t in_stride_t,
+                                                                int64_t in_stride_h, EncArgs a)
+{
+    const int64_t total = T * H * Wd;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * kThreads) {
+        const int w = (int)(i % Wd);
+        const int h = (int)((i / Wd) % H);
+        const int64_t t = i / ((int64_t)Wd * H);
+        uint32_t* dst = row_dst(a, t, h);
+        if (dst) dst[w] = codes[t * in_stride_t + (int64_t)h * in_stride_h + w];
+    }
+}
+
+int num_cus()
+{
+    static int cached = 0;
+    if (cached) return cached;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        prop.multiProcessorCount > 0)
+        cached = prop.multiProcessorCount;
+    else
+        cached = 256;
+    return cached;
+}
+
+// Widest slice of hash columns (a multiple of 32 that divides N) whose transposed LDS image
+// stays within `cap` bytes; 0 when not even 32 columns fit.
+int pick_slice(int N, int K, size_t cap)
+{
+    for (int bn = N; bn >= 32; bn -= 32)
+        if (N % bn == 0 && (size_t)bn * (K + kPad) * 2 <= cap) return bn;
+    return 0;
+}
+
+template <typename V, int KS>
+int launch_mfma(EncArgs a, hipStream_t st)
+{
+    constexpr int K = KS * 16;
+    // 0 = not tried, 1 = large LDS allocations allowed, -1 = refused by the runtime
+    static int big_lds = 0;
+    a.BN = pick_slice(a.N, K, 144 * 1024);
+    if ((size_t)a.BN * (K + kPad) * 2 > 64 * 1024) {
+        if (big_lds == 0) {
+            const hipError_t e =
+                hipFuncSetAttribute((const void*)encode_mfma_kernel<V, KS>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+            if (e != hipSuccess) (void)hipGetLastError();
+            big_lds = (e == hipSuccess) ? 1 : -1;
+        }
+        if (big_lds < 0) a.BN = pick_slice(a.N, K, 64 * 1024);
+    }
+    if (a.BN == 0) return ucm::fail(UCM_EUNSUPPORTED, "no LDS slice fits K=%d", K);
+    const size_t lds = (size_t)a.BN * (K + kPad) * 2;
+    const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
+    const int slices = a.N / a.BN;
+    int64_t per = (int64_t)num_cus() * 2 / ((int64_t)slices * a.H);
+    if (per < 1) per = 1;
+    const dim3 grid((unsigned)(tiles < per ? tiles : per), (unsigned)slices, (unsigned)a.H);
+    hipLaunchKernelGGL((encode_mfma_kernel<V, KS>), grid, dim3(kThreads), lds, st, a);
+    return ucm::launch_status("encode_mfma_kernel");
+}
+
+template <typename V>
+int dispatch_mfma(const EncArgs& a, hipStream_t st)
+{
+    switch (a.K) {
+        case 64: return launch_mfma<V, 4>(a, st);
+        case 128: return launch_mfma<V, 8>(a, st);
+        case 256: return launch_mfma<V, 16>(a, st);
+        case 512: return launch_mfma<V, 32>(a, st);
+        default: return ucm::fail(UCM_ERROR, "internal: K %d has no MFMA kernel", a.K);
+    }
+}
+
+int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
+{
+    UCM_REQUIRE(a.x && a.w, "null input");
+    UCM_REQUIRE(a.T >= 0 && a.H > 0 && a.K > 0 && a.N > 0, "bad shape");
+    UCM_REQUIRE(a.H <= 65535, "more than 65535 heads");
+    UCM_REQUIRE(a.N % 32 == 0, "hash_bits %d must be a multiple of 32", a.N);
+    UCM_REQUIRE(a.n_w >= 1 && a.heads_per_w >= 0, "bad weight layout");
+    UCM_REQUIRE(x_dtype >= 0 && x_dtype <= 2 && w_dtype >= 0 && w_dtype <= 2, "unknown dtype");
+    if (a.T == 0) return UCM_OK;
+
+    const bool same16 = (x_dtype == w_dtype) && (x_dtype == UCM_DT_BF16 || x_dtype == UCM_DT_F16);
+    const bool k_ok = a.K == 64 || a.K == 128 || a.K == 256 || a.K == 512;
+    const bool aligned = (((uintptr_t)a.x | (uintptr_t)a.w) & 15) == 0 && a.x_stride_t % 8 == 0 &&
+                         a.x_stride_h % 8 == 0;
+    if (same16 && k_ok && aligned) {
+        return x_dtype == UCM_DT_BF16 ? dispatch_mfma<bf16x8>(a, st) : dispatch_mfma<f16x8>(a, st);
+    }
+    const int64_t total = a.T * a.H * (a.N / 32);
+    int64_t blocks = ucm::ceil_div(total, kThreads);
+    if (blocks > 65535 * 16) blocks = 65535 * 16;
+    hipLaunchKernelGGL(encode_fma_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, a, x_dtype,
+                       w_dtype);
+    return ucm::launch_status("encode_fma_kernel");
+}
+
+int check_cache(const void* slot, const uint32_t* cache, int64_t NB, int BS)
+{
+    UCM_REQUIRE(slot && cache, "null slot_mapping or cache");
+    UCM_REQUIRE(NB > 0 && BS > 0, "bad cache shape");
+    return UCM_OK;
+}
+
+}  // namespace
+
+extern "C" int ucm_hash_encode(const void* x, int x_dtype, int64_t T, int32_t H, int32_t K,
+                               int64_t x_stride_t, int64_t x_stride_h, const void* w, int w_dtype,
+                               int32_t n_w, int32_t heads_per_w, int32_t N_bits, uint32_t* out,
+                               int64_t out_stride_t, int64_t out_stride_h, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(out, "null output");
+    EncArgs a{};
+    a.x = x; a.T = T; a.H = H; a.K = K; a.x_stride_t = x_stride_t; a.x_stride_h = x_stride_h;
+    a.w = w; a.n_w = n_w; a.heads_per_w = heads_per_w; a.N = N_bits;
+    a.out = out; a.out_stride_t = out_stride_t; a.out_stride_h = out_stride_h;
+    return encode_common(a, x_dtype, w_dtype, (hipStream_t)stream);
+}
+
+extern "C" int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int32_t K,
+                                     int64_t x_stride_t, int64_t x_stride_h, const void* w,
+                                     int w_dtype, int32_t n_w, int32_t heads_per_w, int32_t N_bits,
+                                     const void* slot_mapping, int slot_is_i64, uint32_t* cache,
+                                     int64_t NB, int32_t BS, int64_t cs_block, int64_t cs_token,
+                                     int64_t cs_head, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    int rc = check_cache(slot_mapping, cache, NB, BS);
+    if (rc != UCM_OK) return rc;
+    EncArgs a{};
+    a.x = x; a.T = T; a.H = H; a.K = K; a.x_stride_t = x_stride_t; a.x_stride_h = x_stride_h;
+    a.w = w; a.n_w = n_w; a.heads_per_w = heads_per_w; a.N = N_bits;
+    a.slot = slot_mapping; a.slot_is_i64 = slot_is_i64; a.cache = cache; a.NB = NB; a.BS = BS;
+    a.cs_block = cs_block; a.cs_token = cs_token; a.cs_head = cs_head;
+    return encode_common(a, x_dtype, w_dtype, (hipStream_t)stream);
+}
+
+extern "C" int ucm_code_scatter(const uint32_t* codes, int64_t T, int32_t H, int32_t Wd,
+                                int64_t in_stride_t, int64_t in_stride_h, const void* slot_mapping,
+                                int slot_is_i64, uint32_t* cache, int64_t NB, int32_t BS,
+                                int64_t cs_block, int64_t cs_token, int64_t cs_head,
+                                ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(codes, "null codes");
+    UCM_REQUIRE(T >= 0 && H > 0 && Wd > 0, "bad shape");
+    int rc = check_cache(slot_mapping, cache, NB, BS);
+    if (rc != UCM_OK) return rc;
+    if (T == 0) return UCM_OK;
+    EncArgs a{};
+    a.slot = slot_mapping; a.slot_is_i64 = slot_is_i64; a.cache = cache; a.NB = NB; a.BS = BS;
+    a.cs_block = cs_block; a.cs_token = cs_token; a.cs_head = cs_head;
+    const int64_t total = T * H * Wd;
+    int64_t blocks = ucm::ceil_div(total, kThreads);
+    if (blocks > 65535 * 16) blocks = 65535 * 16;
+    hipLaunchKernelGGL(code_scatter_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
+                       (hipStream_t)stream, codes, T, (int)H, (int)Wd, in_stride_t, in_stride_h, a);
+    return ucm::launch_status("code_scatter_kernel");
+}

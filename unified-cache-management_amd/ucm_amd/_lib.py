@@ -1,0 +1,104 @@
+"""ctypes loader of libucm_hip.so and status-to-exception translation."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libucm_hip.so")
+
+UCM_OK = 0
+UCM_ERROR = -1
+UCM_EPARAM = -50000
+UCM_EOOM = -50001
+UCM_EUNSUPPORTED = -50008
+
+DT_BF16, DT_F16, DT_F32 = 0, 1, 2
+TOPK_REDUCE_HEADS, TOPK_RETURN_PHYSICAL, TOPK_SCORE_ORDER, TOPK_DISTANCE = 1, 2, 4, 8
+TRANS_CE, TRANS_SM = 0, 1
+
+_lib = None
+
+i32, i64, u32, u64 = C.c_int32, C.c_int64, C.c_uint32, C.c_uint64
+vp, sz, ci = C.c_void_p, C.c_size_t, C.c_int
+
+_SIGNATURES = {
+    "ucm_version": (ci, []),
+    "ucm_last_error": (C.c_char_p, []),
+    "ucm_hash_encode": (ci, [vp, ci, i64, i32, i32, i64, i64, vp, ci, i32, i32, i32, vp, i64, i64, vp]),
+    "ucm_hash_encode_cache": (ci, [vp, ci, i64, i32, i32, i64, i64, vp, ci, i32, i32, i32, vp, ci,
+                                   vp, i64, i32, i64, i64, i64, vp]),
+    "ucm_code_scatter": (ci, [vp, i64, i32, i32, i64, i64, vp, ci, vp, i64, i32, i64, i64, i64, vp]),
+    "ucm_hamming_topk_workspace_bytes": (sz, [i32, i32, i32]),
+    "ucm_hamming_topk": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
+                              vp, i32, i32, i32, i32, i32, u32, vp, vp, vp, sz, vp]),
+    "ucm_hamming_score": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
+                               vp, i32, i32, i32, i32, i32, ci, vp, ci, vp]),
+    "ucm_update_seq_lens": (ci, [vp, i32, i32, i32, vp, vp]),
+    "ucm_trans_setup": (ci, [i32]),
+    "ucm_trans_stream_create": (ci, [ci, C.POINTER(vp)]),
+    "ucm_trans_stream_destroy": (ci, [vp]),
+    "ucm_trans_stream_handle": (vp, [vp]),
+    "ucm_trans_stream_sync": (ci, [vp]),
+    "ucm_trans_stream_wait_event": (ci, [vp, vp]),
+    "ucm_trans_stream_append_callback": (ci, [vp, vp, vp]),
+    "ucm_trans_d2h": (ci, [vp, vp, vp, sz, ci]),
+    "ucm_trans_h2d": (ci, [vp, vp, vp, sz, ci]),
+    "ucm_trans_gather": (ci, [vp, vp, ci, vp, sz, sz, ci]),
+    "ucm_trans_scatter": (ci, [vp, vp, vp, ci, sz, sz, ci]),
+    "ucm_trans_batch": (ci, [vp, vp, vp, ci, sz, sz, ci]),
+    "ucm_trans_paged_copy": (ci, [vp, vp, vp, i32, vp, i64, vp, ci, ci]),
+    "ucm_trans_host_alloc": (ci, [sz, C.POINTER(vp)]),
+    "ucm_trans_host_free": (ci, [vp]),
+    "ucm_trans_device_alloc": (ci, [sz, C.POINTER(vp)]),
+    "ucm_trans_device_free": (ci, [vp]),
+    "ucm_trans_host_register": (ci, [vp, sz, C.POINTER(vp)]),
+    "ucm_trans_host_unregister": (ci, [vp]),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+
+def lib():
+    """The loaded library.  torch is imported first so that the HIP runtime it ships is the one
+    the library binds to.  Raises if the library has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python unified-cache-management_amd/build.py`"
+                " (there is no CPU fallback)")
+        import torch  # noqa: F401  (loads libamdhip64 before our library resolves it)
+
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def last_error():
+    return lib().ucm_last_error().decode("utf-8", "replace")
+
+
+def check(rc):
+    """Raise like the reference's bindings do: ValueError for parameter errors,
+    NotImplementedError for unsupported cases, RuntimeError otherwise
+    (ucm/shared/trans/cpy/trans.py.cc:35-38 turns a failed Status into RuntimeError)."""
+    if rc == UCM_OK:
+        return
+    msg = f"{rc}, {last_error()}"
+    if rc == UCM_EPARAM:
+        raise ValueError(msg)
+    if rc == UCM_EUNSUPPORTED:
+        raise NotImplementedError(msg)
+    if rc == UCM_EOOM:
+        raise MemoryError(msg)
+    raise RuntimeError(msg)
+
+
+def stream_ptr(device=None):
+    """hipStream_t of torch's current stream on `device` as an integer."""
+    import torch
+
+    return torch.cuda.current_stream(device).cuda_stream
