@@ -167,6 +167,14 @@ int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_str
                       void* out, int out_is_f16,
                       ucm_stream_t stream);
 
+/*
+ * Measurement hook, no counterpart in the reference.  When both events (hipEvent_t) are
+ * non-NULL, every following ucm_hamming_topk call on this thread records `before` right
+ * before and `after` right after its block-score kernel, on the call's stream, so a caller
+ * can time that kernel alone.  Pass NULLs to switch it off.
+ */
+int ucm_hamming_topk_set_profile_events(void* before, void* after);
+
 /* Replaces update_seq_lens (hamming_topk.py:7-12):
  * out[b] = len[b] - ceil(max(len[b] - topk_tok, 0) / BS) * BS. */
 int ucm_update_seq_lens(const int32_t* seq_lens, int32_t B, int32_t topk_tok, int32_t BS,

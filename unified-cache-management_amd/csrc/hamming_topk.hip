@@ -625,6 +625,9 @@ bool dispatch_fast(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
     return true;
 }
 
+thread_local hipEvent_t g_prof_before = nullptr;
+thread_local hipEvent_t g_prof_after = nullptr;
+
 bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
 int common_checks(const uint32_t* q, const uint32_t* kc, const int32_t* lens, int64_t NB, int BS,
@@ -699,6 +702,7 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     a.TB = TB;
     const dim3 grid((unsigned)ucm::ceil_div(max_blocks, TB), (unsigned)B);
 
+    const bool prof = g_prof_before && g_prof_after;
     if (fast) {
         const int pmax = planes_for_group(a.G);
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
@@ -708,12 +712,15 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             rc = ucm::launch_status("plane_kernel");
             if (rc != UCM_OK) return rc;
         }
+        if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_before, st));
         if (cpu == 1) dispatch_fast<1>(a, pmax, grid, st);
         else if (cpu == 2) dispatch_fast<2>(a, pmax, grid, st);
         else dispatch_fast<4>(a, pmax, grid, st);
     } else {
+        if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_before, st));
         hipLaunchKernelGGL(block_score_generic, grid, dim3(kThreads), (size_t)Hq * Wd * 4, st, a);
     }
+    if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_after, st));
     rc = ucm::launch_status("block_score");
     if (rc != UCM_OK) return rc;
 
@@ -727,6 +734,15 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     s.flags = flags; s.out_idx = out_idx; s.out_score = out_score;
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
     return ucm::launch_status("select_kernel");
+}
+
+extern "C" int ucm_hamming_topk_set_profile_events(void* before, void* after)
+{
+    ucm::clear_error();
+    UCM_REQUIRE((before == nullptr) == (after == nullptr), "pass both events or neither");
+    g_prof_before = (hipEvent_t)before;
+    g_prof_after = (hipEvent_t)after;
+    return UCM_OK;
 }
 
 extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "ucm_hamming_topk_workspace_bytes": (sz, [i32, i32, i32]),
     "ucm_hamming_topk": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
                               vp, i32, i32, i32, i32, i32, u32, vp, vp, vp, sz, vp]),
+    "ucm_hamming_topk_set_profile_events": (ci, [vp, vp]),
     "ucm_hamming_score": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
                                vp, i32, i32, i32, i32, i32, ci, vp, ci, vp]),
     "ucm_update_seq_lens": (ci, [vp, i32, i32, i32, vp, vp]),
@@ -102,3 +103,14 @@ def stream_ptr(device=None):
     import torch
 
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def stride(t, dim):
+    """Stride of `dim` in elements; a canonical (dense) value for extent-1 dimensions, whose
+    recorded stride is arbitrary."""
+    if t.shape[dim] > 1:
+        return t.stride(dim)
+    n = 1
+    for d in range(dim + 1, t.dim()):
+        n *= t.shape[d]
+    return n

@@ -46,7 +46,7 @@ def update_seq_lens(seq_lens, topk_token, block_size):
 
 
 def _cache_geometry(k_hash, head_major):
-    st = k_hash.stride()
+    st = [_lib.stride(k_hash, d) for d in range(4)]
     if st[3] != 1:
         raise ValueError("key codes must be contiguous in the last dimension")
     if head_major:
@@ -111,7 +111,7 @@ def hamming_topk(q_hash, k_hash, block_table, seq_lens, k_blocks, sink_token=0, 
         q_hash, k_hash, block_table, seq_lens, head_major)
     if block_table is not None:
         mb = block_table.shape[1] if max_blocks is None else int(max_blocks)
-        ts = block_table.stride(0)
+        ts = max(_lib.stride(block_table, 0), mb)
     else:
         if max_blocks is None:
             raise ValueError("max_blocks is required without a block table")
@@ -127,7 +127,7 @@ def hamming_topk(q_hash, k_hash, block_table, seq_lens, k_blocks, sink_token=0, 
     nbytes = L.ucm_hamming_topk_workspace_bytes(B, Hkv, mb)
     ws = _workspace(q.device, nbytes)
     _lib.check(L.ucm_hamming_topk(
-        q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), NB, BS, Hkv, Wd, ks[0], ks[1], ks[2],
+        q.data_ptr(), _lib.stride(q, 0), _lib.stride(q, 1), k.data_ptr(), NB, BS, Hkv, Wd, ks[0], ks[1], ks[2],
         block_table.data_ptr() if block_table is not None else None, ts, mb, seq_lens.data_ptr(),
         B, Hq, int(k_blocks), int(sink_token), int(recent_token), flags, idx.data_ptr(),
         sc.data_ptr() if sc is not None else None, ws.data_ptr(), ws.numel(),
@@ -149,8 +149,9 @@ def hamming_score(key_codes, query_code, block_table, seq_len, max_seq_len, sink
     out = torch.empty((B, Ho, int(max_seq_len)),
                       dtype=torch.int32 if out_int32 else torch.float16, device=q.device)
     _lib.check(_lib.lib().ucm_hamming_score(
-        q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), NB, BS, Hkv, Wd, ks[0], ks[1], ks[2],
-        block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_len.data_ptr(),
+        q.data_ptr(), _lib.stride(q, 0), _lib.stride(q, 1), k.data_ptr(), NB, BS, Hkv, Wd, ks[0], ks[1], ks[2],
+        block_table.data_ptr(), max(_lib.stride(block_table, 0), block_table.shape[1]),
+        block_table.shape[1], seq_len.data_ptr(),
         B, Hq, int(max_seq_len), int(sink), int(recent), int(bool(reduce_kvhead)), out.data_ptr(),
         int(not out_int32), _lib.stream_ptr(q.device)))
     return out

@@ -120,9 +120,10 @@ class HashEncoder:
         out = torch.empty((T, H, Wd), dtype=torch.int32, device=x.device)
         if T > 0:
             _lib.check(_lib.lib().ucm_hash_encode(
-                x3.data_ptr(), _DT[self.dtype], T, H, self.input_dim, x3.stride(0), x3.stride(1),
+                x3.data_ptr(), _DT[self.dtype], T, H, self.input_dim, _lib.stride(x3, 0),
+                _lib.stride(x3, 1),
                 self._w.data_ptr(), _DT[self.dtype], self._w.shape[0], hpw, self._padded_bits,
-                out.data_ptr(), out.stride(0), out.stride(1), _lib.stream_ptr(x.device)))
+                out.data_ptr(), _lib.stride(out, 0), _lib.stride(out, 1), _lib.stream_ptr(x.device)))
         codes = out.view(torch.uint8)[..., : self.hash_numbers]
         return codes.reshape(*orig_shape, self.hash_numbers)
 
@@ -174,7 +175,7 @@ class HashEncoder:
         if self.hash_bits % 32 != 0:
             raise NotImplementedError("the fused cache write needs hash_bits % 32 == 0")
         u8 = self._reinterpret_cache_as_u8(k_hash_cache)
-        sb, ss, sh, sw = u8.stride()
+        sb, ss, sh, sw = (_lib.stride(u8, d) for d in range(4))
         if sw != 1 or sb % 4 or ss % 4 or sh % 4 or u8.data_ptr() % 4:
             raise ValueError("k_hash_cache codes must be contiguous and 4-byte aligned")
         if slot_mapping.dtype not in (torch.int32, torch.int64):
@@ -183,7 +184,8 @@ class HashEncoder:
         x = self._prep(x)
         if T > 0:
             _lib.check(_lib.lib().ucm_hash_encode_cache(
-                x.data_ptr(), _DT[self.dtype], T, H, self.input_dim, x.stride(0), x.stride(1),
+                x.data_ptr(), _DT[self.dtype], T, H, self.input_dim, _lib.stride(x, 0),
+                _lib.stride(x, 1),
                 self._w.data_ptr(), _DT[self.dtype], self._w.shape[0],
                 self.heads_per_weight if self.num_weights > 1 else 0, self._padded_bits,
                 slot_mapping.data_ptr(), int(slot_mapping.dtype == torch.int64),
@@ -224,13 +226,13 @@ def reshape_and_cache_khash(k_hash_compute, slot_mapping, k_hash, block_size=128
     src = k_hash_compute.contiguous().view(torch.uint8)
     dst = k_hash.view(torch.uint8)
     T, H, Wb = src.shape
-    sb, ss, sh, sw = dst.stride()
+    sb, ss, sh, sw = (_lib.stride(dst, d) for d in range(4))
     if Wb % 4 or sw != 1 or sb % 4 or ss % 4 or sh % 4:
         raise ValueError("codes must be a whole number of 4-byte words and 4-byte aligned")
     slot_mapping = slot_mapping.contiguous()
     if T > 0:
         _lib.check(_lib.lib().ucm_code_scatter(
-            src.data_ptr(), T, H, Wb // 4, src.stride(0) // 4, src.stride(1) // 4,
+            src.data_ptr(), T, H, Wb // 4, _lib.stride(src, 0) // 4, _lib.stride(src, 1) // 4,
             slot_mapping.data_ptr(), int(slot_mapping.dtype == torch.int64), dst.data_ptr(),
             k_hash.shape[0], block_size, sb // 4, ss // 4, sh // 4,
             _lib.stream_ptr(k_hash.device)))
