@@ -175,6 +175,34 @@ int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_str
  */
 int ucm_hamming_topk_set_profile_events(void* before, void* after);
 
+/*
+ * One decode step of the GQA retrieval path in a single call: store the hash codes of the
+ * step's new keys in the paged code cache, hash the step's queries, then score and select.
+ * Replaces the call sequence of GSAOnDevice.attention_begin at decode
+ * (ucm/sparse/gsa_on_device/gsa_on_device.py:564-572 cache_k_hash_gqa_cuda, :773-786
+ * update_decode_topk_gqa_cuda): three launches issued back to back from native code.
+ *
+ * new_keys  [T, Hkv, K] (strides in elements), slot_mapping [T]: as ucm_hash_encode_cache;
+ *           T = 0 skips the cache update.
+ * queries   [B, Hq, K]  (strides in elements); query head h is projected with matrix
+ *           min(h / (Hq/Hkv), n_w - 1) when n_w > 1 — the matrix of its KV head.
+ * w         [n_w, K, N_bits]; n_w is 1 (shared) or Hkv.
+ * q_codes   uint32 [B, Hq, N_bits/32] contiguous scratch that receives the query codes.
+ * Remaining arguments as in ucm_hamming_topk (Wd = N_bits / 32).
+ */
+int ucm_sparse_decode_step(const void* new_keys, int64_t T, int64_t k_stride_t, int64_t k_stride_h,
+                           const void* slot_mapping, int slot_is_i64,
+                           const void* queries, int64_t q_stride_b, int64_t q_stride_h,
+                           int x_dtype, int32_t K,
+                           const void* w, int w_dtype, int32_t n_w, int32_t N_bits,
+                           uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
+                           int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                           const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                           const int32_t* seq_lens, int32_t B, int32_t Hq, int32_t k,
+                           int32_t sink_tok, int32_t recent_tok, uint32_t flags,
+                           uint32_t* q_codes, int32_t* out_idx, int32_t* out_score,
+                           void* workspace, size_t workspace_bytes, ucm_stream_t stream);
+
 /* Replaces update_seq_lens (hamming_topk.py:7-12):
  * out[b] = len[b] - ceil(max(len[b] - topk_tok, 0) / BS) * BS. */
 int ucm_update_seq_lens(const int32_t* seq_lens, int32_t B, int32_t topk_tok, int32_t BS,

@@ -20,12 +20,15 @@
 // its NPU op (csrc/ascend/hamming_dist_top_k/op_kernel/hamming_dist_top_k_base.h:150-347).
 #include "common.h"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWave = 64;
 constexpr int kInf = 0x7fffffff;
 constexpr int kMaxTileHeads = 1024;  // TB * Hkv bound of the LDS min table
+constexpr int kMaxTile = 64;          // TB bound
 constexpr int kSelLdsCap = 8192;     // block scores kept in LDS by select_kernel
 constexpr int kSelSortCap = 2048;    // largest k for score-ordered output
 
@@ -123,19 +126,27 @@ __global__ __launch_bounds__(kThreads) void plane_kernel(const uint32_t* __restr
 //   CPU   : 16-byte pieces per code (1, 2 or 4)
 //   DIRECT: true  -> G = GP query codes kept in registers, xor+popcount per query head
 //           false -> GP = PMAX bit planes in registers
-// A workgroup owns TB consecutive logical blocks of one request; lane l of the wave that
-// handles 64-piece run r reads piece r*64+l, so each load instruction covers 1 KiB of
-// contiguous memory.  (head, piece-in-code) of a lane never changes, so its query material
+//   U     : 1 KiB runs a wave keeps in flight per step
+// A workgroup owns TB consecutive logical blocks of one request.  A block is a sequence of
+// 64-piece "runs" (1 KiB each); lane l of the wave that handles run r reads piece r*64+l, so
+// each load instruction covers 1 KiB of contiguous memory.  Blocks with >= 4 runs are split
+// over the four waves (split = 1), smaller blocks go whole to one wave (split = 0).  The
+// loads of step s+1 are issued before the popcounts of step s, so every wave always has a
+// batch in flight.  (head, piece-in-code) of a lane never changes, so its query material
 // lives in registers for the whole kernel.
 // ---------------------------------------------------------------------------------------
-template <int CPU, bool DIRECT, int GP, int UNROLL>
-__global__ __launch_bounds__(kThreads) void block_score_fast(ScoreArgs a)
+template <int CPU, bool DIRECT, int GP, int U>
+__global__ __launch_bounds__(kThreads) void block_score_fast(ScoreArgs a, int split)
 {
     __shared__ int smin[kMaxTileHeads];
+    __shared__ long long pbs[kMaxTile];  // physical block per tile block, -1 = unusable
     const int b = blockIdx.y;
+    const int j0 = blockIdx.x * a.TB;
+    // table entries never depend on seq_len: read them while seq_len is still in flight
+    if (threadIdx.x < a.TB && j0 + (int)threadIdx.x < a.max_blocks)
+        pbs[threadIdx.x] = physical_block(a, b, j0 + threadIdx.x);
     const int len = a.lens[b];
     const int nblk = num_blocks_of(a, len);
-    const int j0 = blockIdx.x * a.TB;
     if (j0 >= nblk) return;
     const int nb_tile = (a.TB < nblk - j0) ? a.TB : nblk - j0;
 
@@ -167,58 +178,41 @@ __global__ __launch_bounds__(kThreads) void block_score_fast(ScoreArgs a)
     }
     __syncthreads();
 
-    const int CPB = a.BS * period;          // pieces per block, multiple of 64
-    const int runs = nb_tile * (CPB >> 6);  // 64-piece runs in the tile
-    const int runs_per_block = CPB >> 6;
+    const int rpb = (a.BS * period) >> 6;  // runs per block
     const int wid = wave_id();
+    // this wave's blocks: blk_first, +blk_step ...; its runs inside a block: run_first, +run_step
+    const int blk_first = split ? 0 : wid, blk_step = split ? 1 : 4;
+    const int run_first = split ? wid : 0, run_step = split ? 4 : 1;
+    const int rpw = split ? (rpb >> 2) : rpb;  // runs of one block handled by this wave
+    const int bpb = (rpw + U - 1) / U;         // batches (steps) per block
+    const int my_blocks = (nb_tile - blk_first + blk_step - 1) / blk_step;
+    const int nsteps = my_blocks > 0 ? my_blocks * bpb : 0;
 
-    int cur_blk = -1;
-    int m = kInf;
-
-    auto flush = [&](int blk, int mm) {
-        for (int s = period; s < kWave; s <<= 1) {
-            const int o = __shfl_xor(mm, s);
-            mm = o < mm ? o : mm;
+    auto issue = [&](int s, u32x4 (&kv)[U]) {
+        const int bi = s / bpb, batch = s - bi * bpb;
+        const int blk = blk_first + bi * blk_step;
+        const long long pb = pbs[blk];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = batch * U + u;
+            kv[u] = (u32x4)(0u);
+            if (pb >= 0 && k < rpw) {
+                const int run = run_first + k * run_step;
+                const u32x4* src =
+                    reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + (run << 6) + lane;
+                kv[u] = __builtin_nontemporal_load(src);
+            }
         }
-        if (lane < period && part == 0) atomicMin(&smin[blk * a.Hkv + h], mm);
     };
 
-    for (int r0 = wid; r0 < runs; r0 += 4 * UNROLL) {
-        u32x4 kv[UNROLL];
-        int blk_u[UNROLL];
-        int cc_u[UNROLL];
-        bool ok_u[UNROLL];
+    int m = kInf;
+    auto consume = [&](int s, const u32x4 (&kv)[U]) {
+        const int bi = s / bpb, batch = s - bi * bpb;
+        const int blk = blk_first + bi * blk_step;
+        const bool usable = pbs[blk] >= 0;
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int r = r0 + 4 * u;
-            ok_u[u] = false;
-            blk_u[u] = 0;
-            cc_u[u] = 0;
-            kv[u] = (u32x4)(0u);
-            if (r < runs) {
-                const int blk = r / runs_per_block;
-                const int cc = (r - blk * runs_per_block) * 64 + lane;
-                const int64_t pb = physical_block(a, b, j0 + blk);
-                blk_u[u] = blk;
-                cc_u[u] = cc;
-                if (pb >= 0) {
-                    ok_u[u] = true;
-                    const u32x4* src =
-                        reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + cc;
-                    kv[u] = __builtin_nontemporal_load(src);
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int r = r0 + 4 * u;
-            if (r >= runs) break;
-            if (blk_u[u] != cur_blk) {
-                if (cur_blk >= 0) flush(cur_blk, m);
-                cur_blk = blk_u[u];
-                m = kInf;
-            }
-            if (!ok_u[u]) continue;
+        for (int u = 0; u < U; ++u) {
+            const int k = batch * U + u;
             int d;
             if (DIRECT) {
                 d = 0;
@@ -237,14 +231,162 @@ __global__ __launch_bounds__(kThreads) void block_score_fast(ScoreArgs a)
             }
             if (CPU >= 2) d += __shfl_xor(d, 1);
             if (CPU >= 4) d += __shfl_xor(d, 2);
-            const int t = cc_u[u] >> period_shift;
-            const int pos = (j0 + blk_u[u]) * a.BS + t;
-            if (pos < len && d < m) m = d;
+            const int run = run_first + k * run_step;
+            const int t = ((run << 6) + lane) >> period_shift;
+            const int pos = (j0 + blk) * a.BS + t;
+            if (usable && k < rpw && pos < len && d < m) m = d;
+        }
+        if (batch == bpb - 1) {  // last batch of the block: publish this wave's minimum
+            int mm = m;
+            for (int st = period; st < kWave; st <<= 1) {
+                const int o = __shfl_xor(mm, st);
+                mm = o < mm ? o : mm;
+            }
+            if (lane < period && part == 0) atomicMin(&smin[blk * a.Hkv + h], mm);
+            m = kInf;
+        }
+    };
+
+    u32x4 buf0[U], buf1[U];
+    if (nsteps > 0) issue(0, buf0);
+    for (int s = 0; s < nsteps; s += 2) {
+        if (s + 1 < nsteps) issue(s + 1, buf1);
+        consume(s, buf0);
+        if (s + 1 < nsteps) {
+            if (s + 2 < nsteps) issue(s + 2, buf0);
+            consume(s + 1, buf1);
         }
     }
-    if (cur_blk >= 0) flush(cur_blk, m);
     __syncthreads();
-    write_tile_scores(a, b, j0, nb_tile, len, smin);
+
+    const int full = a.G * 32 * a.Wd;
+    for (int i = threadIdx.x; i < nb_tile * a.Hkv; i += kThreads) {
+        const int blk = i / a.Hkv, hh = i - blk * a.Hkv, j = j0 + blk;
+        const int p0 = j * a.BS;
+        const int p1 = (p0 + a.BS < len) ? p0 + a.BS : len;
+        const bool forced = (p0 < a.sink) || (p1 > len - a.recent);
+        int sc;
+        if (pbs[blk] < 0) sc = -1;
+        else if (forced) sc = full;
+        else sc = full - smin[i];
+        a.scores[((int64_t)b * a.Hkv + hh) * a.max_blocks + j] = sc;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// One-block-per-workgroup scorer: the hot shape (a block of at least 4 KiB, split over the
+// four waves).  Same arithmetic as block_score_fast with the head count a compile-time
+// constant, so the lane -> (head, piece) map, the token of a piece and the wave reduction
+// are all shifts and DPP-friendly shuffles.
+// ---------------------------------------------------------------------------------------
+template <int CPU, int HKV, bool DIRECT, int GP>
+__global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
+{
+    constexpr int PERIOD = HKV * CPU;  // pieces per token (a power of two <= 64)
+    __shared__ int smin[HKV];
+    const int b = blockIdx.y, j = blockIdx.x;
+    const int lane = lane_id();
+    const int wid = wave_id();
+    const int h = (lane % PERIOD) / CPU, part = lane % CPU;
+
+    // query material first: it depends on nothing but the request index
+    uint32_t qr[GP][4];
+    int ctot = 0;
+    if (DIRECT) {
+        const uint32_t* qp = a.q + b * a.q_stride_b + (int64_t)h * GP * a.q_stride_h + part * 4;
+#pragma unroll
+        for (int g = 0; g < GP; ++g)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[g][w] = qp[g * a.q_stride_h + w];
+    } else {
+        const uint32_t* pp = a.planes + ((int64_t)b * HKV + h) * GP * a.Wd + part * 4;
+#pragma unroll
+        for (int p = 0; p < GP; ++p)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[p][w] = pp[p * a.Wd + w];
+    }
+
+    const int len = a.lens[b];
+    const int pos0 = j * a.BS;
+    if (pos0 >= len) return;  // j >= ceil(len / BS); the grid never exceeds max_blocks
+    const int64_t pb = physical_block(a, b, j);
+    const int rpw = (a.BS * PERIOD) >> 8;  // runs per wave (a block has 4*rpw runs)
+    const u32x4* base = reinterpret_cast<const u32x4*>(a.kc + (pb < 0 ? 0 : pb) * a.ks_block) + lane;
+
+    // first batch of code loads goes out before anything waits
+    u32x4 kv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) kv[u] = (u32x4)(0u);
+    if (pb >= 0) {
+        if (rpw >= 4) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * u) << 6));
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (u < rpw) kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * u) << 6));
+        }
+    }
+    if (threadIdx.x < HKV) smin[threadIdx.x] = kInf;
+    if (!DIRECT) {
+#pragma unroll
+        for (int p = 0; p < GP; ++p)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) ctot += __popc(qr[p][w]) << p;
+    }
+
+    int m = kInf;
+    if (pb >= 0) {
+        for (int k0 = 0; k0 < rpw; k0 += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int d;
+                if (DIRECT) {
+                    d = 0;
+#pragma unroll
+                    for (int g = 0; g < GP; ++g)
+                        d += __popc(kv[u].x ^ qr[g][0]) + __popc(kv[u].y ^ qr[g][1]) +
+                             __popc(kv[u].z ^ qr[g][2]) + __popc(kv[u].w ^ qr[g][3]);
+                } else {
+                    int acc = 0;
+#pragma unroll
+                    for (int p = 0; p < GP; ++p)
+                        acc += (__popc(kv[u].x & qr[p][0]) + __popc(kv[u].y & qr[p][1]) +
+                                __popc(kv[u].z & qr[p][2]) + __popc(kv[u].w & qr[p][3]))
+                               << p;
+                    d = ctot + a.G * popc4(kv[u]) - 2 * acc;
+                }
+                if (CPU >= 2) d += __shfl_xor(d, 1);
+                if (CPU >= 4) d += __shfl_xor(d, 2);
+                const int t = (((wid + 4 * (k0 + u)) << 6) + lane) / PERIOD;
+                if (k0 + u < rpw && pos0 + t < len && d < m) m = d;
+            }
+            // next batch (blocks larger than 16 KiB)
+            if (k0 + 4 < rpw) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    kv[u] = (u32x4)(0u);
+                    if (k0 + 4 + u < rpw)
+                        kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * (k0 + 4 + u)) << 6));
+                }
+            }
+        }
+#pragma unroll
+        for (int st = PERIOD; st < kWave; st <<= 1) {
+            const int o = __shfl_xor(m, st);
+            m = o < m ? o : m;
+        }
+    }
+    __syncthreads();  // smin initialised
+    if (pb >= 0 && lane < PERIOD && part == 0) atomicMin(&smin[h], m);
+    __syncthreads();
+    if (threadIdx.x < HKV) {
+        const int full = a.G * 32 * a.Wd;
+        const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
+        const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
+        const int sc = pb < 0 ? -1 : (forced ? full : full - smin[threadIdx.x]);
+        a.scores[((int64_t)b * HKV + threadIdx.x) * a.max_blocks + j] = sc;
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -608,21 +750,56 @@ Workspace carve(void* base, int B, int Hkv, int max_blocks)
     return w;
 }
 
-template <int CPU, bool DIRECT, int GP>
-void launch_fast(const ScoreArgs& a, dim3 grid, hipStream_t st)
+int env_int(const char* name, int dflt)
 {
-    hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 4>), grid, dim3(kThreads), 0, st, a);
+    const char* v = getenv(name);
+    return v ? atoi(v) : dflt;
+}
+
+template <int CPU, bool DIRECT, int GP>
+void launch_fast(const ScoreArgs& a, int split, int u, dim3 grid, hipStream_t st)
+{
+    if (u >= 4)
+        hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 4>), grid, dim3(kThreads), 0, st, a, split);
+    else if (u >= 2)
+        hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 2>), grid, dim3(kThreads), 0, st, a, split);
+    else
+        hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 1>), grid, dim3(kThreads), 0, st, a, split);
 }
 
 template <int CPU>
-bool dispatch_fast(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+bool dispatch_fast(const ScoreArgs& a, int pmax, int split, int u, dim3 grid, hipStream_t st)
 {
-    if (a.G == 1) launch_fast<CPU, true, 1>(a, grid, st);
-    else if (a.G == 2) launch_fast<CPU, true, 2>(a, grid, st);
-    else if (a.G == 4) launch_fast<CPU, true, 4>(a, grid, st);
-    else if (pmax == 4) launch_fast<CPU, false, 4>(a, grid, st);
-    else launch_fast<CPU, false, 8>(a, grid, st);
+    if (a.G == 1) launch_fast<CPU, true, 1>(a, split, u, grid, st);
+    else if (a.G == 2) launch_fast<CPU, true, 2>(a, split, u, grid, st);
+    else if (a.G == 4) launch_fast<CPU, true, 4>(a, split, u, grid, st);
+    else if (pmax == 4) launch_fast<CPU, false, 4>(a, split, u, grid, st);
+    else launch_fast<CPU, false, 8>(a, split, u, grid, st);
     return true;
+}
+
+template <int CPU, int HKV>
+void dispatch_one_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+{
+    if (a.G == 1) hipLaunchKernelGGL((block_score_one<CPU, HKV, true, 1>), grid, dim3(kThreads), 0, st, a);
+    else if (a.G == 2) hipLaunchKernelGGL((block_score_one<CPU, HKV, true, 2>), grid, dim3(kThreads), 0, st, a);
+    else if (a.G == 4) hipLaunchKernelGGL((block_score_one<CPU, HKV, true, 4>), grid, dim3(kThreads), 0, st, a);
+    else if (pmax == 4) hipLaunchKernelGGL((block_score_one<CPU, HKV, false, 4>), grid, dim3(kThreads), 0, st, a);
+    else hipLaunchKernelGGL((block_score_one<CPU, HKV, false, 8>), grid, dim3(kThreads), 0, st, a);
+}
+
+// true when a block_score_one instance exists for this (pieces per code, KV heads) pair
+template <int CPU>
+bool dispatch_one(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+{
+    switch (a.Hkv) {
+        case 1: dispatch_one_g<CPU, 1>(a, pmax, grid, st); return true;
+        case 2: dispatch_one_g<CPU, 2>(a, pmax, grid, st); return true;
+        case 4: dispatch_one_g<CPU, 4>(a, pmax, grid, st); return true;
+        case 8: dispatch_one_g<CPU, 8>(a, pmax, grid, st); return true;
+        case 16: if (CPU <= 4) { dispatch_one_g<CPU, 16>(a, pmax, grid, st); return true; } return false;
+        default: return false;
+    }
 }
 
 thread_local hipEvent_t g_prof_before = nullptr;
@@ -699,6 +876,9 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     while (TB > 1 && TB * Hkv > kMaxTileHeads) TB >>= 1;
     // keep at least ~8 workgroups per CU in flight when the problem allows it
     while (TB > 1 && (int64_t)B * ucm::ceil_div(max_blocks, TB) < 2048) TB >>= 1;
+    if (env_int("UCM_TB", 0) > 0) TB = env_int("UCM_TB", 0);
+    if (TB > kMaxTile) TB = kMaxTile;
+    while (TB > 1 && TB * Hkv > kMaxTileHeads) TB >>= 1;
     a.TB = TB;
     const dim3 grid((unsigned)ucm::ceil_div(max_blocks, TB), (unsigned)B);
 
@@ -713,9 +893,25 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             if (rc != UCM_OK) return rc;
         }
         if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_before, st));
-        if (cpu == 1) dispatch_fast<1>(a, pmax, grid, st);
-        else if (cpu == 2) dispatch_fast<2>(a, pmax, grid, st);
-        else dispatch_fast<4>(a, pmax, grid, st);
+        const int rpb = (int)(((int64_t)BS * Hkv * cpu) >> 6);
+        int split = (rpb >= 4 && rpb % 4 == 0) ? 1 : 0;
+        if (env_int("UCM_SPLIT", -1) >= 0) split = env_int("UCM_SPLIT", -1);
+        const int rpw = split ? rpb / 4 : rpb;
+        const int u = env_int("UCM_UNROLL", rpw);
+        // blocks of >= 4 KiB: one block per workgroup with the head count compiled in
+        bool done = false;
+        if (split && Hkv <= 16 && env_int("UCM_ONE", 1)) {
+            a.TB = 1;
+            const dim3 grid1((unsigned)max_blocks, (unsigned)B);
+            if (cpu == 1) done = dispatch_one<1>(a, pmax, grid1, st);
+            else if (cpu == 2) done = dispatch_one<2>(a, pmax, grid1, st);
+            else done = dispatch_one<4>(a, pmax, grid1, st);
+        }
+        if (!done) {
+            if (cpu == 1) dispatch_fast<1>(a, pmax, split, u, grid, st);
+            else if (cpu == 2) dispatch_fast<2>(a, pmax, split, u, grid, st);
+            else dispatch_fast<4>(a, pmax, split, u, grid, st);
+        }
     } else {
         if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_before, st));
         hipLaunchKernelGGL(block_score_generic, grid, dim3(kThreads), (size_t)Hq * Wd * 4, st, a);
@@ -734,6 +930,37 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     s.flags = flags; s.out_idx = out_idx; s.out_score = out_score;
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
     return ucm::launch_status("select_kernel");
+}
+
+extern "C" int ucm_sparse_decode_step(const void* new_keys, int64_t T, int64_t k_stride_t,
+                                      int64_t k_stride_h, const void* slot_mapping,
+                                      int slot_is_i64, const void* queries, int64_t q_stride_b,
+                                      int64_t q_stride_h, int x_dtype, int32_t K, const void* w,
+                                      int w_dtype, int32_t n_w, int32_t N_bits, uint32_t* k_cache,
+                                      int64_t NB, int32_t BS, int32_t Hkv, int64_t ks_block,
+                                      int64_t ks_token, int64_t ks_head,
+                                      const int32_t* block_table, int32_t table_stride,
+                                      int32_t max_blocks, const int32_t* seq_lens, int32_t B,
+                                      int32_t Hq, int32_t k, int32_t sink_tok, int32_t recent_tok,
+                                      uint32_t flags, uint32_t* q_codes, int32_t* out_idx,
+                                      int32_t* out_score, void* workspace, size_t workspace_bytes,
+                                      ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(Hkv > 0 && Hq > 0 && Hq % Hkv == 0, "bad head counts");
+    UCM_REQUIRE(N_bits > 0 && N_bits % 32 == 0, "hash_bits must be a multiple of 32");
+    UCM_REQUIRE(n_w == 1 || n_w == Hkv, "n_w must be 1 or the number of KV heads");
+    UCM_REQUIRE(q_codes, "q_codes is null");
+    const int32_t Wd = N_bits / 32;
+    int rc = ucm::encode_pair(new_keys, T, Hkv, k_stride_t, k_stride_h, slot_mapping, slot_is_i64,
+                              k_cache, NB, BS, ks_block, ks_token, ks_head, queries, B, Hq,
+                              q_stride_b, q_stride_h, q_codes, x_dtype, K, w, w_dtype, n_w, N_bits,
+                              (hipStream_t)stream);
+    if (rc != UCM_OK) return rc;
+    return ucm_hamming_topk(q_codes, (int64_t)Hq * Wd, Wd, k_cache, NB, BS, Hkv, Wd, ks_block,
+                            ks_token, ks_head, block_table, table_stride, max_blocks, seq_lens, B,
+                            Hq, k, sink_tok, recent_tok, flags, out_idx, out_score, workspace,
+                            workspace_bytes, stream);
 }
 
 extern "C" int ucm_hamming_topk_set_profile_events(void* before, void* after)

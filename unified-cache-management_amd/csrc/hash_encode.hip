@@ -169,6 +169,68 @@ __global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
     }
 }
 
+// Latency path for a handful of rows (decode): one wave per (job, head, 32 hash columns,
+// 32 rows).  No LDS and no persistent loop: the B operand is assembled straight from the
+// row-major projection matrix with eight 2-byte loads per k-step, all issued up front, so the
+// whole kernel is one round trip to L2 plus K/16 MFMAs.  Up to two independent jobs (e.g. the
+// step's new keys and its queries) share one launch.
+struct EncJobs {
+    EncArgs job[2];
+    int waves0;  // waves of job 0; waves >= waves0 belong to job 1
+};
+
+template <typename V, int KS>
+__global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
+{
+    constexpr int K = KS * 16;
+    const bool second = (int)blockIdx.x >= js.waves0;
+    const EncArgs& a = second ? js.job[1] : js.job[0];
+    int wv = second ? blockIdx.x - js.waves0 : blockIdx.x;
+    const int ntiles = a.N / 32;
+    const int nt = wv % ntiles;
+    wv /= ntiles;
+    const int h = wv % a.H;
+    const int64_t row0 = (int64_t)(wv / a.H) * kRowsPerWave;
+
+    const int lane = threadIdx.x;
+    const int r = lane & 31, kb = lane >> 5;
+    const uint16_t* wsrc =
+        (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N + nt * 32 + r;
+    int64_t t = row0 + r;
+    const bool row_ok = t < a.T;
+    if (!row_ok) t = a.T - 1;
+    const uint16_t* xr = (const uint16_t*)a.x + (int64_t)h * a.x_stride_h + t * a.x_stride_t + kb * 8;
+
+    V av[KS];
+    uint16_t bw[KS][8];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bw[ks][i] = wsrc[(int64_t)(ks * 16 + kb * 8 + i) * a.N];
+
+    f32x16 acc = {0};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        V bv;
+        __builtin_memcpy(&bv, bw[ks], 16);
+        acc = Mfma<V>::run(av[ks], bv, acc);
+    }
+    uint32_t word = 0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const unsigned long long m = __ballot(acc[v] > 0.0f);
+        const int r0 = 8 * (v / 4) + (v % 4);
+        if (lane == r0) word = (uint32_t)m;
+        if (lane == r0 + 4) word = (uint32_t)(m >> 32);
+    }
+    if (row_ok && lane < 32) {
+        uint32_t* dst = row_dst(a, t, h);
+        if (dst) dst[nt] = word;
+    }
+}
+
 __device__ __forceinline__ float load_as_float(const void* p, int dtype, int64_t i)
 {
     if (dtype == UCM_DT_F32) return ((const float*)p)[i];
@@ -286,7 +348,36 @@ int dispatch_mfma(const EncArgs& a, hipStream_t st)
     }
 }
 
-int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
+constexpr int64_t kSmallRows = 256;  // at most this many rows per head take the latency path
+
+bool mfma_eligible(const EncArgs& a, int x_dtype, int w_dtype)
+{
+    const bool same16 = (x_dtype == w_dtype) && (x_dtype == UCM_DT_BF16 || x_dtype == UCM_DT_F16);
+    const bool k_ok = a.K == 64 || a.K == 128 || a.K == 256 || a.K == 512;
+    const bool aligned = (((uintptr_t)a.x | (uintptr_t)a.w) & 15) == 0 && a.x_stride_t % 8 == 0 &&
+                         a.x_stride_h % 8 == 0;
+    return same16 && k_ok && aligned;
+}
+
+int64_t small_waves(const EncArgs& a)
+{
+    return ucm::ceil_div(a.T, kRowsPerWave) * a.H * (a.N / 32);
+}
+
+template <typename V>
+int launch_small(const EncJobs& js, int64_t waves, int K, hipStream_t st)
+{
+    const dim3 grid((unsigned)waves);
+    switch (K) {
+        case 64: hipLaunchKernelGGL((encode_small_kernel<V, 4>), grid, dim3(64), 0, st, js); break;
+        case 128: hipLaunchKernelGGL((encode_small_kernel<V, 8>), grid, dim3(64), 0, st, js); break;
+        case 256: hipLaunchKernelGGL((encode_small_kernel<V, 16>), grid, dim3(64), 0, st, js); break;
+        default: return ucm::fail(UCM_ERROR, "internal: K %d has no small-row kernel", K);
+    }
+    return ucm::launch_status("encode_small_kernel");
+}
+
+int check_shape(const EncArgs& a, int x_dtype, int w_dtype)
 {
     UCM_REQUIRE(a.x && a.w, "null input");
     UCM_REQUIRE(a.T >= 0 && a.H > 0 && a.K > 0 && a.N > 0, "bad shape");
@@ -294,15 +385,30 @@ int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
     UCM_REQUIRE(a.N % 32 == 0, "hash_bits %d must be a multiple of 32", a.N);
     UCM_REQUIRE(a.n_w >= 1 && a.heads_per_w >= 0, "bad weight layout");
     UCM_REQUIRE(x_dtype >= 0 && x_dtype <= 2 && w_dtype >= 0 && w_dtype <= 2, "unknown dtype");
+    return UCM_OK;
+}
+
+bool small_eligible(const EncArgs& a, int x_dtype, int w_dtype)
+{
+    return mfma_eligible(a, x_dtype, w_dtype) && a.K <= 256 && a.T <= kSmallRows;
+}
+
+int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
+{
+    int rc = check_shape(a, x_dtype, w_dtype);
+    if (rc != UCM_OK) return rc;
     if (a.T == 0) return UCM_OK;
 
-    const bool same16 = (x_dtype == w_dtype) && (x_dtype == UCM_DT_BF16 || x_dtype == UCM_DT_F16);
-    const bool k_ok = a.K == 64 || a.K == 128 || a.K == 256 || a.K == 512;
-    const bool aligned = (((uintptr_t)a.x | (uintptr_t)a.w) & 15) == 0 && a.x_stride_t % 8 == 0 &&
-                         a.x_stride_h % 8 == 0;
-    if (same16 && k_ok && aligned) {
-        return x_dtype == UCM_DT_BF16 ? dispatch_mfma<bf16x8>(a, st) : dispatch_mfma<f16x8>(a, st);
+    if (small_eligible(a, x_dtype, w_dtype)) {
+        EncJobs js{};
+        js.job[0] = a;
+        js.job[1] = a;
+        js.waves0 = (int)small_waves(a);
+        return x_dtype == UCM_DT_BF16 ? launch_small<bf16x8>(js, js.waves0, a.K, st)
+                                      : launch_small<f16x8>(js, js.waves0, a.K, st);
     }
+    if (mfma_eligible(a, x_dtype, w_dtype))
+        return x_dtype == UCM_DT_BF16 ? dispatch_mfma<bf16x8>(a, st) : dispatch_mfma<f16x8>(a, st);
     const int64_t total = a.T * a.H * (a.N / 32);
     int64_t blocks = ucm::ceil_div(total, kThreads);
     if (blocks > 65535 * 16) blocks = 65535 * 16;
@@ -374,3 +480,45 @@ extern "C" int ucm_code_scatter(const uint32_t* codes, int64_t T, int32_t H, int
                        (hipStream_t)stream, codes, T, (int)H, (int)Wd, in_stride_t, in_stride_h, a);
     return ucm::launch_status("code_scatter_kernel");
 }
+
+// Encodes the step's new keys into the paged cache and the step's queries into a dense
+// tensor.  When both are small enough for the latency path they share one launch.
+namespace ucm {
+int encode_pair(const void* keys, int64_t T, int Hkv, int64_t k_stride_t, int64_t k_stride_h,
+                const void* slot, int slot_is_i64, uint32_t* cache, int64_t NB, int BS,
+                int64_t cs_block, int64_t cs_token, int64_t cs_head, const void* queries, int64_t B,
+                int Hq, int64_t q_stride_b, int64_t q_stride_h, uint32_t* q_codes, int x_dtype,
+                int K, const void* w, int w_dtype, int n_w, int N_bits, hipStream_t st)
+{
+    const int Wd = N_bits / 32;
+    EncArgs kq{};
+    kq.x = queries; kq.T = B; kq.H = Hq; kq.K = K; kq.x_stride_t = q_stride_b; kq.x_stride_h = q_stride_h;
+    kq.w = w; kq.n_w = n_w; kq.heads_per_w = n_w > 1 ? Hq / Hkv : 0; kq.N = N_bits;
+    kq.out = q_codes; kq.out_stride_t = (int64_t)Hq * Wd; kq.out_stride_h = Wd;
+    int rc = check_shape(kq, x_dtype, w_dtype);
+    if (rc != UCM_OK) return rc;
+    if (T <= 0) return encode_common(kq, x_dtype, w_dtype, st);
+
+    EncArgs kk{};
+    kk.x = keys; kk.T = T; kk.H = Hkv; kk.K = K; kk.x_stride_t = k_stride_t; kk.x_stride_h = k_stride_h;
+    kk.w = w; kk.n_w = n_w; kk.heads_per_w = n_w > 1 ? 1 : 0; kk.N = N_bits;
+    kk.slot = slot; kk.slot_is_i64 = slot_is_i64; kk.cache = cache; kk.NB = NB; kk.BS = BS;
+    kk.cs_block = cs_block; kk.cs_token = cs_token; kk.cs_head = cs_head;
+    rc = check_shape(kk, x_dtype, w_dtype);
+    if (rc != UCM_OK) return rc;
+    rc = check_cache(slot, cache, NB, BS);
+    if (rc != UCM_OK) return rc;
+    if (B > 0 && small_eligible(kk, x_dtype, w_dtype) && small_eligible(kq, x_dtype, w_dtype)) {
+        EncJobs js{};
+        js.job[0] = kk;
+        js.job[1] = kq;
+        js.waves0 = (int)small_waves(kk);
+        const int64_t waves = js.waves0 + small_waves(kq);
+        return x_dtype == UCM_DT_BF16 ? launch_small<bf16x8>(js, waves, K, st)
+                                      : launch_small<f16x8>(js, waves, K, st);
+    }
+    rc = encode_common(kk, x_dtype, w_dtype, st);
+    if (rc != UCM_OK) return rc;
+    return encode_common(kq, x_dtype, w_dtype, st);
+}
+}  // namespace ucm

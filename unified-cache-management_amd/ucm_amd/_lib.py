@@ -31,6 +31,9 @@ _SIGNATURES = {
     "ucm_hamming_topk": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
                               vp, i32, i32, i32, i32, i32, u32, vp, vp, vp, sz, vp]),
     "ucm_hamming_topk_set_profile_events": (ci, [vp, vp]),
+    "ucm_sparse_decode_step": (ci, [vp, i64, i64, i64, vp, ci, vp, i64, i64, ci, i32, vp, ci, i32, i32,
+                                    vp, i64, i32, i32, i64, i64, i64, vp, i32, i32, vp, i32, i32, i32,
+                                    i32, i32, u32, vp, vp, vp, vp, sz, vp]),
     "ucm_hamming_score": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
                                vp, i32, i32, i32, i32, i32, ci, vp, ci, vp]),
     "ucm_update_seq_lens": (ci, [vp, i32, i32, i32, vp, vp]),

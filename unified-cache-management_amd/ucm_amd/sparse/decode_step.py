@@ -1,0 +1,78 @@
+"""One GQA decode step of the retrieval path in a single native call.
+
+Host-side counterpart of what GSAOnDevice.attention_begin does per layer at decode
+(ucm/sparse/gsa_on_device/gsa_on_device.py:850-957): cache_k_hash_gqa_cuda (:564-572) followed
+by update_decode_topk_gqa_cuda (:773-786).  All buffers are allocated once in the constructor;
+`step` allocates nothing, so it can be captured in a HIP graph.
+"""
+import torch
+
+from .. import _lib
+from .hash_encoder import _DT
+
+
+class SparseDecodeStep:
+    def __init__(self, weights, num_q_heads, num_kv_heads, batch, max_blocks, topk_blocks,
+                 block_size=128, sink_token=0, recent_token=0, reduce_heads=False,
+                 return_physical=False):
+        """weights: [K, N] (shared) or [Hkv, K, N] projection, bf16 / fp16 / fp32, on the GPU."""
+        w = weights if weights.dim() == 3 else weights.unsqueeze(0)
+        if w.shape[0] not in (1, num_kv_heads):
+            raise ValueError("weights must be [K,N] or [Hkv,K,N]")
+        if w.dtype not in _DT:
+            raise ValueError(f"unsupported weight dtype {w.dtype}")
+        self.w = w.contiguous()
+        self.K, self.N = int(w.shape[1]), int(w.shape[2])
+        if self.N % 32:
+            raise ValueError("hash_bits must be a multiple of 32")
+        self.Hq, self.Hkv, self.B = int(num_q_heads), int(num_kv_heads), int(batch)
+        self.max_blocks, self.k, self.BS = int(max_blocks), int(topk_blocks), int(block_size)
+        self.sink, self.recent = int(sink_token), int(recent_token)
+        self.flags = ((_lib.TOPK_REDUCE_HEADS if reduce_heads else 0)
+                      | (_lib.TOPK_RETURN_PHYSICAL if return_physical else 0))
+        dev = w.device
+        Ho = 1 if reduce_heads else self.Hkv
+        self.q_codes = torch.empty((self.B, self.Hq, self.N // 32), dtype=torch.int32, device=dev)
+        self.out_idx = torch.empty((self.B, Ho, self.k), dtype=torch.int32, device=dev)
+        self.out_score = torch.empty_like(self.out_idx)
+        nbytes = _lib.lib().ucm_hamming_topk_workspace_bytes(self.B, self.Hkv, self.max_blocks)
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+    def step(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
+        """new_keys [T,Hkv,K] + slot_mapping [T] (T may be 0), queries [B,Hq,K],
+        k_hash_cache int32 [NB,BS,Hkv,N/32], block_table int32 [B,max_blocks], seq_lens int32 [B].
+        Returns (indices, scores) int32 [B, Hkv or 1, k]: views of buffers reused by every call."""
+        if queries.dtype != self.w.dtype or (new_keys is not None and new_keys.dtype != self.w.dtype):
+            raise ValueError("keys, queries and weights must share one dtype")
+        if tuple(queries.shape) != (self.B, self.Hq, self.K):
+            raise ValueError(f"queries must be {(self.B, self.Hq, self.K)}, got {tuple(queries.shape)}")
+        if k_hash_cache.dtype != torch.int32 or k_hash_cache.dim() != 4:
+            raise ValueError("k_hash_cache must be int32 [NB,BS,Hkv,W]")
+        NB, BS, Hkv, Wd = k_hash_cache.shape
+        if BS != self.BS or Hkv != self.Hkv or Wd != self.N // 32:
+            raise ValueError("k_hash_cache shape does not match this step's configuration")
+        if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
+            raise ValueError("block_table and seq_lens must be int32")
+        if block_table.shape[0] != self.B or block_table.shape[1] < self.max_blocks:
+            raise ValueError("block_table must be [B, >= max_blocks]")
+        if queries.stride(-1) != 1 or k_hash_cache.stride(-1) != 1 or block_table.stride(-1) != 1:
+            raise ValueError("innermost dimensions must be contiguous")
+        T = 0 if new_keys is None else int(new_keys.shape[0])
+        if T:
+            if tuple(new_keys.shape[1:]) != (self.Hkv, self.K) or new_keys.stride(-1) != 1:
+                raise ValueError(f"new_keys must be [T,{self.Hkv},{self.K}] with contiguous rows")
+            if slot_mapping.dtype not in (torch.int32, torch.int64) or slot_mapping.numel() != T:
+                raise ValueError("slot_mapping must be int32/int64 [T]")
+        s = _lib.stride
+        _lib.check(_lib.lib().ucm_sparse_decode_step(
+            new_keys.data_ptr() if T else None, T, s(new_keys, 0) if T else 0,
+            s(new_keys, 1) if T else 0, slot_mapping.data_ptr() if T else None,
+            int(T > 0 and slot_mapping.dtype == torch.int64),
+            queries.data_ptr(), s(queries, 0), s(queries, 1), _DT[self.w.dtype], self.K,
+            self.w.data_ptr(), _DT[self.w.dtype], self.w.shape[0], self.N,
+            k_hash_cache.data_ptr(), NB, BS, Hkv, s(k_hash_cache, 0), s(k_hash_cache, 1),
+            s(k_hash_cache, 2), block_table.data_ptr(), max(s(block_table, 0), self.max_blocks),
+            self.max_blocks, seq_lens.data_ptr(), self.B, self.Hq, self.k, self.sink, self.recent,
+            self.flags, self.q_codes.data_ptr(), self.out_idx.data_ptr(), self.out_score.data_ptr(),
+            self.workspace.data_ptr(), self.workspace.numel(), _lib.stream_ptr(queries.device)))
+        return self.out_idx, self.out_score
