@@ -26,6 +26,9 @@ for p in (ROOT, os.path.join(ROOT, "unified-cache-management_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per block-score launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
+# what the counter reads for a 1 GiB copy (profiles/decode_step_config2_hbm_traffic_pmc.txt)
+HBM_TRAFFIC_PER_LAUNCH = 136964265
 
 B, CTX, HQ, HKV, D, BS, TOPK = 32, 32768, 32, 8, 128, 128, 64
 NBLK = CTX // BS          # 256 logical blocks per request
@@ -42,6 +45,9 @@ def parse():
     ap.add_argument("--skip-extras", action="store_true",
                     help="only the headline workload (no encoder / gather side figures)")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="only run a plain device-to-device copy of known size (1 GiB read + 1 GiB "
+                         "written per launch) so that hardware byte counters can be scaled")
     ap.add_argument("--no-graph", action="store_true",
                     help="time eager launches instead of HIP graph replays")
     return ap.parse_args()
@@ -177,6 +183,26 @@ def extras(torch, enc_k, gen):
     return out
 
 
+def pmc_calibration(torch):
+    """Three launches of the library's pointer-table copy kernel, each moving exactly 1 GiB
+    (4096 chunks of 256 KiB) from one device buffer to another."""
+    import numpy as np
+    from ucm_amd.trans import Device
+
+    n, chunk = 4096, 256 * 1024
+    src = torch.empty(n * chunk, dtype=torch.uint8, device="cuda").fill_(3)
+    dst = torch.empty(n * chunk, dtype=torch.uint8, device="cuda")
+    d = Device()
+    d.Setup(0)
+    st = d.MakeSMStream()
+    ptrs = np.arange(n, dtype=np.uint64) * np.uint64(chunk) + np.uint64(src.data_ptr())
+    torch.cuda.synchronize()
+    for _ in range(3):
+        st.DeviceToHostGather(ptrs, dst.data_ptr(), chunk, n)
+    print(json.dumps({"calibration": "table_copy_kernel<0>", "bytes_read_per_launch": n * chunk,
+                      "bytes_written_per_launch": n * chunk, "launches": 3}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -188,6 +214,10 @@ def main():
 
     from ucm_amd import _lib
     from ucm_amd.sparse import HashEncoder, SparseDecodeStep
+
+    if args.pmc_calibration:
+        pmc_calibration(torch)
+        return
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -303,7 +333,7 @@ def main():
         "p90_step_latency_us": step_ms[int(len(step_ms) * 0.9) - 1] * 1e3,
         "roofline": {"bound": "hbm", "kernel": "block_score_one", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": None, "algorithmic_bytes": alg, "kernel_avg_us": kern_avg_ms * 1e3,
+                     "traffic": HBM_TRAFFIC_PER_LAUNCH, "algorithmic_bytes": alg, "kernel_avg_us": kern_avg_ms * 1e3,
                      "kernel_p50_us": sorted(kern_ms)[len(kern_ms) // 2] * 1e3},
     }
     if not args.skip_cpu:
