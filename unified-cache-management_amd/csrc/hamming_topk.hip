@@ -390,6 +390,123 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
 }
 
 // ---------------------------------------------------------------------------------------
+// Small-block scorer: blocks of 1 or 2 KiB (RPB = 1 or 2 runs of 64 pieces), e.g. 64-token
+// blocks of one 256-bit latent code.  A workgroup owns TB consecutive blocks; every wave takes
+// 4/RPB whole blocks per round and issues their 4 loads at once, so no block is shared between
+// waves (plain LDS stores, no atomics).  Head count and pieces per code are compile-time.
+// ---------------------------------------------------------------------------------------
+template <int CPU, int HKV, bool DIRECT, int GP, int RPB>
+__global__ __launch_bounds__(kThreads) void block_score_small(ScoreArgs a)
+{
+    constexpr int PERIOD = HKV * CPU;
+    constexpr int UB = 4 / RPB;  // blocks per wave and round
+    __shared__ int smin[kMaxTileHeads];
+    __shared__ long long pbs[kMaxTile];
+    const int b = blockIdx.y;
+    const int j0 = blockIdx.x * a.TB;
+    if (threadIdx.x < a.TB && j0 + (int)threadIdx.x < a.max_blocks)
+        pbs[threadIdx.x] = physical_block(a, b, j0 + threadIdx.x);
+    const int lane = lane_id();
+    const int wid = wave_id();
+    const int h = (lane % PERIOD) / CPU, part = lane % CPU;
+
+    uint32_t qr[GP][4];
+    if (DIRECT) {
+        const uint32_t* qp = a.q + b * a.q_stride_b + (int64_t)h * GP * a.q_stride_h + part * 4;
+#pragma unroll
+        for (int g = 0; g < GP; ++g)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[g][w] = qp[g * a.q_stride_h + w];
+    } else {
+        const uint32_t* pp = a.planes + ((int64_t)b * HKV + h) * GP * a.Wd + part * 4;
+#pragma unroll
+        for (int p = 0; p < GP; ++p)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[p][w] = pp[p * a.Wd + w];
+    }
+    const int len = a.lens[b];
+    const int nblk = num_blocks_of(a, len);
+    if (j0 >= nblk) return;
+    const int nb_tile = (a.TB < nblk - j0) ? a.TB : nblk - j0;
+    __syncthreads();  // pbs visible
+
+    int ctot = 0;
+    if (!DIRECT) {
+#pragma unroll
+        for (int p = 0; p < GP; ++p)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) ctot += __popc(qr[p][w]) << p;
+    }
+
+    for (int blk0 = wid * UB; blk0 < nb_tile; blk0 += 4 * UB) {
+        u32x4 kv[4];
+        bool ok[UB];
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub) {
+            const int blk = blk0 + ub;
+            const long long pb = blk < nb_tile ? pbs[blk] : -1;
+            ok[ub] = pb >= 0;
+#pragma unroll
+            for (int r = 0; r < RPB; ++r) {
+                kv[ub * RPB + r] = (u32x4)(0u);
+                if (ok[ub])
+                    kv[ub * RPB + r] = __builtin_nontemporal_load(
+                        reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + (r << 6) + lane);
+            }
+        }
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub) {
+            const int blk = blk0 + ub;
+            int m = kInf;
+#pragma unroll
+            for (int r = 0; r < RPB; ++r) {
+                const u32x4 k4 = kv[ub * RPB + r];
+                int d;
+                if (DIRECT) {
+                    d = 0;
+#pragma unroll
+                    for (int g = 0; g < GP; ++g)
+                        d += __popc(k4.x ^ qr[g][0]) + __popc(k4.y ^ qr[g][1]) +
+                             __popc(k4.z ^ qr[g][2]) + __popc(k4.w ^ qr[g][3]);
+                } else {
+                    int acc = 0;
+#pragma unroll
+                    for (int p = 0; p < GP; ++p)
+                        acc += (__popc(k4.x & qr[p][0]) + __popc(k4.y & qr[p][1]) +
+                                __popc(k4.z & qr[p][2]) + __popc(k4.w & qr[p][3]))
+                               << p;
+                    d = ctot + a.G * popc4(k4) - 2 * acc;
+                }
+                if (CPU >= 2) d += __shfl_xor(d, 1);
+                if (CPU >= 4) d += __shfl_xor(d, 2);
+                const int t = ((r << 6) + lane) / PERIOD;
+                if ((j0 + blk) * a.BS + t < len && d < m) m = d;
+            }
+#pragma unroll
+            for (int st = PERIOD; st < kWave; st <<= 1) {
+                const int o = __shfl_xor(m, st);
+                m = o < m ? o : m;
+            }
+            if (blk < nb_tile && lane < PERIOD && part == 0) smin[blk * HKV + h] = ok[ub] ? m : kInf;
+        }
+    }
+    __syncthreads();
+
+    const int full = a.G * 32 * a.Wd;
+    for (int i = threadIdx.x; i < nb_tile * HKV; i += kThreads) {
+        const int blk = i / HKV, hh = i % HKV, j = j0 + blk;
+        const int p0 = j * a.BS;
+        const int p1 = (p0 + a.BS < len) ? p0 + a.BS : len;
+        const bool forced = (p0 < a.sink) || (p1 > len - a.recent);
+        int sc;
+        if (pbs[blk] < 0) sc = -1;
+        else if (forced) sc = full;
+        else sc = full - smin[i];
+        a.scores[((int64_t)b * HKV + hh) * a.max_blocks + j] = sc;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Generic block scorer: any strides, code width, head count and group size.  One thread per
 // (token, head) code, word-by-word loads; query codes staged in LDS.
 // ---------------------------------------------------------------------------------------
@@ -788,6 +905,29 @@ void dispatch_one_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
     else hipLaunchKernelGGL((block_score_one<CPU, HKV, false, 8>), grid, dim3(kThreads), 0, st, a);
 }
 
+template <int CPU, int HKV, int RPB>
+void dispatch_small_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+{
+    if (a.G == 1) hipLaunchKernelGGL((block_score_small<CPU, HKV, true, 1, RPB>), grid, dim3(kThreads), 0, st, a);
+    else if (a.G == 2) hipLaunchKernelGGL((block_score_small<CPU, HKV, true, 2, RPB>), grid, dim3(kThreads), 0, st, a);
+    else if (a.G == 4) hipLaunchKernelGGL((block_score_small<CPU, HKV, true, 4, RPB>), grid, dim3(kThreads), 0, st, a);
+    else if (pmax == 4) hipLaunchKernelGGL((block_score_small<CPU, HKV, false, 4, RPB>), grid, dim3(kThreads), 0, st, a);
+    else hipLaunchKernelGGL((block_score_small<CPU, HKV, false, 8, RPB>), grid, dim3(kThreads), 0, st, a);
+}
+
+// Blocks of 1 or 2 KiB with 1, 2 or 4 KV heads; false when no instance exists.
+template <int CPU>
+bool dispatch_small(const ScoreArgs& a, int rpb, int pmax, dim3 grid, hipStream_t st)
+{
+    if (rpb != 1 && rpb != 2) return false;
+    switch (a.Hkv) {
+        case 1: if (rpb == 1) dispatch_small_g<CPU, 1, 1>(a, pmax, grid, st); else dispatch_small_g<CPU, 1, 2>(a, pmax, grid, st); return true;
+        case 2: if (rpb == 1) dispatch_small_g<CPU, 2, 1>(a, pmax, grid, st); else dispatch_small_g<CPU, 2, 2>(a, pmax, grid, st); return true;
+        case 4: if (rpb == 1) dispatch_small_g<CPU, 4, 1>(a, pmax, grid, st); else dispatch_small_g<CPU, 4, 2>(a, pmax, grid, st); return true;
+        default: return false;
+    }
+}
+
 // true when a block_score_one instance exists for this (pieces per code, KV heads) pair
 template <int CPU>
 bool dispatch_one(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
@@ -906,6 +1046,19 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             if (cpu == 1) done = dispatch_one<1>(a, pmax, grid1, st);
             else if (cpu == 2) done = dispatch_one<2>(a, pmax, grid1, st);
             else done = dispatch_one<4>(a, pmax, grid1, st);
+        }
+        if (!done) a.TB = TB;
+        if (!done && !split && env_int("UCM_SMALL", 1)) {
+            // 8 blocks per workgroup: every wave gets one round of 4 loads
+            int tbs = env_int("UCM_TB", 8);
+            if (tbs > kMaxTile) tbs = kMaxTile;
+            while (tbs > 1 && tbs * Hkv > kMaxTileHeads) tbs >>= 1;
+            a.TB = tbs;
+            const dim3 grids((unsigned)ucm::ceil_div(max_blocks, tbs), (unsigned)B);
+            if (cpu == 1) done = dispatch_small<1>(a, rpb, pmax, grids, st);
+            else if (cpu == 2) done = dispatch_small<2>(a, rpb, pmax, grids, st);
+            else done = dispatch_small<4>(a, rpb, pmax, grids, st);
+            if (!done) a.TB = TB;
         }
         if (!done) {
             if (cpu == 1) dispatch_fast<1>(a, pmax, split, u, grid, st);
