@@ -1,0 +1,152 @@
+"""GPU tests of the reference-shaped surfaces around the operators: the retrieval worker API,
+the sparse plugin hooks and the KV store interface."""
+import os
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_topk_matches_unordered_ties, rng_for
+from oracle import c_api
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "hash_retrieval_ref.npz")
+
+
+@pytest.mark.parametrize("case,k", [("ragged", 5), ("ragged", 10), ("tail", 12), ("zero", 3)])
+def test_retrieval_worker_matches_the_reference_backend_outputs(case, k):
+    """Same submit/wait/get_result calls as the reference's worker, compared with the outputs the
+    reference's CPU backend produced for these inputs (golden fixture) and with the oracle."""
+    from ucm_amd.sparse.retrieval_worker import HashRetrievalWorker, HashRetrievalWorkerBackend
+
+    gold = np.load(GOLD)
+    data, query = gold[f"{case}_data"], gold[f"{case}_query"]
+    if case == "ragged":
+        indexes = gold["ragged_indexes"]
+        ref_i, ref_d = gold[f"ragged_idx_k{k}"], gold[f"ragged_dist_k{k}"]
+    else:
+        indexes = np.tile(np.arange(data.shape[0], dtype=np.int32), (query.shape[0], 1))
+        ref_i, ref_d = gold[f"{case}_idx"], gold[f"{case}_dist"]
+    worker = HashRetrievalWorker(HashRetrievalWorkerBackend(data, {0: [0]}))
+    rid = worker.submit(torch.from_numpy(query), k, indexes)
+    worker.wait(rid)
+    assert worker.poll(rid)
+    res = worker.get_result(rid)
+    with pytest.raises(RuntimeError):
+        worker.get_result(rid)  # consumed once
+    oi, od, on = c_api.hash_retrieval(data, query, indexes, k)
+    for r in range(query.shape[0]):
+        kk = int(on[r])
+        assert np.array_equal(res["indices"][r, :kk], oi[r, :kk])  # same tie rule as the oracle
+        assert np.array_equal(res["scores"][r, :kk], od[r, :kk])
+        assert np.array_equal(res["scores"][r, :kk], ref_d[r, :kk])
+        fi, fd, fn = c_api.hash_retrieval(data, query[r:r + 1], indexes[r:r + 1], indexes.shape[1])
+        score_of = {int(i): int(s) for i, s in zip(fi[0, : fn[0]], fd[0, : fn[0]])}
+        assert_topk_matches_unordered_ties(res["indices"][r, :kk], res["scores"][r, :kk],
+                                           ref_i[r, :kk], ref_d[r, :kk], all_scores=score_of)
+
+
+def test_retrieval_worker_errors():
+    from ucm_amd.sparse.retrieval_worker import HashRetrievalWorkerBackend
+
+    be = HashRetrievalWorkerBackend(np.zeros((4, 8, 16), np.uint8))
+    with pytest.raises(RuntimeError):
+        be.submit(np.zeros((1, 8), np.uint8), 2, np.zeros((1, 4), np.int32))
+    with pytest.raises(RuntimeError):
+        be.submit(np.zeros((2, 16), np.uint8), 2, np.zeros((1, 4), np.int32))
+    with pytest.raises(RuntimeError):
+        be.wait(99)
+    with pytest.raises(RuntimeError):
+        be.get_result(99)
+
+
+def test_plugin_hooks_swap_and_restore_the_block_table():
+    from ucm_amd.sparse.base import UcmSparseFactory, UcmSparseRole
+
+    B, Hq, Hkv, D, BS, nblk, topk_tok = 3, 32, 8, 128, 128, 24, 1024
+    cfg = {"ucm_sparse_config": {"GSAOnDevice": {
+        "num_q_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "block_size": BS,
+        "vllm_hash_attention_topk": topk_tok, "vllm_hash_attention_rollback_layers": [0],
+        "seed": 5}}}
+    plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+    rng = rng_for(77)
+    NB = B * nblk + 2
+    k_hash = torch.zeros((NB, BS, Hkv, D // 8), dtype=torch.uint8, device="cuda")
+    table = torch.from_numpy(rng.permutation(NB)[: B * nblk].astype(np.int32).reshape(B, nblk)).cuda()
+    lens = torch.tensor([nblk * BS, nblk * BS - 300, 5 * BS + 1], dtype=torch.int32, device="cuda")
+    # prefill: hash every token's key into the code cache through the hook
+    for b in range(B):
+        L = int(lens[b])
+        keys = torch.from_numpy(rng.standard_normal((L, Hkv * D)).astype(np.float32)).to(torch.bfloat16).cuda()
+        pos = torch.arange(L, device="cuda")
+        slots = table[b, pos // BS].long() * BS + pos % BS
+        meta = types.SimpleNamespace(slot_mapping=slots, block_table=table[b:b + 1], seq_lens=lens[b:b + 1])
+        ctx = types.SimpleNamespace(attn_metadata={"model.layers.1.self_attn.attn": meta})
+        plugin.attention_begin(None, keys, None, "model.layers.1.self_attn.attn", ctx,
+                               phase="prefill", k_hash=k_hash)
+    assert int((k_hash != 0).sum()) > 0
+    # decode step on a normal layer
+    q = torch.from_numpy(rng.standard_normal((B, Hq * D)).astype(np.float32)).to(torch.bfloat16).cuda()
+    newk = torch.from_numpy(rng.standard_normal((B, Hkv * D)).astype(np.float32)).to(torch.bfloat16).cuda()
+    pos = lens.long() - 1
+    slots = table[torch.arange(B), pos // BS].long() * BS + pos % BS
+    meta = types.SimpleNamespace(slot_mapping=slots, block_table=table.clone(), seq_lens=lens.clone())
+    ctx = types.SimpleNamespace(attn_metadata={"model.layers.1.self_attn.attn": meta})
+    plugin.attention_begin(q, newk, None, "model.layers.1.self_attn.attn", ctx, phase="decode",
+                           k_hash=k_hash)
+    kblk = topk_tok // BS
+    # expected: oracle on the codes now in the cache, group-mean query code per KV head
+    qc = plugin.hash_code(q.view(B, Hq, D)).cpu().numpy().view(np.uint32)
+    codes = k_hash.cpu().numpy().view(np.uint32).reshape(NB, BS, Hkv, D // 32)
+    oi, _ = c_api.hamming_topk(qc, codes, table.cpu().numpy(), lens.cpu().numpy(), kblk, BS, 4 * BS,
+                               flags=c_api.F_REDUCE_HEADS | c_api.F_PHYSICAL)
+    got = meta.block_table.cpu().numpy()
+    assert np.array_equal(got[:, :kblk], np.maximum(oi[:, 0], 0))
+    assert not got[:, kblk:].any()
+    assert np.array_equal(meta.seq_lens.cpu().numpy(), c_api.update_seq_lens(lens.cpu().numpy(), topk_tok, BS))
+    plugin.attention_finished(q, newk, None, None, "model.layers.1.self_attn.attn", ctx, phase="decode")
+    assert torch.equal(meta.block_table, table) and torch.equal(meta.seq_lens, lens)
+    # a rollback layer keeps the full table
+    meta0 = types.SimpleNamespace(slot_mapping=slots, block_table=table.clone(), seq_lens=lens.clone())
+    ctx0 = types.SimpleNamespace(attn_metadata=meta0)
+    plugin.attention_begin(q, newk, None, "model.layers.0.self_attn.attn", ctx0, phase="decode",
+                           k_hash=k_hash)
+    assert torch.equal(meta0.block_table, table)
+
+
+def test_host_memory_store_dump_lookup_load_roundtrip():
+    """The store contract of the reference's e2e test (ucm/store/test/e2e/cache_on_empty_test.py:
+    46-79): dump -> lookup -> load -> bit-exact."""
+    from ucm_amd.store import HostMemoryStore
+
+    L, NB, chunk = 4, 16, 8192
+    rng = rng_for(88)
+    src = [torch.from_numpy(rng.integers(0, 256, size=(2, NB, chunk), dtype=np.uint8)).cuda() for _ in range(L)]
+    dst = [torch.zeros_like(t) for t in src]
+    store = HostMemoryStore({"tensor_size_list": [chunk] * (2 * L), "capacity_blocks": 8})
+    ids = [bytes([i]) * 16 for i in range(5)]
+    blocks = [3, 7, 0, 15, 9]
+    new_blocks = [1, 2, 4, 5, 6]
+
+    def addrs(tensors, blks):
+        return np.array([[t[kv, b].data_ptr() for t in tensors for kv in (0, 1)] for b in blks], np.uint64)
+
+    ev = torch.cuda.Event()
+    ev.record()
+    task = store.dump_data(ids, [0] * 5, addrs(src, blocks), ev.cuda_event)
+    store.wait(task)
+    assert store.check(task)
+    assert store.lookup(ids + [b"x" * 16]) == [True] * 5 + [False]
+    assert store.lookup_on_prefix(ids[:2] + [b"y" * 16] + ids[2:]) == 1
+    want = np.concatenate([src[l][kv, blocks[0]].cpu().numpy() for l in range(L) for kv in (0, 1)])
+    assert np.array_equal(store.slot_view(ids[0]), want)
+    task = store.load_data(ids, [0] * 5, addrs(dst, new_blocks))
+    store.wait(task)
+    for l in range(L):
+        assert torch.equal(dst[l][:, new_blocks], src[l][:, blocks])
+        rest = [b for b in range(NB) if b not in new_blocks]
+        assert not dst[l][:, rest].any()
+    with pytest.raises(RuntimeError):
+        store.load_data([b"z" * 16], [0], addrs(dst, [0]))

@@ -1,0 +1,126 @@
+"""GSAOnDevice-shaped driver of the MI355X operators (GQA decode path).
+
+A thin counterpart of the reference plugin's worker-side hot path
+(ucm/sparse/gsa_on_device/gsa_on_device.py): `attention_begin` stores the hash codes of the
+step's keys (cache_k_hash_gqa_cuda, :564-572) and, at decode, replaces the layer's block table
+and seq_lens with the top-k blocks (update_decode_topk_gqa_cuda, :773-811);
+`attention_finished` puts the originals back (:959-995).  Engine metadata is duck-typed: the
+layer's `attn_metadata` needs `slot_mapping`, `block_table` and `seq_lens` attributes.  The
+scheduler-side hooks, prefix-cache rehash, MLA metadata surgery and layer-skip profiling of
+the reference are outside this build.
+
+Configuration (`ucm_sparse_config["GSAOnDevice"]`), names from
+gsa_on_device_config.py:36-98 where they exist:
+    num_q_heads, num_kv_heads, head_dim, block_size, hash_bits (default head_dim),
+    vllm_hash_attention_topk (tokens kept), sink_tokens (default block_size),
+    recent_tokens (default 4 * block_size), vllm_hash_attention_rollback_layers,
+    gpu_seq_len_threshold, dtype ("bfloat16"|"float16"|"float32"), device, seed
+"""
+from typing import List, Optional, Union
+
+import torch
+
+from .base import UcmSparseBase, UcmSparseMetadata, UcmSparseRole
+from .hamming_topk import cuda_hamming_topk, update_seq_lens
+from .hash_encoder import HashEncoder
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}
+
+
+class GSAOnDeviceMetadata(UcmSparseMetadata):
+    pass
+
+
+class GSAOnDevice(UcmSparseBase):
+    def __init__(self, vllm_config, role: UcmSparseRole):
+        super().__init__(vllm_config, role)
+        cfg = getattr(vllm_config, "ucm_sparse_config", None)
+        if cfg is None:
+            cfg = vllm_config["ucm_sparse_config"]
+        cfg = cfg["GSAOnDevice"]
+        self.num_q_heads = int(cfg["num_q_heads"])
+        self.num_key_heads = int(cfg["num_kv_heads"])
+        self.head_dim = int(cfg["head_dim"])
+        self.block_size = int(cfg.get("block_size", 128))
+        self.hash_bits = int(cfg.get("hash_bits", self.head_dim))
+        self.hash_topk_tokens = int(cfg.get("vllm_hash_attention_topk", 2048))
+        self.sink_tokens = int(cfg.get("sink_tokens", self.block_size))
+        self.recent_tokens = int(cfg.get("recent_tokens", 4 * self.block_size))
+        self.hash_rollback_layers = list(cfg.get("vllm_hash_attention_rollback_layers", []))
+        self.seq_len_threshold = int(cfg.get("gpu_seq_len_threshold", 0))
+        self.device = torch.device(cfg.get("device", "cuda:0"))
+        self.dtype = _DTYPES[cfg.get("dtype", "bfloat16")]
+        if "seed" in cfg:
+            torch.manual_seed(int(cfg["seed"]))
+        self.is_mla = False
+        self.gsa_enabled = True
+        self.hash_encoder = HashEncoder(self.head_dim, self.hash_bits, self.dtype, self.device)
+        self._saved = {}
+
+    # ---- helpers mirroring the reference's names ----
+    def get_layer_attn_metadata(self, forward_context, layer_name: str):
+        attn_meta = forward_context.attn_metadata
+        return attn_meta[layer_name] if isinstance(attn_meta, dict) else attn_meta
+
+    def get_layer_state(self, layer_name: str):
+        layer_id = int(layer_name.split(".")[2])
+        return layer_id in self.hash_rollback_layers, False
+
+    def hash_code(self, query: torch.Tensor) -> torch.Tensor:
+        """Group-mean query -> one code per KV head (gsa_on_device.py:396-412)."""
+        if self.num_q_heads > self.num_key_heads:
+            query = query.view(query.shape[0], self.num_key_heads,
+                               self.num_q_heads // self.num_key_heads, query.shape[2]).mean(2)
+        elif self.num_q_heads < self.num_key_heads:
+            query = torch.repeat_interleave(query, self.num_key_heads // self.num_q_heads, dim=1)
+        return self.hash_encoder.compute_hash(query)
+
+    def cache_k_hash_gqa(self, key, attn_metadata, k_hash):
+        slots = attn_metadata.slot_mapping.flatten()
+        n = slots.numel()
+        self.hash_encoder.compute_hash_and_cache(
+            key[:n].view(n, self.num_key_heads, self.head_dim), slots, k_hash,
+            block_size=self.block_size)
+
+    # ---- hooks ----
+    def attention_begin(self, query, key, value, layer_name: str, forward_context, output=None,
+                        phase: Optional[str] = None, k_hash=None, decode_ql_nope=None,
+                        decode_q_pe=None):
+        if not self.gsa_enabled or k_hash is None:
+            return query, key, value, output
+        attn_metadata = self.get_layer_attn_metadata(forward_context, layer_name)
+        self.cache_k_hash_gqa(key, attn_metadata, k_hash)
+        is_rollback_layer, _ = self.get_layer_state(layer_name)
+        if phase == "decode" and not is_rollback_layer:
+            num_reqs = attn_metadata.seq_lens.shape[0]
+            q = query[:num_reqs].view(num_reqs, self.num_q_heads, self.head_dim)
+            q_hash = self.hash_code(q)
+            topk_table = cuda_hamming_topk(
+                q_hash.unsqueeze(1), k_hash, attn_metadata.block_table, attn_metadata.seq_lens,
+                topk_token=self.hash_topk_tokens, sink_token=self.sink_tokens,
+                recent_token=self.recent_tokens, is_mla=self.is_mla)
+            self._saved[layer_name] = (attn_metadata.block_table, attn_metadata.seq_lens)
+            topk = topk_table.shape[1]
+            new_table = torch.zeros_like(attn_metadata.block_table)
+            new_table[:, :topk] = topk_table
+            new_lens = update_seq_lens(attn_metadata.seq_lens, self.hash_topk_tokens, self.block_size)
+            if self.seq_len_threshold > 0:  # short requests keep their full table
+                short = attn_metadata.seq_lens < self.seq_len_threshold
+                new_table = torch.where(short[:, None], attn_metadata.block_table, new_table)
+                new_lens = torch.where(short, attn_metadata.seq_lens, new_lens)
+            attn_metadata.block_table = new_table
+            attn_metadata.seq_lens = new_lens
+        return query, key, value, output
+
+    def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context,
+                           phase: Optional[str] = None) -> None:
+        saved = self._saved.pop(layer_name, None)
+        if saved is not None:
+            attn_metadata = self.get_layer_attn_metadata(forward_context, layer_name)
+            attn_metadata.block_table, attn_metadata.seq_lens = saved
+
+    def request_begin(self, request_id: Union[int, str], prompt_token_ids: List[int]):
+        pass
+
+    def build_sparse_meta(self, scheduler_output, requests, input_batch, attn_metadata):
+        return GSAOnDeviceMetadata()
