@@ -740,6 +740,103 @@ __global__ __launch_bounds__(kThreads) void select_kernel(SelectArgs a)
 }
 
 // ---------------------------------------------------------------------------------------
+// Wave-level selection for rows of at most 64*EL block scores (index-ordered output only).
+// One wave per (request, KV head) row, no LDS and no barriers: a binary search on the score
+// value with ballot counts finds the k-th largest score, two wave prefix sums place the winners
+// in ascending index order, ties to the lower index.  Same results as select_kernel.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ int wave_excl_scan(int v, int* total)
+{
+    int inc = v;
+#pragma unroll
+    for (int s = 1; s < kWave; s <<= 1) {
+        const int o = __shfl_up(inc, s);
+        if (lane_id() >= s) inc += o;
+    }
+    *total = __shfl(inc, kWave - 1);
+    return inc - v;
+}
+
+template <int EL>
+__global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int rows_total)
+{
+    const int rowid = blockIdx.x * (kThreads / kWave) + wave_id();
+    if (rowid >= rows_total) return;
+    const int b = rowid / a.Ho, ho = rowid % a.Ho;
+    const int lane = lane_id();
+    const int len = a.lens[b];
+    int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
+    if (n > a.max_blocks) n = a.max_blocks;
+    int32_t* oi = a.out_idx + ((int64_t)b * a.Ho + ho) * a.k;
+    int32_t* os = a.out_score ? a.out_score + ((int64_t)b * a.Ho + ho) * a.k : nullptr;
+    const int kk = a.k < n ? a.k : n;
+    for (int i = kk + lane; i < a.k; i += kWave) {
+        oi[i] = -1;
+        if (os) os[i] = 0;
+    }
+    if (n == 0) return;
+    const bool reduce = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
+    const int32_t* row = a.scores + ((int64_t)b * a.Hkv + (reduce ? 0 : ho)) * a.max_blocks;
+    int v[EL];
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        const int j = lane * EL + e;
+        int x = -0x7fffffff;  // below every real score (>= -1): never selected
+        if (j < n) {
+            x = row[j];
+            if (reduce)
+                for (int h = 1; h < a.Hkv; ++h) {
+                    const int o = row[(int64_t)h * a.max_blocks + j];
+                    x = o > x ? o : x;
+                }
+        }
+        v[e] = x;
+    }
+    auto count_ge = [&](int t) {
+        int c = 0;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) c += __popcll(__ballot(v[e] >= t));
+        return c;
+    };
+    int lo = -1, hi = a.full;  // count_ge(lo) >= kk always holds
+    while (lo < hi) {
+        const int mid = lo + ((hi - lo + 1) >> 1);
+        if (count_ge(mid) >= kk) lo = mid;
+        else hi = mid - 1;
+    }
+    const int thr = lo;
+    const int need = kk - count_ge(thr + 1);  // ties at thr to take, lowest indices first
+    int eq = 0, gt = 0;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        eq += (v[e] == thr);
+        gt += (v[e] > thr);
+    }
+    int tot;
+    const int eq_before = wave_excl_scan(eq, &tot);
+    int eq_take = need - eq_before;
+    eq_take = eq_take < 0 ? 0 : (eq_take > eq ? eq : eq_take);
+    int pos = wave_excl_scan(gt + eq_take, &tot);
+    int eq_seen = 0;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        bool take = v[e] > thr;
+        if (v[e] == thr) {
+            take = eq_seen < eq_take;
+            ++eq_seen;
+        }
+        if (take && pos < a.k) {
+            const int j = lane * EL + e;
+            oi[pos] = (a.flags & UCM_TOPK_RETURN_PHYSICAL)
+                          ? (a.table ? a.table[(int64_t)b * a.table_stride + j] : b * a.max_blocks + j)
+                          : j;
+            if (os) os[pos] = (a.flags & UCM_TOPK_DISTANCE) ? a.full - v[e] : v[e];
+            ++pos;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Per-token scores in the reference scorer's output shape.
 // ---------------------------------------------------------------------------------------
 struct TokenArgs {
@@ -1081,6 +1178,16 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     s.key_bits = 1;
     while ((1ll << s.key_bits) <= (int64_t)s.full + 1) ++s.key_bits;
     s.flags = flags; s.out_idx = out_idx; s.out_score = out_score;
+    const int rows_total = B * s.Ho;
+    const dim3 wgrid((unsigned)ucm::ceil_div(rows_total, kThreads / kWave));
+    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256 && env_int("UCM_WSEL", 1)) {
+        hipLaunchKernelGGL(select_wave_kernel<4>, wgrid, dim3(kThreads), 0, st, s, rows_total);
+        return ucm::launch_status("select_wave_kernel");
+    }
+    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 1024 && env_int("UCM_WSEL", 1)) {
+        hipLaunchKernelGGL(select_wave_kernel<16>, wgrid, dim3(kThreads), 0, st, s, rows_total);
+        return ucm::launch_status("select_wave_kernel");
+    }
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
     return ucm::launch_status("select_kernel");
 }

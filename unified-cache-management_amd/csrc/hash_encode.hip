@@ -47,7 +47,8 @@ struct EncArgs {
     int64_t NB;
     int BS;
     int64_t cs_block, cs_token, cs_head;
-    int BN;  // hash columns per workgroup slice
+    int BN;        // hash columns per workgroup slice
+    int bs_shift;  // log2(BS) when BS is a power of two, else -1
 };
 
 __device__ __forceinline__ int weight_index(const EncArgs& a, int h)
@@ -62,7 +63,57 @@ __device__ __forceinline__ uint32_t* row_dst(const EncArgs& a, int64_t t, int h)
     if (!a.cache) return a.out + t * a.out_stride_t + (int64_t)h * a.out_stride_h;
     const int64_t s = a.slot_is_i64 ? ((const int64_t*)a.slot)[t] : (int64_t)((const int32_t*)a.slot)[t];
     if (s < 0 || s >= a.NB * (int64_t)a.BS) return nullptr;
-    return a.cache + (s / a.BS) * a.cs_block + (s % a.BS) * a.cs_token + (int64_t)h * a.cs_head;
+    int64_t blk, tok;
+    if (a.bs_shift >= 0) {  // the usual case: no integer division
+        blk = s >> a.bs_shift;
+        tok = s & (a.BS - 1);
+    } else if (s < 0x7fffffff) {
+        blk = (uint32_t)s / (uint32_t)a.BS;
+        tok = (uint32_t)s % (uint32_t)a.BS;
+    } else {
+        blk = s / a.BS;
+        tok = s % a.BS;
+    }
+    return a.cache + blk * a.cs_block + tok * a.cs_token + (int64_t)h * a.cs_head;
+}
+
+// Sign-packs four accumulator registers of a 32x32 MFMA tile.  The 64-bit lane mask of
+// "acc > 0" is two finished output words (32 columns of rows R and R+4); v_writelane_b32 drops
+// each into the lane that owns the row, leaving the other lanes untouched.  The wait states
+// between the vector compares that produce the masks and the lane writes that read them are
+// inserted by hand: the compiler does not look inside inline assembly.
+template <int R>
+__device__ __forceinline__ uint32_t pack_rows4(uint32_t word, float a0, float a1, float a2, float a3)
+{
+    const unsigned long long m0 = __ballot(a0 > 0.0f), m1 = __ballot(a1 > 0.0f);
+    const unsigned long long m2 = __ballot(a2 > 0.0f), m3 = __ballot(a3 > 0.0f);
+    asm("s_nop 4\n\t"
+        "v_writelane_b32 %0, %1, %9\n\ts_nop 0\n\t"
+        "v_writelane_b32 %0, %2, %10\n\ts_nop 0\n\t"
+        "v_writelane_b32 %0, %3, %11\n\ts_nop 0\n\t"
+        "v_writelane_b32 %0, %4, %12\n\ts_nop 0\n\t"
+        "v_writelane_b32 %0, %5, %13\n\ts_nop 0\n\t"
+        "v_writelane_b32 %0, %6, %14\n\ts_nop 0\n\t"
+        "v_writelane_b32 %0, %7, %15\n\ts_nop 0\n\t"
+        "v_writelane_b32 %0, %8, %16"
+        : "+v"(word)
+        : "s"((uint32_t)m0), "s"((uint32_t)m1), "s"((uint32_t)m2), "s"((uint32_t)m3),
+          "s"((uint32_t)(m0 >> 32)), "s"((uint32_t)(m1 >> 32)), "s"((uint32_t)(m2 >> 32)),
+          "s"((uint32_t)(m3 >> 32)),
+          "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3), "n"(R + 4), "n"(R + 5), "n"(R + 6), "n"(R + 7));
+    return word;
+}
+
+// Accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the tile:
+// registers 4g..4g+3 are rows 8g..8g+3 (low mask halves) and 8g+4..8g+7 (high halves).
+__device__ __forceinline__ uint32_t pack_tile(const f32x16& acc)
+{
+    uint32_t word = 0;
+    word = pack_rows4<0>(word, acc[0], acc[1], acc[2], acc[3]);
+    word = pack_rows4<8>(word, acc[4], acc[5], acc[6], acc[7]);
+    word = pack_rows4<16>(word, acc[8], acc[9], acc[10], acc[11]);
+    word = pack_rows4<24>(word, acc[12], acc[13], acc[14], acc[15]);
+    return word;
 }
 
 template <typename V>
@@ -96,15 +147,23 @@ __global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
     const int bn = (a.N - n0 < a.BN) ? a.N - n0 : a.BN;  // columns in this slice
     const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N;
 
-    // W[k][n0 + 8j .. +8] -> wt[8j + i][k]
-    for (int idx = threadIdx.x; idx < K * (bn / 8); idx += kThreads) {
-        const int k = idx / (bn / 8), j = idx % (bn / 8);
-        const u32x4 v = *reinterpret_cast<const u32x4*>(wsrc + (int64_t)k * a.N + n0 + 8 * j);
-        const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+    // W[k0..k0+8][n0+8j..+8] -> wt[8j+c][k0..k0+8]: each thread transposes 8x8 patches of 16-bit
+    // elements in registers (byte permutes) and writes eight 16-byte LDS rows
+    for (int idx = threadIdx.x; idx < (K / 8) * (bn / 8); idx += kThreads) {
+        const int kq = idx / (bn / 8), j = idx % (bn / 8);
+        const uint16_t* src = wsrc + (int64_t)(kq * 8) * a.N + n0 + 8 * j;
+        u32x4 row[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            wt[(8 * j + 2 * i) * KP + k] = (uint16_t)(wv[i] & 0xffffu);
-            wt[(8 * j + 2 * i + 1) * KP + k] = (uint16_t)(wv[i] >> 16);
+        for (int i = 0; i < 8; ++i) row[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * a.N);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+            u32x4 o;
+            o.x = __builtin_amdgcn_perm(row[1][c >> 1], row[0][c >> 1], sel);
+            o.y = __builtin_amdgcn_perm(row[3][c >> 1], row[2][c >> 1], sel);
+            o.z = __builtin_amdgcn_perm(row[5][c >> 1], row[4][c >> 1], sel);
+            o.w = __builtin_amdgcn_perm(row[7][c >> 1], row[6][c >> 1], sel);
+            *reinterpret_cast<u32x4*>(wt + (8 * j + c) * KP + kq * 8) = o;
         }
     }
     __syncthreads();
@@ -117,18 +176,29 @@ __global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
     const int nt_count = bn / 32;
     const int word0 = n0 / 32;
 
+    // A operands of the wave's 32 rows of a tile; rows past T re-read the last row (discarded)
+    auto load_tile = [&](int64_t tile, V (&dstv)[KS]) {
+        int64_t t = tile * kRowsPerWg + wave * kRowsPerWave + r;
+        if (t >= a.T) t = a.T - 1;
+        const uint16_t* xr = xbase + t * a.x_stride_t + kb * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dstv[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
+    };
+    constexpr bool kPrefetch = KS <= 16;  // the next tile's operands fit in registers
+    V av[KS];
+    V nx[kPrefetch ? KS : 1];
+    if (blockIdx.x < tiles) load_tile(blockIdx.x, av);
+
     for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
         const int64_t row0 = tile * kRowsPerWg + wave * kRowsPerWave;
-        if (row0 >= a.T) continue;
-        int64_t t = row0 + r;
+        const int64_t next = tile + gridDim.x;
+        if constexpr (kPrefetch) {
+            if (next < tiles) load_tile(next, nx);
+        } else {
+            if (tile != (int64_t)blockIdx.x) load_tile(tile, av);
+        }
+        const int64_t t = row0 + r;
         const bool row_ok = t < a.T;
-        if (!row_ok) t = a.T - 1;  // read a valid row, discard its result
-        const uint16_t* xr = xbase + t * a.x_stride_t + kb * 8;
-        V av[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-            av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
-
         uint32_t* dst = (row_ok && lane < 32) ? row_dst(a, t, h) : nullptr;
 
         for (int nt0 = 0; nt0 < nt_count; nt0 += 4) {
@@ -145,14 +215,7 @@ __global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
                     acc = Mfma<V>::run(av[ks], bv, acc);
                 }
                 // accumulator v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
-                uint32_t word = 0;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const unsigned long long m = __ballot(acc[v] > 0.0f);
-                    const int r0 = 8 * (v / 4) + (v % 4);
-                    if (lane == r0) word = (uint32_t)m;
-                    if (lane == r0 + 4) word = (uint32_t)(m >> 32);
-                }
+                const uint32_t word = pack_tile(acc);
                 words[q] = word;
             }
             if (dst) {
@@ -164,6 +227,12 @@ __global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
                 } else {
                     for (int q = 0; q < nq; ++q) d[q] = words[q];
                 }
+            }
+        }
+        if constexpr (kPrefetch) {
+            if (next < tiles) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) av[ks] = nx[ks];
             }
         }
     }
@@ -217,14 +286,7 @@ __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
         __builtin_memcpy(&bv, bw[ks], 16);
         acc = Mfma<V>::run(av[ks], bv, acc);
     }
-    uint32_t word = 0;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const unsigned long long m = __ballot(acc[v] > 0.0f);
-        const int r0 = 8 * (v / 4) + (v % 4);
-        if (lane == r0) word = (uint32_t)m;
-        if (lane == r0 + 4) word = (uint32_t)(m >> 32);
-    }
+    const uint32_t word = pack_tile(acc);
     if (row_ok && lane < 32) {
         uint32_t* dst = row_dst(a, t, h);
         if (dst) dst[nt] = word;
@@ -329,7 +391,7 @@ int launch_mfma(EncArgs a, hipStream_t st)
     const size_t lds = (size_t)a.BN * (K + kPad) * 2;
     const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
     const int slices = a.N / a.BN;
-    int64_t per = (int64_t)num_cus() * 2 / ((int64_t)slices * a.H);
+    int64_t per = (int64_t)num_cus() * 4 / ((int64_t)slices * a.H);
     if (per < 1) per = 1;
     const dim3 grid((unsigned)(tiles < per ? tiles : per), (unsigned)slices, (unsigned)a.H);
     hipLaunchKernelGGL((encode_mfma_kernel<V, KS>), grid, dim3(kThreads), lds, st, a);
@@ -377,6 +439,12 @@ int launch_small(const EncJobs& js, int64_t waves, int K, hipStream_t st)
     return ucm::launch_status("encode_small_kernel");
 }
 
+void set_block_shift(EncArgs& a)
+{
+    a.bs_shift = -1;
+    if (a.BS > 0 && (a.BS & (a.BS - 1)) == 0) a.bs_shift = __builtin_ctz((unsigned)a.BS);
+}
+
 int check_shape(const EncArgs& a, int x_dtype, int w_dtype)
 {
     UCM_REQUIRE(a.x && a.w, "null input");
@@ -395,6 +463,7 @@ bool small_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 
 int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
 {
+    set_block_shift(a);
     int rc = check_shape(a, x_dtype, w_dtype);
     if (rc != UCM_OK) return rc;
     if (a.T == 0) return UCM_OK;
@@ -473,6 +542,7 @@ extern "C" int ucm_code_scatter(const uint32_t* codes, int64_t T, int32_t H, int
     EncArgs a{};
     a.slot = slot_mapping; a.slot_is_i64 = slot_is_i64; a.cache = cache; a.NB = NB; a.BS = BS;
     a.cs_block = cs_block; a.cs_token = cs_token; a.cs_head = cs_head;
+    set_block_shift(a);
     const int64_t total = T * H * Wd;
     int64_t blocks = ucm::ceil_div(total, kThreads);
     if (blocks > 65535 * 16) blocks = 65535 * 16;
@@ -510,6 +580,8 @@ int encode_pair(const void* keys, int64_t T, int Hkv, int64_t k_stride_t, int64_
     if (rc != UCM_OK) return rc;
     if (B > 0 && small_eligible(kk, x_dtype, w_dtype) && small_eligible(kq, x_dtype, w_dtype)) {
         EncJobs js{};
+        set_block_shift(kk);
+        set_block_shift(kq);
         js.job[0] = kk;
         js.job[1] = kq;
         js.waves0 = (int)small_waves(kk);
