@@ -169,9 +169,10 @@ int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_str
 
 /*
  * Measurement hook, no counterpart in the reference.  When both events (hipEvent_t) are
- * non-NULL, every following ucm_hamming_topk call on this thread records `before` right
- * before and `after` right after its block-score kernel, on the call's stream, so a caller
- * can time that kernel alone.  Pass NULLs to switch it off.
+ * non-NULL, every following ucm_hamming_topk call on this thread launches its block-score
+ * kernel with `before` / `after` as that dispatch's own start and stop events
+ * (hipExtLaunchKernel), so hipEventElapsedTime(before, after) is the kernel's execution time.
+ * Pass NULLs to switch it off.
  */
 int ucm_hamming_topk_set_profile_events(void* before, void* after);
 

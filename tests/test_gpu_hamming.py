@@ -90,6 +90,9 @@ FAST_CASES = [
     (110, 4, 32, 8, 4, 128, [0, 128, 127, 16384], 64),  # empty request, k > nblk, long
     (111, 2, 32, 8, 4, 128, [131072, 100000], 128),  # 1024 blocks per request
     (112, 2, 128, 1, 8, 64, [65536, 30000], 128),    # config 5 shape at 2 requests
+    (113, 2, 16, 4, 4, 48, [1000, 48], 5),           # 3 KiB blocks: several whole blocks per wave
+    (114, 1, 64, 32, 4, 128, [2000], 6),             # 32 KV heads: 64 KiB blocks split over waves
+    (115, 2, 20, 4, 8, 16, [700, 50], 4),            # 2 KiB blocks, G=5, 256-bit codes, 4 heads
 ]
 
 

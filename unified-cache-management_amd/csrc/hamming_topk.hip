@@ -18,9 +18,9 @@
 // csrc/cuda/ham_dist/paged_ham_dist_mla.cu:148-247 of the reference (block min of the
 // group-summed distance, sink/recent keep, +inf past seq_len), in the similarity form of
 // its NPU op (csrc/ascend/hamming_dist_top_k/op_kernel/hamming_dist_top_k_base.h:150-347).
-#include "common.h"
+#include <hip/hip_ext.h>
 
-#include <cstdlib>
+#include "common.h"
 
 namespace {
 
@@ -964,21 +964,31 @@ Workspace carve(void* base, int B, int Hkv, int max_blocks)
     return w;
 }
 
-int env_int(const char* name, int dflt)
+// Profiling hook: when set, the block-score launch carries these events as the kernel's own
+// start/stop markers (timestamps of the dispatch itself, without the launch latency an event
+// recorded on the stream would add).
+thread_local hipEvent_t g_prof_before = nullptr;
+thread_local hipEvent_t g_prof_after = nullptr;
+
+template <typename K, typename... Args>
+void launch_score(K kernel, dim3 grid, size_t lds, hipStream_t st, Args... args)
 {
-    const char* v = getenv(name);
-    return v ? atoi(v) : dflt;
+    if (g_prof_before && g_prof_after)
+        hipExtLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, st, g_prof_before, g_prof_after, 0,
+                              args...);
+    else
+        hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, st, args...);
 }
 
 template <int CPU, bool DIRECT, int GP>
 void launch_fast(const ScoreArgs& a, int split, int u, dim3 grid, hipStream_t st)
 {
     if (u >= 4)
-        hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 4>), grid, dim3(kThreads), 0, st, a, split);
+        launch_score(block_score_fast<CPU, DIRECT, GP, 4>, grid, 0, st, a, split);
     else if (u >= 2)
-        hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 2>), grid, dim3(kThreads), 0, st, a, split);
+        launch_score(block_score_fast<CPU, DIRECT, GP, 2>, grid, 0, st, a, split);
     else
-        hipLaunchKernelGGL((block_score_fast<CPU, DIRECT, GP, 1>), grid, dim3(kThreads), 0, st, a, split);
+        launch_score(block_score_fast<CPU, DIRECT, GP, 1>, grid, 0, st, a, split);
 }
 
 template <int CPU>
@@ -995,21 +1005,21 @@ bool dispatch_fast(const ScoreArgs& a, int pmax, int split, int u, dim3 grid, hi
 template <int CPU, int HKV>
 void dispatch_one_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
-    if (a.G == 1) hipLaunchKernelGGL((block_score_one<CPU, HKV, true, 1>), grid, dim3(kThreads), 0, st, a);
-    else if (a.G == 2) hipLaunchKernelGGL((block_score_one<CPU, HKV, true, 2>), grid, dim3(kThreads), 0, st, a);
-    else if (a.G == 4) hipLaunchKernelGGL((block_score_one<CPU, HKV, true, 4>), grid, dim3(kThreads), 0, st, a);
-    else if (pmax == 4) hipLaunchKernelGGL((block_score_one<CPU, HKV, false, 4>), grid, dim3(kThreads), 0, st, a);
-    else hipLaunchKernelGGL((block_score_one<CPU, HKV, false, 8>), grid, dim3(kThreads), 0, st, a);
+    if (a.G == 1) launch_score(block_score_one<CPU, HKV, true, 1>, grid, 0, st, a);
+    else if (a.G == 2) launch_score(block_score_one<CPU, HKV, true, 2>, grid, 0, st, a);
+    else if (a.G == 4) launch_score(block_score_one<CPU, HKV, true, 4>, grid, 0, st, a);
+    else if (pmax == 4) launch_score(block_score_one<CPU, HKV, false, 4>, grid, 0, st, a);
+    else launch_score(block_score_one<CPU, HKV, false, 8>, grid, 0, st, a);
 }
 
 template <int CPU, int HKV, int RPB>
 void dispatch_small_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
-    if (a.G == 1) hipLaunchKernelGGL((block_score_small<CPU, HKV, true, 1, RPB>), grid, dim3(kThreads), 0, st, a);
-    else if (a.G == 2) hipLaunchKernelGGL((block_score_small<CPU, HKV, true, 2, RPB>), grid, dim3(kThreads), 0, st, a);
-    else if (a.G == 4) hipLaunchKernelGGL((block_score_small<CPU, HKV, true, 4, RPB>), grid, dim3(kThreads), 0, st, a);
-    else if (pmax == 4) hipLaunchKernelGGL((block_score_small<CPU, HKV, false, 4, RPB>), grid, dim3(kThreads), 0, st, a);
-    else hipLaunchKernelGGL((block_score_small<CPU, HKV, false, 8, RPB>), grid, dim3(kThreads), 0, st, a);
+    if (a.G == 1) launch_score(block_score_small<CPU, HKV, true, 1, RPB>, grid, 0, st, a);
+    else if (a.G == 2) launch_score(block_score_small<CPU, HKV, true, 2, RPB>, grid, 0, st, a);
+    else if (a.G == 4) launch_score(block_score_small<CPU, HKV, true, 4, RPB>, grid, 0, st, a);
+    else if (pmax == 4) launch_score(block_score_small<CPU, HKV, false, 4, RPB>, grid, 0, st, a);
+    else launch_score(block_score_small<CPU, HKV, false, 8, RPB>, grid, 0, st, a);
 }
 
 // Blocks of 1 or 2 KiB with 1, 2 or 4 KV heads; false when no instance exists.
@@ -1038,9 +1048,6 @@ bool dispatch_one(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
         default: return false;
     }
 }
-
-thread_local hipEvent_t g_prof_before = nullptr;
-thread_local hipEvent_t g_prof_after = nullptr;
 
 bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
@@ -1113,13 +1120,11 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     while (TB > 1 && TB * Hkv > kMaxTileHeads) TB >>= 1;
     // keep at least ~8 workgroups per CU in flight when the problem allows it
     while (TB > 1 && (int64_t)B * ucm::ceil_div(max_blocks, TB) < 2048) TB >>= 1;
-    if (env_int("UCM_TB", 0) > 0) TB = env_int("UCM_TB", 0);
     if (TB > kMaxTile) TB = kMaxTile;
     while (TB > 1 && TB * Hkv > kMaxTileHeads) TB >>= 1;
     a.TB = TB;
     const dim3 grid((unsigned)ucm::ceil_div(max_blocks, TB), (unsigned)B);
 
-    const bool prof = g_prof_before && g_prof_after;
     if (fast) {
         const int pmax = planes_for_group(a.G);
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
@@ -1129,15 +1134,13 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             rc = ucm::launch_status("plane_kernel");
             if (rc != UCM_OK) return rc;
         }
-        if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_before, st));
         const int rpb = (int)(((int64_t)BS * Hkv * cpu) >> 6);
-        int split = (rpb >= 4 && rpb % 4 == 0) ? 1 : 0;
-        if (env_int("UCM_SPLIT", -1) >= 0) split = env_int("UCM_SPLIT", -1);
+        const int split = (rpb >= 4 && rpb % 4 == 0) ? 1 : 0;
         const int rpw = split ? rpb / 4 : rpb;
-        const int u = env_int("UCM_UNROLL", rpw);
+        const int u = rpw;
         // blocks of >= 4 KiB: one block per workgroup with the head count compiled in
         bool done = false;
-        if (split && Hkv <= 16 && env_int("UCM_ONE", 1)) {
+        if (split && Hkv <= 16) {
             a.TB = 1;
             const dim3 grid1((unsigned)max_blocks, (unsigned)B);
             if (cpu == 1) done = dispatch_one<1>(a, pmax, grid1, st);
@@ -1145,9 +1148,9 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             else done = dispatch_one<4>(a, pmax, grid1, st);
         }
         if (!done) a.TB = TB;
-        if (!done && !split && env_int("UCM_SMALL", 1)) {
-            // 8 blocks per workgroup: every wave gets one round of 4 loads
-            int tbs = env_int("UCM_TB", 8);
+        if (!done && !split) {
+            // 16 blocks per workgroup: every wave gets two rounds of 4 loads
+            int tbs = 16;
             if (tbs > kMaxTile) tbs = kMaxTile;
             while (tbs > 1 && tbs * Hkv > kMaxTileHeads) tbs >>= 1;
             a.TB = tbs;
@@ -1163,10 +1166,8 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             else dispatch_fast<4>(a, pmax, split, u, grid, st);
         }
     } else {
-        if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_before, st));
-        hipLaunchKernelGGL(block_score_generic, grid, dim3(kThreads), (size_t)Hq * Wd * 4, st, a);
+        launch_score(block_score_generic, grid, (size_t)Hq * Wd * 4, st, a);
     }
-    if (prof) UCM_HIP_TRY(hipEventRecord(g_prof_after, st));
     rc = ucm::launch_status("block_score");
     if (rc != UCM_OK) return rc;
 
@@ -1180,11 +1181,11 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     s.flags = flags; s.out_idx = out_idx; s.out_score = out_score;
     const int rows_total = B * s.Ho;
     const dim3 wgrid((unsigned)ucm::ceil_div(rows_total, kThreads / kWave));
-    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256 && env_int("UCM_WSEL", 1)) {
+    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256) {
         hipLaunchKernelGGL(select_wave_kernel<4>, wgrid, dim3(kThreads), 0, st, s, rows_total);
         return ucm::launch_status("select_wave_kernel");
     }
-    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 1024 && env_int("UCM_WSEL", 1)) {
+    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 1024) {
         hipLaunchKernelGGL(select_wave_kernel<16>, wgrid, dim3(kThreads), 0, st, s, rows_total);
         return ucm::launch_status("select_wave_kernel");
     }
