@@ -279,11 +279,12 @@ __global__ __launch_bounds__(kThreads) void block_score_fast(ScoreArgs a, int sp
 // constant, so the lane -> (head, piece) map, the token of a piece and the wave reduction
 // are all shifts and DPP-friendly shuffles.
 // ---------------------------------------------------------------------------------------
-template <int CPU, int HKV, bool DIRECT, int GP>
+template <int CPU, int HKV, bool DIRECT, int GP, bool EXACT>
 __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
 {
+    // EXACT: the block is exactly 16 KiB (4 runs per wave): one batch of loads, no loop
     constexpr int PERIOD = HKV * CPU;  // pieces per token (a power of two <= 64)
-    __shared__ int smin[HKV];
+    __shared__ int smin[kThreads / kWave][HKV];  // one row of partial minima per wave
     const int b = blockIdx.y, j = blockIdx.x;
     const int lane = lane_id();
     const int wid = wave_id();
@@ -310,7 +311,7 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
     const int pos0 = j * a.BS;
     if (pos0 >= len) return;  // j >= ceil(len / BS); the grid never exceeds max_blocks
     const int64_t pb = physical_block(a, b, j);
-    const int rpw = (a.BS * PERIOD) >> 8;  // runs per wave (a block has 4*rpw runs)
+    const int rpw = EXACT ? 4 : (a.BS * PERIOD) >> 8;  // runs per wave (a block has 4*rpw runs)
     const u32x4* base = reinterpret_cast<const u32x4*>(a.kc + (pb < 0 ? 0 : pb) * a.ks_block) + lane;
 
     // first batch of code loads goes out before anything waits
@@ -318,7 +319,7 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
 #pragma unroll
     for (int u = 0; u < 4; ++u) kv[u] = (u32x4)(0u);
     if (pb >= 0) {
-        if (rpw >= 4) {
+        if (EXACT || rpw >= 4) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * u) << 6));
         } else {
@@ -327,7 +328,6 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
                 if (u < rpw) kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * u) << 6));
         }
     }
-    if (threadIdx.x < HKV) smin[threadIdx.x] = kInf;
     if (!DIRECT) {
 #pragma unroll
         for (int p = 0; p < GP; ++p)
@@ -359,10 +359,10 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
                 if (CPU >= 2) d += __shfl_xor(d, 1);
                 if (CPU >= 4) d += __shfl_xor(d, 2);
                 const int t = (((wid + 4 * (k0 + u)) << 6) + lane) / PERIOD;
-                if (k0 + u < rpw && pos0 + t < len && d < m) m = d;
+                if ((EXACT || k0 + u < rpw) && pos0 + t < len && d < m) m = d;
             }
             // next batch (blocks larger than 16 KiB)
-            if (k0 + 4 < rpw) {
+            if (!EXACT && k0 + 4 < rpw) {
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     kv[u] = (u32x4)(0u);
@@ -377,14 +377,16 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
             m = o < m ? o : m;
         }
     }
-    __syncthreads();  // smin initialised
-    if (pb >= 0 && lane < PERIOD && part == 0) atomicMin(&smin[h], m);
+    if (lane < PERIOD && part == 0) smin[wid][h] = m;
     __syncthreads();
     if (threadIdx.x < HKV) {
+        int dmin = smin[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < kThreads / kWave; ++w) dmin = smin[w][threadIdx.x] < dmin ? smin[w][threadIdx.x] : dmin;
         const int full = a.G * 32 * a.Wd;
         const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
         const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
-        const int sc = pb < 0 ? -1 : (forced ? full : full - smin[threadIdx.x]);
+        const int sc = pb < 0 ? -1 : (forced ? full : full - dmin);
         a.scores[((int64_t)b * HKV + threadIdx.x) * a.max_blocks + j] = sc;
     }
 }
@@ -1002,14 +1004,21 @@ bool dispatch_fast(const ScoreArgs& a, int pmax, int split, int u, dim3 grid, hi
     return true;
 }
 
+template <int CPU, int HKV, bool EXACT>
+void dispatch_one_e(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+{
+    if (a.G == 1) launch_score(block_score_one<CPU, HKV, true, 1, EXACT>, grid, 0, st, a);
+    else if (a.G == 2) launch_score(block_score_one<CPU, HKV, true, 2, EXACT>, grid, 0, st, a);
+    else if (a.G == 4) launch_score(block_score_one<CPU, HKV, true, 4, EXACT>, grid, 0, st, a);
+    else if (pmax == 4) launch_score(block_score_one<CPU, HKV, false, 4, EXACT>, grid, 0, st, a);
+    else launch_score(block_score_one<CPU, HKV, false, 8, EXACT>, grid, 0, st, a);
+}
+
 template <int CPU, int HKV>
 void dispatch_one_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
-    if (a.G == 1) launch_score(block_score_one<CPU, HKV, true, 1>, grid, 0, st, a);
-    else if (a.G == 2) launch_score(block_score_one<CPU, HKV, true, 2>, grid, 0, st, a);
-    else if (a.G == 4) launch_score(block_score_one<CPU, HKV, true, 4>, grid, 0, st, a);
-    else if (pmax == 4) launch_score(block_score_one<CPU, HKV, false, 4>, grid, 0, st, a);
-    else launch_score(block_score_one<CPU, HKV, false, 8>, grid, 0, st, a);
+    if (((int64_t)a.BS * HKV * CPU) >> 8 == 4) dispatch_one_e<CPU, HKV, true>(a, pmax, grid, st);
+    else dispatch_one_e<CPU, HKV, false>(a, pmax, grid, st);
 }
 
 template <int CPU, int HKV, int RPB>
