@@ -303,6 +303,8 @@ def main():
     for e in ev_b + ev_a:
         e.record()  # creates the underlying hipEvent_t so its handle can be handed to the library
     torch.cuda.synchronize()
+    for i in range(args.warmup):  # untimed: the eager pass starts after a host-side pause
+        step(i)
     for i in range(args.steps):
         L.ucm_hamming_topk_set_profile_events(ev_b[i].cuda_event, ev_a[i].cuda_event)
         idx, sc = step(args.warmup + i)
@@ -340,13 +342,15 @@ def main():
                    "cache_rotation": R, "step": "encode 32 new keys + encode 32x32 queries + score + select",
                    "timed_region": (f"hipGraph replays, {GS} consecutive steps per graph"
                                     if graphs is not None else "eager launches"),
-                   "roofline_pass": "same steps launched eagerly, HIP events around the block-score kernel"},
+                   "roofline_pass": "same steps launched eagerly, dispatch start/stop events of the block-score kernel"},
         "p50_step_latency_us": step_ms[len(step_ms) // 2] * 1e3,
         "p90_step_latency_us": step_ms[max(0, int(len(step_ms) * 0.9) - 1)] * 1e3,
         "roofline": {"bound": "hbm", "kernel": "block_score_one", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": HBM_TRAFFIC_PER_LAUNCH, "algorithmic_bytes": alg, "kernel_avg_us": kern_avg_ms * 1e3,
-                     "kernel_p50_us": sorted(kern_ms)[len(kern_ms) // 2] * 1e3},
+                     "kernel_p50_us": sorted(kern_ms)[len(kern_ms) // 2] * 1e3,
+                     "kernel_p90_us": sorted(kern_ms)[int(len(kern_ms) * 0.9)] * 1e3,
+                     "kernel_max_us": max(kern_ms) * 1e3},
     }
     if not args.skip_cpu:
         line["cpu_baseline"] = cpu_baseline(torch, caches[0], tables[0], qc, lens)

@@ -132,6 +132,73 @@ def test_compute_hash_and_cache(dtype, slot_dtype):
         assert_codes_match(codes[:, h], x[:, h].float().numpy(), W[h].float().numpy())
 
 
+# Row counts above 256 per head take the tiled MFMA kernel; the shapes below reach each of its
+# compile-time variants: column tiles per group 4/2/1, unrolled and run-time group counts,
+# the pipelined path (K <= 128) and the line-by-line path (K >= 256), partial last tiles and
+# workgroups whose run of tiles ends past the tensor.
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,N", [(257, 128, 128), (515, 128, 128), (1000, 128, 256), (4100, 128, 128),
+                                   (700, 128, 512), (300, 128, 192), (300, 128, 96), (640, 128, 64),
+                                   (385, 128, 32), (513, 64, 64), (900, 64, 128), (300, 64, 32),
+                                   (600, 256, 128), (300, 512, 256), (2049, 512, 128)])
+def test_tiled_kernel_shapes(dtype, M, K, N):
+    rng = rng_for(2000 + M + K + N)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    W = torch.from_numpy(rng.standard_normal((K, N)).astype(np.float32)).to(dtype)
+    enc = make_encoder(K, N, dtype, W)
+    codes = enc.compute_hash(x.cuda())
+    assert tuple(codes.shape) == (M, N // 8)
+    assert_codes_match(codes.cpu().numpy(), x.float().numpy(), W.float().numpy())
+
+
+@pytest.mark.parametrize("slot_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("T,H,BS", [(700, 8, 128), (1029, 4, 48), (300, 2, 16)])
+def test_tiled_kernel_paged_store(slot_dtype, T, H, BS):
+    """Fused cache write of the tiled kernel: permuted and invalid slots, a block size that is
+    not a power of two, head-interleaved input rows, cells outside the slots untouched."""
+    rng = rng_for(12 + T)
+    K = N = 128
+    NB = (T + BS - 1) // BS + 3
+    x = bf16_round(rng.standard_normal((T, H, K)))
+    W = bf16_round(rng.standard_normal((H, K, N)))
+    slots = rng.permutation(NB * BS)[:T].astype(np.int64)
+    slots[3] = -1
+    slots[T // 2] = NB * BS
+    slots[T - 1] = NB * BS + 77
+    enc = make_encoder(K, N, torch.bfloat16, W, n_w=H, hpw=1)
+    cache = torch.full((NB, BS, H, N // 8), 0xAB, dtype=torch.uint8, device="cuda")
+    enc.compute_hash_and_cache(x.cuda(), torch.from_numpy(slots).to(slot_dtype).cuda(), cache,
+                               block_size=BS)
+    codes = np.stack([brute.hash_encode(x[:, h].float().numpy(), W[h].float().numpy())
+                      for h in range(H)], axis=1)  # [T,H,4] uint32
+    expect = np.full((NB, BS, H, N // 32), 0xABABABAB, np.uint32)
+    c_api.code_scatter(np.ascontiguousarray(codes), slots, expect, BS)
+    got = cache.cpu().numpy().view(np.uint32)
+    if not np.array_equal(got, expect):
+        # differences may only be margin bits of rows that were written
+        gpu_codes = enc.compute_hash(x.cuda(), per_head=True).cpu().numpy()
+        for h in range(H):
+            assert_codes_match(gpu_codes[:, h], x[:, h].float().numpy(), W[h].float().numpy())
+        expect2 = np.full((NB, BS, H, N // 32), 0xABABABAB, np.uint32)
+        c_api.code_scatter(np.ascontiguousarray(gpu_codes).view(np.uint32), slots, expect2, BS)
+        assert np.array_equal(got, expect2)
+
+
+def test_tiled_kernel_strided_rows_and_dense_heads():
+    """Rows that are a slice of a wider tensor (row pitch 3*K) and a dense per-head output."""
+    rng = rng_for(13)
+    T, H, K, N = 520, 3, 128, 128
+    wide = bf16_round(rng.standard_normal((T, H, 3 * K))).cuda()
+    x = wide[:, :, K:2 * K]
+    W = bf16_round(rng.standard_normal((K, N)))
+    enc = make_encoder(K, N, torch.bfloat16, W)
+    c = enc.compute_hash(x, per_head=True).cpu().numpy()  # keeps the row pitch; one matrix
+    assert c.shape == (T, H, N // 8)
+    xs = x.float().cpu().numpy()
+    for h in range(H):
+        assert_codes_match(c[:, h], xs[:, h], W.float().numpy())
+
+
 def test_cache_as_bf16_view_and_shared_weight():
     """The plugin allocates the code cache as bfloat16 [NB,BS,H,hash_numbers/2]
     (hash_encoder.py:509-546) and uses one projection for all heads."""

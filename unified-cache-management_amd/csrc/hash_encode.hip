@@ -4,12 +4,16 @@
 // Follows the reference's HashEncoder (ucm/sparse/gsa_on_device/hash_encoder.py:359-370 for
 // the arithmetic and bit order, :263-356 for the fused cache write, :136-195 for the code
 // scatter).  Design for MI355X:
-//   * bf16 / fp16 inputs go through v_mfma_f32_32x32x16_{bf16,f16}: a wave owns 32 rows, keeps
-//     their K values in registers (A operand, one 16-byte load per lane and k-step) and walks
-//     the hash columns 32 at a time; the projection matrix slice lives in LDS, transposed so a
-//     B operand is one 16-byte LDS read;
-//   * the sign of an accumulator register is a v_cmp whose 64-bit lane mask already IS two
-//     packed output words (32 columns of two rows), so packing costs no shuffles;
+//   * bf16 / fp16 inputs go through v_mfma_f32_32x32x16_{bf16,f16}; a wave owns 32 rows and
+//     walks the hash columns 32 at a time; the projection matrix slice lives in LDS, transposed
+//     so that an operand is one 16-byte LDS read;
+//   * rows are fetched with fully coalesced loads (8 rows x one 128-byte line per instruction,
+//     two row tiles in flight per wave) and redistributed to the MFMA operand layout through a
+//     swizzled 4 KiB LDS patch per wave: loading straight in operand layout touches every
+//     cache line from four instructions and costs about a third of the bandwidth;
+//   * the MFMA runs transposed (projection matrix as A, input rows as B), so a lane's 16
+//     accumulators are 16 hash bits of one row: the signs are packed in-lane, interleaved with
+//     the next column tile's MFMAs, and one half-wave swap joins the two halves of a word;
 //   * the row's words are written with one store, either to a dense [T,H,Wd] tensor or to
 //     cache[slot/BS, slot%BS, h, :].
 // Everything else (fp32 operands, odd shapes, unaligned rows) takes a plain FMA kernel.
@@ -22,7 +26,11 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kRowsPerWave = 32;
-constexpr int kRowsPerWg = 128;
+constexpr int kMfmaThreads = 256;                                // encode_mfma_kernel workgroup
+constexpr int kMfmaWaves = kMfmaThreads / 64;
+constexpr int kRowsPerWg = kMfmaWaves * kRowsPerWave;            // 128 rows per workgroup tile
+constexpr int kTilesPerWg = 4;                                   // row tiles a workgroup encodes
+constexpr int kStageBytes = kRowsPerWave * 128;                  // per wave: one 128-byte line of 32 rows
 constexpr int kPad = 8;  // elements of padding per LDS row (16 bytes)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -37,10 +45,10 @@ struct EncArgs {
     int64_t x_stride_t, x_stride_h;
     const void* w;
     int n_w, heads_per_w, N;
-    // dense output
+    // dense output (host side only: normalize_output() folds it into the paged form)
     uint32_t* out;
     int64_t out_stride_t, out_stride_h;
-    // paged output (cache != null)
+    // paged output; slot == null means slot(t) = t
     const void* slot;
     int slot_is_i64;
     uint32_t* cache;
@@ -57,11 +65,51 @@ __device__ __forceinline__ int weight_index(const EncArgs& a, int h)
     return wi < a.n_w ? wi : a.n_w - 1;
 }
 
-// Destination of the code words of row (t, h), or null when the row must be skipped.
-__device__ __forceinline__ uint32_t* row_dst(const EncArgs& a, int64_t t, int h)
+// A dense [T, H, Wd] output is handled as a paged one with one token per block and the
+// identity slot mapping (normalize_output() on the host), so the kernels know one layout.
+//
+// Raw slot of row t as read from memory: the row index itself when there is no slot array.
+// Split from the address arithmetic so that a kernel can issue the read long before it needs
+// the value; a 32-bit slot is widened only in slot_dst().
+struct RawSlot {
+    uint32_t lo, hi;
+};
+__device__ __forceinline__ RawSlot fetch_slot(const EncArgs& a, int64_t t)
 {
-    if (!a.cache) return a.out + t * a.out_stride_t + (int64_t)h * a.out_stride_h;
-    const int64_t s = a.slot_is_i64 ? ((const int64_t*)a.slot)[t] : (int64_t)((const int32_t*)a.slot)[t];
+    RawSlot s;
+    if (!a.slot) {
+        s.lo = (uint32_t)t;
+        s.hi = (uint32_t)((uint64_t)t >> 32);
+    } else if (a.slot_is_i64) {
+        const uint2 v = ((const uint2*)a.slot)[t];
+        s.lo = v.x;
+        s.hi = v.y;
+    } else {
+        s.lo = ((const uint32_t*)a.slot)[t];
+        s.hi = 0;
+    }
+    return s;
+}
+
+// Branch-free variant for a kernel that prefetches slots: two unconditional 4-byte reads whose
+// results land in fixed registers (a value merged from several branches would have to be
+// waited for at the merge).  Without a slot array the reads hit the input rows instead (valid
+// memory: the caller guarantees rows of at least 16 bytes) and slot_dst_of() ignores them.
+__device__ __forceinline__ RawSlot fetch_slot_flat(const EncArgs& a, int64_t t)
+{
+    const char* p = a.slot ? (const char*)a.slot : (const char*)a.x;
+    const int sh = a.slot_is_i64 ? 3 : 2;
+    const char* q = p + (t << sh);
+    RawSlot s;
+    s.lo = *(const uint32_t*)q;
+    s.hi = *(const uint32_t*)(q + (a.slot_is_i64 ? 4 : 0));
+    return s;
+}
+
+// Destination of the code words of head h of the row with slot s, or null when the row must
+// be skipped (slot outside the cache).
+__device__ __forceinline__ uint32_t* slot_dst(const EncArgs& a, int64_t s, int h)
+{
     if (s < 0 || s >= a.NB * (int64_t)a.BS) return nullptr;
     int64_t blk, tok;
     if (a.bs_shift >= 0) {  // the usual case: no integer division
@@ -77,43 +125,47 @@ __device__ __forceinline__ uint32_t* row_dst(const EncArgs& a, int64_t t, int h)
     return a.cache + blk * a.cs_block + tok * a.cs_token + (int64_t)h * a.cs_head;
 }
 
-// Sign-packs four accumulator registers of a 32x32 MFMA tile.  The 64-bit lane mask of
-// "acc > 0" is two finished output words (32 columns of rows R and R+4); v_writelane_b32 drops
-// each into the lane that owns the row, leaving the other lanes untouched.  The wait states
-// between the vector compares that produce the masks and the lane writes that read them are
-// inserted by hand: the compiler does not look inside inline assembly.
-template <int R>
-__device__ __forceinline__ uint32_t pack_rows4(uint32_t word, float a0, float a1, float a2, float a3)
+// Slot value of row t from its raw words.
+__device__ __forceinline__ int64_t slot_value(const EncArgs& a, RawSlot raw, int64_t t)
 {
-    const unsigned long long m0 = __ballot(a0 > 0.0f), m1 = __ballot(a1 > 0.0f);
-    const unsigned long long m2 = __ballot(a2 > 0.0f), m3 = __ballot(a3 > 0.0f);
-    asm("s_nop 4\n\t"
-        "v_writelane_b32 %0, %1, %9\n\ts_nop 0\n\t"
-        "v_writelane_b32 %0, %2, %10\n\ts_nop 0\n\t"
-        "v_writelane_b32 %0, %3, %11\n\ts_nop 0\n\t"
-        "v_writelane_b32 %0, %4, %12\n\ts_nop 0\n\t"
-        "v_writelane_b32 %0, %5, %13\n\ts_nop 0\n\t"
-        "v_writelane_b32 %0, %6, %14\n\ts_nop 0\n\t"
-        "v_writelane_b32 %0, %7, %15\n\ts_nop 0\n\t"
-        "v_writelane_b32 %0, %8, %16"
-        : "+v"(word)
-        : "s"((uint32_t)m0), "s"((uint32_t)m1), "s"((uint32_t)m2), "s"((uint32_t)m3),
-          "s"((uint32_t)(m0 >> 32)), "s"((uint32_t)(m1 >> 32)), "s"((uint32_t)(m2 >> 32)),
-          "s"((uint32_t)(m3 >> 32)),
-          "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3), "n"(R + 4), "n"(R + 5), "n"(R + 6), "n"(R + 7));
-    return word;
+    if (!a.slot) return t;
+    return a.slot_is_i64 ? (int64_t)(((uint64_t)raw.hi << 32) | raw.lo) : (int64_t)(int32_t)raw.lo;
 }
 
-// Accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the tile:
-// registers 4g..4g+3 are rows 8g..8g+3 (low mask halves) and 8g+4..8g+7 (high halves).
-__device__ __forceinline__ uint32_t pack_tile(const f32x16& acc)
+__device__ __forceinline__ uint32_t* row_dst(const EncArgs& a, int64_t t, int h)
 {
-    uint32_t word = 0;
-    word = pack_rows4<0>(word, acc[0], acc[1], acc[2], acc[3]);
-    word = pack_rows4<8>(word, acc[4], acc[5], acc[6], acc[7]);
-    word = pack_rows4<16>(word, acc[8], acc[9], acc[10], acc[11]);
-    word = pack_rows4<24>(word, acc[12], acc[13], acc[14], acc[15]);
-    return word;
+    return slot_dst(a, slot_value(a, fetch_slot(a, t), t), h);
+}
+
+// The MFMA is issued with the projection matrix as its A operand and the input rows as B, so
+// accumulator register v of lane l is hash column 8*(v/4) + 4*(l/32) + v%4 of input row l%32:
+// a lane holds 16 of the 32 sign bits of ONE row's output word and packs them in-lane.
+// Plain C++ on purpose: the wait states between an MFMA and the first read of its result, and
+// between a compare and the use of its mask, are inserted by the compiler only for
+// instructions it can see.
+//
+// Half of the row's word: bit 8g + j is the sign of accumulator 4g + j (g, j in 0..3).  Two
+// independent chains (g = 3,2 and g = 1,0) halve the dependent-instruction latency.
+__device__ __forceinline__ uint32_t pack_half(const f32x16& acc)
+{
+    uint32_t hi = 0, lo = 0;
+#pragma unroll
+    for (int g = 1; g >= 0; --g) {
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+            hi |= (acc[4 * (g + 2) + j] > 0.0f ? 1u : 0u) << (8 * g + j);
+            lo |= (acc[4 * g + j] > 0.0f ? 1u : 0u) << (8 * g + j);
+        }
+    }
+    return (hi << 16) | lo;
+}
+
+// Lanes l and l+32 hold the two interleaved halves (nibbles 0,2,4,6 and 1,3,5,7) of row l%32's
+// word; `w` must already be shifted left by 4 in the upper lanes.  Returns the full word in both.
+__device__ __forceinline__ uint32_t join_halves(uint32_t w)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return r[0] | r[1];
 }
 
 template <typename V>
@@ -133,13 +185,20 @@ struct Mfma<f16x8> {
     }
 };
 
-// V: 8-element vector type of the 16-bit input format.  KS = K / 16.
-// grid = (row-tile workers, column slices, heads); a workgroup loads its W slice into LDS once
-// and then walks row tiles of 128 rows (32 per wave) with a grid stride.
-template <typename V, int KS>
-__global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
+// V: 8-element vector type of the 16-bit input format.  KS = K / 16.  NQ: column tiles of 32
+// handled per group (divides the slice's tile count; 4 gives one 16-byte store per row).  NG:
+// groups per slice when known at compile time (the group loop is then unrolled, which keeps
+// the compiler from draining all outstanding loads in front of it), 0 = run-time count.
+// grid = (groups of kTilesPerWg row tiles, column slices, heads); a workgroup stages its W slice
+// in LDS once and then encodes its run of row tiles (128 rows each, 32 per wave).  Two waves
+// per SIMD: the register budget holds two row tiles in flight per wave next to the one being
+// computed.  The pipelined path is straight-line code with the same loads on every path, so
+// that the compiler can count outstanding loads exactly and never waits for a prefetch it has
+// just issued.
+template <typename V, int KS, int NQ, int NG>
+__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 3))) void encode_mfma_kernel(EncArgs a)
 {
-    extern __shared__ uint16_t wt[];  // [BN][K + kPad], k contiguous
+    extern __shared__ uint16_t wt[];  // [BN][K + kPad], k contiguous; then the waves' staging
     constexpr int K = KS * 16;
     constexpr int KP = K + kPad;
     const int h = blockIdx.z;
@@ -147,14 +206,101 @@ __global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
     const int bn = (a.N - n0 < a.BN) ? a.N - n0 : a.BN;  // columns in this slice
     const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N;
 
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 31, kb = lane >> 5;
+    const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)h * a.x_stride_h;
+    const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
+    const int64_t first = (int64_t)blockIdx.x * kTilesPerWg;  // this workgroup's run of tiles
+
+    // Rows are fetched one 128-byte line at a time: a load instruction covers 8 rows x 128
+    // contiguous bytes (lane l: row 8j + l/8, 16-byte chunk l%8), so every cache line is touched
+    // by exactly one instruction.  Register 4L + j of a lane then holds a piece of line L that
+    // belongs to another lane's MFMA column; to_operands() redistributes through LDS.
+    // Rows past T re-read the last row (their results are discarded).  Addresses are a uniform
+    // 64-bit tile base plus a 32-bit lane offset (the host checks that a tile of rows spans
+    // less than 2 GiB).
+    auto row_offset = [&](int64_t tile, int j) -> uint32_t {
+        const int q = wave * kRowsPerWave + 8 * j + (lane >> 3);
+        const int64_t left = a.T - 1 - tile * kRowsPerWg;  // last valid row, relative to the tile
+        const uint32_t qq = (int64_t)q > left ? (uint32_t)left : (uint32_t)q;
+        return (qq * (uint32_t)a.x_stride_t + (lane & 7) * 8) * 2u;
+    };
+    // `real` = false issues the same number of loads against one cache line of the tensor's
+    // first row: the prefetch ring then has one instruction sequence on every path, which lets
+    // the compiler count outstanding loads exactly instead of waiting for all of them.
+    auto load_tile = [&](int64_t tile, V (&dstv)[KS], bool real) {
+        // masks instead of branches: both cases must be the same instruction stream
+        const uint32_t m = real ? ~0u : 0u;
+        const int64_t tc = real ? tile : (int64_t)0;
+        const char* tb = reinterpret_cast<const char*>(xbase + tc * kRowsPerWg * a.x_stride_t);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t off = row_offset(tc, j) & m;
+#pragma unroll
+            for (int L = 0; L < KS / 4; ++L)
+                dstv[4 * L + j] = __builtin_nontemporal_load(
+                    reinterpret_cast<const V*>(tb + off + ((L * 128) & m)));
+        }
+    };
+    // Per wave 4 KiB of LDS: [32 rows][8 chunks of 16 bytes], chunk c of row q stored at slot
+    // c ^ swz(q), swz(q) = (q ^ (q >> 3)) & 7, so that the row-major writes and the column reads
+    // (consecutive rows, one chunk each) spread over all banks whether the hardware serves 8 or
+    // 16 lanes of a 128-bit access per cycle.  Only this wave touches the region and a wave's
+    // LDS operations execute in order, so no workgroup barrier is needed.
+    uint8_t* stage = reinterpret_cast<uint8_t*>(wt) + (size_t)a.BN * KP * 2 + wave * kStageBytes;
+    const int wq = lane >> 3;  // row within a group of 8 written by this lane
+    uint32_t w_off[4], r_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int q = 8 * j + wq;
+        w_off[j] = q * 128 + (((lane & 7) ^ ((q ^ (q >> 3)) & 7)) << 4);
+        r_off[j] = r * 128 + (((2 * j + kb) ^ ((r ^ (r >> 3)) & 7)) << 4);
+    }
+    auto stage_line = [&](const V (&src)[KS], V (&dstv)[KS], int L) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<V*>(stage + w_off[j]) = src[4 * L + j];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) dstv[4 * L + s4] = *reinterpret_cast<const V*>(stage + r_off[s4]);
+        __builtin_amdgcn_wave_barrier();
+    };
+    auto to_operands = [&](const V (&src)[KS], V (&dstv)[KS]) {
+#pragma unroll
+        for (int L = 0; L < KS / 4; ++L) stage_line(src, dstv, L);
+    };
+    // Wide rows: no register prefetch; fetch, stage and redistribute line by line.
+    auto load_operands = [&](int64_t tile, V (&dstv)[KS]) {
+        const char* tb = reinterpret_cast<const char*>(xbase + tile * kRowsPerWg * a.x_stride_t);
+        uint32_t off[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) off[j] = row_offset(tile, j);
+#pragma unroll
+        for (int L = 0; L < KS / 4; ++L) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<V*>(stage + w_off[j]) = *reinterpret_cast<const V*>(tb + off[j] + L * 128);
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4) dstv[4 * L + s4] = *reinterpret_cast<const V*>(stage + r_off[s4]);
+            __builtin_amdgcn_wave_barrier();
+        }
+    };
+    constexpr bool kPrefetch = KS <= 8;  // two tiles of rows fit in registers
+    V av[KS];                            // MFMA operands of the current tile
+    V raw0[kPrefetch ? KS : 1];          // rows of the next two tiles as fetched
+    V raw1[kPrefetch ? KS : 1];
+
     // W[k0..k0+8][n0+8j..+8] -> wt[8j+c][k0..k0+8]: each thread transposes 8x8 patches of 16-bit
-    // elements in registers (byte permutes) and writes eight 16-byte LDS rows
-    for (int idx = threadIdx.x; idx < (K / 8) * (bn / 8); idx += kThreads) {
+    // elements in registers (byte permutes) and writes eight 16-byte LDS rows.
+    auto patch_load = [&](int idx, u32x4 (&row)[8]) {
         const int kq = idx / (bn / 8), j = idx % (bn / 8);
         const uint16_t* src = wsrc + (int64_t)(kq * 8) * a.N + n0 + 8 * j;
-        u32x4 row[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) row[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * a.N);
+    };
+    auto patch_store = [&](int idx, const u32x4 (&row)[8]) {
+        const int kq = idx / (bn / 8), j = idx % (bn / 8);
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
@@ -165,75 +311,126 @@ __global__ __launch_bounds__(kThreads) void encode_mfma_kernel(EncArgs a)
             o.w = __builtin_amdgcn_perm(row[7][c >> 1], row[6][c >> 1], sel);
             *reinterpret_cast<u32x4*>(wt + (8 * j + c) * KP + kq * 8) = o;
         }
+    };
+    constexpr bool kPipelined = kPrefetch && NG > 0;
+    if constexpr (kPipelined) {
+        // slice width known at compile time: no loop, no divergence (surplus threads redo a
+        // patch); the first two tiles' rows go out right behind the first patch loads
+        constexpr int kPatches = (K / 8) * (NQ * NG * 4);
+        constexpr int kRounds = (kPatches + kMfmaThreads - 1) / kMfmaThreads;
+#pragma unroll
+        for (int it = 0; it < kRounds; ++it) {
+            const int idx = (threadIdx.x + it * kMfmaThreads) % kPatches;
+            u32x4 row[8];
+            patch_load(idx, row);
+            if (it == 0) {
+                load_tile(first, raw0, first < tiles);
+                load_tile(first + 1, raw1, first + 1 < tiles);
+            }
+            patch_store(idx, row);
+        }
+    } else {
+        const int npatch = (K / 8) * (bn / 8);
+        for (int idx = threadIdx.x; idx < npatch; idx += kMfmaThreads) {
+            u32x4 row[8];
+            patch_load(idx, row);
+            patch_store(idx, row);
+        }
     }
     __syncthreads();
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int r = lane & 31, kb = lane >> 5;
-    const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)h * a.x_stride_h;
-    const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
     const int nt_count = bn / 32;
     const int word0 = n0 / 32;
 
-    // A operands of the wave's 32 rows of a tile; rows past T re-read the last row (discarded)
-    auto load_tile = [&](int64_t tile, V (&dstv)[KS]) {
-        int64_t t = tile * kRowsPerWg + wave * kRowsPerWave + r;
-        if (t >= a.T) t = a.T - 1;
-        const uint16_t* xr = xbase + t * a.x_stride_t + kb * 8;
+    // 32 hash columns x 32 rows: K/16 MFMAs into one accumulator tile
+    auto project = [&](int nt) {
+        f32x16 acc = {0};
+        const uint16_t* bp = wt + (nt * 32 + r) * KP + kb * 8;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dstv[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
-    };
-    constexpr bool kPrefetch = KS <= 16;  // the next tile's operands fit in registers
-    V av[KS];
-    V nx[kPrefetch ? KS : 1];
-    if (blockIdx.x < tiles) load_tile(blockIdx.x, av);
-
-    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-        const int64_t row0 = tile * kRowsPerWg + wave * kRowsPerWave;
-        const int64_t next = tile + gridDim.x;
-        if constexpr (kPrefetch) {
-            if (next < tiles) load_tile(next, nx);
-        } else {
-            if (tile != (int64_t)blockIdx.x) load_tile(tile, av);
+        for (int k0 = 0; k0 < KS; k0 += 4) {
+            V bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) bv[i] = *reinterpret_cast<const V*>(bp + (k0 + i) * 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc = Mfma<V>::run(bv[i], av[k0 + i], acc);
         }
-        const int64_t t = row0 + r;
-        const bool row_ok = t < a.T;
-        uint32_t* dst = (row_ok && lane < 32) ? row_dst(a, t, h) : nullptr;
-
-        for (int nt0 = 0; nt0 < nt_count; nt0 += 4) {
-            uint32_t words[4] = {0, 0, 0, 0};
+        return acc;
+    };
+    // All column tiles of the wave's 32 rows of `tile`, from the operands in av.
+    auto encode_rows = [&](int64_t tile, uint32_t* dst) {
+        // NQ column tiles per group, straight-line: the sign packing of one tile is independent
+        // of the next tile's MFMAs, so the two can overlap
+        auto group = [&](int nt0) {
+            uint32_t words[NQ];
+            f32x16 cur = project(nt0);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int nt = nt0 + q;
-                if (nt >= nt_count) break;
-                f32x16 acc = {0};
-                const uint16_t* bp = wt + (nt * 32 + r) * KP + kb * 8;
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const V bv = *reinterpret_cast<const V*>(bp + ks * 16);
-                    acc = Mfma<V>::run(av[ks], bv, acc);
-                }
-                // accumulator v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
-                const uint32_t word = pack_tile(acc);
-                words[q] = word;
+            for (int q = 1; q < NQ; ++q) {
+                const f32x16 nxt = project(nt0 + q);
+                words[q - 1] = pack_half(cur);
+                cur = nxt;
             }
+            words[NQ - 1] = pack_half(cur);
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) words[q] = join_halves(kb ? words[q] << 4 : words[q]);
             if (dst) {
-                const int nq = (nt_count - nt0 < 4) ? nt_count - nt0 : 4;
                 uint32_t* d = dst + word0 + nt0;
-                if (nq == 4 && (((uintptr_t)d) & 15) == 0) {
-                    u32x4 v = {words[0], words[1], words[2], words[3]};
+                if (NQ == 4 && (((uintptr_t)d) & 15) == 0) {
+                    u32x4 v = {words[0], words[1 % NQ], words[2 % NQ], words[3 % NQ]};
                     *reinterpret_cast<u32x4*>(d) = v;
                 } else {
-                    for (int q = 0; q < nq; ++q) d[q] = words[q];
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) d[q] = words[q];
                 }
             }
-        }
-        if constexpr (kPrefetch) {
-            if (next < tiles) {
+        };
+        if constexpr (NG > 0) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) av[ks] = nx[ks];
+            for (int g = 0; g < NG; ++g) group(g * NQ);
+        } else {
+            for (int nt0 = 0; nt0 < nt_count; nt0 += NQ) group(nt0);
+        }
+    };
+    // Lanes 0..31 own one row each.  The row's slot is fetched together with the tile's rows,
+    // two tiles ahead, so that its value never has to be waited for behind younger loads
+    // (a wave's loads return in issue order).
+    auto tile_slot = [&](int64_t tile) -> RawSlot {
+        int64_t t = tile * kRowsPerWg + wave * kRowsPerWave + r;
+        if (t >= a.T) t = a.T - 1;  // in-bounds read; the row itself is masked in slot_target()
+        return fetch_slot_flat(a, t);
+    };
+    auto slot_target = [&](int64_t tile, RawSlot s) -> uint32_t* {
+        const int64_t t = tile * kRowsPerWg + wave * kRowsPerWave + r;
+        return (t < a.T && lane < 32) ? slot_dst(a, slot_value(a, s, t), h) : nullptr;
+    };
+
+    if constexpr (kPipelined) {
+        // ring of two fetched tiles, fully unrolled; tiles past the end are dummy loads and
+        // masked stores
+        RawSlot slot0 = tile_slot(first < tiles ? first : tiles - 1);
+        RawSlot slot1 = tile_slot(first + 1 < tiles ? first + 1 : tiles - 1);
+#pragma unroll
+        for (int i = 0; i < kTilesPerWg; i += 2) {
+            const int64_t t0 = first + i, t1 = first + i + 1;
+            to_operands(raw0, av);
+            uint32_t* dst = t0 < tiles ? slot_target(t0, slot0) : nullptr;
+            if (i + 2 < kTilesPerWg) {
+                slot0 = tile_slot(t0 + 2 < tiles ? t0 + 2 : tiles - 1);
+                load_tile(t0 + 2, raw0, t0 + 2 < tiles);
             }
+            encode_rows(t0, dst);
+            to_operands(raw1, av);
+            dst = t1 < tiles ? slot_target(t1, slot1) : nullptr;
+            if (i + 3 < kTilesPerWg) {
+                slot1 = tile_slot(t1 + 2 < tiles ? t1 + 2 : tiles - 1);
+                load_tile(t1 + 2, raw1, t1 + 2 < tiles);
+            }
+            encode_rows(t1, dst);
+        }
+    } else {
+        for (int64_t tile = first; tile < first + kTilesPerWg && tile < tiles; ++tile) {
+            const RawSlot sl = tile_slot(tile);
+            load_operands(tile, av);
+            encode_rows(tile, slot_target(tile, sl));
         }
     }
 }
@@ -284,9 +481,10 @@ __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
     for (int ks = 0; ks < KS; ++ks) {
         V bv;
         __builtin_memcpy(&bv, bw[ks], 16);
-        acc = Mfma<V>::run(av[ks], bv, acc);
+        acc = Mfma<V>::run(bv, av[ks], acc);
     }
-    const uint32_t word = pack_tile(acc);
+    const uint32_t half = pack_half(acc);
+    const uint32_t word = join_halves(kb ? half << 4 : half);
     if (row_ok && lane < 32) {
         uint32_t* dst = row_dst(a, t, h);
         if (dst) dst[nt] = word;
@@ -347,20 +545,6 @@ __global__ __launch_bounds__(kThreads) void code_scatter_kernel(const uint32_t* 
     }
 }
 
-int num_cus()
-{
-    static int cached = 0;
-    if (cached) return cached;
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-        prop.multiProcessorCount > 0)
-        cached = prop.multiProcessorCount;
-    else
-        cached = 256;
-    return cached;
-}
-
 // Widest slice of hash columns (a multiple of 32 that divides N) whose transposed LDS image
 // stays within `cap` bytes; 0 when not even 32 columns fit.
 int pick_slice(int N, int K, size_t cap)
@@ -370,32 +554,49 @@ int pick_slice(int N, int K, size_t cap)
     return 0;
 }
 
-template <typename V, int KS>
-int launch_mfma(EncArgs a, hipStream_t st)
+template <typename V, int KS, int NQ, int NG>
+int launch_mfma_q(const EncArgs& a, size_t lds, const dim3& grid, hipStream_t st)
 {
-    constexpr int K = KS * 16;
     // 0 = not tried, 1 = large LDS allocations allowed, -1 = refused by the runtime
     static int big_lds = 0;
-    a.BN = pick_slice(a.N, K, 144 * 1024);
-    if ((size_t)a.BN * (K + kPad) * 2 > 64 * 1024) {
+    if (lds > 64 * 1024) {
         if (big_lds == 0) {
             const hipError_t e =
-                hipFuncSetAttribute((const void*)encode_mfma_kernel<V, KS>,
+                hipFuncSetAttribute((const void*)encode_mfma_kernel<V, KS, NQ, NG>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
             if (e != hipSuccess) (void)hipGetLastError();
             big_lds = (e == hipSuccess) ? 1 : -1;
         }
-        if (big_lds < 0) a.BN = pick_slice(a.N, K, 64 * 1024);
+        if (big_lds < 0) return UCM_EUNSUPPORTED;
     }
-    if (a.BN == 0) return ucm::fail(UCM_EUNSUPPORTED, "no LDS slice fits K=%d", K);
-    const size_t lds = (size_t)a.BN * (K + kPad) * 2;
-    const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
-    const int slices = a.N / a.BN;
-    int64_t per = (int64_t)num_cus() * 4 / ((int64_t)slices * a.H);
-    if (per < 1) per = 1;
-    const dim3 grid((unsigned)(tiles < per ? tiles : per), (unsigned)slices, (unsigned)a.H);
-    hipLaunchKernelGGL((encode_mfma_kernel<V, KS>), grid, dim3(kThreads), lds, st, a);
+    hipLaunchKernelGGL((encode_mfma_kernel<V, KS, NQ, NG>), grid, dim3(kMfmaThreads), lds, st, a);
     return ucm::launch_status("encode_mfma_kernel");
+}
+
+template <typename V, int KS>
+int launch_mfma(EncArgs a, hipStream_t st)
+{
+    constexpr int K = KS * 16;
+    constexpr size_t kStage = (size_t)kMfmaWaves * kStageBytes;
+    for (size_t cap : {(size_t)144 * 1024, (size_t)64 * 1024}) {
+        a.BN = pick_slice(a.N, K, cap - kStage);
+        if (a.BN == 0) return ucm::fail(UCM_EUNSUPPORTED, "no LDS slice fits K=%d", K);
+        const size_t lds = (size_t)a.BN * (K + kPad) * 2 + kStage;
+        const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
+        const int slices = a.N / a.BN;
+        const dim3 grid((unsigned)ucm::ceil_div(tiles, kTilesPerWg), (unsigned)slices, (unsigned)a.H);
+        const int nt = a.BN / 32;
+        const int rc = nt == 4       ? launch_mfma_q<V, KS, 4, 1>(a, lds, grid, st)
+                       : nt == 8     ? launch_mfma_q<V, KS, 4, 2>(a, lds, grid, st)
+                       : nt % 4 == 0 ? launch_mfma_q<V, KS, 4, 0>(a, lds, grid, st)
+                       : nt == 2     ? launch_mfma_q<V, KS, 2, 1>(a, lds, grid, st)
+                       : nt == 1     ? launch_mfma_q<V, KS, 1, 1>(a, lds, grid, st)
+                       : nt % 2 == 0 ? launch_mfma_q<V, KS, 2, 0>(a, lds, grid, st)
+                                     : launch_mfma_q<V, KS, 1, 0>(a, lds, grid, st);
+        // a refused large-LDS opt-in falls back to the slice that fits the default 64 KiB
+        if (rc != UCM_EUNSUPPORTED || lds <= 64 * 1024) return rc;
+    }
+    return ucm::fail(UCM_EUNSUPPORTED, "no LDS slice fits K=%d", K);
 }
 
 template <typename V>
@@ -416,8 +617,10 @@ bool mfma_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 {
     const bool same16 = (x_dtype == w_dtype) && (x_dtype == UCM_DT_BF16 || x_dtype == UCM_DT_F16);
     const bool k_ok = a.K == 64 || a.K == 128 || a.K == 256 || a.K == 512;
+    // 16-byte row pieces; a tile of rows must span less than 2 GiB (32-bit lane offsets)
     const bool aligned = (((uintptr_t)a.x | (uintptr_t)a.w) & 15) == 0 && a.x_stride_t % 8 == 0 &&
-                         a.x_stride_h % 8 == 0;
+                         a.x_stride_h % 8 == 0 && a.x_stride_t >= 0 &&
+                         a.x_stride_t < ((int64_t)1 << 31) / (2 * kRowsPerWg);
     return same16 && k_ok && aligned;
 }
 
@@ -439,8 +642,23 @@ int launch_small(const EncJobs& js, int64_t waves, int K, hipStream_t st)
     return ucm::launch_status("encode_small_kernel");
 }
 
+// Folds a dense output into the paged form: block = row, one token per block, identity slots.
+void normalize_output(EncArgs& a)
+{
+    if (a.cache) return;
+    a.cache = a.out;
+    a.slot = nullptr;
+    a.slot_is_i64 = 1;
+    a.NB = a.T > 0 ? a.T : 1;
+    a.BS = 1;
+    a.cs_block = a.out_stride_t;
+    a.cs_token = 0;
+    a.cs_head = a.out_stride_h;
+}
+
 void set_block_shift(EncArgs& a)
 {
+    normalize_output(a);
     a.bs_shift = -1;
     if (a.BS > 0 && (a.BS & (a.BS - 1)) == 0) a.bs_shift = __builtin_ctz((unsigned)a.BS);
 }
