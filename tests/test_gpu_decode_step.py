@@ -57,6 +57,25 @@ def test_fused_step_equals_separate_operators_and_oracle(per_head_w):
     assert np.array_equal(idx.cpu().numpy(), oi) and np.array_equal(sc.cpu().numpy(), osc)
 
 
+def test_bound_step_follows_tensor_contents():
+    """bind() freezes the arguments, not the data: new queries in the same tensor give the new
+    answer, identical to an unbound step()."""
+    from ucm_amd.sparse import SparseDecodeStep
+
+    W, cache, table, lens, keys, qs, slots, enc_k, enc_q = build(3)
+    B, Hq, Hkv, nblk, K = 4, 32, 8, 6, 3
+    st = SparseDecodeStep(W, Hq, Hkv, B, nblk, K)
+    run = st.bind(keys, slots, qs, cache, table, lens)
+    i1, s1 = (t.clone() for t in run())
+    e1, f1 = (t.clone() for t in st.step(keys, slots, qs, cache, table, lens))
+    assert torch.equal(i1, e1) and torch.equal(s1, f1)
+    qs.copy_(torch.flip(qs, dims=[0]))
+    i2, s2 = (t.clone() for t in run())
+    e2, f2 = (t.clone() for t in st.step(keys, slots, qs, cache, table, lens))
+    assert torch.equal(i2, e2) and torch.equal(s2, f2)
+    assert not torch.equal(s1, s2)
+
+
 def test_step_without_new_keys_leaves_cache_untouched():
     from ucm_amd.sparse import SparseDecodeStep
 

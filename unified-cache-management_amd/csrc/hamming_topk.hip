@@ -290,11 +290,27 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
     const int wid = wave_id();
     const int h = (lane % PERIOD) / CPU, part = lane % CPU;
 
-    // query material first: it depends on nothing but the request index
+    // The two request-level scalars do not depend on each other: both reads go out together
+    // (without a table the entry read is a harmless second read of the length).
+    // Selected with masks, not branches: a branch would put the reads on separate paths and
+    // serialise their latencies.
+    const uintptr_t has_table = a.table ? ~(uintptr_t)0 : 0;
+    const uintptr_t ea = (reinterpret_cast<uintptr_t>(a.table + ((int64_t)b * a.table_stride + j)) & has_table) |
+                         (reinterpret_cast<uintptr_t>(a.lens + b) & ~has_table);
+    int entry = *reinterpret_cast<const int32_t*>(ea);
+    int len = a.lens[b];
+    // Scheduling fence: both scalars and the arguments the code loads need must be in
+    // registers here, which makes the compiler fetch all of them up front (two dependent
+    // rounds of scalar reads) instead of one after the other along the early-exit tests.
+    // (Pointers stay out of it: one that passes through would lose its address space.)
+    int64_t ks_block0 = a.ks_block, nb0 = a.NB, q_stride_b0 = a.q_stride_b;
+    asm volatile("" : "+s"(entry), "+s"(len), "+s"(ks_block0), "+s"(nb0), "+s"(q_stride_b0));
+
+    // query material next: it depends on nothing but the request index
     uint32_t qr[GP][4];
     int ctot = 0;
     if (DIRECT) {
-        const uint32_t* qp = a.q + b * a.q_stride_b + (int64_t)h * GP * a.q_stride_h + part * 4;
+        const uint32_t* qp = a.q + b * q_stride_b0 + (int64_t)h * GP * a.q_stride_h + part * 4;
 #pragma unroll
         for (int g = 0; g < GP; ++g)
 #pragma unroll
@@ -307,12 +323,14 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
             for (int w = 0; w < 4; ++w) qr[p][w] = pp[p * a.Wd + w];
     }
 
-    const int len = a.lens[b];
+    // physical block, or -1 when the entry is unusable; the address arithmetic sits in front of
+    // the early exit so that every kernel argument is fetched in one go at the top
+    int64_t pb = ((int64_t)entry & (int64_t)has_table) | (((int64_t)b * a.max_blocks + j) & ~(int64_t)has_table);
+    if (pb < 0 || pb >= nb0) pb = -1;
+    const int rpw = EXACT ? 4 : (a.BS * PERIOD) >> 8;  // runs per wave (a block has 4*rpw runs)
+    const u32x4* base = reinterpret_cast<const u32x4*>(a.kc + (pb < 0 ? 0 : pb) * ks_block0) + lane;
     const int pos0 = j * a.BS;
     if (pos0 >= len) return;  // j >= ceil(len / BS); the grid never exceeds max_blocks
-    const int64_t pb = physical_block(a, b, j);
-    const int rpw = EXACT ? 4 : (a.BS * PERIOD) >> 8;  // runs per wave (a block has 4*rpw runs)
-    const u32x4* base = reinterpret_cast<const u32x4*>(a.kc + (pb < 0 ? 0 : pb) * a.ks_block) + lane;
 
     // first batch of code loads goes out before anything waits
     u32x4 kv[4];

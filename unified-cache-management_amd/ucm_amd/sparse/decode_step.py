@@ -38,10 +38,8 @@ class SparseDecodeStep:
         nbytes = _lib.lib().ucm_hamming_topk_workspace_bytes(self.B, self.Hkv, self.max_blocks)
         self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
 
-    def step(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
-        """new_keys [T,Hkv,K] + slot_mapping [T] (T may be 0), queries [B,Hq,K],
-        k_hash_cache int32 [NB,BS,Hkv,N/32], block_table int32 [B,max_blocks], seq_lens int32 [B].
-        Returns (indices, scores) int32 [B, Hkv or 1, k]: views of buffers reused by every call."""
+    def _arguments(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
+        """Checks the tensors and returns the C call's arguments (all but the stream)."""
         if queries.dtype != self.w.dtype or (new_keys is not None and new_keys.dtype != self.w.dtype):
             raise ValueError("keys, queries and weights must share one dtype")
         if tuple(queries.shape) != (self.B, self.Hq, self.K):
@@ -64,7 +62,7 @@ class SparseDecodeStep:
             if slot_mapping.dtype not in (torch.int32, torch.int64) or slot_mapping.numel() != T:
                 raise ValueError("slot_mapping must be int32/int64 [T]")
         s = _lib.stride
-        _lib.check(_lib.lib().ucm_sparse_decode_step(
+        return (
             new_keys.data_ptr() if T else None, T, s(new_keys, 0) if T else 0,
             s(new_keys, 1) if T else 0, slot_mapping.data_ptr() if T else None,
             int(T > 0 and slot_mapping.dtype == torch.int64),
@@ -74,5 +72,28 @@ class SparseDecodeStep:
             s(k_hash_cache, 2), block_table.data_ptr(), max(s(block_table, 0), self.max_blocks),
             self.max_blocks, seq_lens.data_ptr(), self.B, self.Hq, self.k, self.sink, self.recent,
             self.flags, self.q_codes.data_ptr(), self.out_idx.data_ptr(), self.out_score.data_ptr(),
-            self.workspace.data_ptr(), self.workspace.numel(), _lib.stream_ptr(queries.device)))
+            self.workspace.data_ptr(), self.workspace.numel())
+
+    def step(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
+        """new_keys [T,Hkv,K] + slot_mapping [T] (T may be 0), queries [B,Hq,K],
+        k_hash_cache int32 [NB,BS,Hkv,N/32], block_table int32 [B,max_blocks], seq_lens int32 [B].
+        Returns (indices, scores) int32 [B, Hkv or 1, k]: views of buffers reused by every call."""
+        args = self._arguments(new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens)
+        _lib.check(_lib.lib().ucm_sparse_decode_step(*args, _lib.stream_ptr(queries.device)))
         return self.out_idx, self.out_score
+
+    def bind(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
+        """Validates once and returns `run()`: each call issues the step on torch's current
+        stream with the same tensors (whose contents may change between calls) at a few
+        microseconds of host time, for serving loops that would otherwise be bound by the
+        argument checks.  The tensors must stay alive as long as `run` is used."""
+        args = self._arguments(new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens)
+        keep = (new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens)
+        fn, dev, stream_ptr, check = _lib.lib().ucm_sparse_decode_step, queries.device, _lib.stream_ptr, _lib.check
+        result = (self.out_idx, self.out_score)
+
+        def run(_keep=keep):
+            check(fn(*args, stream_ptr(dev)))
+            return result
+
+        return run
