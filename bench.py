@@ -138,6 +138,37 @@ def extras(torch, enc_k, gen):
                       "hbm_frac": enc_bytes / ms / 1e6 / HBM_PEAK_GBPS}
     del keys, cache
 
+    # --- prefix-cache rehash: keys of 256 blocks read in place from a paged key cache, against
+    #     the reference's recipe (gather the blocks into a copy, then encode with a slot map) ---
+    NBK = 1024
+    kcache = torch.empty((NBK, BS, HKV, D), dtype=torch.bfloat16, device="cuda").normal_(generator=gen)
+    codes = torch.empty((NBK, BS, HKV, WD), dtype=torch.int32, device="cuda")
+    perms = [torch.randperm(NBK, generator=gen, device="cuda")[:NBLK].to(torch.int32) for _ in range(4)]
+    tok = torch.arange(CTX, device="cuda")
+
+    def fused(i):
+        enc_k.compute_hash_from_paged_cache(kcache, perms[i % 4], CTX, codes, BS)
+
+    def recipe(i):
+        ids = perms[i % 4]
+        gathered = kcache[ids.long()].reshape(-1, HKV, D)
+        slot_map = ids.long()[tok // BS] * BS + tok % BS
+        enc_k.compute_hash_and_cache(gathered, slot_map, codes, BS)
+
+    for name, fn in (("fused", fused), ("reference_recipe", recipe)):
+        for i in range(4):
+            fn(i)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(reps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out.setdefault("prefix_rehash", {})[name] = {
+            "tokens": CTX, "ms": ms, "key_GBps": rows * D * 2 / ms / 1e6}
+    del kcache, codes
+
     # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---
     L, NBP, n_req, n_sel = 32, 256, 4, 64
     chunk = BS * HKV * D * 2  # 256 KiB

@@ -84,6 +84,29 @@ int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int3
                           ucm_stream_t stream);
 
 /*
+ * Re-encodes keys that already sit in the paged KV cache (prefix-cache hit): replaces the
+ * gather `kv_cache[0][0][prefix_block_ids]` followed by compute_hash_and_cache with the
+ * prefix slot mapping (ucm/sparse/gsa_on_device/gsa_on_device.py:574-588; the slot rule is
+ * rebuild_prefix_cache_info_for_req, :1142-1174: slot(i) = block_ids[i / BS] * BS + i % BS).
+ * The keys are read in place — no gathered copy — and token i % BS of key block
+ * block_ids[i / BS] gets its code at the same block and token of the code cache.
+ *
+ * k_cache    [NBk, BS, H, K] of x_dtype; strides (block, token, head) in elements, the K
+ *            values of a row are contiguous.
+ * block_ids  [n_blocks] int32, device memory; n_tokens <= n_blocks * BS tokens are encoded
+ *            (the last block may be partial).  Ids outside [0, min(NBk, NB)) are skipped.
+ * cache      uint32 code cache [NB, BS, H, N_bits/32]; strides in 32-bit words.
+ */
+int ucm_hash_encode_paged(const void* k_cache, int x_dtype, int64_t NBk, int32_t BS, int32_t H,
+                          int32_t K, int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                          const int32_t* block_ids, int64_t n_blocks, int64_t n_tokens,
+                          const void* w, int w_dtype, int32_t n_w, int32_t heads_per_w,
+                          int32_t N_bits,
+                          uint32_t* cache, int64_t NB,
+                          int64_t cs_block, int64_t cs_token, int64_t cs_head,
+                          ucm_stream_t stream);
+
+/*
  * Replaces reshape_and_cache_khash_triton (hash_encoder.py:136-261): scatter already
  * computed codes [T, H, Wd] into the paged code cache by slot.
  */

@@ -88,6 +88,24 @@ def hash_encode_cache(x, W, heads_per_w, slot, cache, BS):
     return cache
 
 
+def hash_encode_paged(k_cache, block_ids, n_tokens, W, heads_per_w, cache):
+    """k_cache [NBk,BS,H,K] f32, block_ids [n] int32, W [n_w,K,N] f32, cache uint32
+    [NB,BS,H,Wd] (modified)."""
+    k_cache = _c(k_cache, np.float32)
+    W = _c(W, np.float32)
+    block_ids = _c(block_ids, np.int32)
+    assert cache.dtype == np.uint32 and cache.flags.c_contiguous
+    NBk, BS, H, K = k_cache.shape
+    n_w, _, N = W.shape
+    st = [s // 4 for s in cache.strides]
+    lib().oracle_hash_encode_paged(_p(k_cache), C.c_int64(NBk), C.c_int32(BS), C.c_int32(H),
+                                   C.c_int32(K), _p(block_ids), C.c_int64(n_tokens), _p(W),
+                                   C.c_int32(n_w), C.c_int32(heads_per_w), C.c_int32(N), _p(cache),
+                                   C.c_int64(cache.shape[0]), C.c_int64(st[0]), C.c_int64(st[1]),
+                                   C.c_int64(st[2]))
+    return cache
+
+
 def code_scatter(codes, slot, cache, BS):
     codes = _c(codes, np.uint32)
     slot = _c(slot, np.int64)

@@ -82,6 +82,30 @@ void oracle_hash_encode_cache(const float* x, int64_t T, int32_t H, int32_t K, c
     free(tmp);
 }
 
+/*
+ * Prefix-cache rehash.  gsa_on_device.py:574-588: the key blocks `block_ids` are gathered from
+ * the paged KV cache (kv_cache[0][0][prefix_block_ids], reshaped to [-1, H, K]), the first
+ * n_tokens rows are encoded and stored with the prefix slot mapping, which
+ * rebuild_prefix_cache_info_for_req (:1142-1174) builds as
+ *     slot(i) = block_ids[i / BS] * BS + i % BS.
+ * k_cache [NBk,BS,H,K] fp32 contiguous.  A block id outside either cache drops its rows (the
+ * reference would fault on the gather; the slot test of :338-344 covers the code cache side).
+ */
+void oracle_hash_encode_paged(const float* k_cache, int64_t NBk, int32_t BS, int32_t H, int32_t K,
+                              const int32_t* block_ids, int64_t n_tokens, const float* W,
+                              int32_t n_w, int32_t heads_per_w, int32_t N, uint32_t* cache,
+                              int64_t NB, int64_t cs_block, int64_t cs_token, int64_t cs_head)
+{
+    for (int64_t i = 0; i < n_tokens; ++i) {
+        const int64_t blk = block_ids[i / BS];
+        if (blk < 0 || blk >= NBk || blk >= NB) continue;
+        const int64_t slot = blk * BS + i % BS;
+        const float* row = k_cache + (blk * BS + i % BS) * (int64_t)H * K;  /* the gathered row i */
+        oracle_hash_encode_cache(row, 1, H, K, W, n_w, heads_per_w, N, &slot, cache, NB, BS,
+                                 cs_block, cs_token, cs_head);
+    }
+}
+
 /* Scatter of precomputed codes.  hash_encoder.py:136-195 (_reshape_and_cache_khash_kernel). */
 void oracle_code_scatter(const uint32_t* codes, int64_t T, int32_t H, int32_t Wd,
                          const int64_t* slot, uint32_t* cache, int64_t NB, int32_t BS,

@@ -199,6 +199,78 @@ def test_tiled_kernel_strided_rows_and_dense_heads():
         assert_codes_match(c[:, h], xs[:, h], W.float().numpy())
 
 
+@pytest.mark.parametrize("dtype,BS,H,n_blocks,n_tokens,per_head", [
+    (torch.bfloat16, 128, 8, 9, 1100, True),    # tiled kernel, partial last block
+    (torch.float16, 128, 2, 40, 5120, False),   # several workgroups per head
+    (torch.bfloat16, 64, 4, 3, 130, False),     # few rows: latency kernel
+    (torch.bfloat16, 32, 4, 20, 640, True),     # a wave per block
+    (torch.bfloat16, 48, 2, 12, 570, False),    # block size not a multiple of 32: FMA kernel
+    (torch.float32, 16, 2, 5, 77, False),       # fp32: FMA kernel
+])
+def test_rehash_from_paged_cache(dtype, BS, H, n_blocks, n_tokens, per_head):
+    """Prefix-cache rehash against the CPU checker and against the reference's own recipe run
+    on the GPU (gather the blocks, then compute_hash_and_cache with the prefix slot mapping)."""
+    rng = rng_for(300 + BS + n_blocks)
+    K = N = 128
+    NBk, NB = n_blocks + 6, n_blocks + 4
+    kc = torch.from_numpy(rng.standard_normal((NBk, BS, H, K)).astype(np.float32)).to(dtype)
+    W = torch.from_numpy(rng.standard_normal((H if per_head else 1, K, N)).astype(np.float32)).to(dtype)
+    ids = rng.permutation(NB)[:n_blocks].astype(np.int32)
+    if n_blocks >= 5:
+        ids[1] = -1            # unusable entries drop their tokens
+        ids[3] = NB + 1        # valid in the KV cache, outside the code cache
+    enc = make_encoder(K, N, dtype, W if per_head else W[0], n_w=H if per_head else 1, hpw=1)
+    cache = torch.full((NB, BS, H, N // 8), 0xAB, dtype=torch.uint8, device="cuda")
+    out = enc.compute_hash_from_paged_cache(kc.cuda(), torch.from_numpy(ids).cuda(), n_tokens, cache,
+                                            block_size=BS)
+    assert out is cache
+    got = cache.cpu().numpy().view(np.uint32)
+
+    # the reference's recipe on the GPU: gather, slot mapping, fused encode + store
+    cache2 = torch.full_like(cache, 0xAB)
+    tok = np.arange(n_tokens)
+    slots = ids[tok // BS].astype(np.int64) * BS + tok % BS
+    slots[(ids[tok // BS] < 0) | (ids[tok // BS] >= NB)] = -1
+    gathered = kc.cuda()[torch.from_numpy(np.clip(ids, 0, NBk - 1)).long().cuda()].reshape(-1, H, K)[:n_tokens]
+    enc.compute_hash_and_cache(gathered.contiguous(), torch.from_numpy(slots).cuda(), cache2, block_size=BS)
+    assert torch.equal(cache, cache2)
+
+    # CPU checker (bits may differ only inside the margin)
+    expect = np.full((NB, BS, H, N // 32), 0xABABABAB, np.uint32)
+    c_api.hash_encode_paged(kc.float().numpy(), ids, n_tokens, W.float().numpy(),
+                            1 if per_head else 0, expect)
+    if not np.array_equal(got, expect):
+        kcn, Wn = kc.float().numpy(), W.float().numpy()
+        for i in range(n_tokens):
+            b = int(ids[i // BS])
+            if b < 0 or b >= NB:
+                continue
+            for h in range(H):
+                assert_codes_match(got[b, i % BS, h:h + 1].view(np.uint8),
+                                   kcn[b, i % BS, h:h + 1], Wn[h if per_head else 0])
+    # cells of skipped and unlisted blocks stay untouched
+    listed = {int(b) for b in ids if 0 <= b < NB}
+    for b in range(NB):
+        if b not in listed:
+            assert (got[b] == 0xABABABAB).all()
+
+
+def test_rehash_argument_errors():
+    enc = make_encoder(128, 128, torch.bfloat16, torch.eye(128))
+    kc = torch.zeros((4, 64, 2, 128), dtype=torch.bfloat16, device="cuda")
+    cache = torch.zeros((4, 64, 2, 16), dtype=torch.uint8, device="cuda")
+    ids = torch.tensor([0, 1], dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        enc.compute_hash_from_paged_cache(kc, ids, 129, cache, block_size=64)   # > 2 blocks
+    with pytest.raises(ValueError):
+        enc.compute_hash_from_paged_cache(kc, ids.long(), 10, cache, block_size=64)
+    with pytest.raises(ValueError):
+        enc.compute_hash_from_paged_cache(kc, ids, 10, cache, block_size=128)
+    with pytest.raises(ValueError):
+        enc.compute_hash_from_paged_cache(kc.float(), ids, 10, cache, block_size=64)
+    assert enc.compute_hash_from_paged_cache(kc, ids, 0, cache, block_size=64) is cache
+
+
 def test_cache_as_bf16_view_and_shared_weight():
     """The plugin allocates the code cache as bfloat16 [NB,BS,H,hash_numbers/2]
     (hash_encoder.py:509-546) and uses one projection for all heads."""

@@ -116,6 +116,45 @@ def test_plugin_hooks_swap_and_restore_the_block_table():
     assert torch.equal(meta0.block_table, table)
 
 
+def test_plugin_rehashes_a_prefix_cache_hit_from_the_key_cache():
+    """Two requests whose prompt prefixes were loaded from the store into the paged KV cache:
+    the hook must produce, for the prefix tokens, the codes a full prefill of the same keys
+    would have produced (gsa_on_device.py:574-588), next to the codes of the new tokens."""
+    from ucm_amd.sparse.base import UcmSparseFactory, UcmSparseRole
+
+    Hq, Hkv, D, BS = 32, 8, 128, 64
+    cfg = {"ucm_sparse_config": {"GSAOnDevice": {
+        "num_q_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "block_size": BS, "seed": 6}}}
+    plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+    rng = rng_for(78)
+    NB = 40
+    name = "model.layers.1.self_attn.attn"
+    k_cache = torch.from_numpy(rng.standard_normal((NB, BS, Hkv, D)).astype(np.float32)).to(torch.bfloat16).cuda()
+    rows = torch.from_numpy(rng.permutation(NB)[:24].astype(np.int32).reshape(2, 12)).cuda()
+    prompts, qlens = [9 * BS + 17, 6 * BS], [BS + 17, 2 * BS]   # prefixes of 8 and 4 blocks
+    # new tokens of the step (their keys also sit in the KV cache, as after the cache write)
+    pos = [torch.arange(p - q, p, device="cuda") for p, q in zip(prompts, qlens)]
+    slots = torch.cat([rows[b, ps // BS].long() * BS + ps % BS for b, ps in enumerate(pos)])
+    keys = k_cache.view(NB * BS, Hkv * D)[slots]
+    k_hash = torch.zeros((NB, BS, Hkv, D // 8), dtype=torch.uint8, device="cuda")
+    plugin.set_prefix_cache_hits([(rows[0], prompts[0], qlens[0]), (rows[1], prompts[1], qlens[1])])
+    assert plugin.has_pc_hit and plugin.prefix_block_ids.numel() == 12
+    assert plugin.prefix_slot_mapping.numel() == 8 * BS + 4 * BS
+    meta = types.SimpleNamespace(slot_mapping=slots, block_table=rows, seq_lens=None)
+    layer = types.SimpleNamespace(kv_cache=[(k_cache, None)])
+    ctx = types.SimpleNamespace(attn_metadata={name: meta}, no_compile_layers={name: layer}, virtual_engine=0)
+    plugin.attention_begin(None, keys, None, name, ctx, phase="prefill", k_hash=k_hash)
+    # expected: every prompt token's key hashed at its slot
+    expect = torch.zeros_like(k_hash)
+    allpos = [torch.arange(p, device="cuda") for p in prompts]
+    allslots = torch.cat([rows[b, ps // BS].long() * BS + ps % BS for b, ps in enumerate(allpos)])
+    plugin.hash_encoder.compute_hash_and_cache(
+        k_cache.view(NB * BS, Hkv, D)[allslots], allslots, expect, block_size=BS)
+    assert torch.equal(k_hash, expect)
+    # the slot mapping the mirror reports equals the reference's formula
+    assert torch.equal(plugin.prefix_slot_mapping[: 8 * BS], allslots[: 8 * BS])
+
+
 def test_host_memory_store_dump_lookup_load_roundtrip():
     """The store contract of the reference's e2e test (ucm/store/test/e2e/cache_on_empty_test.py:
     46-79): dump -> lookup -> load -> bit-exact."""

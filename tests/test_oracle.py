@@ -301,6 +301,32 @@ def test_encode_cache_and_scatter():
     assert np.array_equal(cache2, expect)
 
 
+def test_encode_paged_is_gather_plus_prefix_slot_mapping():
+    """The rehash of keys that sit in the paged KV cache must equal the reference's recipe
+    written out with numpy: gather the blocks, keep the first n tokens, slot(i) =
+    block_ids[i // BS] * BS + i % BS (gsa_on_device.py:574-588, :1142-1174).  The slot rule is
+    also checked by hand on one token."""
+    rng = rng_for(44)
+    NBk, NB, BS, H, K, N = 7, 6, 4, 2, 32, 64
+    kc = rng.standard_normal((NBk, BS, H, K)).astype(np.float32)
+    W = rng.standard_normal((1, K, N)).astype(np.float32)
+    ids = np.array([5, 2, 6, 0], np.int32)  # 6 exists in the KV cache but not in the code cache
+    n_tokens = 14                          # the last block is half used
+    cache = np.full((NB, BS, H, N // 32), 0xDEADBEEF, np.uint32)
+    c_api.hash_encode_paged(kc, ids, n_tokens, W, 0, cache)
+    gathered = kc[np.clip(ids, 0, NBk - 1)].reshape(-1, H, K)[:n_tokens]
+    token_idx = np.arange(n_tokens)
+    slots = ids[token_idx // BS].astype(np.int64) * BS + token_idx % BS
+    slots[ids[token_idx // BS] >= NB] = -1
+    expect = np.full_like(cache, 0xDEADBEEF)
+    c_api.hash_encode_cache(gathered, W, 0, slots, expect, BS)
+    assert np.array_equal(cache, expect)
+    # token 5 = token 1 of block ids[1] = 2 -> slot 9
+    assert np.array_equal(cache[2, 1, 0], c_api.hash_encode(kc[2, 1, :1], W[0])[0])
+    assert (cache[0, 2:] == 0xDEADBEEF).all()  # tokens 14, 15 of the last block were not encoded
+    assert (cache[[1, 3, 4]] == 0xDEADBEEF).all()
+
+
 def test_gather_scatter_roundtrip_and_addresses():
     rng = rng_for(43)
     size, n = 48, 7

@@ -43,6 +43,11 @@ struct EncArgs {
     int64_t T;
     int H, K;
     int64_t x_stride_t, x_stride_h;
+    // paged input (src_blocks != null): row t is token t % BS of block src_blocks[t / BS] of a
+    // [NBsrc, BS, H, K] tensor with block stride xs_block; its code goes to the same block and
+    // token of the code cache
+    const int32_t* src_blocks;
+    int64_t xs_block, NBsrc;
     const void* w;
     int n_w, heads_per_w, N;
     // dense output (host side only: normalize_output() folds it into the paged form)
@@ -65,6 +70,33 @@ __device__ __forceinline__ int weight_index(const EncArgs& a, int h)
     return wi < a.n_w ? wi : a.n_w - 1;
 }
 
+// t -> (t / BS, t % BS) without a division when BS is a power of two.
+__device__ __forceinline__ void split_token(const EncArgs& a, int64_t t, int64_t& blk, int64_t& tok)
+{
+    if (a.bs_shift >= 0) {
+        blk = t >> a.bs_shift;
+        tok = t & (a.BS - 1);
+    } else if (t < 0x7fffffff) {
+        blk = (uint32_t)t / (uint32_t)a.BS;
+        tok = (uint32_t)t % (uint32_t)a.BS;
+    } else {
+        blk = t / a.BS;
+        tok = t % a.BS;
+    }
+}
+
+// Element offset of input row (t, h); for a paged input an unusable block id reads block 0
+// (the row is dropped when it is stored).
+__device__ __forceinline__ int64_t src_offset(const EncArgs& a, int64_t t, int h)
+{
+    if (!a.src_blocks) return t * a.x_stride_t + (int64_t)h * a.x_stride_h;
+    int64_t bi, tok;
+    split_token(a, t, bi, tok);
+    int64_t blk = a.src_blocks[bi];
+    if (blk < 0 || blk >= a.NBsrc) blk = 0;
+    return blk * a.xs_block + tok * a.x_stride_t + (int64_t)h * a.x_stride_h;
+}
+
 // A dense [T, H, Wd] output is handled as a paged one with one token per block and the
 // identity slot mapping (normalize_output() on the host), so the kernels know one layout.
 //
@@ -77,7 +109,12 @@ struct RawSlot {
 __device__ __forceinline__ RawSlot fetch_slot(const EncArgs& a, int64_t t)
 {
     RawSlot s;
-    if (!a.slot) {
+    if (a.src_blocks) {
+        int64_t bi, tok;
+        split_token(a, t, bi, tok);
+        s.lo = (uint32_t)a.src_blocks[bi];
+        s.hi = 0;
+    } else if (!a.slot) {
         s.lo = (uint32_t)t;
         s.hi = (uint32_t)((uint64_t)t >> 32);
     } else if (a.slot_is_i64) {
@@ -94,15 +131,24 @@ __device__ __forceinline__ RawSlot fetch_slot(const EncArgs& a, int64_t t)
 // Branch-free variant for a kernel that prefetches slots: two unconditional 4-byte reads whose
 // results land in fixed registers (a value merged from several branches would have to be
 // waited for at the merge).  Without a slot array the reads hit the input rows instead (valid
-// memory: the caller guarantees rows of at least 16 bytes) and slot_dst_of() ignores them.
+// memory: the caller guarantees rows of at least 16 bytes) and slot_value() ignores them.
 __device__ __forceinline__ RawSlot fetch_slot_flat(const EncArgs& a, int64_t t)
 {
     const char* p = a.slot ? (const char*)a.slot : (const char*)a.x;
-    const int sh = a.slot_is_i64 ? 3 : 2;
-    const char* q = p + (t << sh);
+    int sh = a.slot_is_i64 ? 3 : 2;
+    int hi_off = a.slot_is_i64 ? 4 : 0;
+    int64_t i = t;
+    if (a.src_blocks) {  // the "slot array" of a paged input is its block list
+        int64_t tok;
+        split_token(a, t, i, tok);
+        p = (const char*)a.src_blocks;
+        sh = 2;
+        hi_off = 0;
+    }
+    const char* q = p + (i << sh);
     RawSlot s;
     s.lo = *(const uint32_t*)q;
-    s.hi = *(const uint32_t*)(q + (a.slot_is_i64 ? 4 : 0));
+    s.hi = *(const uint32_t*)(q + hi_off);
     return s;
 }
 
@@ -128,6 +174,13 @@ __device__ __forceinline__ uint32_t* slot_dst(const EncArgs& a, int64_t s, int h
 // Slot value of row t from its raw words.
 __device__ __forceinline__ int64_t slot_value(const EncArgs& a, RawSlot raw, int64_t t)
 {
+    if (a.src_blocks) {
+        const int64_t blk = (int32_t)raw.lo;
+        if (blk < 0 || blk >= a.NBsrc) return -1;
+        int64_t bi, tok;
+        split_token(a, t, bi, tok);
+        return blk * a.BS + tok;
+    }
     if (!a.slot) return t;
     return a.slot_is_i64 ? (int64_t)(((uint64_t)raw.hi << 32) | raw.lo) : (int64_t)(int32_t)raw.lo;
 }
@@ -207,7 +260,7 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
     const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 31, kb = lane >> 5;
     const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)h * a.x_stride_h;
     const int64_t tiles = (a.T + kRowsPerWg - 1) / kRowsPerWg;
@@ -218,22 +271,43 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
     // by exactly one instruction.  Register 4L + j of a lane then holds a piece of line L that
     // belongs to another lane's MFMA column; to_operands() redistributes through LDS.
     // Rows past T re-read the last row (their results are discarded).  Addresses are a uniform
-    // 64-bit tile base plus a 32-bit lane offset (the host checks that a tile of rows spans
-    // less than 2 GiB).
+    // 64-bit base per wave plus a 32-bit lane offset (the host checks that 32 rows span less
+    // than 2 GiB).  With a paged input the wave's 32 rows lie in one block (the host checks that
+    // the block size is a multiple of 32) whose id is read once per tile.
+    auto wave_row0 = [&](int64_t tile) -> int64_t {
+        const int64_t row0 = tile * kRowsPerWg + wave * kRowsPerWave;
+        return row0 < a.T ? row0 : a.T - 1;
+    };
+    auto wave_block = [&](int64_t tile) -> int {  // paged input only
+        int64_t bi, tok;
+        split_token(a, wave_row0(tile), bi, tok);
+        return a.src_blocks[bi];
+    };
+    auto wave_base = [&](int64_t tile, int sblk) -> const char* {
+        const int64_t row0 = wave_row0(tile);
+        int64_t off = row0 * a.x_stride_t;
+        if (a.src_blocks) {
+            int64_t bi, tok;
+            split_token(a, row0, bi, tok);
+            const int64_t blk = (sblk < 0 || sblk >= a.NBsrc) ? 0 : sblk;
+            off = blk * a.xs_block + tok * a.x_stride_t;
+        }
+        return reinterpret_cast<const char*>(xbase + off);
+    };
     auto row_offset = [&](int64_t tile, int j) -> uint32_t {
-        const int q = wave * kRowsPerWave + 8 * j + (lane >> 3);
-        const int64_t left = a.T - 1 - tile * kRowsPerWg;  // last valid row, relative to the tile
+        const int q = 8 * j + (lane >> 3);
+        const int64_t left = a.T - 1 - wave_row0(tile);  // last valid row, relative to the wave's first
         const uint32_t qq = (int64_t)q > left ? (uint32_t)left : (uint32_t)q;
         return (qq * (uint32_t)a.x_stride_t + (lane & 7) * 8) * 2u;
     };
     // `real` = false issues the same number of loads against one cache line of the tensor's
     // first row: the prefetch ring then has one instruction sequence on every path, which lets
     // the compiler count outstanding loads exactly instead of waiting for all of them.
-    auto load_tile = [&](int64_t tile, V (&dstv)[KS], bool real) {
+    auto load_tile = [&](int64_t tile, int sblk, V (&dstv)[KS], bool real) {
         // masks instead of branches: both cases must be the same instruction stream
         const uint32_t m = real ? ~0u : 0u;
         const int64_t tc = real ? tile : (int64_t)0;
-        const char* tb = reinterpret_cast<const char*>(xbase + tc * kRowsPerWg * a.x_stride_t);
+        const char* tb = real ? wave_base(tc, sblk) : reinterpret_cast<const char*>(xbase);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t off = row_offset(tc, j) & m;
@@ -271,7 +345,7 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
     };
     // Wide rows: no register prefetch; fetch, stage and redistribute line by line.
     auto load_operands = [&](int64_t tile, V (&dstv)[KS]) {
-        const char* tb = reinterpret_cast<const char*>(xbase + tile * kRowsPerWg * a.x_stride_t);
+        const char* tb = wave_base(tile, a.src_blocks ? wave_block(tile) : 0);
         uint32_t off[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) off[j] = row_offset(tile, j);
@@ -313,6 +387,15 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
         }
     };
     constexpr bool kPipelined = kPrefetch && NG > 0;
+    // paged input: the block ids of the wave's rows in each of the workgroup's tiles, up front
+    int sblk[kTilesPerWg] = {0, 0, 0, 0};
+    if constexpr (kPipelined) {
+        if (a.src_blocks) {
+#pragma unroll
+            for (int i = 0; i < kTilesPerWg; ++i)
+                sblk[i] = wave_block(first + i < tiles ? first + i : tiles - 1);
+        }
+    }
     if constexpr (kPipelined) {
         // slice width known at compile time: no loop, no divergence (surplus threads redo a
         // patch); the first two tiles' rows go out right behind the first patch loads
@@ -324,8 +407,8 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
             u32x4 row[8];
             patch_load(idx, row);
             if (it == 0) {
-                load_tile(first, raw0, first < tiles);
-                load_tile(first + 1, raw1, first + 1 < tiles);
+                load_tile(first, sblk[0], raw0, first < tiles);
+                load_tile(first + 1, sblk[1], raw1, first + 1 < tiles);
             }
             patch_store(idx, row);
         }
@@ -415,14 +498,14 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
             uint32_t* dst = t0 < tiles ? slot_target(t0, slot0) : nullptr;
             if (i + 2 < kTilesPerWg) {
                 slot0 = tile_slot(t0 + 2 < tiles ? t0 + 2 : tiles - 1);
-                load_tile(t0 + 2, raw0, t0 + 2 < tiles);
+                load_tile(t0 + 2, sblk[(i + 2) % kTilesPerWg], raw0, t0 + 2 < tiles);
             }
             encode_rows(t0, dst);
             to_operands(raw1, av);
             dst = t1 < tiles ? slot_target(t1, slot1) : nullptr;
             if (i + 3 < kTilesPerWg) {
                 slot1 = tile_slot(t1 + 2 < tiles ? t1 + 2 : tiles - 1);
-                load_tile(t1 + 2, raw1, t1 + 2 < tiles);
+                load_tile(t1 + 2, sblk[(i + 3) % kTilesPerWg], raw1, t1 + 2 < tiles);
             }
             encode_rows(t1, dst);
         }
@@ -465,7 +548,7 @@ __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
     int64_t t = row0 + r;
     const bool row_ok = t < a.T;
     if (!row_ok) t = a.T - 1;
-    const uint16_t* xr = (const uint16_t*)a.x + (int64_t)h * a.x_stride_h + t * a.x_stride_t + kb * 8;
+    const uint16_t* xr = (const uint16_t*)a.x + src_offset(a, t, h) + kb * 8;
 
     V av[KS];
     uint16_t bw[KS][8];
@@ -511,7 +594,7 @@ __global__ __launch_bounds__(kThreads) void encode_fma_kernel(EncArgs a, int x_d
         const int64_t t = i / ((int64_t)Wd * a.H);
         uint32_t* dst = row_dst(a, t, h);
         if (!dst) continue;
-        const int64_t xo = t * a.x_stride_t + (int64_t)h * a.x_stride_h;
+        const int64_t xo = src_offset(a, t, h);
         const int64_t wo = (int64_t)weight_index(a, h) * a.K * a.N + w * 32;
         float acc[32];
 #pragma unroll
@@ -617,11 +700,13 @@ bool mfma_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 {
     const bool same16 = (x_dtype == w_dtype) && (x_dtype == UCM_DT_BF16 || x_dtype == UCM_DT_F16);
     const bool k_ok = a.K == 64 || a.K == 128 || a.K == 256 || a.K == 512;
-    // 16-byte row pieces; a tile of rows must span less than 2 GiB (32-bit lane offsets)
+    // 16-byte row pieces; a wave's 32 rows must span less than 2 GiB (32-bit lane offsets)
     const bool aligned = (((uintptr_t)a.x | (uintptr_t)a.w) & 15) == 0 && a.x_stride_t % 8 == 0 &&
                          a.x_stride_h % 8 == 0 && a.x_stride_t >= 0 &&
-                         a.x_stride_t < ((int64_t)1 << 31) / (2 * kRowsPerWg);
-    return same16 && k_ok && aligned;
+                         a.x_stride_t < ((int64_t)1 << 31) / (2 * kRowsPerWave);
+    // paged input: a wave's 32 rows must lie in one block
+    const bool paged_ok = !a.src_blocks || (a.BS % kRowsPerWave == 0 && a.xs_block % 8 == 0);
+    return same16 && k_ok && aligned && paged_ok;
 }
 
 int64_t small_waves(const EncArgs& a)
@@ -741,6 +826,30 @@ extern "C" int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int3
     a.x = x; a.T = T; a.H = H; a.K = K; a.x_stride_t = x_stride_t; a.x_stride_h = x_stride_h;
     a.w = w; a.n_w = n_w; a.heads_per_w = heads_per_w; a.N = N_bits;
     a.slot = slot_mapping; a.slot_is_i64 = slot_is_i64; a.cache = cache; a.NB = NB; a.BS = BS;
+    a.cs_block = cs_block; a.cs_token = cs_token; a.cs_head = cs_head;
+    return encode_common(a, x_dtype, w_dtype, (hipStream_t)stream);
+}
+
+extern "C" int ucm_hash_encode_paged(const void* k_cache, int x_dtype, int64_t NBk, int32_t BS,
+                                     int32_t H, int32_t K, int64_t ks_block, int64_t ks_token,
+                                     int64_t ks_head, const int32_t* block_ids, int64_t n_blocks,
+                                     int64_t n_tokens, const void* w, int w_dtype, int32_t n_w,
+                                     int32_t heads_per_w, int32_t N_bits, uint32_t* cache,
+                                     int64_t NB, int64_t cs_block, int64_t cs_token,
+                                     int64_t cs_head, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(cache && NB > 0 && BS > 0 && NBk > 0, "bad cache shape");
+    UCM_REQUIRE(n_blocks >= 0 && n_tokens >= 0 && n_tokens <= n_blocks * (int64_t)BS,
+                "n_tokens %lld does not fit %lld blocks of %d", (long long)n_tokens,
+                (long long)n_blocks, (int)BS);
+    UCM_REQUIRE(n_tokens == 0 || block_ids, "null block_ids");
+    EncArgs a{};
+    a.x = k_cache; a.T = n_tokens; a.H = H; a.K = K; a.x_stride_t = ks_token; a.x_stride_h = ks_head;
+    a.src_blocks = block_ids; a.xs_block = ks_block;
+    a.NBsrc = NBk < NB ? NBk : NB;  // an id must be valid in both caches
+    a.w = w; a.n_w = n_w; a.heads_per_w = heads_per_w; a.N = N_bits;
+    a.slot = nullptr; a.slot_is_i64 = 0; a.cache = cache; a.NB = NB; a.BS = BS;
     a.cs_block = cs_block; a.cs_token = cs_token; a.cs_head = cs_head;
     return encode_common(a, x_dtype, w_dtype, (hipStream_t)stream);
 }

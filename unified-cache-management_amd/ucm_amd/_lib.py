@@ -26,6 +26,8 @@ _SIGNATURES = {
     "ucm_hash_encode": (ci, [vp, ci, i64, i32, i32, i64, i64, vp, ci, i32, i32, i32, vp, i64, i64, vp]),
     "ucm_hash_encode_cache": (ci, [vp, ci, i64, i32, i32, i64, i64, vp, ci, i32, i32, i32, vp, ci,
                                    vp, i64, i32, i64, i64, i64, vp]),
+    "ucm_hash_encode_paged": (ci, [vp, ci, i64, i32, i32, i32, i64, i64, i64, vp, i64, i64, vp, ci,
+                                   i32, i32, i32, vp, i64, i64, i64, i64, vp]),
     "ucm_code_scatter": (ci, [vp, i64, i32, i32, i64, i64, vp, ci, vp, i64, i32, i64, i64, i64, vp]),
     "ucm_hamming_topk_workspace_bytes": (sz, [i32, i32, i32]),
     "ucm_hamming_topk": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,

@@ -5,9 +5,11 @@ A thin counterpart of the reference plugin's worker-side hot path
 step's keys (cache_k_hash_gqa_cuda, :564-572) and, at decode, replaces the layer's block table
 and seq_lens with the top-k blocks (update_decode_topk_gqa_cuda, :773-811);
 `attention_finished` puts the originals back (:959-995).  Engine metadata is duck-typed: the
-layer's `attn_metadata` needs `slot_mapping`, `block_table` and `seq_lens` attributes.  The
-scheduler-side hooks, prefix-cache rehash, MLA metadata surgery and layer-skip profiling of
-the reference are outside this build.
+layer's `attn_metadata` needs `slot_mapping`, `block_table` and `seq_lens` attributes.
+After a prefix-cache hit (`set_prefix_cache_hits`, the bookkeeping of build_sparse_meta,
+:1322-1366) the keys that were loaded into the paged KV cache are re-encoded in place
+(cache_k_hash_gqa_cuda's `has_pc_hit` branch, :574-588).  The scheduler-side hooks, MLA
+metadata surgery and layer-skip profiling of the reference are outside this build.
 
 Configuration (`ucm_sparse_config["GSAOnDevice"]`), names from
 gsa_on_device_config.py:36-98 where they exist:
@@ -56,6 +58,10 @@ class GSAOnDevice(UcmSparseBase):
         self.gsa_enabled = True
         self.hash_encoder = HashEncoder(self.head_dim, self.hash_bits, self.dtype, self.device)
         self._saved = {}
+        self.has_pc_hit = False
+        self.prefix_block_ids = None      # int32 [sum of prefix blocks], all hit requests
+        self.prefix_slot_mapping = None   # int64 [sum of prefix tokens]
+        self._prefix_segments = []        # (first block, blocks, tokens) per hit request
 
     # ---- helpers mirroring the reference's names ----
     def get_layer_attn_metadata(self, forward_context, layer_name: str):
@@ -75,12 +81,56 @@ class GSAOnDevice(UcmSparseBase):
             query = torch.repeat_interleave(query, self.num_key_heads // self.num_q_heads, dim=1)
         return self.hash_encoder.compute_hash(query)
 
-    def cache_k_hash_gqa(self, key, attn_metadata, k_hash):
+    def rebuild_prefix_cache_info_for_req(self, block_table_row, num_prompt_tokens, qlen,
+                                          block_size):
+        """(num_prefix_tokens, num_prefix_blocks, prefix_block_ids, prefix_slot_mapping) of a
+        request whose first num_prompt_tokens - qlen tokens came from the store
+        (gsa_on_device.py:1142-1174)."""
+        assert 0 <= qlen <= num_prompt_tokens
+        num_prefix_tokens = num_prompt_tokens - qlen
+        if num_prefix_tokens <= 0:
+            empty = block_table_row[:0]
+            return 0, 0, empty, empty
+        num_prefix_blocks = (num_prefix_tokens + block_size - 1) // block_size
+        prefix_block_ids = block_table_row[:num_prefix_blocks]
+        token_idx = torch.arange(num_prefix_tokens, device=block_table_row.device)
+        prefix_slot_mapping = (prefix_block_ids.index_select(0, token_idx // block_size).to(torch.int64)
+                               * block_size + token_idx % block_size)
+        return num_prefix_tokens, num_prefix_blocks, prefix_block_ids, prefix_slot_mapping
+
+    def set_prefix_cache_hits(self, hits):
+        """hits: iterable of (block_table_row, num_prompt_tokens, qlen) for the requests of this
+        step whose prompt prefix was loaded from the store; sets has_pc_hit, prefix_block_ids
+        and prefix_slot_mapping like build_sparse_meta (gsa_on_device.py:1322-1366)."""
+        ids, slots, self._prefix_segments = [], [], []
+        first = 0
+        for row, num_prompt_tokens, qlen in hits:
+            n_tok, n_blk, blk, slot = self.rebuild_prefix_cache_info_for_req(
+                row, int(num_prompt_tokens), int(qlen), self.block_size)
+            if n_tok > 0:
+                ids.append(blk.to(torch.int32))
+                slots.append(slot)
+                self._prefix_segments.append((first, n_blk, n_tok))
+                first += n_blk
+        self.has_pc_hit = bool(ids)
+        self.prefix_block_ids = torch.cat(ids) if ids else None
+        self.prefix_slot_mapping = torch.cat(slots) if slots else None
+
+    def cache_k_hash_gqa(self, key, attn_metadata, k_hash, k_cache=None):
         slots = attn_metadata.slot_mapping.flatten()
         n = slots.numel()
         self.hash_encoder.compute_hash_and_cache(
             key[:n].view(n, self.num_key_heads, self.head_dim), slots, k_hash,
             block_size=self.block_size)
+        if self.has_pc_hit:
+            # keys of the prefix are read where they lie in the paged KV cache (the reference
+            # gathers them into a copy first, gsa_on_device.py:574-588)
+            if k_cache is None:
+                raise ValueError("a prefix-cache hit needs the layer's key cache")
+            for first, n_blk, n_tok in self._prefix_segments:
+                self.hash_encoder.compute_hash_from_paged_cache(
+                    k_cache, self.prefix_block_ids[first:first + n_blk], n_tok, k_hash,
+                    block_size=self.block_size)
 
     # ---- hooks ----
     def attention_begin(self, query, key, value, layer_name: str, forward_context, output=None,
@@ -89,7 +139,12 @@ class GSAOnDevice(UcmSparseBase):
         if not self.gsa_enabled or k_hash is None:
             return query, key, value, output
         attn_metadata = self.get_layer_attn_metadata(forward_context, layer_name)
-        self.cache_k_hash_gqa(key, attn_metadata, k_hash)
+        k_cache = None
+        if self.has_pc_hit:
+            # kv_cache[0] is the key cache [NB, BS, Hkv, D] (gsa_on_device.py:576-579)
+            attn = forward_context.no_compile_layers[layer_name]
+            k_cache = attn.kv_cache[forward_context.virtual_engine][0]
+        self.cache_k_hash_gqa(key, attn_metadata, k_hash, k_cache)
         is_rollback_layer, _ = self.get_layer_state(layer_name)
         if phase == "decode" and not is_rollback_layer:
             num_reqs = attn_metadata.seq_lens.shape[0]

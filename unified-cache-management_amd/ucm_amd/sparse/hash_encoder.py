@@ -192,6 +192,57 @@ class HashEncoder:
                 u8.data_ptr(), NB, BS, sb // 4, ss // 4, sh // 4, _lib.stream_ptr(x.device)))
         return k_hash_cache
 
+    def compute_hash_from_paged_cache(self, k_cache: torch.Tensor, block_ids: torch.Tensor,
+                                      num_tokens: int, k_hash_cache: torch.Tensor,
+                                      block_size: int = 128) -> torch.Tensor:
+        """Prefix-cache rehash: encode the first `num_tokens` tokens of the key blocks
+        `block_ids` of the paged KV cache k_cache [NB,BS,H,K] in place and store each code at
+        the same block and token of k_hash_cache [NB',BS,H,W].
+
+        One call for what the reference does with a gathered copy
+        (`kv_cache[0][0][prefix_block_ids]`, reshape, compute_hash_and_cache with the prefix
+        slot mapping, gsa_on_device.py:574-588); slot(i) = block_ids[i // BS] * BS + i % BS
+        as in rebuild_prefix_cache_info_for_req (:1142-1174).  Returns k_hash_cache."""
+        if k_cache.ndim != 4:
+            raise ValueError(f"k_cache must be [NB,BS,H,K], got {k_cache.shape}")
+        if k_hash_cache.ndim != 4:
+            raise ValueError(f"k_hash_cache must be rank-4, got {k_hash_cache.shape}")
+        if block_ids.ndim != 1 or block_ids.dtype != torch.int32:
+            raise ValueError("block_ids must be int32 [n_blocks]")
+        self._check_x(k_cache)
+        if block_ids.device != k_cache.device or k_hash_cache.device != k_cache.device:
+            raise ValueError(f"all tensors must be on {self.device}")
+        if k_cache.dtype != self.dtype:
+            raise ValueError(f"k_cache dtype {k_cache.dtype} != encoder dtype {self.dtype}")
+        NBk, BS, H, _ = k_cache.shape
+        NB, BSc, Hc, _ = k_hash_cache.shape
+        if BS != block_size or BSc != block_size:
+            raise ValueError(f"block sizes {BS}, {BSc} != block_size={block_size}")
+        if Hc != H:
+            raise ValueError(f"k_hash_cache.shape[2]={Hc} != H={H}")
+        n_blocks = int(block_ids.shape[0])
+        num_tokens = int(num_tokens)
+        if num_tokens < 0 or num_tokens > n_blocks * BS:
+            raise ValueError(f"num_tokens {num_tokens} does not fit {n_blocks} blocks of {BS}")
+        if self.hash_bits % 32 != 0:
+            raise NotImplementedError("the fused cache write needs hash_bits % 32 == 0")
+        if k_cache.stride(-1) != 1:
+            raise ValueError("the K values of a row must be contiguous")
+        u8 = self._reinterpret_cache_as_u8(k_hash_cache)
+        sb, ss, sh, sw = (_lib.stride(u8, d) for d in range(4))
+        if sw != 1 or sb % 4 or ss % 4 or sh % 4 or u8.data_ptr() % 4:
+            raise ValueError("k_hash_cache codes must be contiguous and 4-byte aligned")
+        block_ids = block_ids.contiguous()
+        if num_tokens > 0:
+            _lib.check(_lib.lib().ucm_hash_encode_paged(
+                k_cache.data_ptr(), _DT[self.dtype], NBk, BS, H, self.input_dim,
+                _lib.stride(k_cache, 0), _lib.stride(k_cache, 1), _lib.stride(k_cache, 2),
+                block_ids.data_ptr(), n_blocks, num_tokens,
+                self._w.data_ptr(), _DT[self.dtype], self._w.shape[0],
+                self.heads_per_weight if self.num_weights > 1 else 0, self._padded_bits,
+                u8.data_ptr(), NB, sb // 4, ss // 4, sh // 4, _lib.stream_ptr(k_cache.device)))
+        return k_hash_cache
+
     def reshape_and_cache(self, k_hash_compute: torch.Tensor, slot_mapping: torch.Tensor,
                           k_hash: torch.Tensor, block_size: int = 128) -> torch.Tensor:
         """Scatter precomputed codes [T,H,W] into the paged cache [NB,BS,H,W]
