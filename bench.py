@@ -213,6 +213,34 @@ def extras(torch, enc_k, gen):
     out["d2h_copy_engine_flat"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
     ms = timed(lambda: st.PagedScatterAsync(host.data_ptr(), base, sizes, ids), 2)
     out["scatter_from_pinned_host_kernel"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
+    del host, dev_flat
+
+    # --- the same blocks through the native cache store (task queues + pinned staging nodes):
+    #     submit -> wait, one request (64 blocks = 1 GiB) per task, as the connector's
+    #     save_speed / load_speed are measured ---
+    from ucm_amd.store import CacheStore
+
+    n_tensors = 2 * L
+    store = CacheStore({"tensor_size_list": [chunk] * n_tensors,
+                        "buffer_capacity_bytes": len(ids) * n_tensors * chunk})
+    rows = (ids.astype(np.uint64)[:, None] * sizes[None, :] + base[None, :])  # [blocks, tensors]
+    bids = [int(i).to_bytes(8, "little") * 2 for i in range(len(ids))]
+    per_task = n_sel
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    tasks = [store.dump_data(bids[i:i + per_task], [0] * per_task, rows[i:i + per_task])
+             for i in range(0, len(ids), per_task)]
+    for t in tasks:
+        store.wait(t)
+    t1 = time.perf_counter()
+    tasks = [store.load_data(bids[i:i + per_task], [0] * per_task, rows[i:i + per_task])
+             for i in range(0, len(ids), per_task)]
+    for t in tasks:
+        store.wait(t)
+    t2 = time.perf_counter()
+    out["cache_store"] = {"payload_GiB": payload / 2**30, "tasks": len(tasks),
+                          "dump_GBps": payload / (t1 - t0) / 1e9, "load_GBps": payload / (t2 - t1) / 1e9}
+    store.close()
     return out
 
 

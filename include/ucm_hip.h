@@ -26,6 +26,7 @@ extern "C" {
 #define UCM_EPARAM       (-50000)
 #define UCM_EOOM         (-50001)
 #define UCM_EOSERROR     (-50002)
+#define UCM_ENOOBJ       (-50005)
 #define UCM_EUNSUPPORTED (-50008)
 #define UCM_ETIMEOUT     (-50010)
 
@@ -306,6 +307,76 @@ int ucm_trans_device_alloc(size_t size, void** out);
 int ucm_trans_device_free(void* p);
 int ucm_trans_host_register(void* host, size_t size, void** device_alias);
 int ucm_trans_host_unregister(void* host);
+
+/* ------------------------------------------------------------------------------------
+ * 4. Cache store: pinned-host staging cache in front of a slower store backend — the caller
+ *    of the gather / scatter path (ucm/store/cache/cc/).
+ * ------------------------------------------------------------------------------------ */
+
+typedef struct ucm_cache_store ucm_cache_store_t;
+
+/*
+ * The slower tier behind the staging cache: the part of the reference's StoreV1 interface
+ * (ucm/store/ucmstore_v1.h) that CacheStore calls on its `store_backend`
+ * (dump_queue.cc:129, load_queue.cc:103, buffer_manager.h:103).  All hooks may be NULL; with a
+ * NULL table the pinned buffer is the only tier.  `block_ids` are n x 16 bytes, `host` holds n
+ * pointers to shards of `shard_size` bytes in pinned memory that stays valid until wait()
+ * returns.  dump/load return a positive handle, or a negative status.
+ */
+typedef struct ucm_cache_backend {
+    void* ctx;
+    int (*lookup)(void* ctx, const uint8_t* block_ids, size_t n, uint8_t* found);
+    int64_t (*dump)(void* ctx, const uint8_t* block_ids, const uint64_t* shard_idx,
+                    void* const* host, size_t n, size_t shard_size);
+    int64_t (*load)(void* ctx, const uint8_t* block_ids, const uint64_t* shard_idx,
+                    void* const* host, size_t n, size_t shard_size);
+    int (*wait)(void* ctx, int64_t handle);
+} ucm_cache_backend_t;
+
+/*
+ * CacheStore::Setup (cache_store.cc:37-57) with the fields of its Config
+ * (global_config.h:33-48): a shard is the concatenation of `n_tensors` pieces of
+ * `tensor_sizes[i]` bytes (tensor_size_list), `buffer_bytes` of pinned memory hold
+ * buffer_bytes / shard_size shards (cache_buffer_capacity_gb), `waiting_queue_depth` bounds
+ * the submitted-but-not-started tasks of each direction, `timeout_ms` is Wait's limit
+ * (0 = 30000).  Starts the dump and load worker threads.
+ */
+int ucm_cache_store_create(int32_t device_id, const size_t* tensor_sizes, size_t n_tensors,
+                           size_t buffer_bytes, size_t waiting_queue_depth, size_t timeout_ms,
+                           const ucm_cache_backend_t* backend, ucm_cache_store_t** out);
+int ucm_cache_store_destroy(ucm_cache_store_t* store);
+/* staging nodes the buffer holds */
+size_t ucm_cache_store_nodes(ucm_cache_store_t* store);
+
+/* CacheStore::Lookup / LookupOnPrefix (cache_store.cc:59-70, buffer_manager.h:66-127):
+ * found[i] = block i is in the staging cache (its shard 0) or in the backend;
+ * *last_found = index of the last block of the leading run that is present, -1 if none. */
+int ucm_cache_store_lookup(ucm_cache_store_t* store, const uint8_t* block_ids, size_t n,
+                           uint8_t* found);
+int ucm_cache_store_lookup_on_prefix(ucm_cache_store_t* store, const uint8_t* block_ids, size_t n,
+                                     int64_t* last_found);
+
+/*
+ * CacheStore::Dump / Load (cache_store.cc:72-89; DumpQueue::DumpOneTask dump_queue.cc:92-143,
+ * LoadQueue::DispatchOneTask / TransferOneTask load_queue.cc:77-160).  A task is n shards;
+ * shard i is (block_ids[16 i .. 16 i + 15], shard_idx[i]) and lives on the device as n_tensors
+ * pieces at device_addrs[i * n_tensors + t].  Both calls only enqueue and return a task id.
+ * Dump: waits for `prerequisite_event` (hipEvent_t, may be NULL) on the store's stream, copies
+ * every shard that no other task is already staging into its pinned node with one kernel
+ * launch, then hands the nodes to the backend.  Load: shards that are not resident are first
+ * fetched from the backend into their node; the task fails if one is in neither tier.
+ */
+int ucm_cache_store_dump(ucm_cache_store_t* store, const uint8_t* block_ids,
+                         const uint64_t* shard_idx, void* const* device_addrs, size_t n,
+                         void* prerequisite_event, int64_t* task);
+int ucm_cache_store_load(ucm_cache_store_t* store, const uint8_t* block_ids,
+                         const uint64_t* shard_idx, void* const* device_addrs, size_t n,
+                         int64_t* task);
+/* CacheStore::Check / Wait (cache_store.cc:90-101; task_wrapper.h:62-107): Check reports
+ * whether the task has finished (either way); Wait blocks up to timeout_ms, forgets the task
+ * and returns UCM_OK, UCM_ERROR (the task failed), UCM_ETIMEOUT or UCM_ENOOBJ (unknown id). */
+int ucm_cache_store_check(ucm_cache_store_t* store, int64_t task, int* finished);
+int ucm_cache_store_wait(ucm_cache_store_t* store, int64_t task);
 
 #ifdef __cplusplus
 }

@@ -9,7 +9,9 @@ UCM_OK = 0
 UCM_ERROR = -1
 UCM_EPARAM = -50000
 UCM_EOOM = -50001
+UCM_ENOOBJ = -50005
 UCM_EUNSUPPORTED = -50008
+UCM_ETIMEOUT = -50010
 
 DT_BF16, DT_F16, DT_F32 = 0, 1, 2
 TOPK_REDUCE_HEADS, TOPK_RETURN_PHYSICAL, TOPK_SCORE_ORDER, TOPK_DISTANCE = 1, 2, 4, 8
@@ -58,6 +60,15 @@ _SIGNATURES = {
     "ucm_trans_device_free": (ci, [vp]),
     "ucm_trans_host_register": (ci, [vp, sz, C.POINTER(vp)]),
     "ucm_trans_host_unregister": (ci, [vp]),
+    "ucm_cache_store_create": (ci, [i32, vp, sz, sz, sz, sz, vp, C.POINTER(vp)]),
+    "ucm_cache_store_destroy": (ci, [vp]),
+    "ucm_cache_store_nodes": (sz, [vp]),
+    "ucm_cache_store_lookup": (ci, [vp, vp, sz, vp]),
+    "ucm_cache_store_lookup_on_prefix": (ci, [vp, vp, sz, C.POINTER(i64)]),
+    "ucm_cache_store_dump": (ci, [vp, vp, vp, vp, sz, vp, C.POINTER(i64)]),
+    "ucm_cache_store_load": (ci, [vp, vp, vp, vp, sz, C.POINTER(i64)]),
+    "ucm_cache_store_check": (ci, [vp, i64, C.POINTER(ci)]),
+    "ucm_cache_store_wait": (ci, [vp, i64]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
