@@ -111,6 +111,37 @@ def cpu_baseline(torch, cache, table, qcodes, lens, seconds_budget=20.0):
                       f"one thread per request over {cores} threads (oracle/ucm_oracle.c)"}
 
 
+def cpu_side_baselines(torch):
+    """Host-CPU figures for the two side paths, on bounded samples: the reference's CPU form of
+    the encoder (torch.matmul in fp32 + pack, hash_encoder.py:359-370) on all cores, and the
+    pointer-table memcpy loop of its CPU trans backend (the checker's gather)."""
+    import numpy as np
+    from oracle import c_api
+
+    out = {}
+    rows = 65536
+    x = torch.randn((rows, D), dtype=torch.float32)
+    w = torch.randn((D, D), dtype=torch.float32)
+    masks = (1 << torch.arange(8, dtype=torch.int32)).to(torch.uint8)
+    torch.matmul(x[:1024], w)
+    t0 = time.perf_counter()
+    bits = torch.matmul(x, w) > 0
+    packed = (bits.view(rows, D // 8, 8).to(torch.uint8) * masks).sum(-1, dtype=torch.uint8)
+    t1 = time.perf_counter()
+    out["encoder_cpu_torch"] = {"rows": rows, "threads": torch.get_num_threads(), "ms": (t1 - t0) * 1e3,
+                                "rows_per_s": rows / (t1 - t0), "checksum": int(packed.sum())}
+    n, size = 1024, 256 * 1024
+    pool = np.random.default_rng(5).integers(0, 256, size=(n, size), dtype=np.uint8)
+    chunks = [pool[i] for i in np.random.default_rng(6).permutation(n)]
+    c_api.gather(chunks[:8], size)
+    t0 = time.perf_counter()
+    c_api.gather(chunks, size)
+    t1 = time.perf_counter()
+    out["gather_cpu_memcpy"] = {"payload_MiB": n * size / 2**20, "threads": 1, "ms": (t1 - t0) * 1e3,
+                                "GBps": n * size / (t1 - t0) / 1e9}
+    return out
+
+
 def extras(torch, enc_k, gen):
     """Side figures: encoder at cache-build shape, device gather, pinned-host dump."""
     import numpy as np
@@ -405,6 +436,7 @@ def main():
                    "timed_region": (f"hipGraph replays, {GS} consecutive steps per graph"
                                     if graphs is not None else "eager launches"),
                    "roofline_pass": "same steps launched eagerly, dispatch start/stop events of the block-score kernel"},
+        "token_head_codes_per_s": tokens * HKV / (ms_per_step / 1e3),
         "p50_step_latency_us": step_ms[len(step_ms) // 2] * 1e3,
         "p90_step_latency_us": step_ms[max(0, int(len(step_ms) * 0.9) - 1)] * 1e3,
         "roofline": {"bound": "hbm", "kernel": "block_score_one", "achieved": achieved,
@@ -421,6 +453,8 @@ def main():
         del caches[1:], tables[1:]
         torch.cuda.empty_cache()
         line["extras"] = extras(torch, enc_k, gen)
+        if not args.skip_cpu:
+            line["extras"].update(cpu_side_baselines(torch))
     print(json.dumps(line))
 
 
