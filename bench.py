@@ -130,6 +130,14 @@ def cpu_side_baselines(torch):
     t1 = time.perf_counter()
     out["encoder_cpu_torch"] = {"rows": rows, "threads": torch.get_num_threads(), "ms": (t1 - t0) * 1e3,
                                 "rows_per_s": rows / (t1 - t0), "checksum": int(packed.sum())}
+    rng = np.random.default_rng(7)
+    vec = rng.random((25600, 1024), dtype=np.float32)
+    qq = rng.random((2, 1024), dtype=np.float32)
+    cand = np.stack([rng.permutation(25600)[:8000] for _ in range(2)]).astype(np.int32)
+    t0 = time.perf_counter()
+    c_api.dot_topk(vec, qq, cand, 3000)
+    t1 = time.perf_counter()
+    out["esa_dot_topk_cpu"] = {"threads": 1, "ms": (t1 - t0) * 1e3}
     n, size = 1024, 256 * 1024
     pool = np.random.default_rng(5).integers(0, 256, size=(n, size), dtype=np.uint8)
     chunks = [pool[i] for i in np.random.default_rng(6).permutation(n)]
@@ -140,6 +148,12 @@ def cpu_side_baselines(torch):
     out["gather_cpu_memcpy"] = {"payload_MiB": n * size / 2**20, "threads": 1, "ms": (t1 - t0) * 1e3,
                                 "GBps": n * size / (t1 - t0) / 1e9}
     return out
+
+
+def _esa_ws(B, max_n):
+    from ucm_amd import _lib
+
+    return int(_lib.lib().ucm_dot_topk_workspace_bytes(B, max_n))
 
 
 def extras(torch, enc_k, gen):
@@ -199,6 +213,28 @@ def extras(torch, enc_k, gen):
         out.setdefault("prefix_rehash", {})[name] = {
             "tokens": CTX, "ms": ms, "key_GBps": rows * D * 2 / ms / 1e6}
     del kcache, codes
+
+    # --- float retrieval (ESA): the shape of the reference's own driver
+    #     (esa/retrieval/retrieval_worker.py:45-60): 25600 block vectors of dim 1024, 2 requests,
+    #     8000 candidates each, top-3000 ---
+    from ucm_amd.sparse.esa_retrieval_worker import dot_topk
+
+    vecs = torch.rand((25600, 1024), generator=gen, device="cuda", dtype=torch.float32)
+    qv = torch.rand((2, 1024), generator=gen, device="cuda", dtype=torch.float32)
+    cand = torch.stack([torch.randperm(25600, generator=gen, device="cuda")[:8000] for _ in range(2)]).to(torch.int32)
+    ws = torch.empty(_esa_ws(2, 8000), dtype=torch.uint8, device="cuda")
+    for _ in range(3):
+        dot_topk(vecs, qv, cand, 3000, ws)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        dot_topk(vecs, qv, cand, 3000, ws)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    out["esa_dot_topk"] = {"candidates": 2 * 8000, "dim": 1024, "topk": 3000, "ms": ms,
+                           "gather_GBps": 2 * 8000 * 4096 / ms / 1e6}
+    del vecs
 
     # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---
     L, NBP, n_req, n_sel = 32, 256, 4, 64

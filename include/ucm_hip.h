@@ -309,6 +309,30 @@ int ucm_trans_host_register(void* host, size_t size, void** device_alias);
 int ucm_trans_host_unregister(void* host);
 
 /* ------------------------------------------------------------------------------------
+ * 3b. Float retrieval (ESA): dot-product top-k over a candidate list
+ * ------------------------------------------------------------------------------------ */
+
+/*
+ * GPU form of the reference's ESA retrieval backend
+ * (ucm/sparse/esa/retrieval/cpy/retrieval_backend.cpp:207-227; submit :83-113): for request b,
+ * every candidate indexes[b, j] != -1 is scored with dot(query[b, :], data[candidate, :]) and
+ * the min(n_candidates, topk) best are returned in descending score order.
+ *
+ * data      fp32 [n_items, dim] (block representatives), device memory, 16-byte aligned.
+ * query     fp32 [B, dim], indexes int32 [B, max_n]; entries -1 or outside [0, n_items) are
+ *           no candidates.  topk <= 4096, dim <= 16384.
+ * out_idx   int32 [B, topk], out_score fp32 [B, topk]; positions past a request's candidate
+ *           count hold -1 / 0.  Equal scores keep list order (the reference leaves ties open).
+ * Scores are fp32 sums taken in a different order than the reference's sequential loop: they
+ * agree to ~1e-6 relative to sum |q_d x_d|.
+ */
+size_t ucm_dot_topk_workspace_bytes(int32_t B, int32_t max_n);
+int ucm_dot_topk(const float* data, int64_t n_items, int32_t dim, const float* query,
+                 const int32_t* indexes, int32_t B, int32_t max_n, int32_t topk,
+                 int32_t* out_idx, float* out_score, void* workspace, size_t workspace_bytes,
+                 ucm_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
  * 4. Cache store: pinned-host staging cache in front of a slower store backend — the caller
  *    of the gather / scatter path (ucm/store/cache/cc/).
  * ------------------------------------------------------------------------------------ */

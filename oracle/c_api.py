@@ -35,15 +35,16 @@ def lib():
     return _LIB
 
 
-def ref_backend():
-    """The reference's hash_retrieval_backend module compiled from its own source
-    (ucm/sparse/gsa_on_device/csrc/cuda/hash_retrieval/cpy/hash_retrieval_backend.cpp),
-    or None when oracle/_ref holds no build."""
+def ref_backend(name="hash_retrieval_backend"):
+    """A CPU retrieval backend of the reference compiled from its own source into oracle/_ref
+    (see the Makefile), or None when no build is there.  Names: "hash_retrieval_backend"
+    (ucm/sparse/gsa_on_device/csrc/cuda/hash_retrieval/cpy/hash_retrieval_backend.cpp) and
+    "retrieval_backend" (ucm/sparse/esa/retrieval/cpy/retrieval_backend.cpp)."""
     ext = sysconfig.get_config_var("EXT_SUFFIX")
-    path = os.path.join(_HERE, "_ref", "hash_retrieval_backend" + ext)
+    path = os.path.join(_HERE, "_ref", name + ext)
     if not os.path.exists(path):
         return None
-    spec = importlib.util.spec_from_file_location("hash_retrieval_backend", path)
+    spec = importlib.util.spec_from_file_location(name, path)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     return mod
@@ -244,3 +245,19 @@ def paged_copy(base, col_bytes, block_ids, flat, to_cache):
     lib().oracle_paged_copy(_p(base), _p(col_bytes), C.c_int32(base.shape[0]), _p(block_ids),
                             C.c_int64(block_ids.shape[0]), _p(flat), C.c_int(int(to_cache)))
     return flat
+
+
+def dot_topk(data, query, indexes, topk):
+    """data [n,dim] f32, query [B,dim] f32, indexes [B,max_n] int32 (-1 = none) ->
+    (indices int32 [B,topk], scores f32 [B,topk])."""
+    data = _c(data, np.float32)
+    query = _c(query, np.float32)
+    indexes = _c(indexes, np.int32)
+    n, dim = data.shape
+    B, max_n = indexes.shape
+    assert query.shape == (B, dim)
+    oi = np.zeros((B, topk), np.int32)
+    osc = np.zeros((B, topk), np.float32)
+    lib().oracle_dot_topk(_p(data), C.c_int64(n), C.c_int32(dim), _p(query), _p(indexes),
+                          C.c_int32(B), C.c_int32(max_n), C.c_int32(topk), _p(oi), _p(osc))
+    return oi, osc

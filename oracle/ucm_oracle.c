@@ -479,3 +479,60 @@ void oracle_paged_copy(const uint64_t* base, const uint64_t* col_bytes, int32_t 
             off += (size_t)col_bytes[c];
         }
 }
+
+/* ------------------------------------------------------------------------------------
+ * Float retrieval (ESA).  retrieval_backend.cpp:207-227: per request, every allowed index is
+ * scored with a sequential fp32 dot product (no fused multiply-add: the reference module is
+ * built for baseline x86-64), the pairs are partially sorted by descending score and the
+ * first min(n_allowed, topk) returned.  Entries -1 of `indexes` are dropped when the request
+ * is submitted (:96-104).  Ties: the reference's partial_sort leaves them open; here equal
+ * scores keep list order.  out rows are padded with -1 / 0.
+ * ------------------------------------------------------------------------------------ */
+__attribute__((optimize("fp-contract=off"))) static float seq_dot(const float* q, const float* x,
+                                                                  int32_t dim)
+{
+    float score = 0.0f;
+    for (int32_t d = 0; d < dim; ++d) {
+        const float p = q[d] * x[d];
+        score = score + p;
+    }
+    return score;
+}
+
+typedef struct {
+    float score;
+    int32_t pos;
+} dot_pair;
+
+static int dot_pair_cmp(const void* a, const void* b)
+{
+    const dot_pair* x = (const dot_pair*)a;
+    const dot_pair* y = (const dot_pair*)b;
+    if (x->score > y->score) return -1;
+    if (x->score < y->score) return 1;
+    return (x->pos > y->pos) - (x->pos < y->pos);
+}
+
+void oracle_dot_topk(const float* data, int64_t n_items, int32_t dim, const float* query,
+                     const int32_t* indexes, int32_t B, int32_t max_n, int32_t topk,
+                     int32_t* out_idx, float* out_score)
+{
+    dot_pair* pairs = (dot_pair*)malloc(sizeof(dot_pair) * (size_t)(max_n > 0 ? max_n : 1));
+    for (int32_t b = 0; b < B; ++b) {
+        int32_t n = 0;
+        for (int32_t j = 0; j < max_n; ++j) {
+            const int32_t item = indexes[(int64_t)b * max_n + j];
+            if (item < 0 || item >= n_items) continue;
+            pairs[n].score = seq_dot(query + (int64_t)b * dim, data + (int64_t)item * dim, dim);
+            pairs[n].pos = j;
+            ++n;
+        }
+        qsort(pairs, (size_t)n, sizeof(dot_pair), dot_pair_cmp);
+        for (int32_t t = 0; t < topk; ++t) {
+            const int has = t < n;
+            out_idx[(int64_t)b * topk + t] = has ? indexes[(int64_t)b * max_n + pairs[t].pos] : -1;
+            out_score[(int64_t)b * topk + t] = has ? pairs[t].score : 0.0f;
+        }
+    }
+    free(pairs);
+}

@@ -61,6 +61,8 @@ _SIGNATURES = {
     "ucm_trans_device_free": (ci, [vp]),
     "ucm_trans_host_register": (ci, [vp, sz, C.POINTER(vp)]),
     "ucm_trans_host_unregister": (ci, [vp]),
+    "ucm_dot_topk_workspace_bytes": (sz, [i32, i32]),
+    "ucm_dot_topk": (ci, [vp, i64, i32, vp, vp, i32, i32, i32, vp, vp, vp, sz, vp]),
     "ucm_cache_store_create": (ci, [i32, vp, sz, sz, sz, sz, vp, C.POINTER(vp)]),
     "ucm_cache_store_destroy": (ci, [vp]),
     "ucm_cache_store_nodes": (sz, [vp]),
