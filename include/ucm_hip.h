@@ -332,6 +332,29 @@ int ucm_dot_topk(const float* data, int64_t n_items, int32_t dim, const float* q
                  int32_t* out_idx, float* out_score, void* workspace, size_t workspace_bytes,
                  ucm_stream_t stream);
 
+/*
+ * GPU form of KVStar's block retrieval
+ * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:816-985;
+ * submitted through AsyncRetrieveByCPU, py_intf/py_intf.cpp:13-52): attention-probability mass
+ * per KV block for a group of query tokens, then the topk blocks.
+ *
+ * query         fp16 [X, Hq, d_orig] contiguous (the last X query tokens of the request).
+ * blk_repre     fp16 [n_blocks, M, Hkv, d] contiguous: M representative keys per block.
+ * pruned_index  int64 [Hkv, d] or NULL: channel j of KV head h's keys corresponds to channel
+ *               pruned_index[h, j] of the queries; NULL requires d == d_orig.
+ * For every (x, H): p = softmax over all n_blocks * M representatives of q[x, H] . k[s, H/g]
+ * (left unnormalised when the sum of exponentials is <= 1e-9, as the reference does);
+ * score[n] = sum of p over x, H and the M representatives of block n.
+ * out_idx / out_score  [topk]: blocks by descending score, -1 / 0 past n_blocks; equal scores
+ *               in ascending block order.  topk <= 4096, d <= 1024, X * Hq <= 65535.
+ */
+size_t ucm_kvstar_topk_workspace_bytes(int32_t X, int32_t Hq, int64_t n_blocks, int32_t M);
+int ucm_kvstar_topk(const void* query, int32_t X, int32_t Hq, int32_t d_orig,
+                    const void* blk_repre, int64_t n_blocks, int32_t M, int32_t Hkv, int32_t d,
+                    const int64_t* pruned_index, int32_t topk,
+                    int32_t* out_idx, float* out_score, void* workspace, size_t workspace_bytes,
+                    ucm_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * 4. Cache store: pinned-host staging cache in front of a slower store backend — the caller
  *    of the gather / scatter path (ucm/store/cache/cc/).

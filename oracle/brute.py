@@ -106,3 +106,22 @@ def update_seq_lens(lens, topk_tok, BS):
     lens = np.asarray(lens, np.int64)
     drop = (np.clip(lens - topk_tok, 0, None) + BS - 1) // BS
     return (lens - drop * BS).astype(np.int32)
+
+
+def kvstar_block_scores(query_f16, blk_repre_f16, pruned_index=None):
+    """float64 restatement of the KVStar block score (simd_compute_kernel.cpp:816-952) with
+    library routines: einsum for q.k, a max-shifted softmax over all representatives, a reshape
+    and sum per block.  Returns [n_blocks] float64."""
+    q = np.asarray(query_f16, np.float16).astype(np.float64)      # [X, Hq, d_orig]
+    k = np.asarray(blk_repre_f16, np.float16).astype(np.float64)  # [n, M, Hkv, d]
+    n, M, Hkv, d = k.shape
+    X, Hq, _ = q.shape
+    g = Hq // Hkv
+    if pruned_index is not None:
+        pr = np.asarray(pruned_index, np.int64)                   # [Hkv, d]
+        q = np.stack([q[:, H, pr[H // g]] for H in range(Hq)], axis=1)
+    kh = np.repeat(k.reshape(n * M, Hkv, d), g, axis=1)           # [S, Hq, d]
+    sc = np.einsum("xhd,shd->xhs", q, kh)
+    sc = np.exp(sc - sc.max(axis=2, keepdims=True))
+    sc = sc / sc.sum(axis=2, keepdims=True)
+    return sc.reshape(X * Hq, n, M).sum(axis=(0, 2))

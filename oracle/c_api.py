@@ -261,3 +261,28 @@ def dot_topk(data, query, indexes, topk):
     lib().oracle_dot_topk(_p(data), C.c_int64(n), C.c_int32(dim), _p(query), _p(indexes),
                           C.c_int32(B), C.c_int32(max_n), C.c_int32(topk), _p(oi), _p(osc))
     return oi, osc
+
+
+def kvstar_topk(query_f16, blk_repre_f16, topk, pruned_index=None):
+    """query fp16 [X,Hq,d_orig], blk_repre fp16 [n,M,Hkv,d], pruned_index int64 [Hkv,d] or None
+    -> (indices int64 [count], scores f32 [count], all block scores f32 [n])."""
+    q = _c(query_f16, np.float16)
+    k = _c(blk_repre_f16, np.float16)
+    X, Hq, d_orig = q.shape
+    n, M, Hkv, d = k.shape
+    pr = _c(pruned_index, np.int64) if pruned_index is not None else None
+    oi = np.zeros(max(topk, 1), np.int64)
+    osc = np.zeros(max(topk, 1), np.float32)
+    cnt = C.c_int32(0)
+    allsc = np.zeros(n, np.float32)
+    lib().oracle_kvstar_topk(_p(q), C.c_int32(X), C.c_int32(Hq), C.c_int32(d_orig), _p(k),
+                             C.c_int64(n), C.c_int32(M), C.c_int32(Hkv), C.c_int32(d), _p(pr),
+                             C.c_int32(topk), _p(oi), _p(osc), C.byref(cnt), _p(allsc))
+    return oi[:cnt.value], osc[:cnt.value], allsc
+
+
+def half_to_float(bits_u16):
+    h = _c(bits_u16, np.uint16)
+    out = np.zeros(h.shape, np.float32)
+    lib().oracle_half_to_float(_p(h), C.c_int64(h.size), _p(out))
+    return out

@@ -536,3 +536,143 @@ void oracle_dot_topk(const float* data, int64_t n_items, int32_t dim, const floa
     }
     free(pairs);
 }
+
+/* ------------------------------------------------------------------------------------
+ * KVStar block retrieval.  kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp
+ * :816-985 (scalar_impl::execute_impl), statement by statement: channel pruning of the queries
+ * (:846-872), sequential fp32 q.k over all S = n_blocks * M representatives (:885-911), softmax
+ * per (token, q head) with the "sum_exp > 1e-9" guard (:913-942), block sums accumulated row by
+ * row (:944-952), a size-topk min-heap of (score, block) pairs with strict-greater replacement,
+ * emptied back to front (:954-977).  fp16 -> fp32 as fp16_to_float (:780-812).
+ * all_scores (optional) receives the n_blocks block scores.
+ * ------------------------------------------------------------------------------------ */
+static float half_bits_to_float(uint16_t h)
+{
+    const uint32_t s = ((uint32_t)h & 0x8000u) << 16, e = (h >> 10) & 0x1Fu, m = h & 0x3FFu;
+    uint32_t bits;
+    if (e == 0) {
+        if (m == 0) {
+            bits = s;
+        } else {  /* subnormal: normalise */
+            uint32_t mm = m, ee = 113;
+            while (!(mm & 0x400u)) {
+                mm <<= 1;
+                --ee;
+            }
+            bits = s | (ee << 23) | ((mm & 0x3FFu) << 13);
+        }
+    } else if (e == 0x1Fu) {
+        bits = s | 0x7F800000u | (m << 13);
+    } else {
+        bits = s | ((e + 112u) << 23) | (m << 13);
+    }
+    float f;
+    memcpy(&f, &bits, sizeof(f));
+    return f;
+}
+
+void oracle_half_to_float(const uint16_t* h, int64_t n, float* out)
+{
+    for (int64_t i = 0; i < n; ++i) out[i] = half_bits_to_float(h[i]);
+}
+
+typedef struct {
+    float score;
+    int64_t idx;
+} kv_pair;
+
+static int kv_pair_less(kv_pair a, kv_pair b)  /* std::pair ordering */
+{
+    return a.score < b.score || (a.score == b.score && a.idx < b.idx);
+}
+
+static void heap_sift_down(kv_pair* h, int64_t n, int64_t i)
+{
+    for (;;) {
+        int64_t l = 2 * i + 1, r = l + 1, m = i;
+        if (l < n && kv_pair_less(h[l], h[m])) m = l;
+        if (r < n && kv_pair_less(h[r], h[m])) m = r;
+        if (m == i) return;
+        kv_pair t = h[i];
+        h[i] = h[m];
+        h[m] = t;
+        i = m;
+    }
+}
+
+__attribute__((optimize("fp-contract=off")))
+void oracle_kvstar_topk(const uint16_t* q, int32_t X, int32_t Hq, int32_t d_orig, const uint16_t* k,
+                        int64_t n_blocks, int32_t M, int32_t Hkv, int32_t d, const int64_t* pruned,
+                        int32_t topk, int64_t* out_idx, float* out_score, int32_t* out_count,
+                        float* all_scores)
+{
+    const int32_t g = Hq / Hkv;
+    const int64_t S = n_blocks * M, rows = (int64_t)X * Hq;
+    float* sc = (float*)malloc(sizeof(float) * (size_t)(rows * S));
+    float* qrow = (float*)malloc(sizeof(float) * (size_t)d);
+    for (int64_t x = 0; x < X; ++x)
+        for (int32_t h = 0; h < Hkv; ++h)
+            for (int32_t gg = 0; gg < g; ++gg) {
+                const int32_t H = h * g + gg;
+                for (int32_t j = 0; j < d; ++j) {
+                    const int64_t src = pruned ? pruned[(int64_t)h * d + j] : j;
+                    qrow[j] = half_bits_to_float(q[(x * Hq + H) * (int64_t)d_orig + src]);
+                }
+                for (int64_t s = 0; s < S; ++s) {
+                    const uint16_t* kv = k + (s * Hkv + h) * (int64_t)d;
+                    float score = 0.0f;
+                    for (int32_t j = 0; j < d; ++j) {
+                        const float p = qrow[j] * half_bits_to_float(kv[j]);
+                        score = score + p;
+                    }
+                    sc[(x * Hq + H) * S + s] = score;
+                }
+            }
+    for (int64_t i = 0; i < rows; ++i) {
+        float* cur = sc + i * S;
+        float mx = cur[0];
+        for (int64_t s = 1; s < S; ++s)
+            if (cur[s] > mx) mx = cur[s];
+        float sum = 0.0f;
+        for (int64_t s = 0; s < S; ++s) {
+            cur[s] = expf(cur[s] - mx);
+            sum = sum + cur[s];
+        }
+        if (sum > 1e-9)
+            for (int64_t s = 0; s < S; ++s) cur[s] = cur[s] / sum;
+    }
+    float* fin = (float*)calloc((size_t)n_blocks, sizeof(float));
+    for (int64_t i = 0; i < rows; ++i)
+        for (int64_t s = 0; s < S; ++s) fin[s / M] = fin[s / M] + sc[i * S + s];
+    if (all_scores) memcpy(all_scores, fin, sizeof(float) * (size_t)n_blocks);
+    kv_pair* heap = (kv_pair*)malloc(sizeof(kv_pair) * (size_t)(topk > 0 ? topk : 1));
+    int64_t hn = 0;
+    for (int64_t n = 0; n < n_blocks; ++n) {
+        const kv_pair p = {fin[n], n};
+        if (hn < topk) {  /* push */
+            int64_t i = hn++;
+            heap[i] = p;
+            while (i > 0 && kv_pair_less(heap[i], heap[(i - 1) / 2])) {
+                kv_pair t = heap[i];
+                heap[i] = heap[(i - 1) / 2];
+                heap[(i - 1) / 2] = t;
+                i = (i - 1) / 2;
+            }
+        } else if (hn > 0 && fin[n] > heap[0].score) {  /* replace the minimum */
+            heap[0] = p;
+            heap_sift_down(heap, hn, 0);
+        }
+    }
+    *out_count = (int32_t)hn;
+    for (int64_t pos = hn - 1; pos >= 0; --pos) {  /* smallest pair goes last */
+        out_idx[pos] = heap[0].idx;
+        out_score[pos] = heap[0].score;
+        heap[0] = heap[hn - 1];
+        --hn;
+        heap_sift_down(heap, hn, 0);
+    }
+    free(heap);
+    free(fin);
+    free(qrow);
+    free(sc);
+}

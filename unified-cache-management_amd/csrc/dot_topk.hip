@@ -15,24 +15,14 @@
 // Scores differ from the reference's in the last bits (the partial sums are added in a
 // different order); the tolerance is stated where the results are compared.
 #include "common.h"
+#include "float_topk.h"
 
 namespace {
 
 constexpr int kDotThreads = 256;
 constexpr int kRowsPerWave = 4;
-constexpr int kSortThreads = 1024;
-constexpr int kMaxTopk = 4096;  // winners sorted in LDS: 8 bytes each (32 KiB)
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-// Order-preserving key of a score: larger score <-> larger key.  0 is reserved for "no
-// candidate", 1 for NaN (below every number, above nothing else).
-__device__ __forceinline__ uint32_t score_key(float s)
-{
-    if (s != s) return 1u;
-    const uint32_t u = __float_as_uint(s);
-    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
 
 struct DotArgs {
     const float* data;
@@ -85,133 +75,6 @@ __global__ __launch_bounds__(kDotThreads) void dot_score_kernel(DotArgs a)
     }
 }
 
-struct SortArgs {
-    const uint32_t* keys;   // [B][max_n]
-    const float* scores;    // [B][max_n]
-    const int32_t* idx;     // [B][max_n]
-    int max_n, topk, cap;   // cap = power of two >= topk: LDS elements
-    int32_t* out_idx;       // [B][topk]
-    float* out_score;       // [B][topk]
-};
-
-// Exclusive prefix sum of one int per thread over the 1024-thread workgroup.
-__device__ __forceinline__ int scan1024(int v, int* wsum, int* total)
-{
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    int inc = v;
-#pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-        const int o = __shfl_up(inc, s);
-        if (lane >= s) inc += o;
-    }
-    __syncthreads();
-    if (lane == 63) wsum[w] = inc;
-    __syncthreads();
-    int base = 0, tot = 0;
-    for (int i = 0; i < kSortThreads / 64; ++i) {
-        const int x = wsum[i];
-        if (i < w) base += x;
-        tot += x;
-    }
-    *total = tot;
-    return base + inc - v;
-}
-
-__global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
-{
-    extern __shared__ unsigned long long win[];  // [cap] (key << 32) | ~position
-    __shared__ int hist[256];
-    __shared__ int wsum[kSortThreads / 64];
-    __shared__ int s_digit, s_need, s_count;
-    const int b = blockIdx.x;
-    const uint32_t* keys = a.keys + (int64_t)b * a.max_n;
-    const int tid = threadIdx.x;
-
-    // candidates present
-    int mine = 0;
-    for (int i = tid; i < a.max_n; i += kSortThreads) mine += keys[i] != 0u;
-    int n_valid;
-    (void)scan1024(mine, wsum, &n_valid);
-    const int kk = n_valid < a.topk ? n_valid : a.topk;
-
-    // ---- radix search, 8 bits a pass, for the kk-th largest key among the candidates ----
-    uint32_t prefix = 0, mask = 0;
-    int need = kk;
-    for (int shift = 24; shift >= 0 && kk > 0; shift -= 8) {
-        if (tid < 256) hist[tid] = 0;
-        __syncthreads();
-        for (int i = tid; i < a.max_n; i += kSortThreads) {
-            const uint32_t k = keys[i];
-            if (k != 0u && (k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255], 1);
-        }
-        __syncthreads();
-        if (tid == 0) {
-            int d = 255, acc = 0;
-            for (; d > 0; --d) {
-                if (acc + hist[d] >= need) break;
-                acc += hist[d];
-            }
-            s_digit = d;
-            s_need = need - acc;  // still to take among keys with this digit
-        }
-        __syncthreads();
-        prefix |= (uint32_t)s_digit << shift;
-        mask |= 255u << shift;
-        need = s_need;
-        __syncthreads();
-    }
-    const uint32_t thr = prefix;  // the kk-th largest key; `need` of the keys equal to it are taken
-
-    // ---- winners into LDS: every key above the threshold, the first `need` equal to it ----
-    for (int i = tid; i < a.cap; i += kSortThreads) win[i] = 0ull;
-    if (tid == 0) s_count = 0;
-    __syncthreads();
-    int eq_before = 0;  // keys equal to the threshold in earlier chunks
-    for (int base = 0; base < a.max_n && kk > 0; base += kSortThreads) {
-        const int i = base + tid;
-        const uint32_t k = i < a.max_n ? keys[i] : 0u;
-        const bool gt = k > thr && k != 0u;
-        const bool eq = k == thr && k != 0u;
-        int eq_total;
-        const int eq_rank = eq_before + scan1024(eq ? 1 : 0, wsum, &eq_total);
-        if (gt || (eq && eq_rank < need)) {
-            const int slot = atomicAdd(&s_count, 1);
-            win[slot] = ((unsigned long long)k << 32) | (uint32_t)(~(uint32_t)i);
-        }
-        eq_before += eq_total;
-    }
-    __syncthreads();
-
-    // ---- bitonic sort, descending: larger key first, then smaller position ----
-    for (int size = 2; size <= a.cap; size <<= 1) {
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            for (int t = tid; t < a.cap / 2; t += kSortThreads) {
-                const int lo = 2 * t - (t & (stride - 1));
-                const int hi = lo + stride;
-                const bool desc = (lo & size) == 0;
-                const unsigned long long x = win[lo], y = win[hi];
-                if ((x < y) == desc) {
-                    win[lo] = y;
-                    win[hi] = x;
-                }
-            }
-            __syncthreads();
-        }
-    }
-
-    for (int t = tid; t < a.topk; t += kSortThreads) {
-        int32_t oi = -1;
-        float os = 0.0f;
-        if (t < kk) {
-            const int pos = (int)(~(uint32_t)(win[t] & 0xffffffffull));
-            oi = a.idx[(int64_t)b * a.max_n + pos];
-            os = a.scores[(int64_t)b * a.max_n + pos];
-        }
-        a.out_idx[(int64_t)b * a.topk + t] = oi;
-        a.out_score[(int64_t)b * a.topk + t] = os;
-    }
-}
-
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace
@@ -250,10 +113,6 @@ extern "C" int ucm_dot_topk(const float* data, int64_t n_items, int32_t dim, con
     if (rc != UCM_OK) return rc;
     SortArgs s{};
     s.keys = d.keys; s.scores = d.scores; s.idx = indexes; s.max_n = max_n; s.topk = topk;
-    int cap = 2;
-    while (cap < topk) cap <<= 1;
-    s.cap = cap;
     s.out_idx = out_idx; s.out_score = out_score;
-    hipLaunchKernelGGL(topk_sort_kernel, dim3((unsigned)B), dim3(kSortThreads), (size_t)cap * 8, st, s);
-    return ucm::launch_status("topk_sort_kernel");
+    return launch_topk_sort(s, B, st);
 }

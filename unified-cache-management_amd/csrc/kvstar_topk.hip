@@ -1,0 +1,231 @@
+// KVStar block retrieval for gfx950: attention-probability mass per KV block, then top-k.
+//
+// GPU counterpart of the reference's CPU kernel
+// (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:816-985, the
+// scalar form; its NEON / AVX forms compute the same quantities in other summation orders):
+//   1. optional channel pruning of the queries: q'[x, H, j] = q[x, H, pruned_index[H / g, j]];
+//   2. scores[x, H, s] = q'[x, H, :] . k[s, H / g, :] over the S = n_blocks * M block
+//      representatives, fp16 inputs, fp32 accumulation;
+//   3. softmax over s for every (x, H) (left unnormalised when the sum of exponentials is
+//      <= 1e-9, as the reference does);
+//   4. block score[n] = sum over x, H and the M representatives of block n;
+//   5. the topk blocks by descending score.
+// Kernels: qk_score_kernel (one thread per (s, kv head), the head's query rows broadcast from
+// LDS, K read once: the HBM-bound part), row_stats_kernel (max and sum of exponentials per
+// (x, H) row), block_mass_kernel (probabilities summed over rows in a fixed order, then over a
+// block's representatives: deterministic, no atomics) and the shared top-k selection.
+// Sums are taken in a different order than the reference's loops; the tolerance is stated
+// where the results are compared.  Equal scores come out in ascending block order (the
+// reference's heap pops them in descending block order).
+#include <hip/hip_fp16.h>
+
+#include "common.h"
+#include "float_topk.h"
+
+namespace {
+
+constexpr int kQkThreads = 256;
+constexpr int kRowTile = 16;  // query rows of one KV head scored per pass over a K vector
+
+struct QkArgs {
+    const __half* q;        // [X, Hq, d_orig]
+    const __half* k;        // [S, Hkv, d]
+    const int64_t* pruned;  // [Hkv, d] or null
+    int X, Hq, Hkv, g, d_orig, d;
+    int64_t S;
+    float* scores;          // [X * Hq, S]
+};
+
+// grid = (ceil(S / 256), Hkv, ceil(X * g / kRowTile)); LDS: kRowTile rows of d floats
+__global__ __launch_bounds__(kQkThreads) void qk_score_kernel(QkArgs a)
+{
+    extern __shared__ float qs[];  // [kRowTile][d]
+    const int h = blockIdx.y;
+    const int row0 = blockIdx.z * kRowTile;  // first (x, gg) pair of this pass
+    const int rows = a.X * a.g;
+    // stage the pass's query rows of KV head h: row r = x * g + gg  <->  q head H = h * g + gg
+    for (int i = threadIdx.x; i < kRowTile * a.d; i += kQkThreads) {
+        const int r = row0 + i / a.d, j = i % a.d;
+        float v = 0.0f;
+        if (r < rows) {
+            const int x = r / a.g, H = h * a.g + r % a.g;
+            int64_t src = a.pruned ? a.pruned[(int64_t)h * a.d + j] : j;
+            src = src < 0 ? 0 : (src >= a.d_orig ? a.d_orig - 1 : src);  // stay inside the row
+            v = __half2float(a.q[((int64_t)x * a.Hq + H) * a.d_orig + src]);
+        }
+        qs[i] = v;
+    }
+    __syncthreads();
+    const int64_t s = (int64_t)blockIdx.x * kQkThreads + threadIdx.x;
+    if (s >= a.S) return;
+    const __half* kv = a.k + (s * a.Hkv + h) * a.d;
+    float acc[kRowTile];
+#pragma unroll
+    for (int r = 0; r < kRowTile; ++r) acc[r] = 0.0f;
+    if ((a.d & 7) == 0) {  // 16-byte pieces of the K vector
+        for (int j = 0; j < a.d; j += 8) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(kv + j);
+            __half hv[8];
+            __builtin_memcpy(hv, &raw, 16);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float kf = __half2float(hv[i]);
+#pragma unroll
+                for (int r = 0; r < kRowTile; ++r)
+                    acc[r] = __builtin_fmaf(qs[r * a.d + j + i], kf, acc[r]);
+            }
+        }
+    } else {
+        for (int j = 0; j < a.d; ++j) {
+            const float kf = __half2float(kv[j]);
+#pragma unroll
+            for (int r = 0; r < kRowTile; ++r) acc[r] = __builtin_fmaf(qs[r * a.d + j], kf, acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kRowTile; ++r) {
+        const int rr = row0 + r;
+        if (rr < rows) {
+            const int x = rr / a.g, H = h * a.g + rr % a.g;
+            a.scores[((int64_t)x * a.Hq + H) * a.S + s] = acc[r];
+        }
+    }
+}
+
+// One workgroup per (x, H) row: max over s and sum of exp(score - max).
+__global__ __launch_bounds__(kQkThreads) void row_stats_kernel(const float* __restrict__ scores,
+                                                               int64_t S, float* __restrict__ stats)
+{
+    __shared__ float red[kQkThreads / 64];
+    const float* row = scores + (int64_t)blockIdx.x * S;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    float m = -INFINITY;
+    for (int64_t s = threadIdx.x; s < S; s += kQkThreads) m = fmaxf(m, row[s]);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if (lane == 0) red[w] = m;
+    __syncthreads();
+    m = red[0];
+    for (int i = 1; i < kQkThreads / 64; ++i) m = fmaxf(m, red[i]);
+    __syncthreads();
+    float sum = 0.0f;
+    for (int64_t s = threadIdx.x; s < S; s += kQkThreads) sum += expf(row[s] - m);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+    if (lane == 0) red[w] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.0f;
+        for (int i = 0; i < kQkThreads / 64; ++i) t += red[i];
+        stats[2 * blockIdx.x] = m;
+        // the reference normalises only when the sum exceeds 1e-9
+        stats[2 * blockIdx.x + 1] = t > 1e-9f ? 1.0f / t : 1.0f;
+    }
+}
+
+// One thread per block n: probabilities of its M representatives summed over all rows.
+__global__ __launch_bounds__(kQkThreads) void block_mass_kernel(const float* __restrict__ scores,
+                                                                const float* __restrict__ stats,
+                                                                int rows, int64_t S, int M,
+                                                                int64_t n_blocks,
+                                                                float* __restrict__ mass,
+                                                                uint32_t* __restrict__ keys,
+                                                                int32_t* __restrict__ ident)
+{
+    const int64_t n = (int64_t)blockIdx.x * kQkThreads + threadIdx.x;
+    if (n >= n_blocks) return;
+    float total = 0.0f;
+    for (int r = 0; r < rows; ++r) {
+        const float mx = stats[2 * r], inv = stats[2 * r + 1];
+        const float* row = scores + (int64_t)r * S + n * M;
+        for (int m = 0; m < M; ++m) total += expf(row[m] - mx) * inv;
+    }
+    mass[n] = total;
+    keys[n] = score_key(total);
+    ident[n] = (int32_t)n;
+}
+
+size_t align256k(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct KvstarWs {
+    float* scores;
+    float* stats;
+    float* mass;
+    uint32_t* keys;
+    int32_t* ident;
+    size_t bytes;
+};
+
+KvstarWs carve_kvstar(void* base, int64_t rows, int64_t S, int64_t n_blocks)
+{
+    KvstarWs w{};
+    size_t off = 0;
+    w.scores = (float*)((char*)base + off);
+    off += align256k((size_t)rows * S * 4);
+    w.stats = (float*)((char*)base + off);
+    off += align256k((size_t)rows * 8);
+    w.mass = (float*)((char*)base + off);
+    off += align256k((size_t)n_blocks * 4);
+    w.keys = (uint32_t*)((char*)base + off);
+    off += align256k((size_t)n_blocks * 4);
+    w.ident = (int32_t*)((char*)base + off);
+    off += align256k((size_t)n_blocks * 4);
+    w.bytes = off;
+    return w;
+}
+
+}  // namespace
+
+extern "C" size_t ucm_kvstar_topk_workspace_bytes(int32_t X, int32_t Hq, int64_t n_blocks, int32_t M)
+{
+    if (X <= 0 || Hq <= 0 || n_blocks <= 0 || M <= 0) return 256;
+    return carve_kvstar(nullptr, (int64_t)X * Hq, n_blocks * M, n_blocks).bytes;
+}
+
+extern "C" int ucm_kvstar_topk(const void* query, int32_t X, int32_t Hq, int32_t d_orig,
+                               const void* blk_repre, int64_t n_blocks, int32_t M, int32_t Hkv,
+                               int32_t d, const int64_t* pruned_index, int32_t topk,
+                               int32_t* out_idx, float* out_score, void* workspace,
+                               size_t workspace_bytes, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(query && blk_repre && out_idx && out_score, "null pointer");
+    UCM_REQUIRE(X > 0 && Hq > 0 && Hkv > 0 && d > 0 && d_orig > 0 && n_blocks > 0 && M > 0,
+                "non-positive shape");
+    UCM_REQUIRE(Hq % Hkv == 0, "Num_q_heads must be a divisible by num_kv_heads.");
+    UCM_REQUIRE(pruned_index || d == d_orig,
+                "Dimension mismatch: No dPrunedIndex, but Q and K head dims differ.");
+    UCM_REQUIRE(topk > 0, "topk %d must be positive", topk);
+    if (topk > kMaxTopk) return ucm::fail(UCM_EUNSUPPORTED, "topk %d above %d", topk, kMaxTopk);
+    UCM_REQUIRE((size_t)kRowTile * d * 4 <= 64 * 1024, "head dim %d above 1024", d);
+    UCM_REQUIRE(n_blocks <= INT32_MAX && n_blocks * M <= INT32_MAX, "too many block representatives");
+    const int64_t rows = (int64_t)X * Hq, S = n_blocks * M;
+    UCM_REQUIRE(rows <= 65535, "more than 65535 query rows");
+    UCM_REQUIRE(workspace && workspace_bytes >= ucm_kvstar_topk_workspace_bytes(X, Hq, n_blocks, M),
+                "workspace too small");
+    UCM_REQUIRE((((uintptr_t)blk_repre | (uintptr_t)workspace) & 15) == 0, "block representatives must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const KvstarWs w = carve_kvstar(workspace, rows, S, n_blocks);
+    QkArgs a{};
+    a.q = (const __half*)query; a.k = (const __half*)blk_repre; a.pruned = pruned_index;
+    a.X = X; a.Hq = Hq; a.Hkv = Hkv; a.g = Hq / Hkv; a.d_orig = d_orig; a.d = d; a.S = S;
+    a.scores = w.scores;
+    const dim3 grid((unsigned)ucm::ceil_div(S, kQkThreads), (unsigned)Hkv,
+                    (unsigned)ucm::ceil_div((int64_t)X * a.g, kRowTile));
+    UCM_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "too many heads or query rows");
+    hipLaunchKernelGGL(qk_score_kernel, grid, dim3(kQkThreads), (size_t)kRowTile * d * 4, st, a);
+    int rc = ucm::launch_status("qk_score_kernel");
+    if (rc != UCM_OK) return rc;
+    hipLaunchKernelGGL(row_stats_kernel, dim3((unsigned)rows), dim3(kQkThreads), 0, st, w.scores, S, w.stats);
+    rc = ucm::launch_status("row_stats_kernel");
+    if (rc != UCM_OK) return rc;
+    hipLaunchKernelGGL(block_mass_kernel, dim3((unsigned)ucm::ceil_div(n_blocks, kQkThreads)),
+                       dim3(kQkThreads), 0, st, w.scores, w.stats, (int)rows, S, (int)M, n_blocks,
+                       w.mass, w.keys, w.ident);
+    rc = ucm::launch_status("block_mass_kernel");
+    if (rc != UCM_OK) return rc;
+    SortArgs s{};
+    s.keys = w.keys; s.scores = w.mass; s.idx = w.ident; s.max_n = (int)n_blocks; s.topk = topk;
+    s.out_idx = out_idx; s.out_score = out_score;
+    return launch_topk_sort(s, 1, st);
+}

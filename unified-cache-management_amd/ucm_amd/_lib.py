@@ -63,6 +63,8 @@ _SIGNATURES = {
     "ucm_trans_host_unregister": (ci, [vp]),
     "ucm_dot_topk_workspace_bytes": (sz, [i32, i32]),
     "ucm_dot_topk": (ci, [vp, i64, i32, vp, vp, i32, i32, i32, vp, vp, vp, sz, vp]),
+    "ucm_kvstar_topk_workspace_bytes": (sz, [i32, i32, i64, i32]),
+    "ucm_kvstar_topk": (ci, [vp, i32, i32, i32, vp, i64, i32, i32, i32, vp, i32, vp, vp, vp, sz, vp]),
     "ucm_cache_store_create": (ci, [i32, vp, sz, sz, sz, sz, vp, C.POINTER(vp)]),
     "ucm_cache_store_destroy": (ci, [vp]),
     "ucm_cache_store_nodes": (sz, [vp]),
