@@ -144,6 +144,11 @@ def cpu_side_baselines(torch):
     c_api.dot_topk(vec, qq, cand, 3000)
     t1 = time.perf_counter()
     out["esa_dot_topk_cpu"] = {"threads": 1, "ms": (t1 - t0) * 1e3}
+    kq, kk, kp = _kvstar_case(np)
+    t0 = time.perf_counter()
+    c_api.kvstar_topk(kq, kk, 64, kp)
+    t1 = time.perf_counter()
+    out["kvstar_topk_cpu"] = {"threads": 1, "ms": (t1 - t0) * 1e3}
     n, size = 1024, 256 * 1024
     pool = np.random.default_rng(5).integers(0, 256, size=(n, size), dtype=np.uint8)
     chunks = [pool[i] for i in np.random.default_rng(6).permutation(n)]
@@ -156,10 +161,25 @@ def cpu_side_baselines(torch):
     return out
 
 
-def _esa_ws(B, max_n):
+def _kvstar_case(np):
+    """The reference example's KVStar shape (examples/offline_inference_kvstar.py:81-99): 32k
+    context in 128-token blocks less the fixed windows, 2-token merge -> 64 representatives per
+    block, channels pruned to a quarter, a group of 8 queries, 32 q heads over 8 kv heads."""
+    rng = np.random.default_rng(9)
+    q = (rng.standard_normal((8, 32, 128)) * 0.5).astype(np.float16)
+    k = (rng.standard_normal((253, 64, 8, 32)) * 0.5).astype(np.float16)
+    pr = np.stack([np.sort(rng.permutation(128)[:32]) for _ in range(8)]).astype(np.int64)
+    return q, k, pr
+
+
+def _lib_mod():
     from ucm_amd import _lib
 
-    return int(_lib.lib().ucm_dot_topk_workspace_bytes(B, max_n))
+    return _lib
+
+
+def _esa_ws(B, max_n):
+    return int(_lib_mod().lib().ucm_dot_topk_workspace_bytes(B, max_n))
 
 
 def extras(torch, enc_k, gen):
@@ -241,6 +261,23 @@ def extras(torch, enc_k, gen):
     out["esa_dot_topk"] = {"candidates": 2 * 8000, "dim": 1024, "topk": 3000, "ms": ms,
                            "gather_GBps": 2 * 8000 * 4096 / ms / 1e6}
     del vecs
+
+    # --- float retrieval (KVStar) ---
+    from ucm_amd.sparse.kvstar_retrieve import kvstar_topk
+
+    kq, kk, kp = (torch.from_numpy(t).cuda() for t in _kvstar_case(np))
+    kws = torch.empty(_lib_mod().lib().ucm_kvstar_topk_workspace_bytes(8, 32, 253, 64), dtype=torch.uint8,
+                      device="cuda")
+    for _ in range(3):
+        kvstar_topk(kq, kk, kp, 64, kws)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        kvstar_topk(kq, kk, kp, 64, kws)
+    e1.record()
+    torch.cuda.synchronize()
+    out["kvstar_topk"] = {"queries": 8, "q_heads": 32, "blocks": 253, "representatives": 253 * 64,
+                          "dim": 32, "topk": 64, "ms": e0.elapsed_time(e1) / reps}
 
     # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---
     L, NBP, n_req, n_sel = 32, 256, 4, 64

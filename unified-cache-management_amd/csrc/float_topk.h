@@ -81,14 +81,14 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
             if (k != 0u && (k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255], 1);
         }
         __syncthreads();
-        if (tid == 0) {
-            int d = 255, acc = 0;
-            for (; d > 0; --d) {
-                if (acc + hist[d] >= need) break;
-                acc += hist[d];
-            }
-            s_digit = d;
-            s_need = need - acc;  // still to take among keys with this digit
+        // digits in descending order, one per thread: the chosen digit is where the running
+        // count first reaches `need`
+        const int cnt = tid < 256 ? hist[255 - tid] : 0;
+        int all;
+        const int before = scan1024(cnt, wsum, &all);
+        if (tid < 256 && before < need && before + cnt >= need) {
+            s_digit = 255 - tid;
+            s_need = need - before;  // still to take among keys with this digit
         }
         __syncthreads();
         prefix |= (uint32_t)s_digit << shift;

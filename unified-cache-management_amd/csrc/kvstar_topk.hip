@@ -25,6 +25,7 @@
 namespace {
 
 constexpr int kQkThreads = 256;
+constexpr int kStatThreads = 1024;
 constexpr int kRowTile = 16;  // query rows of one KV head scored per pass over a K vector
 
 struct QkArgs {
@@ -39,7 +40,7 @@ struct QkArgs {
 // grid = (ceil(S / 256), Hkv, ceil(X * g / kRowTile)); LDS: kRowTile rows of d floats
 __global__ __launch_bounds__(kQkThreads) void qk_score_kernel(QkArgs a)
 {
-    extern __shared__ float qs[];  // [kRowTile][d]
+    extern __shared__ __align__(16) float qs[];  // [kRowTile][d]
     const int h = blockIdx.y;
     const int row0 = blockIdx.z * kRowTile;  // first (x, gg) pair of this pass
     const int rows = a.X * a.g;
@@ -67,12 +68,23 @@ __global__ __launch_bounds__(kQkThreads) void qk_score_kernel(QkArgs a)
             const uint4 raw = *reinterpret_cast<const uint4*>(kv + j);
             __half hv[8];
             __builtin_memcpy(hv, &raw, 16);
+            float kf[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float kf = __half2float(hv[i]);
+            for (int i = 0; i < 8; ++i) kf[i] = __half2float(hv[i]);
 #pragma unroll
-                for (int r = 0; r < kRowTile; ++r)
-                    acc[r] = __builtin_fmaf(qs[r * a.d + j + i], kf, acc[r]);
+            for (int r = 0; r < kRowTile; ++r) {  // 16-byte LDS reads, the same address in all lanes
+                const float4 qa = *reinterpret_cast<const float4*>(qs + r * a.d + j);
+                const float4 qb = *reinterpret_cast<const float4*>(qs + r * a.d + j + 4);
+                float t = acc[r];
+                t = __builtin_fmaf(qa.x, kf[0], t);
+                t = __builtin_fmaf(qa.y, kf[1], t);
+                t = __builtin_fmaf(qa.z, kf[2], t);
+                t = __builtin_fmaf(qa.w, kf[3], t);
+                t = __builtin_fmaf(qb.x, kf[4], t);
+                t = __builtin_fmaf(qb.y, kf[5], t);
+                t = __builtin_fmaf(qb.z, kf[6], t);
+                t = __builtin_fmaf(qb.w, kf[7], t);
+                acc[r] = t;
             }
         }
     } else {
@@ -93,56 +105,65 @@ __global__ __launch_bounds__(kQkThreads) void qk_score_kernel(QkArgs a)
 }
 
 // One workgroup per (x, H) row: max over s and sum of exp(score - max).
-__global__ __launch_bounds__(kQkThreads) void row_stats_kernel(const float* __restrict__ scores,
-                                                               int64_t S, float* __restrict__ stats)
+__global__ __launch_bounds__(kStatThreads) void row_stats_kernel(const float* __restrict__ scores,
+                                                                 int64_t S, float* __restrict__ stats)
 {
-    __shared__ float red[kQkThreads / 64];
+    __shared__ float red[kStatThreads / 64];
     const float* row = scores + (int64_t)blockIdx.x * S;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     float m = -INFINITY;
-    for (int64_t s = threadIdx.x; s < S; s += kQkThreads) m = fmaxf(m, row[s]);
+    for (int64_t s = threadIdx.x; s < S; s += kStatThreads) m = fmaxf(m, row[s]);
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
     if (lane == 0) red[w] = m;
     __syncthreads();
     m = red[0];
-    for (int i = 1; i < kQkThreads / 64; ++i) m = fmaxf(m, red[i]);
+    for (int i = 1; i < kStatThreads / 64; ++i) m = fmaxf(m, red[i]);
     __syncthreads();
     float sum = 0.0f;
-    for (int64_t s = threadIdx.x; s < S; s += kQkThreads) sum += expf(row[s] - m);
+    for (int64_t s = threadIdx.x; s < S; s += kStatThreads) sum += expf(row[s] - m);
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
     if (lane == 0) red[w] = sum;
     __syncthreads();
     if (threadIdx.x == 0) {
         float t = 0.0f;
-        for (int i = 0; i < kQkThreads / 64; ++i) t += red[i];
+        for (int i = 0; i < kStatThreads / 64; ++i) t += red[i];
         stats[2 * blockIdx.x] = m;
         // the reference normalises only when the sum exceeds 1e-9
         stats[2 * blockIdx.x + 1] = t > 1e-9f ? 1.0f / t : 1.0f;
     }
 }
 
-// One thread per block n: probabilities of its M representatives summed over all rows.
-__global__ __launch_bounds__(kQkThreads) void block_mass_kernel(const float* __restrict__ scores,
-                                                                const float* __restrict__ stats,
-                                                                int rows, int64_t S, int M,
-                                                                int64_t n_blocks,
-                                                                float* __restrict__ mass,
-                                                                uint32_t* __restrict__ keys,
-                                                                int32_t* __restrict__ ident)
+// One workgroup per block n: probabilities of its M representatives summed over all rows, in a
+// fixed order (strided partial sums, xor-shuffle tree, then the waves in turn).
+__global__ __launch_bounds__(kStatThreads) void block_mass_kernel(const float* __restrict__ scores,
+                                                                  const float* __restrict__ stats,
+                                                                  int rows, int64_t S, int M,
+                                                                  float* __restrict__ mass,
+                                                                  uint32_t* __restrict__ keys,
+                                                                  int32_t* __restrict__ ident)
 {
-    const int64_t n = (int64_t)blockIdx.x * kQkThreads + threadIdx.x;
-    if (n >= n_blocks) return;
-    float total = 0.0f;
-    for (int r = 0; r < rows; ++r) {
-        const float mx = stats[2 * r], inv = stats[2 * r + 1];
-        const float* row = scores + (int64_t)r * S + n * M;
-        for (int m = 0; m < M; ++m) total += expf(row[m] - mx) * inv;
+    __shared__ float red[kStatThreads / 64];
+    const int64_t n = blockIdx.x;
+    const float* base = scores + n * M;
+    const int total = rows * M;
+    float part = 0.0f;
+    for (int e = threadIdx.x; e < total; e += kStatThreads) {
+        const int r = e / M, m = e - r * M;
+        part += expf(base[(int64_t)r * S + m] - stats[2 * r]) * stats[2 * r + 1];
     }
-    mass[n] = total;
-    keys[n] = score_key(total);
-    ident[n] = (int32_t)n;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.0f;
+        for (int i = 0; i < kStatThreads / 64; ++i) t += red[i];
+        mass[n] = t;
+        keys[n] = score_key(t);
+        ident[n] = (int32_t)n;
+    }
 }
 
 size_t align256k(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -200,7 +221,7 @@ extern "C" int ucm_kvstar_topk(const void* query, int32_t X, int32_t Hq, int32_t
     UCM_REQUIRE((size_t)kRowTile * d * 4 <= 64 * 1024, "head dim %d above 1024", d);
     UCM_REQUIRE(n_blocks <= INT32_MAX && n_blocks * M <= INT32_MAX, "too many block representatives");
     const int64_t rows = (int64_t)X * Hq, S = n_blocks * M;
-    UCM_REQUIRE(rows <= 65535, "more than 65535 query rows");
+    UCM_REQUIRE(rows <= 65535 && rows * M <= INT32_MAX, "too many query rows");
     UCM_REQUIRE(workspace && workspace_bytes >= ucm_kvstar_topk_workspace_bytes(X, Hq, n_blocks, M),
                 "workspace too small");
     UCM_REQUIRE((((uintptr_t)blk_repre | (uintptr_t)workspace) & 15) == 0, "block representatives must be 16-byte aligned");
@@ -216,12 +237,11 @@ extern "C" int ucm_kvstar_topk(const void* query, int32_t X, int32_t Hq, int32_t
     hipLaunchKernelGGL(qk_score_kernel, grid, dim3(kQkThreads), (size_t)kRowTile * d * 4, st, a);
     int rc = ucm::launch_status("qk_score_kernel");
     if (rc != UCM_OK) return rc;
-    hipLaunchKernelGGL(row_stats_kernel, dim3((unsigned)rows), dim3(kQkThreads), 0, st, w.scores, S, w.stats);
+    hipLaunchKernelGGL(row_stats_kernel, dim3((unsigned)rows), dim3(kStatThreads), 0, st, w.scores, S, w.stats);
     rc = ucm::launch_status("row_stats_kernel");
     if (rc != UCM_OK) return rc;
-    hipLaunchKernelGGL(block_mass_kernel, dim3((unsigned)ucm::ceil_div(n_blocks, kQkThreads)),
-                       dim3(kQkThreads), 0, st, w.scores, w.stats, (int)rows, S, (int)M, n_blocks,
-                       w.mass, w.keys, w.ident);
+    hipLaunchKernelGGL(block_mass_kernel, dim3((unsigned)n_blocks), dim3(kStatThreads), 0, st, w.scores,
+                       w.stats, (int)rows, S, (int)M, w.mass, w.keys, w.ident);
     rc = ucm::launch_status("block_mass_kernel");
     if (rc != UCM_OK) return rc;
     SortArgs s{};
