@@ -351,6 +351,44 @@ def extras(torch, enc_k, gen):
     out["cache_store"] = {"payload_GiB": payload / 2**30, "tasks": len(tasks),
                           "dump_GBps": payload / (t1 - t0) / 1e9, "load_GBps": payload / (t2 - t1) / 1e9}
     store.close()
+
+    # --- "Cache|Posix" pipeline: the same shards on to block files in a temporary directory
+    #     (page cache included: a figure of the software path, not of a disk) ---
+    import shutil
+    import tempfile
+
+    from ucm_amd.store import UcmPipelineStore
+
+    root = tempfile.mkdtemp(prefix="ucm_bench_posix_")
+    try:
+        shard = n_tensors * chunk
+        n_blk, per_task = 32, 8
+        pipe = UcmPipelineStore({"store_pipeline": "Cache|Posix", "storage_backends": [root], "device_id": 0,
+                                 "tensor_size": chunk, "shard_size": shard, "block_size": shard,
+                                 "data_dir_shard_bytes": 2, "posix_data_trans_concurrency": 16,
+                                 "buffer_capacity_bytes": 2 * per_task * shard})
+        watcher = UcmPipelineStore({"store_pipeline": "Posix", "storage_backends": [root],
+                                    "data_dir_shard_bytes": 2})
+        pbids = [(1000 + i).to_bytes(8, "little") * 2 for i in range(n_blk)]
+        t0 = time.perf_counter()
+        for i in range(0, n_blk, per_task):
+            pipe.wait(pipe.dump_data(pbids[i:i + per_task], [0] * per_task, rows[i:i + per_task]))
+            while watcher.lookup_on_prefix(pbids[i:i + per_task]) + 1 < per_task:  # files committed
+                time.sleep(0.0005)
+        t1 = time.perf_counter()
+        for i in range(0, n_blk, per_task):
+            pipe.wait(pipe.load_data(pbids[i:i + per_task], [0] * per_task, rows[i:i + per_task]))
+        t2 = time.perf_counter()
+        pbytes = n_blk * shard
+        out["cache_posix_pipeline"] = {"payload_GiB": pbytes / 2**30, "dir": os.path.dirname(root),
+                                       "dump_to_files_GBps": pbytes / (t1 - t0) / 1e9,
+                                       "load_from_files_GBps": pbytes / (t2 - t1) / 1e9}
+        pipe.close()
+        watcher.close()
+    except Exception as e:  # noqa: BLE001 - a side figure must not take the headline down
+        out["cache_posix_pipeline"] = {"error": str(e)[:200]}
+    finally:
+        shutil.rmtree(root, ignore_errors=True)
     return out
 
 

@@ -425,6 +425,84 @@ int ucm_cache_store_load(ucm_cache_store_t* store, const uint8_t* block_ids,
 int ucm_cache_store_check(ucm_cache_store_t* store, int64_t task, int* finished);
 int ucm_cache_store_wait(ucm_cache_store_t* store, int64_t task);
 
+/* ======================================================================================
+ * 5. Posix store: one file per block in the reference's on-disk format
+ *    (ucm/store/posix/cc/).  Host-only: addresses are host pointers and no GPU is needed.
+ *
+ *    File of a block = <backend>/<dir>/<32 lowercase hex digits of the 16-byte id>, where
+ *    <dir> is the first data_dir_shard_bytes digits of the name, or "data" when that is 0
+ *    (space_layout.cc:88-99); with several backends the block lives in backend
+ *    std::hash<std::string_view>(id) % n (space_layout.cc:164-170).  Shard `index` is the byte
+ *    range [index * shard_size, (index + 1) * shard_size): its tensors, tensor_size bytes each,
+ *    one after the other (trans_queue.cc:127-169).  A file is written as <name>.tmp and
+ *    renamed when the block's last shard has been written (trans_queue.cc:117-119,
+ *    space_layout.cc:101-111).
+ * ====================================================================================== */
+typedef struct ucm_posix_store ucm_posix_store_t;
+
+/* Fields of the reference's Config (posix/cc/global_config.h:33-56) under the names of its
+ * dictionary keys (posix_store.cc:104-129).  capacity_bytes stands for posix_capacity_gb. */
+typedef struct ucm_posix_config {
+    const char* const* storage_backends; /* existing directories; the first one gets the shard
+                                            directories created, the others must hold them */
+    size_t n_backends;
+    int32_t device_id;             /* >= 0: dump / load enabled; -1: lookup only, and blocks
+                                      found by a lookup get their mtime refreshed */
+    int32_t io_direct;             /* O_DIRECT: addresses, sizes and offsets 4096-aligned */
+    size_t tensor_size, shard_size, block_size;
+    size_t data_trans_concurrency; /* threads per direction (posix_data_trans_concurrency) */
+    size_t lookup_concurrency;     /* posix_lookup_concurrency */
+    size_t timeout_ms;             /* 0 = 30000 */
+    size_t data_dir_shard_bytes;   /* 0..5 hex digits of directory sharding */
+    int32_t gc_enable;             /* posix_gc_enable; active only with capacity_bytes > 0 */
+    int32_t reserved;
+    size_t capacity_bytes;
+    double gc_recycle_percent;            /* share of a directory's files removed per pass */
+    double gc_trigger_threshold_ratio;    /* of capacity / block_size / directories */
+    double gc_shard_sample_ratio;         /* directories counted to decide */
+    size_t gc_max_recycle_count_per_shard;
+    size_t gc_check_interval_sec;
+} ucm_posix_config_t;
+
+/* PosixStore::Setup (posix_store.cc:37-56) incl. CheckConfig (:131-193): UCM_EPARAM for the
+ * configurations the reference rejects. */
+int ucm_posix_store_create(const ucm_posix_config_t* config, ucm_posix_store_t** out);
+int ucm_posix_store_destroy(ucm_posix_store_t* store);
+/* SpaceLayout::DataFilePath (space_layout.cc:88-99): the path of the block's file, with the
+ * ".tmp" suffix when `activated`.  Returns the path length (the text is cut to cap - 1). */
+int64_t ucm_posix_store_data_file_path(ucm_posix_store_t* store, const uint8_t* block_id,
+                                       int32_t activated, char* buf, size_t cap);
+/* SpaceLayout::CommitFile (space_layout.cc:101-111): rename <name>.tmp to <name>
+ * (success != 0) or remove it.  UCM_ENOOBJ when there is no such .tmp file. */
+int ucm_posix_store_commit(ucm_posix_store_t* store, const uint8_t* block_id, int32_t success);
+/* SpaceManager::LookupOnPrefix / Lookup (space_manager.cc:56-95): *last_found = index of the
+ * last block of the leading run whose files exist (readable and writable), -1 if none;
+ * found[i] = i <= *last_found (blocks after the first miss are reported absent). */
+int ucm_posix_store_lookup_on_prefix(ucm_posix_store_t* store, const uint8_t* block_ids, size_t n,
+                                     int64_t* last_found);
+int ucm_posix_store_lookup(ucm_posix_store_t* store, const uint8_t* block_ids, size_t n,
+                           uint8_t* found);
+/* PosixStore::Dump / Load (posix_store.cc:75-93; TransQueue trans_queue.cc:66-169): shard i is
+ * (block_ids[16 i ..], shard_idx[i]) with shard_size / tensor_size host addresses at
+ * host_addrs[i * tensors_per_shard + t].  Both only enqueue and return a task id. */
+int ucm_posix_store_dump(ucm_posix_store_t* store, const uint8_t* block_ids,
+                         const uint64_t* shard_idx, void* const* host_addrs, size_t n,
+                         int64_t* task);
+int ucm_posix_store_load(ucm_posix_store_t* store, const uint8_t* block_ids,
+                         const uint64_t* shard_idx, void* const* host_addrs, size_t n,
+                         int64_t* task);
+/* PosixStore::Check / Wait (posix_store.cc:94-103): as ucm_cache_store_check / _wait. */
+int ucm_posix_store_check(ucm_posix_store_t* store, int64_t task, int32_t* finished);
+int ucm_posix_store_wait(ucm_posix_store_t* store, int64_t task);
+/* One turn of the collector's loop now (ShardGarbageCollector::GCCheckLoop, shard_gc.cc:85-108):
+ * sample directories, and while the average file count is at or above the threshold remove
+ * each directory's oldest files by mtime.  *removed = files removed by this call. */
+int ucm_posix_store_gc_once(ucm_posix_store_t* store, uint64_t* removed);
+/* Fills the hooks that put this store beneath a cache store (the reference's "Cache|Posix"
+ * pipeline, ucm/store/pipeline/connector.py:180-188; there as here the posix store is then
+ * configured with tensor_size = shard_size).  `store` must outlive the cache store. */
+int ucm_posix_store_backend(ucm_posix_store_t* store, ucm_cache_backend_t* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,7 +11,8 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-SRC = ["common.hip", "hamming_topk.hip", "hash_encode.hip", "trans.hip", "cache_store.hip", "dot_topk.hip", "kvstar_topk.hip"]
+SRC = ["common.hip", "hamming_topk.hip", "hash_encode.hip", "trans.hip", "cache_store.hip", "dot_topk.hip", "kvstar_topk.hip",
+       "posix_store.hip"]
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libucm_hip.so")
 

@@ -74,7 +74,43 @@ _SIGNATURES = {
     "ucm_cache_store_load": (ci, [vp, vp, vp, vp, sz, C.POINTER(i64)]),
     "ucm_cache_store_check": (ci, [vp, i64, C.POINTER(ci)]),
     "ucm_cache_store_wait": (ci, [vp, i64]),
+    "ucm_posix_store_create": (ci, [vp, C.POINTER(vp)]),
+    "ucm_posix_store_destroy": (ci, [vp]),
+    "ucm_posix_store_data_file_path": (i64, [vp, vp, i32, C.c_char_p, sz]),
+    "ucm_posix_store_commit": (ci, [vp, vp, i32]),
+    "ucm_posix_store_lookup_on_prefix": (ci, [vp, vp, sz, C.POINTER(i64)]),
+    "ucm_posix_store_lookup": (ci, [vp, vp, sz, vp]),
+    "ucm_posix_store_dump": (ci, [vp, vp, vp, vp, sz, C.POINTER(i64)]),
+    "ucm_posix_store_load": (ci, [vp, vp, vp, vp, sz, C.POINTER(i64)]),
+    "ucm_posix_store_check": (ci, [vp, i64, C.POINTER(i32)]),
+    "ucm_posix_store_wait": (ci, [vp, i64]),
+    "ucm_posix_store_gc_once": (ci, [vp, C.POINTER(u64)]),
+    "ucm_posix_store_backend": (ci, [vp, vp]),
 }
+
+
+class PosixConfig(C.Structure):
+    """ucm_posix_config_t"""
+    _fields_ = [
+        ("storage_backends", C.POINTER(C.c_char_p)), ("n_backends", sz),
+        ("device_id", i32), ("io_direct", i32),
+        ("tensor_size", sz), ("shard_size", sz), ("block_size", sz),
+        ("data_trans_concurrency", sz), ("lookup_concurrency", sz), ("timeout_ms", sz),
+        ("data_dir_shard_bytes", sz),
+        ("gc_enable", i32), ("reserved", i32), ("capacity_bytes", sz),
+        ("gc_recycle_percent", C.c_double), ("gc_trigger_threshold_ratio", C.c_double),
+        ("gc_shard_sample_ratio", C.c_double),
+        ("gc_max_recycle_count_per_shard", sz), ("gc_check_interval_sec", sz),
+    ]
+
+
+class CacheBackend(C.Structure):
+    """ucm_cache_backend_t"""
+    LOOKUP = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p)
+    MOVE = C.CFUNCTYPE(C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t)
+    WAIT = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int64)
+    _fields_ = [("ctx", C.c_void_p), ("lookup", LOOKUP), ("dump", MOVE), ("load", MOVE), ("wait", WAIT)]
+
 
 EXPORTS = tuple(_SIGNATURES)
 

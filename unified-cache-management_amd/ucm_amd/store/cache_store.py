@@ -9,9 +9,10 @@ config keys (names from cache_store.cc:104-131 where they exist):
     tensor_size_list [bytes per tensor of a shard ...]  or  tensor_size + shard_size
     cache_buffer_capacity_gb  or  buffer_capacity_bytes     pinned staging memory
     device_id (default 0), waiting_queue_depth (default 8192), timeout_ms (default 30000)
-    store_backend: optional object with lookup(ids) -> [bool], dump(ids, shard_idx, views) and
+    store_backend: optional; either a PosixStore (chained natively through its C hooks) or any
+        object with lookup(ids) -> [bool], dump(ids, shard_idx, views) and
         load(ids, shard_idx, views); `views` are writable uint8 numpy views of the pinned
-        shards.  It stands where the reference passes the next StoreV1* (a posix store, ...).
+        shards.  It stands where the reference passes the next StoreV1*.
 """
 import ctypes as C
 import threading
@@ -23,13 +24,7 @@ from .. import _lib
 from .base import Task, UcmKVStoreBaseV1
 
 
-class _Backend(C.Structure):
-    _LOOKUP = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p)
-    _MOVE = C.CFUNCTYPE(C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
-                        C.c_size_t)
-    _WAIT = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int64)
-    _fields_ = [("ctx", C.c_void_p), ("lookup", _LOOKUP), ("dump", _MOVE), ("load", _MOVE),
-                ("wait", _WAIT)]
+_Backend = _lib.CacheBackend
 
 
 def _ids_array(block_ids: List[bytes]) -> np.ndarray:
@@ -66,7 +61,11 @@ class CacheStore(UcmKVStoreBaseV1):
         self._py_backend = config.get("store_backend")
         self._cb = None
         backend_ptr = None
-        if self._py_backend is not None:
+        if hasattr(self._py_backend, "native_backend"):
+            # a native store (the posix store): its own C hooks, no Python in the data path
+            self._cb = self._py_backend.native_backend(self.shard_size)
+            backend_ptr = C.addressof(self._cb)
+        elif self._py_backend is not None:
             self._cb = self._make_callbacks(self._py_backend)
             backend_ptr = C.addressof(self._cb)
         handle = C.c_void_p()
@@ -118,10 +117,10 @@ class CacheStore(UcmKVStoreBaseV1):
 
         cb = _Backend()
         cb.ctx = None
-        cb.lookup = _Backend._LOOKUP(lookup)
-        cb.dump = _Backend._MOVE(mover(be.dump))
-        cb.load = _Backend._MOVE(mover(be.load))
-        cb.wait = _Backend._WAIT(lambda _ctx, _h: 0)  # the Python hooks are synchronous
+        cb.lookup = _Backend.LOOKUP(lookup)
+        cb.dump = _Backend.MOVE(mover(be.dump))
+        cb.load = _Backend.MOVE(mover(be.load))
+        cb.wait = _Backend.WAIT(lambda _ctx, _h: 0)  # the Python hooks are synchronous
         return cb
 
     def close(self):
