@@ -6,7 +6,7 @@ unmodified).  The fixture holds inputs (or their seed + sha256 when large) and t
 backend's outputs; tests compare the C oracle and the HIP library against it.
 
 Cases
-  c1_gqa   BASELINE config 1: 1 request, 32 q heads / 8 KV heads, 8192 tokens in 64 blocks of
+  c1_gqa   BASELINE.json config 1: 1 request, 32 q heads / 8 KV heads, 8192 tokens in 64 blocks of
            128, 128-bit codes, top-16.  The backend has no head or group notion, so the GQA
            group sum is obtained through
                dist(concat_g q_g, tile_G(k)) = sum_g dist(q_g, k)
@@ -45,7 +45,7 @@ def run_ref(mod, data_u8, query_u8, indexes, k):
 
 
 def c1_inputs(seed=1001):
-    """Shared with the tests: BASELINE config 1 inputs from one PCG64 stream."""
+    """Shared with the tests: BASELINE.json config 1 inputs from one PCG64 stream."""
     rng = np.random.Generator(np.random.PCG64(seed))
     keys = rng.integers(0, 2**32, size=(64, 128, 8, 4), dtype=np.uint32)
     q = rng.integers(0, 2**32, size=(1, 32, 4), dtype=np.uint32)

@@ -94,7 +94,7 @@ def test_zero_and_nan_rows_give_zero_bits():
 
 
 def test_per_head_weights_gqa_queries():
-    """BASELINE config 2 query side: 32 q heads, one projection per KV head (group of 4)."""
+    """BASELINE.json config 2 query side: 32 q heads, one projection per KV head (group of 4)."""
     rng = rng_for(8)
     B, Hq, Hkv, K, N = 6, 32, 8, 128, 128
     x = bf16_round(rng.standard_normal((B, Hq, K)))

@@ -1,4 +1,4 @@
-"""GPU parity at the full BASELINE sizes (configs 2-5).
+"""GPU parity at the full sizes of BASELINE.json (configs 2-5).
 
 Where the CPU oracle finishes in seconds the comparison is complete and bit-exact; on top of
 that each test checks size-independent properties of the domain: ascending indices, every

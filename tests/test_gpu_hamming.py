@@ -56,7 +56,7 @@ def check(q, kc, table, lens, k, sink=0, recent=0, head_major=False, **kw):
 
 
 def test_config1_golden_and_oracle():
-    """BASELINE config 1 against the reference CPU backend's recorded output."""
+    """BASELINE.json config 1 against the reference CPU backend's recorded output."""
     from golden.make_golden import c1_inputs
 
     gold = np.load(GOLD)

@@ -93,7 +93,7 @@ def test_odd_sizes_and_unaligned_chunks(device, size):
 
 
 def test_kv_cache_gather_scatter_small_config4(device):
-    """BASELINE config 4 at reduced size: layers x {K,V} x [NB,BS,H,D] bf16 cache; gather the
+    """BASELINE.json config 4 at reduced size: layers x {K,V} x [NB,BS,H,D] bf16 cache; gather the
     selected blocks of several requests into one pinned buffer, scatter into fresh blocks of
     a second cache, compare byte for byte, check untouched blocks stay untouched."""
     L, NB, BS, H, D = 4, 24, 16, 8, 128
