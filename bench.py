@@ -111,10 +111,57 @@ def cpu_baseline(torch, cache, table, qcodes, lens, seconds_budget=10.0):
     for _ in range(20):
         c_api.hamming_topk(q[:1], kc, tb[:1], ln[:1], TOPK, nthreads=1)
     one = 20 * CTX / (time.perf_counter() - t0)
-    return {"value": tok_s, "unit": "scored KV tokens/s", "cores": cores, "kind": "port",
-            "one_thread_value": one,
-            "sample": f"all {sample_b} requests x {CTX} tokens of the same workload, {reps} passes, "
-                      f"one thread per request over {cores} threads (oracle/ucm_oracle.c)"}
+    out = {"value": tok_s, "unit": "scored KV tokens/s", "cores": cores, "kind": "port",
+           "one_thread_value": one,
+           "sample": f"all {sample_b} requests x {CTX} tokens of the same workload, {reps} passes, "
+                     f"one thread per request over {cores} threads (oracle/ucm_oracle.c)"}
+    try:
+        ref = reference_backend_baseline(np, c_api, kc, tb, q, cores)
+    except Exception as e:  # noqa: BLE001 - an extra figure; the port above is the baseline
+        ref = {"error": str(e)[:200]}
+    if ref is not None:
+        out["reference_backend"] = ref
+    return out
+
+
+def reference_backend_baseline(np, c_api, kc, tb, q, threads, requests=2, seconds=4.0):
+    """The reference's own CPU retrieval backend (hash_retrieval_backend.cpp compiled unmodified
+    into oracle/_ref by oracle/Makefile, where that build exists) on a sample of the same
+    codes.  The backend scores flat byte codes with no head or group notion, so one submit is
+    one (request, KV head): its 256 blocks x 128 tokens with the 16-byte code repeated G times,
+    against the group's G query codes laid end to end — dist(concat_g q_g, tile_G k) = sum_g
+    dist(q_g, k), the same group sum the GPU scorer takes.  Its worker threads each take one
+    submit at a time; `threads` of them run."""
+    mod = c_api.ref_backend()
+    if mod is None:
+        return None
+    G = HQ // HKV
+    data = np.empty((requests * HKV * NBLK, BS, 16 * G), np.uint8)
+    queries, allowed = [], []
+    for r in range(requests):
+        blocks = kc[tb[r, :NBLK]]  # [NBLK, BS, HKV, WD] in logical order
+        for h in range(HKV):
+            base = (r * HKV + h) * NBLK
+            kh = np.ascontiguousarray(blocks[:, :, h, :]).view(np.uint8).reshape(NBLK, BS, 16)
+            data[base:base + NBLK] = np.tile(kh, (1, 1, G))
+            queries.append(np.ascontiguousarray(q[r, h * G:(h + 1) * G]).view(np.uint8).reshape(1, -1))
+            allowed.append((np.arange(NBLK, dtype=np.int32) + base).reshape(1, -1))
+    be = mod.HashRetrievalWorkerBackend(data, {0: list(range(threads))})
+    reps, t_total = 0, 0.0
+    while reps < 2 or t_total < seconds:
+        t0 = time.perf_counter()
+        ids = [be.submit(qq, TOPK, al) for qq, al in zip(queries, allowed)]
+        for i in ids:
+            be.wait(i)
+            be.get_result(i)
+        t_total += time.perf_counter() - t0
+        reps += 1
+    del be
+    return {"value": requests * CTX * reps / t_total, "unit": "scored KV tokens/s", "cores": threads,
+            "kind": "reference",
+            "sample": f"{requests} requests x {CTX} tokens x {HKV} KV heads of the same codes, one submit "
+                      f"per (request, KV head), {reps} passes, {threads} worker threads "
+                      "(hash_retrieval_backend.cpp)"}
 
 
 def cpu_side_baselines(torch):

@@ -72,6 +72,47 @@ def test_config2_batch32_x_32k_top64_bit_exact():
     assert torch.equal(idx, idx2) and torch.equal(sc, sc2)
 
 
+def test_config2_against_the_reference_cpu_backend_itself():
+    """Config 2 at full size against the reference's own CPU backend (hash_retrieval_backend.cpp
+    compiled unmodified into oracle/_ref; skipped where that build is absent).  The backend has
+    no head or group notion: one submit per (request, KV head) with the 16-byte codes repeated
+    G times against the group's query codes laid end to end, so that its distance is the GQA
+    group sum.  It returns block distances ascending; ties are in unspecified order, so the
+    comparison is on the sorted distances and, away from ties at the threshold, the index sets."""
+    from ucm_amd.sparse import hamming_topk
+
+    mod = c_api.ref_backend()
+    if mod is None:
+        pytest.skip("oracle/_ref is not built")
+    B, CTX, HQ, HKV, WD, BS, K = 32, 32768, 32, 8, 4, 128, 64
+    NBLK, G = CTX // BS, HQ // HKV
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1202)
+    cache = gpu_codes(gen, (B * NBLK, BS, HKV, WD))
+    q = gpu_codes(gen, (B, HQ, WD))
+    table = torch.randperm(B * NBLK, device="cuda", generator=gen).to(torch.int32).reshape(B, NBLK)
+    lens = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
+    idx, sc = hamming_topk(q, cache, table, lens, K)
+    idx, sc = idx.cpu().numpy(), sc.cpu().numpy()
+    kc, qq, tb = np_u32(cache), np_u32(q), table.cpu().numpy()
+    for b in (0, 13, 31):
+        blocks = kc[tb[b]]  # [NBLK, BS, HKV, WD] in logical order
+        for h in range(HKV):
+            kh = np.ascontiguousarray(blocks[:, :, h, :]).view(np.uint8).reshape(NBLK, BS, 16)
+            be = mod.HashRetrievalWorkerBackend(np.tile(kh, (1, 1, G)), {0: [0]})
+            rid = be.submit(np.ascontiguousarray(qq[b, h * G:(h + 1) * G]).view(np.uint8).reshape(1, -1), K,
+                            np.arange(NBLK, dtype=np.int32).reshape(1, -1))
+            be.wait(rid)
+            res = be.get_result(rid)
+            ref_idx = np.array(res["indices"], np.int64)[0]
+            ref_dist = np.array(res["scores"], np.int64)[0]
+            del be
+            sim = G * 32 * WD - ref_dist  # the GPU reports similarity
+            assert np.array_equal(np.sort(sim)[::-1], np.sort(sc[b, h])[::-1])
+            thr = sim.min()
+            assert set(ref_idx[sim > thr]) == set(idx[b, h][sc[b, h] > thr])
+
+
 def test_config3_long_ragged_top128_ascending_with_scores():
     from ucm_amd.sparse import hamming_topk
 
