@@ -57,6 +57,8 @@ def check(q, k, pr, topk):
     (2, 4, 1, 64, 300, 1, 300),    # MQA, every block returned
     (17, 8, 8, 128, 513, 2, 64),   # more than one row tile, blocks past one workgroup
     (1, 1, 1, 8, 1, 1, 1),         # smallest problem
+    (20, 8, 2, 32, 70, 3, 9),      # 80 query rows per KV head: three row tiles, ragged last tiles
+    (3, 4, 2, 48, 33, 1, 5),       # three k-steps, one representative past a 32-wide tile
 ])
 def test_matches_checker(X, Hq, Hkv, d, n, M, topk):
     q, k = make(X * 1000 + n, X, Hq, Hkv, d, n, M)

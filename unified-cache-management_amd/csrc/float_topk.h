@@ -148,9 +148,47 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
     }
 }
 
+// Short rows (max_n <= 1024, e.g. the blocks of one request): every candidate counts the
+// candidates that come before it in the output order (larger key, or equal key and earlier
+// position) and writes itself at that rank.  No search and no sort: n broadcast reads from LDS
+// per thread.  Same output as topk_sort_kernel.
+__global__ __launch_bounds__(kSortThreads) void topk_rank_kernel(SortArgs a)
+{
+    __shared__ __align__(16) uint32_t k_lds[kSortThreads];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const uint32_t* keys = a.keys + (int64_t)b * a.max_n;
+    const uint32_t mine = tid < a.max_n ? keys[tid] : 0u;
+    k_lds[tid] = mine;
+    for (int t = tid; t < a.topk; t += kSortThreads) {  // slots no candidate reaches
+        a.out_idx[(int64_t)b * a.topk + t] = -1;
+        a.out_score[(int64_t)b * a.topk + t] = 0.0f;
+    }
+    __syncthreads();  // also orders the fill above before the winners' writes below
+    if (mine == 0u) return;
+    int rank = 0;
+    const int n4 = a.max_n & ~3;
+    for (int j = 0; j < n4; j += 4) {
+        const uint4 o = *reinterpret_cast<const uint4*>(k_lds + j);
+        rank += (o.x > mine || (o.x == mine && j < tid)) + (o.y > mine || (o.y == mine && j + 1 < tid)) +
+                (o.z > mine || (o.z == mine && j + 2 < tid)) + (o.w > mine || (o.w == mine && j + 3 < tid));
+    }
+    for (int j = n4; j < a.max_n; ++j) {
+        const uint32_t o = k_lds[j];
+        rank += (o > mine || (o == mine && j < tid));
+    }
+    if (rank < a.topk) {
+        a.out_idx[(int64_t)b * a.topk + rank] = a.idx[(int64_t)b * a.max_n + tid];
+        a.out_score[(int64_t)b * a.topk + rank] = a.scores[(int64_t)b * a.max_n + tid];
+    }
+}
+
 // cap = power of two >= topk
 inline int launch_topk_sort(const SortArgs& in, int rows, hipStream_t st)
 {
+    if (in.max_n <= kSortThreads) {
+        hipLaunchKernelGGL(topk_rank_kernel, dim3((unsigned)rows), dim3(kSortThreads), 0, st, in);
+        return ucm::launch_status("topk_rank_kernel");
+    }
     SortArgs s = in;
     int cap = 2;
     while (cap < s.topk) cap <<= 1;

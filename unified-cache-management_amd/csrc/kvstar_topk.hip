@@ -24,7 +24,7 @@
 
 namespace {
 
-constexpr int kQkThreads = 256;
+constexpr int kQkThreads = 256;  // the matrix-core kernel stages 32 query rows with 8 threads each
 constexpr int kStatThreads = 1024;
 constexpr int kRowTile = 16;  // query rows of one KV head scored per pass over a K vector
 
@@ -41,9 +41,14 @@ struct QkArgs {
 __global__ __launch_bounds__(kQkThreads) void qk_score_kernel(QkArgs a)
 {
     extern __shared__ __align__(16) float qs[];  // [kRowTile][d]
+    __shared__ int orow[kRowTile];               // score row x * Hq + H of each query row, -1 = none
     const int h = blockIdx.y;
     const int row0 = blockIdx.z * kRowTile;  // first (x, gg) pair of this pass
     const int rows = a.X * a.g;
+    if (threadIdx.x < kRowTile) {
+        const int rr = row0 + threadIdx.x;
+        orow[threadIdx.x] = rr < rows ? (rr / a.g) * a.Hq + h * a.g + rr % a.g : -1;
+    }
     // stage the pass's query rows of KV head h: row r = x * g + gg  <->  q head H = h * g + gg
     for (int i = threadIdx.x; i < kRowTile * a.d; i += kQkThreads) {
         const int r = row0 + i / a.d, j = i % a.d;
@@ -96,42 +101,117 @@ __global__ __launch_bounds__(kQkThreads) void qk_score_kernel(QkArgs a)
     }
 #pragma unroll
     for (int r = 0; r < kRowTile; ++r) {
-        const int rr = row0 + r;
-        if (rr < rows) {
-            const int x = rr / a.g, H = h * a.g + rr % a.g;
-            a.scores[((int64_t)x * a.Hq + H) * a.S + s] = acc[r];
-        }
+        const int o = orow[r];
+        if (o >= 0) a.scores[(int64_t)o * a.S + s] = acc[r];
     }
 }
 
-// One workgroup per (x, H) row: max over s and sum of exp(score - max).
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// q.k on the matrix cores for head dims that are multiples of 16: one workgroup per (128
+// representatives, KV head, 32 query rows); the query tile (channel-pruned) is gathered once
+// into LDS, then each wave takes 32 representatives: d / 16 v_mfma_f32_32x32x16_f16 with the
+// query tile as the A operand (lane: row lane % 32, eight channels of the k-step, one 16-byte
+// LDS read) and the representatives as the B operand (one 16-byte global load per lane and
+// k-step).  Accumulator v of a lane is
+// score[row 8 (v / 4) + 4 (lane / 32) + v % 4][representative lane % 32]: lanes 0..31 store 32
+// consecutive floats of one score row.  grid = (ceil(S / 128), Hkv, ceil(X g / 32));
+// LDS = 32 rows of (d + 8) halves.
+__global__ __launch_bounds__(kQkThreads) void qk_mfma_kernel(QkArgs a)
+{
+    extern __shared__ __align__(16) _Float16 qt[];  // [32][d + 8]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = blockIdx.y;
+    const int rows = a.X * a.g;
+    const int dp = a.d + 8;  // row pitch: 16 bytes of padding spread the rows over the banks
+    const _Float16* q = reinterpret_cast<const _Float16*>(a.q);
+    {
+        // eight threads per query row, each taking every eighth channel: one division per thread
+        const int rl = threadIdx.x >> 3;
+        const int rr = blockIdx.z * 32 + rl;
+        const bool ok = rr < rows;
+        const _Float16* qrow = q + ((int64_t)(ok ? rr / a.g : 0) * a.Hq + h * a.g + (ok ? rr % a.g : 0)) * a.d_orig;
+        for (int j = threadIdx.x & 7; j < a.d; j += 8) {
+            int64_t src = a.pruned ? a.pruned[(int64_t)h * a.d + j] : j;
+            src = src < 0 ? 0 : (src >= a.d_orig ? a.d_orig - 1 : src);  // stay inside the row
+            qt[rl * dp + j] = ok ? qrow[src] : (_Float16)0;
+        }
+    }
+    __syncthreads();
+    const int64_t s0 = ((int64_t)blockIdx.x * (kQkThreads / 64) + wave) * 32;
+    if (s0 >= a.S) return;  // wave-uniform, after the only barrier
+    int64_t s = s0 + (lane & 31);
+    const bool s_ok = s < a.S;
+    if (!s_ok) s = a.S - 1;
+    const int kb = (lane >> 5) * 8;  // channels kb .. kb + 7 of a k-step
+    const __half* kv = a.k + (s * a.Hkv + h) * a.d + kb;
+    const _Float16* qa_row = qt + (lane & 31) * dp + kb;
+    f32x16 acc = {0};
+    for (int c = 0; c < a.d; c += 16) {
+        const f16x8 qa = *reinterpret_cast<const f16x8*>(qa_row + c);
+        const f16x8 kk = *reinterpret_cast<const f16x8*>(kv + c);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa, kk, acc, 0, 0, 0);
+    }
+    // score row of query row lane % 32 (one division per lane, handed round by shuffles:
+    // sixteen divisions per lane in the store loop cost more than the matrix products)
+    const int r = blockIdx.z * 32 + (lane & 31);
+    const int orow = r < rows ? (r / a.g) * a.Hq + h * a.g + r % a.g : -1;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int o = __shfl(orow, 8 * (v / 4) + 4 * (lane >> 5) + (v % 4));
+        if (s_ok && o >= 0) a.scores[(int64_t)o * a.S + s] = acc[v];
+    }
+}
+
+// Running (max, sum of exp(x - max)) pairs merge associatively; a side that has seen nothing
+// carries max = -inf and sum = 0.
+__device__ __forceinline__ void merge_stats(float& m, float& sum, float om, float osum)
+{
+    const float nm = fmaxf(m, om);
+    if (nm == -INFINITY) return;
+    sum = sum * expf(m - nm) + osum * expf(om - nm);
+    m = nm;
+}
+
+// One workgroup per (x, H) row: max over s and sum of exp(score - max), in one pass over the
+// row (eight loads in flight per thread, running pairs merged at the end).
 __global__ __launch_bounds__(kStatThreads) void row_stats_kernel(const float* __restrict__ scores,
                                                                  int64_t S, float* __restrict__ stats)
 {
-    __shared__ float red[kStatThreads / 64];
+    __shared__ float red_m[kStatThreads / 64], red_s[kStatThreads / 64];
     const float* row = scores + (int64_t)blockIdx.x * S;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    float m = -INFINITY;
-    for (int64_t s = threadIdx.x; s < S; s += kStatThreads) m = fmaxf(m, row[s]);
+    float m = -INFINITY, sum = 0.0f;
+    for (int64_t base = threadIdx.x; base < S; base += 8 * kStatThreads) {
+        float v[8];
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-    if (lane == 0) red[w] = m;
-    __syncthreads();
-    m = red[0];
-    for (int i = 1; i < kStatThreads / 64; ++i) m = fmaxf(m, red[i]);
-    __syncthreads();
-    float sum = 0.0f;
-    for (int64_t s = threadIdx.x; s < S; s += kStatThreads) sum += expf(row[s] - m);
+        for (int i = 0; i < 8; ++i) {
+            const int64_t s = base + (int64_t)i * kStatThreads;
+            v[i] = s < S ? row[s] : -INFINITY;
+        }
+        float cm = v[0];
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
-    if (lane == 0) red[w] = sum;
+        for (int i = 1; i < 8; ++i) cm = fmaxf(cm, v[i]);
+        if (cm == -INFINITY) continue;
+        float cs = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) cs += expf(v[i] - cm);
+        merge_stats(m, sum, cm, cs);
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) merge_stats(m, sum, __shfl_xor(m, o), __shfl_xor(sum, o));
+    if (lane == 0) {
+        red_m[w] = m;
+        red_s[w] = sum;
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
-        float t = 0.0f;
-        for (int i = 0; i < kStatThreads / 64; ++i) t += red[i];
-        stats[2 * blockIdx.x] = m;
+        float tm = red_m[0], ts = red_s[0];
+        for (int i = 1; i < kStatThreads / 64; ++i) merge_stats(tm, ts, red_m[i], red_s[i]);
+        stats[2 * blockIdx.x] = tm;
         // the reference normalises only when the sum exceeds 1e-9
-        stats[2 * blockIdx.x + 1] = t > 1e-9f ? 1.0f / t : 1.0f;
+        stats[2 * blockIdx.x + 1] = ts > 1e-9f ? 1.0f / ts : 1.0f;
     }
 }
 
@@ -149,9 +229,18 @@ __global__ __launch_bounds__(kStatThreads) void block_mass_kernel(const float* _
     const float* base = scores + n * M;
     const int total = rows * M;
     float part = 0.0f;
+    // element e = r * M + m; e advances by the workgroup size: (r, m) follow without a division
+    const int dr = kStatThreads / M, dm = kStatThreads % M;
+    int r = threadIdx.x / M, m = threadIdx.x % M;
+#pragma unroll 4
     for (int e = threadIdx.x; e < total; e += kStatThreads) {
-        const int r = e / M, m = e - r * M;
         part += expf(base[(int64_t)r * S + m] - stats[2 * r]) * stats[2 * r + 1];
+        r += dr;
+        m += dm;
+        if (m >= M) {
+            m -= M;
+            ++r;
+        }
     }
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o);
@@ -234,8 +323,17 @@ extern "C" int ucm_kvstar_topk(const void* query, int32_t X, int32_t Hq, int32_t
     const dim3 grid((unsigned)ucm::ceil_div(S, kQkThreads), (unsigned)Hkv,
                     (unsigned)ucm::ceil_div((int64_t)X * a.g, kRowTile));
     UCM_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "too many heads or query rows");
-    hipLaunchKernelGGL(qk_score_kernel, grid, dim3(kQkThreads), (size_t)kRowTile * d * 4, st, a);
-    int rc = ucm::launch_status("qk_score_kernel");
+    int rc;
+    if (d % 16 == 0 && d <= 512) {
+        const dim3 mgrid((unsigned)ucm::ceil_div(S, 32 * (kQkThreads / 64)), (unsigned)Hkv,
+                         (unsigned)ucm::ceil_div((int64_t)X * a.g, 32));
+        UCM_REQUIRE(mgrid.z <= 65535, "too many query rows");
+        hipLaunchKernelGGL(qk_mfma_kernel, mgrid, dim3(kQkThreads), (size_t)32 * (d + 8) * 2, st, a);
+        rc = ucm::launch_status("qk_mfma_kernel");
+    } else {
+        hipLaunchKernelGGL(qk_score_kernel, grid, dim3(kQkThreads), (size_t)kRowTile * d * 4, st, a);
+        rc = ucm::launch_status("qk_score_kernel");
+    }
     if (rc != UCM_OK) return rc;
     hipLaunchKernelGGL(row_stats_kernel, dim3((unsigned)rows), dim3(kStatThreads), 0, st, w.scores, S, w.stats);
     rc = ucm::launch_status("row_stats_kernel");
