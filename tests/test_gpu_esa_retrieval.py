@@ -93,6 +93,11 @@ def test_integer_inputs_are_bit_exact_and_ties_keep_list_order():
     (400, 30, 4, 77, 10),            # dim % 4 != 0: scalar loads
     (64, 4096, 1, 64, 7),            # long rows
     (20000, 64, 8, 6000, 4096),      # the largest k
+    (30000, 32, 2, 10000, 500),      # more than 8192 candidates: keys re-read from memory per phase
+    (9000, 16, 2, 8192, 100),        # exactly what the register path holds
+    (9000, 16, 2, 8193, 100),        # one more
+    (2000, 16, 3, 1024, 40),         # the longest row of the counting path
+    (2000, 16, 3, 1025, 40),         # the shortest row of the search-and-sort path
 ])
 def test_random_shapes(n_items, dim, B, max_n, k):
     rng = rng_for(n_items + dim + B)

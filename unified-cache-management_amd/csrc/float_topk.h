@@ -1,8 +1,8 @@
 // Selection shared by the float retrieval paths: the k best of a row of fp32 scores in
 // descending order.  One 1024-thread workgroup per row: four 8-bit radix passes over
 // order-preserving 32-bit keys find the k-th largest, winners are compacted into LDS (ties at
-// the threshold in list order) and a bitonic sort orders (key, position) pairs, so equal
-// scores come out in list order.  Included by the translation units that launch it.
+// the threshold in list order) and ordered as (key, position) pairs by segment-wise bitonic
+// networks followed by pairwise merges, so equal scores come out in list order.  Included by the translation units that launch it.
 #pragma once
 
 #include "common.h"
@@ -11,6 +11,7 @@ namespace {
 
 constexpr int kSortThreads = 1024;
 constexpr int kMaxTopk = 4096;  // winners sorted in LDS: 8 bytes each (32 KiB)
+constexpr int kRegKeys = 8;     // keys a thread keeps in registers: rows of up to 8192 candidates
 
 // Order-preserving key of a score: larger score <-> larger key.  0 is reserved for "no
 // candidate", 1 for NaN (below every number, above nothing else).
@@ -53,19 +54,55 @@ __device__ __forceinline__ int scan1024(int v, int* wsum, int* total)
     return base + inc - v;
 }
 
+// REG: the row has at most kRegKeys * 1024 candidates and every thread keeps its keys in
+// registers for all phases (one round trip to memory instead of one per phase and chunk).
+template <bool REG>
 __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
 {
     extern __shared__ unsigned long long win[];  // [cap] (key << 32) | ~position
     __shared__ int hist[256];
     __shared__ int wsum[kSortThreads / 64];
-    __shared__ int s_digit, s_need, s_count;
+    __shared__ int s_digit, s_need;
     const int b = blockIdx.x;
     const uint32_t* keys = a.keys + (int64_t)b * a.max_n;
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63;
+
+    // REG: thread t holds list positions t * kRegKeys .. + kRegKeys - 1 (consecutive, so that one
+    // prefix sum over per-thread counts orders the whole list)
+    uint32_t kreg[REG ? kRegKeys : 1];
+    if constexpr (REG) {
+        static_assert(kRegKeys == 8, "two 16-byte loads per thread");
+        const bool vec = (reinterpret_cast<uintptr_t>(keys) & 15) == 0;  // uniform
+        if (vec && (tid + 1) * kRegKeys <= a.max_n) {
+            const uint4 lo = *reinterpret_cast<const uint4*>(keys + tid * kRegKeys);
+            const uint4 hi = *reinterpret_cast<const uint4*>(keys + tid * kRegKeys + 4);
+            kreg[0] = lo.x; kreg[1] = lo.y; kreg[2] = lo.z; kreg[3] = lo.w;
+            kreg[4] = hi.x; kreg[5] = hi.y; kreg[6] = hi.z; kreg[7] = hi.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < kRegKeys; ++e) {
+                const int i = tid * kRegKeys + e;
+                kreg[e] = i < a.max_n ? keys[i] : 0u;
+            }
+        }
+    }
+    // f(chunk, key) over the thread's keys; uniform control flow.  Without REG chunk e covers
+    // list positions e * 1024 + tid.
+    auto for_chunks = [&](auto&& f) {
+        if constexpr (REG) {
+#pragma unroll
+            for (int e = 0; e < kRegKeys; ++e) f(e, kreg[e]);
+        } else {
+            for (int e = 0; e * kSortThreads < a.max_n; ++e) {
+                const int i = e * kSortThreads + tid;
+                f(e, i < a.max_n ? keys[i] : 0u);
+            }
+        }
+    };
 
     // candidates present
     int mine = 0;
-    for (int i = tid; i < a.max_n; i += kSortThreads) mine += keys[i] != 0u;
+    for_chunks([&](int, uint32_t k) { mine += k != 0u; });
     int n_valid;
     (void)scan1024(mine, wsum, &n_valid);
     const int kk = n_valid < a.topk ? n_valid : a.topk;
@@ -76,10 +113,22 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
     for (int shift = 24; shift >= 0 && kk > 0; shift -= 8) {
         if (tid < 256) hist[tid] = 0;
         __syncthreads();
-        for (int i = tid; i < a.max_n; i += kSortThreads) {
-            const uint32_t k = keys[i];
-            if (k != 0u && (k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255], 1);
-        }
+        for_chunks([&](int, uint32_t k) {
+            const bool in = k != 0u && (k & mask) == prefix;
+            const int d = (k >> shift) & 255;
+            // scores of one magnitude share their leading digits: when a whole wave holds one
+            // digit its first lane adds the count (64 lanes adding to one LDS word serialise)
+            const unsigned long long act = __ballot(in);
+            if (act != 0ull) {
+                const int first = __ffsll((long long)act) - 1;
+                const int d0 = __shfl(d, first);
+                if (__ballot(in && d == d0) == act) {
+                    if (lane == first) atomicAdd(&hist[d0], __popcll(act));
+                } else if (in) {
+                    atomicAdd(&hist[d], 1);
+                }
+            }
+        });
         __syncthreads();
         // digits in descending order, one per thread: the chosen digit is where the running
         // count first reaches `need`
@@ -98,33 +147,68 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
     }
     const uint32_t thr = prefix;  // the kk-th largest key; `need` of the keys equal to it are taken
 
-    // ---- winners into LDS: every key above the threshold, the first `need` equal to it ----
+    // ---- winners into LDS: every key above the threshold, then the first `need` equal to it.
+    //      Slots come from a prefix sum over the list (both counts packed into one scan), not
+    //      from a shared counter: thousands of increments of one LDS word would serialise ----
     for (int i = tid; i < a.cap; i += kSortThreads) win[i] = 0ull;
-    if (tid == 0) s_count = 0;
     __syncthreads();
-    int eq_before = 0;  // keys equal to the threshold in earlier chunks
-    for (int base = 0; base < a.max_n && kk > 0; base += kSortThreads) {
-        const int i = base + tid;
-        const uint32_t k = i < a.max_n ? keys[i] : 0u;
-        const bool gt = k > thr && k != 0u;
-        const bool eq = k == thr && k != 0u;
-        int eq_total;
-        const int eq_rank = eq_before + scan1024(eq ? 1 : 0, wsum, &eq_total);
-        if (gt || (eq && eq_rank < need)) {
-            const int slot = atomicAdd(&s_count, 1);
-            win[slot] = ((unsigned long long)k << 32) | (uint32_t)(~(uint32_t)i);
+    const int n_gt = kk - need;  // keys above the threshold
+    int gt_before = 0, eq_before = 0;
+    if (kk > 0) {
+        if constexpr (REG) {
+            int my_gt = 0, my_eq = 0;
+#pragma unroll
+            for (int e = 0; e < kRegKeys; ++e) {
+                my_gt += kreg[e] > thr && kreg[e] != 0u;
+                my_eq += kreg[e] == thr && kreg[e] != 0u;
+            }
+            int total;
+            const int before = scan1024(my_gt | (my_eq << 16), wsum, &total);
+            int gt_at = before & 0xffff, eq_at = before >> 16;
+#pragma unroll
+            for (int e = 0; e < kRegKeys; ++e) {
+                const uint32_t k = kreg[e];
+                const int i = tid * kRegKeys + e;
+                int slot = -1;
+                if (k > thr && k != 0u) slot = gt_at++;
+                else if (k == thr && k != 0u) {
+                    if (eq_at < need) slot = n_gt + eq_at;
+                    ++eq_at;
+                }
+                if (slot >= 0) win[slot] = ((unsigned long long)k << 32) | (uint32_t)(~(uint32_t)i);
+            }
+        } else {
+            for_chunks([&](int e, uint32_t k) {
+                const int i = e * kSortThreads + tid;
+                const bool gt = k > thr && k != 0u;
+                const bool eq = k == thr && k != 0u;
+                int total;
+                const int before = scan1024((gt ? 1 : 0) | (eq ? 1 << 16 : 0), wsum, &total);
+                const int eq_rank = eq_before + (before >> 16);
+                int slot = -1;
+                if (gt) slot = gt_before + (before & 0xffff);
+                else if (eq && eq_rank < need) slot = n_gt + eq_rank;
+                if (slot >= 0) win[slot] = ((unsigned long long)k << 32) | (uint32_t)(~(uint32_t)i);
+                gt_before += total & 0xffff;
+                eq_before += total >> 16;
+            });
         }
-        eq_before += eq_total;
     }
     __syncthreads();
 
-    // ---- bitonic sort, descending: larger key first, then smaller position ----
-    for (int size = 2; size <= a.cap; size <<= 1) {
+    // ---- order the winners, descending: larger key first, then smaller position ----
+    // (a) bitonic networks over aligned segments of 256 entries, every segment descending;
+    // (b) sorted runs merged pairwise: an entry's place in the merged run is its place in its own
+    //     run plus the number of entries of the sibling run that go before it (binary search; the
+    //     left run wins ties, which only the empty slots have).  For 4096 entries that is 36 + 2 * 4
+    //     barriers where one network over everything takes 78.
+    const int seg = a.cap < 256 ? a.cap : 256;
+    for (int size = 2; size <= seg; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             for (int t = tid; t < a.cap / 2; t += kSortThreads) {
                 const int lo = 2 * t - (t & (stride - 1));
                 const int hi = lo + stride;
-                const bool desc = (lo & size) == 0;
+                const bool desc = size == seg || (lo & size) == 0;
                 const unsigned long long x = win[lo], y = win[hi];
                 if ((x < y) == desc) {
                     win[lo] = y;
@@ -133,6 +217,36 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
             }
             __syncthreads();
         }
+    }
+    for (int run = seg; run < a.cap; run <<= 1) {
+        constexpr int kPer = kMaxTopk / kSortThreads;  // entries per thread at the largest cap
+        unsigned long long x[kPer];
+        int dst[kPer];
+        const int sh = __builtin_ctz(run);
+#pragma unroll
+        for (int e = 0; e < kPer; ++e) {
+            const int i = tid + e * kSortThreads;
+            dst[e] = -1;
+            if (i < a.cap) {
+                x[e] = win[i];
+                const int r = i >> sh, at = i & (run - 1);
+                const unsigned long long* sib = win + (r ^ 1) * run;
+                const bool left = (r & 1) == 0;
+                int lo = 0, hi = run;  // entries of the sibling run that go before x[e]
+                while (lo < hi) {
+                    const int mid = (lo + hi) >> 1;
+                    const unsigned long long o = sib[mid];
+                    if (o > x[e] || (!left && o == x[e])) lo = mid + 1;
+                    else hi = mid;
+                }
+                dst[e] = (r >> 1) * 2 * run + at + lo;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < kPer; ++e)
+            if (dst[e] >= 0) win[dst[e]] = x[e];
+        __syncthreads();
     }
 
     for (int t = tid; t < a.topk; t += kSortThreads) {
@@ -193,7 +307,10 @@ inline int launch_topk_sort(const SortArgs& in, int rows, hipStream_t st)
     int cap = 2;
     while (cap < s.topk) cap <<= 1;
     s.cap = cap;
-    hipLaunchKernelGGL(topk_sort_kernel, dim3((unsigned)rows), dim3(kSortThreads), (size_t)cap * 8, st, s);
+    if (s.max_n <= kRegKeys * kSortThreads)
+        hipLaunchKernelGGL(topk_sort_kernel<true>, dim3((unsigned)rows), dim3(kSortThreads), (size_t)cap * 8, st, s);
+    else
+        hipLaunchKernelGGL(topk_sort_kernel<false>, dim3((unsigned)rows), dim3(kSortThreads), (size_t)cap * 8, st, s);
     return ucm::launch_status("topk_sort_kernel");
 }
 
