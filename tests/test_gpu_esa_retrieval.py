@@ -113,6 +113,35 @@ def test_random_shapes(n_items, dim, B, max_n, k):
     check(data, query, indexes, k)
 
 
+@pytest.mark.parametrize("max_n,k,values", [
+    (5000, 2000, 9),      # nine distinct scores: every bucket of the ordering fast path overflows
+    (8000, 3000, 1),      # all scores equal: the output is the list order
+    (3000, 2500, 400),    # a few hundred distinct scores: crowded and sparse buckets mixed
+    (20000, 4096, 30),    # the same past the register-resident size
+])
+def test_many_equal_scores_are_bit_exact_in_list_order(max_n, k, values):
+    """Integer-valued data make the scores exact in any summation order, so outputs must equal
+    the checker's bit for bit, including the order among equal scores (list order)."""
+    rng = rng_for(max_n + values)
+    n_items, dim = 25000, 8
+    data = rng.integers(0, 2, size=(n_items, dim)).astype(np.float32)
+    if values == 1:
+        data[:] = 1.0
+    elif values > 9:
+        data[:, 0] = rng.integers(0, values, n_items)
+    query = np.ones((2, dim), np.float32)
+    indexes = np.stack([rng.permutation(n_items)[:max_n] for _ in range(2)]).astype(np.int32)
+    gi, gs = gpu_dot_topk(data, query, indexes, k)
+    oi, osc = c_api.dot_topk(data, query, indexes, k)
+    assert np.array_equal(gs, osc)
+    # equal scores: the checker's order among ties is its partial_sort's; list order is this
+    # library's contract, so compare against a stable sort of the exact scores
+    exact = (data[indexes] * query[:, None, :]).sum(-1)
+    for b in range(2):
+        order = np.argsort(-exact[b], kind="stable")[:k]
+        assert np.array_equal(gi[b], indexes[b][order])
+
+
 def test_fewer_candidates_than_k_and_empty_rows():
     rng = rng_for(9)
     data = rng.standard_normal((100, 64)).astype(np.float32)

@@ -11,6 +11,8 @@ namespace {
 
 constexpr int kSortThreads = 1024;
 constexpr int kMaxTopk = 4096;  // winners sorted in LDS: 8 bytes each (32 KiB)
+constexpr int kBuckets = 1024;   // equal-width key buckets of the ordering fast path (one per thread)
+constexpr int kBucketMax = 48;   // entries a bucket may hold on that path
 constexpr int kRegKeys = 8;     // keys a thread keeps in registers: rows of up to 8192 candidates
 
 // Order-preserving key of a score: larger score <-> larger key.  0 is reserved for "no
@@ -63,6 +65,7 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
     __shared__ int hist[256];
     __shared__ int wsum[kSortThreads / 64];
     __shared__ int s_digit, s_need;
+    __shared__ int bcount[kBuckets], bfill[kBuckets], bbase[kBuckets];
     const int b = blockIdx.x;
     const uint32_t* keys = a.keys + (int64_t)b * a.max_n;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -197,49 +200,68 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
     __syncthreads();
 
     // ---- order the winners, descending: larger key first, then smaller position ----
-    // (a) bitonic networks over aligned segments of 256 entries, every segment descending;
-    // (b) sorted runs merged pairwise: an entry's place in the merged run is its place in its own
-    //     run plus the number of entries of the sibling run that go before it (binary search; the
-    //     left run wins ties, which only the empty slots have).  For 4096 entries that is 36 + 2 * 4
-    //     barriers where one network over everything takes 78.
-    const int seg = a.cap < 256 ? a.cap : 256;
-    for (int size = 2; size <= seg; size <<= 1) {
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            for (int t = tid; t < a.cap / 2; t += kSortThreads) {
-                const int lo = 2 * t - (t & (stride - 1));
-                const int hi = lo + stride;
-                const bool desc = size == seg || (lo & size) == 0;
-                const unsigned long long x = win[lo], y = win[hi];
-                if ((x < y) == desc) {
-                    win[lo] = y;
-                    win[hi] = x;
-                }
-            }
-            __syncthreads();
+    // Fast path: the winners' keys lie in [thr, kmax]; 1024 equal-width buckets over that range
+    // (descending), a prefix sum over the bucket counts, every winner dropped into its bucket,
+    // then ranked among the few entries that share it.  Six barriers and a handful of LDS accesses
+    // per entry.  A bucket of more than kBucketMax entries (many equal or tightly clustered scores)
+    // sends the row down the general path below.
+    constexpr int kPer = kMaxTopk / kSortThreads;  // entries per thread at the largest cap
+    uint32_t kmax_part = 0u;
+    unsigned long long x[kPer];
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+        const int i = tid + e * kSortThreads;
+        x[e] = i < kk ? win[i] : 0ull;
+        const uint32_t k = (uint32_t)(x[e] >> 32);
+        kmax_part = k > kmax_part ? k : kmax_part;
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)kmax_part, o);
+        kmax_part = other > kmax_part ? other : kmax_part;
+    }
+    if (tid < kBuckets) {
+        bcount[tid] = 0;
+        bfill[tid] = 0;
+    }
+    if (lane == 0) wsum[tid >> 6] = (int)kmax_part;
+    __syncthreads();
+    uint32_t kmax = 0u;
+    for (int w = 0; w < kSortThreads / 64; ++w) kmax = (uint32_t)wsum[w] > kmax ? (uint32_t)wsum[w] : kmax;
+    const uint32_t range = kmax > thr ? kmax - thr : 0u;
+    const int bits = range ? 32 - __builtin_clz(range) : 0;
+    const int bshift = bits > 10 ? bits - 10 : 0;
+    int bucket[kPer];
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+        const int i = tid + e * kSortThreads;
+        bucket[e] = -1;
+        if (i < kk) {
+            bucket[e] = (kBuckets - 1) - (int)(((uint32_t)(x[e] >> 32) - thr) >> bshift);
+            atomicAdd(&bcount[bucket[e]], 1);
         }
     }
-    for (int run = seg; run < a.cap; run <<= 1) {
-        constexpr int kPer = kMaxTopk / kSortThreads;  // entries per thread at the largest cap
-        unsigned long long x[kPer];
+    __syncthreads();
+    const int my_count = tid < kBuckets ? bcount[tid] : 0;
+    int all_winners;
+    const int my_base = scan1024(my_count, wsum, &all_winners);
+    const bool crowded = __syncthreads_or(my_count > kBucketMax);
+    if (!crowded) {
+        if (tid < kBuckets) bbase[tid] = my_base;
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < kPer; ++e)
+            if (bucket[e] >= 0) win[bbase[bucket[e]] + atomicAdd(&bfill[bucket[e]], 1)] = x[e];
+        __syncthreads();
         int dst[kPer];
-        const int sh = __builtin_ctz(run);
 #pragma unroll
         for (int e = 0; e < kPer; ++e) {
-            const int i = tid + e * kSortThreads;
             dst[e] = -1;
-            if (i < a.cap) {
-                x[e] = win[i];
-                const int r = i >> sh, at = i & (run - 1);
-                const unsigned long long* sib = win + (r ^ 1) * run;
-                const bool left = (r & 1) == 0;
-                int lo = 0, hi = run;  // entries of the sibling run that go before x[e]
-                while (lo < hi) {
-                    const int mid = (lo + hi) >> 1;
-                    const unsigned long long o = sib[mid];
-                    if (o > x[e] || (!left && o == x[e])) lo = mid + 1;
-                    else hi = mid;
-                }
-                dst[e] = (r >> 1) * 2 * run + at + lo;
+            if (bucket[e] >= 0) {
+                const int first = bbase[bucket[e]], n = bcount[bucket[e]];
+                int ahead = 0;  // entries of the bucket that go before this one
+                for (int j = 0; j < n; ++j) ahead += win[first + j] > x[e];
+                dst[e] = first + ahead;
             }
         }
         __syncthreads();
@@ -247,6 +269,57 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
         for (int e = 0; e < kPer; ++e)
             if (dst[e] >= 0) win[dst[e]] = x[e];
         __syncthreads();
+    } else {
+        // General path:
+        // (a) bitonic networks over aligned segments of 256 entries, every segment descending;
+        // (b) sorted runs merged pairwise: an entry's place in the merged run is its place in its
+        //     own run plus the number of entries of the sibling run that go before it (binary
+        //     search; the left run wins ties, which only the empty slots have).  For 4096 entries
+        //     that is 36 + 2 * 4 barriers where one network over everything takes 78.
+        const int seg = a.cap < 256 ? a.cap : 256;
+        for (int size = 2; size <= seg; size <<= 1) {
+            for (int stride = size >> 1; stride > 0; stride >>= 1) {
+                for (int t = tid; t < a.cap / 2; t += kSortThreads) {
+                    const int lo = 2 * t - (t & (stride - 1));
+                    const int hi = lo + stride;
+                    const bool desc = size == seg || (lo & size) == 0;
+                    const unsigned long long p = win[lo], q = win[hi];
+                    if ((p < q) == desc) {
+                        win[lo] = q;
+                        win[hi] = p;
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        for (int run = seg; run < a.cap; run <<= 1) {
+            int dst[kPer];
+            const int sh = __builtin_ctz(run);
+#pragma unroll
+            for (int e = 0; e < kPer; ++e) {
+                const int i = tid + e * kSortThreads;
+                dst[e] = -1;
+                if (i < a.cap) {
+                    x[e] = win[i];
+                    const int r = i >> sh, at = i & (run - 1);
+                    const unsigned long long* sib = win + (r ^ 1) * run;
+                    const bool left = (r & 1) == 0;
+                    int lo = 0, hi = run;  // entries of the sibling run that go before x[e]
+                    while (lo < hi) {
+                        const int mid = (lo + hi) >> 1;
+                        const unsigned long long o = sib[mid];
+                        if (o > x[e] || (!left && o == x[e])) lo = mid + 1;
+                        else hi = mid;
+                    }
+                    dst[e] = (r >> 1) * 2 * run + at + lo;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < kPer; ++e)
+                if (dst[e] >= 0) win[dst[e]] = x[e];
+            __syncthreads();
+        }
     }
 
     for (int t = tid; t < a.topk; t += kSortThreads) {
