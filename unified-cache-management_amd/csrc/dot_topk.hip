@@ -45,32 +45,53 @@ __global__ __launch_bounds__(kDotThreads) void dot_score_kernel(DotArgs a)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int first = (blockIdx.x * (kDotThreads / 64) + wave) * kRowsPerWave;
     const bool vec = (a.dim & 3) == 0;
+    // the wave's candidates first, then their rows chunk by chunk with all of the wave's rows in
+    // flight together: two round trips to memory instead of two per row
+    int item[kRowsPerWave];
+    bool ok[kRowsPerWave];
+    const float* row[kRowsPerWave];
+    float acc[kRowsPerWave];
+#pragma unroll
     for (int r = 0; r < kRowsPerWave; ++r) {
         const int j = first + r;
-        if (j >= a.max_n) break;
-        const int item = a.idx[(int64_t)b * a.max_n + j];
-        const bool ok = item >= 0 && item < a.n_items;
-        float acc = 0.0f;
-        if (ok) {
-            const float* row = a.data + (int64_t)item * a.dim;
-            if (vec) {
-                for (int c = lane * 4; c < a.dim; c += 256) {
-                    const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(row + c));
-                    const f32x4 y = *reinterpret_cast<const f32x4*>(qs + c);
-                    acc = __builtin_fmaf(x.x, y.x, acc);
-                    acc = __builtin_fmaf(x.y, y.y, acc);
-                    acc = __builtin_fmaf(x.z, y.z, acc);
-                    acc = __builtin_fmaf(x.w, y.w, acc);
-                }
-            } else {
-                for (int c = lane; c < a.dim; c += 64) acc = __builtin_fmaf(row[c], qs[c], acc);
+        item[r] = j < a.max_n ? a.idx[(int64_t)b * a.max_n + j] : -1;
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        ok[r] = item[r] >= 0 && item[r] < a.n_items;
+        row[r] = a.data + (int64_t)(ok[r] ? item[r] : 0) * a.dim;  // row 0 stands in: always readable
+        acc[r] = 0.0f;
+    }
+    if (vec) {
+        for (int c = lane * 4; c < a.dim; c += 256) {
+            f32x4 x[kRowsPerWave];
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r)
+                x[r] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(row[r] + c));
+            const f32x4 y = *reinterpret_cast<const f32x4*>(qs + c);
+#pragma unroll
+            for (int r = 0; r < kRowsPerWave; ++r) {
+                acc[r] = __builtin_fmaf(x[r].x, y.x, acc[r]);
+                acc[r] = __builtin_fmaf(x[r].y, y.y, acc[r]);
+                acc[r] = __builtin_fmaf(x[r].z, y.z, acc[r]);
+                acc[r] = __builtin_fmaf(x[r].w, y.w, acc[r]);
             }
         }
+    } else {
+        for (int c = lane; c < a.dim; c += 64) {
 #pragma unroll
-        for (int s = 32; s >= 1; s >>= 1) acc += __shfl_xor(acc, s);
-        if (lane == 0) {
-            a.scores[(int64_t)b * a.max_n + j] = ok ? acc : 0.0f;
-            a.keys[(int64_t)b * a.max_n + j] = ok ? score_key(acc) : 0u;
+            for (int r = 0; r < kRowsPerWave; ++r) acc[r] = __builtin_fmaf(row[r][c], qs[c], acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        float t = acc[r];
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) t += __shfl_xor(t, s);
+        const int j = first + r;
+        if (lane == 0 && j < a.max_n) {
+            a.scores[(int64_t)b * a.max_n + j] = ok[r] ? t : 0.0f;
+            a.keys[(int64_t)b * a.max_n + j] = ok[r] ? score_key(t) : 0u;
         }
     }
 }
