@@ -229,6 +229,30 @@ def _esa_ws(B, max_n):
     return int(_lib_mod().lib().ucm_dot_topk_workspace_bytes(B, max_n))
 
 
+def graph_ms(torch, fn, reps=20, replays=5):
+    """Milliseconds per call of fn(i) with `reps` calls captured in one HIP graph and the graph
+    replayed: the launches run back to back on the GPU, so the figure is the kernels' time, not
+    the host's time to issue them one by one from Python."""
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(3):
+            fn(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        for i in range(reps):
+            fn(i)
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (reps * replays)
+
+
 def extras(torch, enc_k, gen):
     """Side figures: encoder at cache-build shape, device gather, pinned-host dump."""
     import numpy as np
@@ -239,16 +263,9 @@ def extras(torch, enc_k, gen):
     keys = torch.randn((CTX, HKV, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
     cache = torch.empty((NBLK, BS, HKV, WD), dtype=torch.int32, device="cuda")
     slots = torch.arange(CTX, device="cuda", dtype=torch.int64)
-    for _ in range(3):
-        enc_k.compute_hash_and_cache(keys, slots, cache, BS)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     reps = 20
-    e0.record()
-    for _ in range(reps):
-        enc_k.compute_hash_and_cache(keys, slots, cache, BS)
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / reps
+    ms = graph_ms(torch, lambda i: enc_k.compute_hash_and_cache(keys, slots, cache, BS))
     rows = CTX * HKV
     enc_bytes = rows * D * 2 + rows * WD * 4 + HKV * D * D * 2
     out["encoder"] = {"rows": rows, "ms": ms, "GBps": enc_bytes / ms / 1e6,
@@ -274,15 +291,7 @@ def extras(torch, enc_k, gen):
         enc_k.compute_hash_and_cache(gathered, slot_map, codes, BS)
 
     for name, fn in (("fused", fused), ("reference_recipe", recipe)):
-        for i in range(4):
-            fn(i)
-        torch.cuda.synchronize()
-        e0.record()
-        for i in range(reps):
-            fn(i)
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / reps
+        ms = graph_ms(torch, fn)
         out.setdefault("prefix_rehash", {})[name] = {
             "tokens": CTX, "ms": ms, "key_GBps": rows * D * 2 / ms / 1e6}
     del kcache, codes
@@ -296,15 +305,7 @@ def extras(torch, enc_k, gen):
     qv = torch.rand((2, 1024), generator=gen, device="cuda", dtype=torch.float32)
     cand = torch.stack([torch.randperm(25600, generator=gen, device="cuda")[:8000] for _ in range(2)]).to(torch.int32)
     ws = torch.empty(_esa_ws(2, 8000), dtype=torch.uint8, device="cuda")
-    for _ in range(3):
-        dot_topk(vecs, qv, cand, 3000, ws)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(reps):
-        dot_topk(vecs, qv, cand, 3000, ws)
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / reps
+    ms = graph_ms(torch, lambda i: dot_topk(vecs, qv, cand, 3000, ws))
     out["esa_dot_topk"] = {"candidates": 2 * 8000, "dim": 1024, "topk": 3000, "ms": ms,
                            "gather_GBps": 2 * 8000 * 4096 / ms / 1e6}
     del vecs
@@ -315,16 +316,9 @@ def extras(torch, enc_k, gen):
     kq, kk, kp = (torch.from_numpy(t).cuda() for t in _kvstar_case(np))
     kws = torch.empty(_lib_mod().lib().ucm_kvstar_topk_workspace_bytes(8, 32, 253, 64), dtype=torch.uint8,
                       device="cuda")
-    for _ in range(3):
-        kvstar_topk(kq, kk, kp, 64, kws)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(reps):
-        kvstar_topk(kq, kk, kp, 64, kws)
-    e1.record()
-    torch.cuda.synchronize()
     out["kvstar_topk"] = {"queries": 8, "q_heads": 32, "blocks": 253, "representatives": 253 * 64,
-                          "dim": 32, "topk": 64, "ms": e0.elapsed_time(e1) / reps}
+                          "dim": 32, "topk": 64,
+                          "ms": graph_ms(torch, lambda i: kvstar_topk(kq, kk, kp, 64, kws))}
 
     # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---
     L, NBP, n_req, n_sel = 32, 256, 4, 64
