@@ -545,6 +545,10 @@ void oracle_dot_topk(const float* data, int64_t n_items, int32_t dim, const floa
  * row (:944-952), a size-topk min-heap of (score, block) pairs with strict-greater replacement,
  * emptied back to front (:954-977).  fp16 -> fp32 as fp16_to_float (:780-812).
  * all_scores (optional) receives the n_blocks block scores.
+ * Pinned by mathematics only (tests/test_oracle_kvstar.py: a float64 library formulation,
+ * closed forms, invariants, the heap's tie order, all 65,536 fp16 patterns): the reference's
+ * translation unit needs its logger (spdlog, fmt), which this image lacks, so it cannot be
+ * compiled for golden vectors, and the reference holds no test vectors for this kernel.
  * ------------------------------------------------------------------------------------ */
 static float half_bits_to_float(uint16_t h)
 {
