@@ -337,35 +337,42 @@ __global__ __launch_bounds__(kSortThreads) void topk_sort_kernel(SortArgs a)
 
 // Short rows (max_n <= 1024, e.g. the blocks of one request): every candidate counts the
 // candidates that come before it in the output order (larger key, or equal key and earlier
-// position) and writes itself at that rank.  No search and no sort: n broadcast reads from LDS
-// per thread.  Same output as topk_sort_kernel.
+// position — one comparison of (key, ~position) pairs) and writes itself at that rank.  No
+// search and no sort.  The 1024 threads share the work: P = 1024 / n (rounded down to a power
+// of two, at most 64) neighbouring lanes split one candidate's comparisons and add their counts
+// with shuffles.  Same output as topk_sort_kernel.
 __global__ __launch_bounds__(kSortThreads) void topk_rank_kernel(SortArgs a)
 {
-    __shared__ __align__(16) uint32_t k_lds[kSortThreads];
+    __shared__ __align__(16) unsigned long long c_lds[kSortThreads];
     const int b = blockIdx.x, tid = threadIdx.x;
     const uint32_t* keys = a.keys + (int64_t)b * a.max_n;
-    const uint32_t mine = tid < a.max_n ? keys[tid] : 0u;
-    k_lds[tid] = mine;
+    {
+        const uint32_t k = tid < a.max_n ? keys[tid] : 0u;
+        c_lds[tid] = k ? ((unsigned long long)k << 32) | (uint32_t)(~(uint32_t)tid) : 0ull;
+    }
     for (int t = tid; t < a.topk; t += kSortThreads) {  // slots no candidate reaches
         a.out_idx[(int64_t)b * a.topk + t] = -1;
         a.out_score[(int64_t)b * a.topk + t] = 0.0f;
     }
     __syncthreads();  // also orders the fill above before the winners' writes below
-    if (mine == 0u) return;
+    int shift = 0;    // P = 1 << shift lanes per candidate
+    while (shift < 6 && (a.max_n << (shift + 1)) <= kSortThreads) ++shift;
+    const int cand = tid >> shift, part = tid & ((1 << shift) - 1);
+    const int span = (((a.max_n + (1 << shift) - 1) >> shift) + 1) & ~1;  // even: 16-byte reads
+    const unsigned long long mine = cand < a.max_n ? c_lds[cand] : 0ull;
     int rank = 0;
-    const int n4 = a.max_n & ~3;
-    for (int j = 0; j < n4; j += 4) {
-        const uint4 o = *reinterpret_cast<const uint4*>(k_lds + j);
-        rank += (o.x > mine || (o.x == mine && j < tid)) + (o.y > mine || (o.y == mine && j + 1 < tid)) +
-                (o.z > mine || (o.z == mine && j + 2 < tid)) + (o.w > mine || (o.w == mine && j + 3 < tid));
+    const int j0 = part * span;
+    int j1 = j0 + span;
+    j1 = j1 < a.max_n ? j1 : a.max_n;
+    for (int j = j0; j + 1 < j1; j += 2) {
+        const ulonglong2 o = *reinterpret_cast<const ulonglong2*>(c_lds + j);
+        rank += (o.x > mine) + (o.y > mine);
     }
-    for (int j = n4; j < a.max_n; ++j) {
-        const uint32_t o = k_lds[j];
-        rank += (o > mine || (o == mine && j < tid));
-    }
-    if (rank < a.topk) {
-        a.out_idx[(int64_t)b * a.topk + rank] = a.idx[(int64_t)b * a.max_n + tid];
-        a.out_score[(int64_t)b * a.topk + rank] = a.scores[(int64_t)b * a.max_n + tid];
+    if (j0 < j1 && ((j1 - j0) & 1)) rank += c_lds[j1 - 1] > mine;
+    for (int o = 1; o < (1 << shift); o <<= 1) rank += __shfl_xor(rank, o);
+    if (part == 0 && mine != 0ull && rank < a.topk) {
+        a.out_idx[(int64_t)b * a.topk + rank] = a.idx[(int64_t)b * a.max_n + cand];
+        a.out_score[(int64_t)b * a.topk + rank] = a.scores[(int64_t)b * a.max_n + cand];
     }
 }
 
