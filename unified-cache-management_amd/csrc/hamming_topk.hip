@@ -784,6 +784,18 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
     if (rowid >= rows_total) return;
     const int b = rowid / a.Ho, ho = rowid % a.Ho;
     const int lane = lane_id();
+    // the row's scores go out before the length is known (in-range positions only, masked
+    // below): one round trip to memory instead of two
+    int raw[EL];
+    {
+        const bool red = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
+        const int32_t* r0 = a.scores + ((int64_t)b * a.Hkv + (red ? 0 : ho)) * a.max_blocks;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int j = lane * EL + e;
+            raw[e] = r0[j < a.max_blocks ? j : 0];
+        }
+    }
     const int len = a.lens[b];
     int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
     if (n > a.max_blocks) n = a.max_blocks;
@@ -803,7 +815,7 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
         const int j = lane * EL + e;
         int x = -0x7fffffff;  // below every real score (>= -1): never selected
         if (j < n) {
-            x = row[j];
+            x = raw[e];
             if (reduce)
                 for (int h = 1; h < a.Hkv; ++h) {
                     const int o = row[(int64_t)h * a.max_blocks + j];
