@@ -1,0 +1,114 @@
+"""Randomised differential tests (fixed seeds): many small random configurations of the scorer /
+top-k and of the encoder's three paths against the CPU checker.  The hand-picked cases elsewhere
+aim at known corners; these sweep combinations nobody thought of.  Bit-exact for the top-k, the
+margin rule (|projection| < 1e-2 * ||x||) for hash bits."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import rng_for
+from oracle import brute, c_api
+
+pytestmark = pytest.mark.gpu
+
+MARGIN_TOL = 1e-2
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_topk_random_configurations(seed):
+    from ucm_amd.sparse import hamming_topk
+
+    rng = rng_for(seed)
+    for _ in range(250):
+        B = int(rng.integers(1, 7))
+        Hkv = int(rng.choice([1, 2, 3, 4, 8]))
+        G = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        Wd = int(rng.choice([1, 2, 4, 6, 8]))
+        BS = int(rng.choice([4, 8, 16, 32, 64, 128]))
+        mb = int(rng.integers(1, 200))
+        NB = B * mb + int(rng.integers(0, 5))
+        kc = rng.integers(0, 2**32, size=(NB, BS, Hkv, Wd), dtype=np.uint32)
+        if rng.integers(0, 4) == 0:
+            kc &= np.uint32(0x01010101)  # low-entropy codes: many equal scores
+        q = rng.integers(0, 2**32, size=(B, Hkv * G, Wd), dtype=np.uint32)
+        use_table = bool(rng.integers(0, 4))
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32) if use_table else None
+        if not use_table:
+            kc = kc[:B * mb]
+        lens = rng.integers(0, mb * BS + 1, size=B).astype(np.int32)
+        if rng.integers(0, 3) == 0:
+            lens[rng.integers(0, B)] = mb * BS
+        k = int(rng.integers(1, min(mb, 128) + 3))
+        sink = int(rng.integers(0, 3)) * BS if rng.integers(0, 3) == 0 else 0
+        recent = int(rng.integers(0, 3)) * BS if rng.integers(0, 3) == 0 else 0
+        reduce_heads, physical = bool(rng.integers(0, 4) == 0), bool(rng.integers(0, 3) == 0)
+        score_order, distance = bool(rng.integers(0, 3) == 0), bool(rng.integers(0, 3) == 0)
+        flags = (c_api.F_REDUCE_HEADS if reduce_heads else 0) | (c_api.F_PHYSICAL if physical else 0) | \
+                (c_api.F_SCORE_ORDER if score_order else 0) | (c_api.F_DISTANCE if distance else 0)
+        what = dict(B=B, Hkv=Hkv, G=G, Wd=Wd, BS=BS, mb=mb, k=k, table=use_table, sink=sink, recent=recent,
+                    flags=flags)
+        oi, osc = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, flags, max_blocks=mb)
+        gi, gs = hamming_topk(torch.from_numpy(q.view(np.int32)).cuda(), torch.from_numpy(kc.view(np.int32)).cuda(),
+                              torch.from_numpy(table).cuda() if use_table else None, torch.from_numpy(lens).cuda(),
+                              k, sink, recent, reduce_heads=reduce_heads, return_physical=physical,
+                              score_order=score_order, distance=distance, max_blocks=mb)
+        assert np.array_equal(gi.cpu().numpy(), oi), what
+        assert np.array_equal(gs.cpu().numpy(), osc), what
+
+
+def _codes_ok(codes_u8, x32, W32):
+    ref = brute.hash_encode(x32, W32).view(np.uint8)
+    got = np.ascontiguousarray(codes_u8)
+    if np.array_equal(got, ref):
+        return True
+    diff = np.unpackbits(got ^ ref, axis=-1, bitorder="little").astype(bool)
+    return not np.any(diff & (brute.margins(x32, W32) >= MARGIN_TOL))
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_encoder_random_configurations(seed):
+    from ucm_amd.sparse import HashEncoder
+
+    rng = rng_for(seed)
+    for _ in range(30):
+        dt = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+        K = int(rng.choice([40, 64, 96, 128, 256, 512]))
+        N = int(rng.choice([32, 64, 96, 128, 256, 512]))
+        H = int(rng.choice([1, 2, 4, 8]))
+        T = int(rng.choice([1, 3, 31, 32, 33, 100, 257, 511, 1024, 1500, 4096]))
+        n_w = int(rng.choice([1, H]))
+        BS = int(rng.choice([8, 16, 32, 64, 128]))
+        what = dict(dt=str(dt), K=K, N=N, H=H, T=T, n_w=n_w, BS=BS)
+        W = torch.from_numpy(rng.standard_normal((n_w, K, N)).astype(np.float32)).to(dt)
+        enc = HashEncoder(K, N, dt, torch.device("cuda:0"), num_weights=n_w, heads_per_weight=1)
+        enc.set_hash_weight(W.cuda() if n_w > 1 else W[0].cuda())
+        x = torch.from_numpy(rng.standard_normal((T, H, K)).astype(np.float32)).to(dt)
+        if rng.integers(0, 5) == 0:
+            x[rng.integers(0, T)] = 0
+        W32, x32 = W.float().numpy(), x.float().numpy()
+        # dense, one matrix per head
+        codes = enc.compute_hash(x.cuda(), per_head=True).cpu().numpy()
+        for h in range(H):
+            assert _codes_ok(codes[:, h], x32[:, h], W32[min(h, n_w - 1)]), ("dense", what, h)
+        # paged store through a random slot mapping, a tenth of the rows dropped
+        NBc = (T + BS - 1) // BS + 2
+        slots = rng.permutation(NBc * BS)[:T].astype(np.int64)
+        drop = rng.random(T) < 0.1
+        slots_d = np.where(drop, -1, slots)
+        cache = torch.full((NBc, BS, H, N // 32), -1, dtype=torch.int32, device="cuda")
+        enc.compute_hash_and_cache(x.cuda(), torch.from_numpy(slots_d).cuda(), cache, BS)
+        c = cache.cpu().numpy().view(np.uint8).reshape(NBc * BS, H, N // 8)
+        for h in range(H):
+            assert _codes_ok(c[slots[~drop], h], x32[~drop, h], W32[min(h, n_w - 1)]), ("paged", what, h)
+            assert np.all(c[slots[drop], h] == 0xff), ("dropped slot written", what, h)
+        # paged input (prefix-cache rehash)
+        nblk = (T + BS - 1) // BS
+        kcache = torch.zeros((nblk + 3, BS, H, K), dtype=dt)
+        ids = rng.permutation(nblk + 3)[:nblk].astype(np.int32)
+        pos = (torch.from_numpy(ids).long().repeat_interleave(BS) * BS + torch.arange(BS).repeat(nblk))[:T]
+        kcache.view(-1, H, K)[pos] = x
+        codes2 = torch.full((nblk + 3, BS, H, N // 32), -1, dtype=torch.int32, device="cuda")
+        enc.compute_hash_from_paged_cache(kcache.cuda(), torch.from_numpy(ids).cuda(), T, codes2, BS)
+        c2 = codes2.cpu().numpy().view(np.uint8).reshape(-1, H, N // 8)
+        for h in range(H):
+            assert _codes_ok(c2[pos.numpy(), h], x32[:, h], W32[min(h, n_w - 1)]), ("rehash", what, h)
