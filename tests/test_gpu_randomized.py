@@ -112,3 +112,63 @@ def test_encoder_random_configurations(seed):
         c2 = codes2.cpu().numpy().view(np.uint8).reshape(-1, H, N // 8)
         for h in range(H):
             assert _codes_ok(c2[pos.numpy(), h], x32[:, h], W32[min(h, n_w - 1)]), ("rehash", what, h)
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_float_retrieval_random_configurations(seed):
+    """KVStar and ESA top-k on random shapes (matrix-core and scalar q.k paths, pruning, the
+    counting / bucket / merge selection paths, holes in the candidate lists, rounded data for
+    ties) against the checker, with the tolerances of test_gpu_kvstar.py and
+    test_gpu_esa_retrieval.py."""
+    from ucm_amd.sparse import kvstar_retrieve
+    from ucm_amd.sparse.esa_retrieval_worker import dot_topk
+
+    rng = rng_for(seed)
+    for _ in range(40):
+        Hkv, g = int(rng.choice([1, 2, 4, 8])), int(rng.choice([1, 2, 4, 7]))
+        Hq, X = Hkv * g, int(rng.integers(1, 12))
+        d, M = int(rng.choice([8, 16, 20, 32, 48, 64, 128])), int(rng.choice([1, 2, 3, 4]))
+        n = int(rng.integers(1, 1200))
+        n = min(n, max(1, 1_500_000 // (M * X * Hq)))
+        topk = int(rng.integers(1, min(n, 200) + 2))
+        pr, d_orig = None, d
+        if rng.integers(0, 3) == 0:
+            d_orig = d + int(rng.integers(1, 40))
+            pr = np.stack([np.sort(rng.permutation(d_orig)[:d]) for _ in range(Hkv)]).astype(np.int64)
+        q = (rng.standard_normal((X, Hq, d_orig)) * 0.5).astype(np.float16)
+        k = (rng.standard_normal((n, M, Hkv, d)) * 0.5).astype(np.float16)
+        what = dict(X=X, Hq=Hq, Hkv=Hkv, d=d, d_orig=d_orig, n=n, M=M, topk=topk)
+        gi, gs = kvstar_retrieve.kvstar_topk(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(),
+                                              torch.from_numpy(pr).cuda() if pr is not None else None, topk)
+        gi, gs = gi.cpu().numpy().astype(np.int64), gs.cpu().numpy()
+        oi, osc, allsc = c_api.kvstar_topk(q, k, topk, pr)
+        tol = 1e-7 + 2e-5 * np.abs(osc)
+        assert gi.shape == oi.shape and len(set(gi.tolist())) == gi.size, what
+        assert np.all(np.abs(gs - osc) <= tol), what
+        for t in np.nonzero(gi != oi)[0]:
+            assert abs(allsc[gi[t]] - allsc[oi[t]]) <= 2 * tol[t], what
+
+        n_items, dim = int(rng.integers(10, 12000)), int(rng.choice([16, 30, 64, 100, 256, 1024]))
+        B = int(rng.integers(1, 4))
+        max_n = int(rng.integers(1, min(n_items, 10000) + 1))
+        kk = int(rng.integers(1, min(max_n, 4096) + 1))
+        data = rng.standard_normal((n_items, dim)).astype(np.float32)
+        query = rng.standard_normal((B, dim)).astype(np.float32)
+        if rng.integers(0, 4) == 0:
+            data, query = np.round(data), np.round(query)  # exact scores, many ties
+        idx = np.stack([rng.permutation(n_items)[:max_n] for _ in range(B)]).astype(np.int32)
+        idx[rng.random(idx.shape) < 0.05] = -1
+        what = dict(n_items=n_items, dim=dim, B=B, max_n=max_n, k=kk)
+        gi, gs = dot_topk(torch.from_numpy(data).cuda(), torch.from_numpy(query).cuda(),
+                          torch.from_numpy(idx).cuda(), kk)
+        gi, gs = gi.cpu().numpy(), gs.cpu().numpy()
+        oi, osc = c_api.dot_topk(data, query, idx, kk)
+        exact = query.astype(np.float64) @ data.astype(np.float64).T
+        for b in range(B):
+            tolb = 1e-5 * (np.abs(query[b].astype(np.float64))[None, :] * np.abs(data.astype(np.float64))).sum(-1)
+            valid = oi[b] >= 0
+            assert np.array_equal(valid, gi[b] >= 0), what
+            assert len(set(gi[b][valid].tolist())) == valid.sum(), what
+            assert np.all(np.abs(gs[b][valid] - osc[b][valid]) <= 2 * tolb[oi[b][valid]].max() + 1e-30), what
+            for t in np.nonzero(valid & (gi[b] != oi[b]))[0]:
+                assert abs(exact[b, gi[b, t]] - exact[b, oi[b, t]]) <= 2 * max(tolb[gi[b, t]], tolb[oi[b, t]]) + 1e-30, what
