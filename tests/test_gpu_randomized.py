@@ -172,3 +172,50 @@ def test_float_retrieval_random_configurations(seed):
             assert np.all(np.abs(gs[b][valid] - osc[b][valid]) <= 2 * tolb[oi[b][valid]].max() + 1e-30), what
             for t in np.nonzero(valid & (gi[b] != oi[b]))[0]:
                 assert abs(exact[b, gi[b, t]] - exact[b, oi[b, t]]) <= 2 * max(tolb[gi[b, t]], tolb[oi[b, t]]) + 1e-30, what
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_block_transfer_random_configurations(seed):
+    """Scatter / gather / batch copies with random chunk sizes (odd ones included), counts,
+    permutations, both stream kinds and both directions; every byte compared, and the bytes a
+    transfer must not touch checked for their fill value."""
+    from ucm_amd.trans import Device
+
+    dev = Device()
+    dev.Setup(0)
+    rng = rng_for(seed)
+    for _ in range(40):
+        size = int(rng.choice([1, 3, 16, 100, 4096, 4097, 36 * 1024, 65536 + 8, 262144]))
+        number = int(rng.integers(1, 400))
+        number = min(number, max(1, (32 << 20) // size))
+        stream = dev.MakeSMStream() if rng.integers(0, 2) else dev.MakeStream()
+        what = dict(size=size, number=number)
+        spare = int(rng.integers(0, 4))
+        pool = torch.full((size * (number + spare),), 0xA5, dtype=torch.uint8, device="cuda")
+        perm = rng.permutation(number + spare)[:number]
+        table = np.array([pool.data_ptr() + int(i) * size for i in perm], dtype=np.uint64)
+        h1 = torch.empty(size * number, dtype=torch.uint8).pin_memory()
+        h1.numpy()[:] = rng.integers(0, 256, size=size * number, dtype=np.uint8)
+        h2 = torch.zeros(size * number, dtype=torch.uint8).pin_memory()
+        torch.cuda.synchronize()
+        stream.HostToDeviceScatterAsync(h1.data_ptr(), table, size, number)
+        stream.DeviceToHostGatherAsync(table, h2.data_ptr(), size, number)
+        stream.Synchronized()
+        assert np.array_equal(h2.numpy(), h1.numpy()), what
+        got = pool.cpu().numpy().reshape(number + spare, size)
+        assert np.array_equal(got[perm], h1.numpy().reshape(number, size)), what
+        untouched = np.setdiff1d(np.arange(number + spare), perm)
+        assert np.all(got[untouched] == 0xA5), what
+        # chunk-to-chunk batch: device chunks to separately placed host chunks and back
+        h3 = torch.zeros(size * number, dtype=torch.uint8).pin_memory()
+        hperm = rng.permutation(number)
+        htable = np.array([h3.data_ptr() + int(i) * size for i in hperm], dtype=np.uint64)
+        stream.DeviceToHostBatchAsync(table, htable, size, number)
+        stream.Synchronized()
+        assert np.array_equal(h3.numpy().reshape(number, size)[hperm], h1.numpy().reshape(number, size)), what
+        pool2 = torch.zeros(size * number, dtype=torch.uint8, device="cuda")
+        table2 = np.array([pool2.data_ptr() + int(i) * size for i in range(number)], dtype=np.uint64)
+        stream.HostToDeviceBatchAsync(htable, table2, size, number)
+        stream.Synchronized()
+        assert np.array_equal(pool2.cpu().numpy(), h1.numpy()), what
+        stream.close()
