@@ -320,6 +320,51 @@ def extras(torch, enc_k, gen):
                           "dim": 32, "topk": 64,
                           "ms": graph_ms(torch, lambda i: kvstar_topk(kq, kk, kp, 64, kws))}
 
+    # --- the other retrieval shapes of BASELINE.json (parity-tested in tests/test_gpu_full_size.py),
+    #     timed here on random codes: top-k = score + select; the per-token scorer alone ---
+    from ucm_amd.sparse import hamming_score, hamming_topk
+
+    def codes(shape):
+        return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device="cuda", generator=gen)
+
+    # config 3: batch 8, lengths uniform in [16384, 131072], 128-bit codes, top-128
+    lens3 = torch.randint(16384, 131072 + 1, (8,), generator=gen, device="cuda").to(torch.int32)
+    nblk3 = (lens3.long() + BS - 1) // BS
+    nb3 = int(nblk3.sum())
+    cache3 = codes((nb3, BS, HKV, WD))
+    table3 = torch.zeros((8, int(nblk3.max())), dtype=torch.int32, device="cuda")
+    perm3 = torch.randperm(nb3, generator=gen, device="cuda").to(torch.int32)
+    o = 0
+    for b in range(8):
+        table3[b, : int(nblk3[b])] = perm3[o:o + int(nblk3[b])]
+        o += int(nblk3[b])
+    q3 = codes((8, HQ, WD))
+    ms = graph_ms(torch, lambda i: hamming_topk(q3, cache3, table3, lens3, 128))
+    tok3 = int(lens3.sum())
+    out["config3_ragged_topk128"] = {"tokens": tok3, "ms": ms, "tokens_per_s": tok3 / ms * 1e3,
+                                     "code_GBps": tok3 * HKV * WD * 4 / ms / 1e6}
+    del cache3, table3
+    # config 5: MLA, one latent head, 128 q heads, 256-bit codes, 16 x 65536 tokens, 64-token blocks, top-128
+    b5, ctx5, bs5, wd5 = 16, 65536, 64, 8
+    cache5 = codes((b5 * ctx5 // bs5, bs5, 1, wd5))
+    table5 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
+    lens5 = torch.full((b5,), ctx5, dtype=torch.int32, device="cuda")
+    q5 = codes((b5, 128, wd5))
+    ms = graph_ms(torch, lambda i: hamming_topk(q5, cache5, table5, lens5, 128))
+    out["config5_mla_topk128"] = {"tokens": b5 * ctx5, "ms": ms, "tokens_per_s": b5 * ctx5 / ms * 1e3,
+                                  "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6}
+    del cache5, table5
+    # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
+    cache2 = codes((NB, BS, HKV, WD))
+    table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, NBLK)
+    lens2 = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
+    q2 = codes((B, HQ, WD))
+    ms = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, False), reps=10)
+    byt = B * CTX * HKV * (WD * 4 + 2)
+    out["token_scores_config2"] = {"tokens": B * CTX, "ms": ms, "tokens_per_s": B * CTX / ms * 1e3,
+                                   "hbm_GBps": byt / ms / 1e6, "hbm_frac": byt / ms / 1e6 / HBM_PEAK_GBPS}
+    del cache2, table2
+
     # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---
     L, NBP, n_req, n_sel = 32, 256, 4, 64
     chunk = BS * HKV * D * 2  # 256 KiB

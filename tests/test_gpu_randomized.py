@@ -219,3 +219,40 @@ def test_block_transfer_random_configurations(seed):
         stream.Synchronized()
         assert np.array_equal(pool2.cpu().numpy(), h1.numpy()), what
         stream.close()
+
+
+@pytest.mark.parametrize("seed", [51, 52])
+def test_per_token_scores_random_configurations(seed):
+    """The per-token scorer (coalesced kernel and general kernel) against the checker: exact
+    int32 distances, and fp16 output wherever the distances stay exactly representable."""
+    from ucm_amd.sparse import hamming_score
+
+    rng = rng_for(seed)
+    for _ in range(120):
+        B = int(rng.integers(1, 5))
+        Hkv = int(rng.choice([1, 2, 3, 4, 8]))
+        G = int(rng.choice([1, 2, 3, 4, 8]))
+        Wd = int(rng.choice([2, 4, 6, 8, 16]))
+        BS = int(rng.choice([4, 16, 32, 64, 128]))
+        mb = int(rng.integers(1, 40))
+        NB = B * mb + 3
+        kc = rng.integers(0, 2**32, size=(NB, BS, Hkv, Wd), dtype=np.uint32)
+        q = rng.integers(0, 2**32, size=(B, Hkv * G, Wd), dtype=np.uint32)
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32)
+        if rng.integers(0, 4) == 0:
+            table[rng.integers(0, B), rng.integers(0, mb)] = NB + 7  # unusable entry
+        lens = rng.integers(0, mb * BS + 1, size=B).astype(np.int32)
+        msl = mb * BS - int(rng.integers(0, BS))
+        msl = max(msl, 1)
+        sink, recent = int(rng.integers(0, 2 * BS)), int(rng.integers(0, 2 * BS))
+        red = bool(rng.integers(0, 4) == 0)
+        what = dict(B=B, Hkv=Hkv, G=G, Wd=Wd, BS=BS, mb=mb, msl=msl, sink=sink, recent=recent, red=red)
+        o = c_api.hamming_score(q, kc, table, lens, msl, sink, recent, red)
+        args = (torch.from_numpy(kc.view(np.int32)).cuda(), torch.from_numpy(q.view(np.int32)).cuda()[:, None],
+                torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda(), msl, sink, recent, red)
+        g = hamming_score(*args, out_int32=True).cpu().numpy()
+        assert np.array_equal(g, o), what
+        if G * Wd * 32 <= 2048:
+            h = hamming_score(*args).cpu().numpy()
+            expect = np.where(o == c_api.INF, np.inf, o.astype(np.float64)).astype(np.float16)
+            assert np.array_equal(h, expect), what

@@ -1272,6 +1272,72 @@ extern "C" int ucm_hamming_topk_set_profile_events(void* before, void* after)
     return UCM_OK;
 }
 
+namespace {
+
+// Per-token scores for the usual layout (token-major codes whose words are a multiple of four,
+// Hkv * Wd / 4 a power of two): one workgroup per (request, logical block).  A thread keeps the
+// (head, 16-byte piece) it is responsible for and walks the block's tokens, so its loads are
+// 16 bytes wide and a wave reads 1 KiB of contiguous codes per instruction, and the G query
+// pieces of its head stay in registers.  Pieces of a wider code are summed across neighbouring
+// lanes; the block's distances are collected in LDS and written out as one contiguous run per
+// head.  Used when G * bits <= 2048, where every partial sum is an integer that fp16 holds
+// exactly, so the reference's piecewise half-precision accumulation equals the exact sum.
+template <int G>
+__global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t)
+{
+    extern __shared__ uint32_t dyn[];  // [Hkv][BS] distances
+    const ScoreArgs& a = t.s;
+    const int b = blockIdx.y, j = blockIdx.x;
+    const int P = a.Wd >> 2, HP = a.Hkv * P;
+    const int sub = threadIdx.x & (HP - 1);
+    const int p_shift = __builtin_ctz(P), hp_shift = __builtin_ctz(HP);
+    const int h = sub >> p_shift, part = sub & (P - 1);
+    uint32_t qw[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            qw[g][i] = a.q[b * a.q_stride_b + (int64_t)(h * G + g) * a.q_stride_h + part * 4 + i];
+    const int len = a.lens[b];
+    const int64_t pb = j < a.max_blocks ? physical_block(a, b, j) : -1;
+    const uint32_t* base = a.kc + (pb < 0 ? 0 : pb) * a.ks_block + sub * 4;
+    const int step = kThreads >> hp_shift;
+    for (int tok = threadIdx.x >> hp_shift; tok < a.BS; tok += step) {
+        int d = 0;
+        if (pb >= 0) {
+            const uint4 kw = *reinterpret_cast<const uint4*>(base + (int64_t)tok * a.ks_token);
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+                d += __popc(kw.x ^ qw[g][0]) + __popc(kw.y ^ qw[g][1]) + __popc(kw.z ^ qw[g][2]) +
+                     __popc(kw.w ^ qw[g][3]);
+        }
+        for (int o = 1; o < P; o <<= 1) d += __shfl_xor(d, o);
+        if (part == 0) dyn[h * a.BS + tok] = (uint32_t)d;
+    }
+    __syncthreads();
+    for (int hh = 0; hh < a.Hkv; ++hh) {
+        for (int tok = threadIdx.x; tok < a.BS; tok += kThreads) {
+            const int pos = j * a.BS + tok;
+            if (pos >= t.max_seq_len) continue;
+            const bool is_inf = pos >= len;
+            const bool keep = (pos < a.sink) || (pos >= len - a.recent && pos < len);
+            const int d = (int)dyn[hh * a.BS + tok];
+            const int64_t o = ((int64_t)b * a.Hkv + hh) * t.max_seq_len + pos;
+            if (t.out_is_f16) {
+                const _Float16 v = is_inf ? (_Float16)__builtin_inff()
+                                          : (keep ? (_Float16)0.0f : (pb >= 0 ? (_Float16)(float)d : (_Float16)__builtin_inff()));
+                uint16_t u;
+                __builtin_memcpy(&u, &v, 2);
+                ((uint16_t*)t.out)[o] = u;
+            } else {
+                ((int32_t*)t.out)[o] = is_inf ? kInf : (keep ? 0 : (pb >= 0 ? d : kInf));
+            }
+        }
+    }
+}
+
+}  // namespace
+
 extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
                                  const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
                                  int32_t Wd, int64_t ks_block, int64_t ks_token, int64_t ks_head,
@@ -1299,6 +1365,22 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
     a.recent = recent_tok; a.TB = 1; a.planes = nullptr; a.scores = nullptr;
     t.max_seq_len = max_seq_len; t.reduce_heads = reduce_heads; t.out_is_f16 = out_is_f16;
     t.out = out;
+    const int G = a.G;
+    const bool fast = !reduce_heads && Wd % 4 == 0 && is_pow2(Wd / 4) && is_pow2(Hkv * (Wd / 4)) &&
+                      Hkv * (Wd / 4) <= kThreads && ks_head == Wd && ks_token == (int64_t)Hkv * Wd &&
+                      ks_block % 4 == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 &&
+                      (G == 1 || G == 2 || G == 4 || G == 8) && (int64_t)G * Wd * 32 <= 2048 &&
+                      (int64_t)BS * Hkv * 4 <= 48 * 1024 && ucm::ceil_div(max_seq_len, BS) <= 0x7fffffff;
+    if (fast) {
+        const dim3 fgrid((unsigned)ucm::ceil_div(max_seq_len, BS), (unsigned)B);
+        const size_t lds = (size_t)BS * Hkv * 4;
+        hipStream_t st = (hipStream_t)stream;
+        if (G == 1) hipLaunchKernelGGL(token_score_fast<1>, fgrid, dim3(kThreads), lds, st, t);
+        else if (G == 2) hipLaunchKernelGGL(token_score_fast<2>, fgrid, dim3(kThreads), lds, st, t);
+        else if (G == 4) hipLaunchKernelGGL(token_score_fast<4>, fgrid, dim3(kThreads), lds, st, t);
+        else hipLaunchKernelGGL(token_score_fast<8>, fgrid, dim3(kThreads), lds, st, t);
+        return ucm::launch_status("token_score_fast");
+    }
     const dim3 grid((unsigned)ucm::ceil_div(max_seq_len, kThreads), (unsigned)B);
     hipLaunchKernelGGL(token_score_kernel, grid, dim3(kThreads), (size_t)Hq * Wd * 4,
                        (hipStream_t)stream, t);
