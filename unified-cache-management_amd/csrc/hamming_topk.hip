@@ -527,6 +527,98 @@ __global__ __launch_bounds__(kThreads) void block_score_small(ScoreArgs a)
 }
 
 // ---------------------------------------------------------------------------------------
+// Blocks of 1 to 8 KiB (16- to 64-token blocks of the usual head layouts) with the query codes
+// compared directly (G = 1, 2, 4): every wave owns whole blocks — U = max(4, RPB) runs of 64
+// pieces, i.e. U / RPB consecutive blocks — so its 4 or 8 loads go out together right after the
+// two scalar reads, the block minimum never leaves the wave (register minimum over the runs,
+// shuffles over the lanes of a head) and the kernel has no LDS, no barrier and no loop.  A
+// workgroup is four such waves: the same 16 KiB in flight as the one-block kernel above, where
+// a workgroup per 2 KiB block would spend most of its time in the prologue.
+// ---------------------------------------------------------------------------------------
+template <int CPU, int HKV, int GP, int RPB>
+__global__ __launch_bounds__(kThreads) void block_score_rows(ScoreArgs a)
+{
+    constexpr int PERIOD = HKV * CPU;        // pieces per token (a power of two <= 64)
+    constexpr int U = RPB > 4 ? RPB : 4;     // runs per wave
+    constexpr int NBW = U / RPB;             // blocks per wave
+    const int b = blockIdx.y;
+    const int lane = lane_id();
+    const int wid = wave_id();
+    const int h = (lane % PERIOD) / CPU, part = lane % CPU;
+    const int jw = (blockIdx.x * (kThreads / kWave) + wid) * NBW;  // the wave's first block
+
+    // table entries of the wave's blocks and the length: independent scalar reads, selected with
+    // masks (no table: the entry read is a harmless second read of the length)
+    const uintptr_t has_table = a.table ? ~(uintptr_t)0 : 0;
+    int entry[NBW];
+#pragma unroll
+    for (int bi = 0; bi < NBW; ++bi) {
+        const int j = jw + bi < a.max_blocks ? jw + bi : a.max_blocks - 1;
+        const uintptr_t ea = (reinterpret_cast<uintptr_t>(a.table + ((int64_t)b * a.table_stride + j)) & has_table) |
+                             (reinterpret_cast<uintptr_t>(a.lens + b) & ~has_table);
+        entry[bi] = *reinterpret_cast<const int32_t*>(ea);
+    }
+    const int len = a.lens[b];
+
+    uint32_t qr[GP][4];
+    {
+        const uint32_t* qp = a.q + b * a.q_stride_b + (int64_t)h * GP * a.q_stride_h + part * 4;
+#pragma unroll
+        for (int g = 0; g < GP; ++g)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[g][w] = qp[g * a.q_stride_h + w];
+    }
+    if ((int64_t)jw * a.BS >= len) return;  // the whole wave lies past the request's last block
+
+    // every load is issued, against block 0 when the entry is unusable (masked below): one
+    // instruction stream, nothing waits before all of them are out
+    int64_t pb[NBW];
+    u32x4 kv[U];
+#pragma unroll
+    for (int bi = 0; bi < NBW; ++bi) {
+        const int j = jw + bi;
+        int64_t v = ((int64_t)entry[bi] & (int64_t)has_table) | (((int64_t)b * a.max_blocks + j) & ~(int64_t)has_table);
+        if (j >= a.max_blocks || v < 0 || v >= a.NB) v = -1;
+        pb[bi] = v;
+        const u32x4* base = reinterpret_cast<const u32x4*>(a.kc + (v < 0 ? 0 : v) * a.ks_block) + lane;
+#pragma unroll
+        for (int r = 0; r < RPB; ++r) kv[bi * RPB + r] = __builtin_nontemporal_load(base + (r << 6));
+    }
+
+    const int full = a.G * 32 * a.Wd;
+#pragma unroll
+    for (int bi = 0; bi < NBW; ++bi) {
+        const int j = jw + bi;
+        const int pos0 = j * a.BS;
+        int m = kInf;
+#pragma unroll
+        for (int r = 0; r < RPB; ++r) {
+            const u32x4 k4 = kv[bi * RPB + r];
+            int d = 0;
+#pragma unroll
+            for (int g = 0; g < GP; ++g)
+                d += __popc(k4.x ^ qr[g][0]) + __popc(k4.y ^ qr[g][1]) + __popc(k4.z ^ qr[g][2]) +
+                     __popc(k4.w ^ qr[g][3]);
+            if (CPU >= 2) d += __shfl_xor(d, 1);
+            if (CPU >= 4) d += __shfl_xor(d, 2);
+            const int t = ((r << 6) + lane) / PERIOD;
+            if (pos0 + t < len && d < m) m = d;
+        }
+#pragma unroll
+        for (int st = PERIOD; st < kWave; st <<= 1) {
+            const int o = __shfl_xor(m, st);
+            m = o < m ? o : m;
+        }
+        if (lane < PERIOD && part == 0 && j < a.max_blocks && pos0 < len) {
+            const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
+            const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
+            const int sc = pb[bi] < 0 ? -1 : (forced ? full : full - m);
+            a.scores[((int64_t)b * HKV + h) * a.max_blocks + j] = sc;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Generic block scorer: any strides, code width, head count and group size.  One thread per
 // (token, head) code, word-by-word loads; query codes staged in LDS.
 // ---------------------------------------------------------------------------------------
@@ -1074,6 +1166,43 @@ bool dispatch_small(const ScoreArgs& a, int rpb, int pmax, dim3 grid, hipStream_
     }
 }
 
+template <int CPU, int HKV, int RPB>
+void dispatch_rows_g(const ScoreArgs& a, dim3 grid, hipStream_t st)
+{
+    if (a.G == 1) launch_score(block_score_rows<CPU, HKV, 1, RPB>, grid, 0, st, a);
+    else if (a.G == 2) launch_score(block_score_rows<CPU, HKV, 2, RPB>, grid, 0, st, a);
+    else launch_score(block_score_rows<CPU, HKV, 4, RPB>, grid, 0, st, a);
+}
+
+template <int CPU, int HKV>
+bool dispatch_rows_h(const ScoreArgs& a, int rpb, int B, hipStream_t st)
+{
+    const int nbw = rpb > 4 ? 1 : 4 / rpb;  // blocks per wave
+    const dim3 grid((unsigned)ucm::ceil_div(a.max_blocks, 4 * nbw), (unsigned)B);
+    switch (rpb) {
+        case 1: dispatch_rows_g<CPU, HKV, 1>(a, grid, st); return true;
+        case 2: dispatch_rows_g<CPU, HKV, 2>(a, grid, st); return true;
+        case 4: dispatch_rows_g<CPU, HKV, 4>(a, grid, st); return true;
+        case 8: dispatch_rows_g<CPU, HKV, 8>(a, grid, st); return true;
+        default: return false;
+    }
+}
+
+// Blocks of 1, 2, 4 or 8 KiB, group size 1, 2 or 4, 1 to 16 KV heads; false when no instance exists.
+template <int CPU>
+bool dispatch_rows(const ScoreArgs& a, int rpb, int B, hipStream_t st)
+{
+    if (!(a.G == 1 || a.G == 2 || a.G == 4)) return false;
+    switch (a.Hkv) {
+        case 1: return dispatch_rows_h<CPU, 1>(a, rpb, B, st);
+        case 2: return dispatch_rows_h<CPU, 2>(a, rpb, B, st);
+        case 4: return dispatch_rows_h<CPU, 4>(a, rpb, B, st);
+        case 8: return dispatch_rows_h<CPU, 8>(a, rpb, B, st);
+        case 16: if (CPU <= 4) return dispatch_rows_h<CPU, 16>(a, rpb, B, st); return false;
+        default: return false;
+    }
+}
+
 // true when a block_score_one instance exists for this (pieces per code, KV heads) pair
 template <int CPU>
 bool dispatch_one(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
@@ -1179,7 +1308,13 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
         const int u = rpw;
         // blocks of >= 4 KiB: one block per workgroup with the head count compiled in
         bool done = false;
-        if (split && Hkv <= 16) {
+        // blocks of at most 8 KiB with directly compared query codes: whole blocks per wave
+        if (direct && rpb <= 8) {
+            if (cpu == 1) done = dispatch_rows<1>(a, rpb, B, st);
+            else if (cpu == 2) done = dispatch_rows<2>(a, rpb, B, st);
+            else done = dispatch_rows<4>(a, rpb, B, st);
+        }
+        if (!done && split && Hkv <= 16) {
             a.TB = 1;
             const dim3 grid1((unsigned)max_blocks, (unsigned)B);
             if (cpu == 1) done = dispatch_one<1>(a, pmax, grid1, st);
