@@ -759,6 +759,104 @@ int check_shape(const EncArgs& a, int x_dtype, int w_dtype)
     return UCM_OK;
 }
 
+// LDS-tiled FMA path for what the matrix-core kernels do not take (fp32 inputs, K that is not
+// 64/128/256/512, row layouts they reject): a workgroup computes 64 rows x TN hash columns of
+// one head, K in chunks of 16 staged in LDS (x transposed, k-major), each thread an 8 x 4
+// micro-tile (32 fp32 accumulators, 32 FMAs per three 16-byte LDS reads).  A row's word is
+// assembled from the eight neighbouring lanes that hold its 32 columns.  DT: element type of x
+// and W (both the same).  grid = (ceil(T / 64), N / TN, H).
+template <int DT, int TN>
+__global__ __launch_bounds__(kThreads) void encode_tiled_kernel(EncArgs a)
+{
+    constexpr int TM = 64, KC = 16;
+    __shared__ __align__(16) float xs[KC][TM];
+    __shared__ __align__(16) float wsm[KC][TN];
+    const int h = blockIdx.z;
+    const int n0 = blockIdx.y * TN;
+    const int64_t t0 = (int64_t)blockIdx.x * TM;
+    const int tid = threadIdx.x;
+    constexpr int CG = TN / 4;            // column groups of 4 (threads along N)
+    constexpr int RG = kThreads / CG;     // row groups
+    constexpr int RPT = TM / RG;          // rows per thread
+    const int tx = tid % CG, ty = tid / CG;
+    const int64_t wbase = (int64_t)weight_index(a, h) * a.K * a.N + n0;
+
+    // the row this thread stages (tid / 4) and its four k positions per chunk
+    const int xr = tid >> 2, xk = (tid & 3) * 4;
+    int64_t xt = t0 + xr;
+    if (xt >= a.T) xt = a.T - 1;  // in-bounds read; the row is dropped at the store
+    const int64_t xo = src_offset(a, xt, h);
+
+    float acc[RPT][4];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
+
+    for (int k0 = 0; k0 < a.K; k0 += KC) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = k0 + xk + i;
+            xs[xk + i][xr] = k < a.K ? load_as_float(a.x, DT, xo + k) : 0.0f;
+        }
+#pragma unroll
+        for (int e = tid; e < KC * TN; e += kThreads) {
+            const int kk = e / TN, c = e % TN;
+            wsm[kk][c] = k0 + kk < a.K ? load_as_float(a.w, DT, wbase + (int64_t)(k0 + kk) * a.N + c) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KC; ++kk) {
+            const float4 wv = *reinterpret_cast<const float4*>(&wsm[kk][tx * 4]);
+            float xv[RPT];
+            if constexpr (RPT >= 4) {
+#pragma unroll
+                for (int r4 = 0; r4 < RPT; r4 += 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(&xs[kk][ty * RPT + r4]);
+                    xv[r4] = v.x; xv[r4 + 1] = v.y; xv[r4 + 2] = v.z; xv[r4 + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < RPT; ++r) xv[r] = xs[kk][ty * RPT + r];
+            }
+#pragma unroll
+            for (int r = 0; r < RPT; ++r) {
+                acc[r][0] = __builtin_fmaf(xv[r], wv.x, acc[r][0]);
+                acc[r][1] = __builtin_fmaf(xv[r], wv.y, acc[r][1]);
+                acc[r][2] = __builtin_fmaf(xv[r], wv.z, acc[r][2]);
+                acc[r][3] = __builtin_fmaf(xv[r], wv.w, acc[r][3]);
+            }
+        }
+        __syncthreads();
+    }
+    // eight neighbouring lanes (tx % 8 = 0..7) hold the 32 columns of one word
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+        uint32_t v = (acc[r][0] > 0.0f ? 1u : 0u) | (acc[r][1] > 0.0f ? 2u : 0u) |
+                     (acc[r][2] > 0.0f ? 4u : 0u) | (acc[r][3] > 0.0f ? 8u : 0u);
+        v <<= 4 * (tx & 7);
+        v |= __shfl_xor(v, 1);
+        v |= __shfl_xor(v, 2);
+        v |= __shfl_xor(v, 4);
+        const int64_t t = t0 + ty * RPT + r;
+        if ((tx & 7) == 0 && t < a.T) {
+            uint32_t* dst = row_dst(a, t, h);
+            if (dst) dst[(n0 >> 5) + (tx >> 3)] = v;
+        }
+    }
+}
+
+template <int DT>
+int launch_tiled(const EncArgs& a, hipStream_t st)
+{
+    const int tn = a.N % 128 == 0 ? 128 : (a.N % 64 == 0 ? 64 : 32);
+    const dim3 grid((unsigned)ucm::ceil_div(a.T, 64), (unsigned)(a.N / tn), (unsigned)a.H);
+    if (tn == 128) hipLaunchKernelGGL((encode_tiled_kernel<DT, 128>), grid, dim3(kThreads), 0, st, a);
+    else if (tn == 64) hipLaunchKernelGGL((encode_tiled_kernel<DT, 64>), grid, dim3(kThreads), 0, st, a);
+    else hipLaunchKernelGGL((encode_tiled_kernel<DT, 32>), grid, dim3(kThreads), 0, st, a);
+    return ucm::launch_status("encode_tiled_kernel");
+}
+
 bool small_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 {
     return mfma_eligible(a, x_dtype, w_dtype) && a.K <= 256 && a.T <= kSmallRows;
@@ -781,6 +879,12 @@ int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
     }
     if (mfma_eligible(a, x_dtype, w_dtype))
         return x_dtype == UCM_DT_BF16 ? dispatch_mfma<bf16x8>(a, st) : dispatch_mfma<f16x8>(a, st);
+    // same element type on both sides, enough rows to fill a tile, grid within limits
+    if (x_dtype == w_dtype && a.T >= 16 && a.H <= 65535 && ucm::ceil_div(a.T, 64) <= 0x7fffffff) {
+        if (x_dtype == UCM_DT_F32) return launch_tiled<UCM_DT_F32>(a, st);
+        if (x_dtype == UCM_DT_F16) return launch_tiled<UCM_DT_F16>(a, st);
+        return launch_tiled<UCM_DT_BF16>(a, st);
+    }
     const int64_t total = a.T * a.H * (a.N / 32);
     int64_t blocks = ucm::ceil_div(total, kThreads);
     if (blocks > 65535 * 16) blocks = 65535 * 16;
