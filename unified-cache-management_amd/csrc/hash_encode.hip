@@ -646,7 +646,7 @@ int launch_mfma_q(const EncArgs& a, size_t lds, const dim3& grid, hipStream_t st
         if (big_lds == 0) {
             const hipError_t e =
                 hipFuncSetAttribute((const void*)encode_mfma_kernel<V, KS, NQ, NG>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) (void)hipGetLastError();
             big_lds = (e == hipSuccess) ? 1 : -1;
         }
@@ -661,7 +661,7 @@ int launch_mfma(EncArgs a, hipStream_t st)
 {
     constexpr int K = KS * 16;
     constexpr size_t kStage = (size_t)kMfmaWaves * kStageBytes;
-    for (size_t cap : {(size_t)144 * 1024, (size_t)64 * 1024}) {
+    for (size_t cap : {(size_t)160 * 1024, (size_t)64 * 1024}) {
         a.BN = pick_slice(a.N, K, cap - kStage);
         if (a.BN == 0) return ucm::fail(UCM_EUNSUPPORTED, "no LDS slice fits K=%d", K);
         const size_t lds = (size_t)a.BN * (K + kPad) * 2 + kStage;
