@@ -180,7 +180,13 @@ int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
  * out_is_f16 = 1 writes IEEE half exactly as the reference (inf = 0x7C00);
  * out_is_f16 = 0 writes int32 with infinity = INT32_MAX.
  * reduce_heads = 1 writes the min over KV heads, shape [B, 1, max_seq_len].
+ * workspace   optional device memory of at least ucm_hamming_score_workspace_bytes(...)
+ *             bytes, 16-byte aligned, contents need no initialisation.  It holds the bit
+ *             planes of the query counts, which the kernel for one KV head and more than 8
+ *             query heads (the latent-attention layout) reads; with NULL that case runs on
+ *             the slower general kernel, with the same results.
  */
+size_t ucm_hamming_score_workspace_bytes(int32_t B, int32_t Hq, int32_t Wd);
 int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
                       const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
                       int64_t ks_block, int64_t ks_token, int64_t ks_head,
@@ -189,6 +195,7 @@ int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_str
                       int32_t B, int32_t Hq, int32_t max_seq_len,
                       int32_t sink_tok, int32_t recent_tok, int reduce_heads,
                       void* out, int out_is_f16,
+                      void* workspace, size_t workspace_bytes,
                       ucm_stream_t stream);
 
 /*

@@ -234,6 +234,56 @@ def test_f16_scores_round_like_sequential_half_adds():
     assert np.array_equal(h, expect)
 
 
+def _half_piece_sums(q, kc, table, lens, msl):
+    """The reference's per-token accumulation (paged_ham_dist_mla.cu:235-241) for one KV head and
+    an even code width: per 64-bit piece the integer group-summed popcount is converted to half
+    and added in half precision, piece 0 first."""
+    B = q.shape[0]
+    BS = kc.shape[1]
+    kp = np.ascontiguousarray(kc).view(np.uint64)  # [NB,BS,1,L]
+    qp = np.ascontiguousarray(q).view(np.uint64)   # [B,G,L]
+    cnt = np.array([bin(i).count("1") for i in range(256)], np.int64)
+    out = np.full((B, 1, msl), np.inf, np.float16)
+    for b in range(B):
+        for p in range(min(int(lens[b]), msl)):
+            pb = table[b, p // BS]
+            if pb < 0 or pb >= kp.shape[0]:
+                continue  # unusable entry: infinity
+            x = kp[pb, p % BS, 0][None, :] ^ qp[b]          # [G,L]
+            parts = cnt[x.view(np.uint8).reshape(x.shape[0], x.shape[1], 8)].sum(axis=(0, 2))
+            acc = np.float16(0)
+            for part in parts:
+                acc = np.float16(acc + np.float16(part))
+            out[b, 0, p] = acc
+    return out
+
+
+@pytest.mark.parametrize("G", [1, 2, 4, 5, 8, 16, 128])
+@pytest.mark.parametrize("Wd,BS", [(18, 64), (18, 128), (18, 16), (18, 1), (6, 32), (2, 64), (34, 8), (64, 4)])
+def test_one_kv_head_even_code_widths(G, Wd, BS):
+    """One KV head with codes that are not a whole number of 16-byte pieces per token — the
+    18-word (512 + 64 bit) codes of the reference's latent-attention path
+    (hamming_topk.py: `k_hash.shape[-1] == 18`) and other even widths: block top-k, exact
+    per-token distances and the half-precision output against the checker."""
+    from ucm_amd.sparse import hamming_score
+
+    lens_list = [BS * 7 + BS // 2 + 1, BS * 21, 1, 0]
+    q, kc, table, lens = make_paged_case(400 + G + Wd, 4, G, 1, Wd, BS, lens_list, table_pad=2)
+    check(q, kc, table, lens, 5)
+    check(q, kc, table, lens, 6, sink=BS, recent=2 * BS, distance=True, score_order=True)
+    table[1, 3] = kc.shape[0] + 1  # unusable entry
+    check(q, kc, table, lens, 22, return_physical=True)
+    msl = table.shape[1] * BS - BS // 2
+    args = (dev(as_i32(kc)), dev(as_i32(q))[:, None], dev(table), dev(lens), msl)
+    for sink, recent in ((0, 0), (BS + 1, 3)):
+        o = c_api.hamming_score(q, kc, table, lens, msl, sink, recent, False)
+        g = hamming_score(*args, sink, recent, False, out_int32=True).cpu().numpy()
+        assert np.array_equal(g, o)
+    h = hamming_score(*args, 0, 0, False).cpu().numpy()
+    expect = _half_piece_sums(q, kc, table, lens, msl)
+    assert np.array_equal(h, expect)
+
+
 def test_update_seq_lens():
     from ucm_amd.sparse import update_seq_lens
 

@@ -31,6 +31,7 @@ constexpr int kMaxTileHeads = 1024;  // TB * Hkv bound of the LDS min table
 constexpr int kMaxTile = 64;          // TB bound
 constexpr int kSelLdsCap = 8192;     // block scores kept in LDS by select_kernel
 constexpr int kSelSortCap = 2048;    // largest k for score-ordered output
+constexpr int kMaxPlaneWords = 64;   // widest code the bit-plane kernels take
 
 struct ScoreArgs {
     const uint32_t* q;
@@ -52,6 +53,7 @@ __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ int popc4(u32x4 v)
 {
@@ -94,28 +96,44 @@ __device__ __forceinline__ void write_tile_scores(const ScoreArgs& a, int b, int
 // Bit planes of the per-bit query counts (group size > 4).
 // planes[b][h][p][w] bit i  =  bit p of  #{ g : q[b, h*G+g, w] has bit i set }.
 // ---------------------------------------------------------------------------------------
+// One workgroup per (request, KV head, 64 bits of the code): lane i of every wave owns bit i of
+// the chunk, the four waves split the G query heads between them (all loads of a wave are
+// independent and go out together), the partial counts meet in LDS and wave 0 turns each
+// count bit into one 64-bit ballot, i.e. two plane words.
 __global__ __launch_bounds__(kThreads) void plane_kernel(const uint32_t* __restrict__ q,
                                                          int64_t q_stride_b, int64_t q_stride_h,
                                                          int Hkv, int G, int Wd, int PMAX,
                                                          uint32_t* __restrict__ planes)
 {
-    const int b = blockIdx.x / Hkv, h = blockIdx.x % Hkv;
-    const uint32_t* qb = q + b * q_stride_b + (int64_t)h * G * q_stride_h;
-    uint32_t* out = planes + ((int64_t)b * Hkv + h) * PMAX * Wd;
-    const int nbits = 32 * Wd;
-    for (int i0 = wave_id() * kWave; i0 < nbits; i0 += kThreads) {
-        const int i = i0 + lane_id();
-        int cnt = 0;
-        if (i < nbits) {
-            const int w = i >> 5, sh = i & 31;
-            for (int g = 0; g < G; ++g) cnt += (qb[g * q_stride_h + w] >> sh) & 1u;
-        }
-        for (int p = 0; p < PMAX; ++p) {
-            const unsigned long long m = __ballot((cnt >> p) & 1);
-            const int w0 = i0 >> 5;
-            if (lane_id() == 0 && w0 < Wd) out[p * Wd + w0] = (uint32_t)m;
-            if (lane_id() == 32 && w0 + 1 < Wd) out[p * Wd + w0 + 1] = (uint32_t)(m >> 32);
-        }
+    __shared__ int part[kThreads];
+    const int chunks = (Wd + 1) >> 1;
+    const int chunk = blockIdx.x % chunks, bh = blockIdx.x / chunks;
+    const int b = bh / Hkv, h = bh % Hkv;
+    const int lane = lane_id(), wid = wave_id();
+    const int w = chunk * 2 + (lane >> 5), sh = lane & 31;
+    const bool ok = w < Wd;
+    const uint32_t* qb = q + b * q_stride_b + (int64_t)h * G * q_stride_h + (ok ? w : 0);
+    int cnt = 0;
+    constexpr int kWaves = kThreads / kWave;
+    int g = wid;
+    for (; g + 7 * kWaves < G; g += 8 * kWaves) {
+        uint32_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = qb[(int64_t)(g + u * kWaves) * q_stride_h];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) cnt += (v[u] >> sh) & 1u;
+    }
+    for (; g < G; g += kWaves) cnt += (qb[(int64_t)g * q_stride_h] >> sh) & 1u;
+    part[threadIdx.x] = cnt;
+    __syncthreads();
+    if (wid != 0) return;
+    cnt = part[lane] + part[lane + kWave] + part[lane + 2 * kWave] + part[lane + 3 * kWave];
+    if (!ok) cnt = 0;
+    uint32_t* out = planes + ((int64_t)b * Hkv + h) * PMAX * Wd + chunk * 2;
+    for (int p = 0; p < PMAX; ++p) {
+        const unsigned long long m = __ballot((cnt >> p) & 1);
+        if (lane == 0) out[p * Wd] = (uint32_t)m;
+        if (lane == 32 && ok) out[p * Wd + 1] = (uint32_t)(m >> 32);
     }
 }
 
@@ -619,6 +637,141 @@ __global__ __launch_bounds__(kThreads) void block_score_rows(ScoreArgs a)
 }
 
 // ---------------------------------------------------------------------------------------
+// One KV head and codes of an even number of words that the 16-byte kernels above cannot take
+// — above all the 18-word codes of a latent-attention cache (512 + 64 hash bits), where a
+// 16-byte piece would straddle two tokens.  The unit is the 8-byte piece: L = Wd / 2 consecutive
+// lanes hold one code and a wave covers TP = 64 / L tokens per pass (18 words: 9 lanes, 7
+// tokens, 63 of 64 lanes busy).  Consecutive lanes read consecutive 8 bytes, so a pass is one
+// contiguous run of TP * Wd * 4 bytes, and the query material of a lane (its two words of every
+// query code, or of every bit plane) never changes.
+// ---------------------------------------------------------------------------------------
+template <bool DIRECT, int GP>
+struct PairQuery {
+    uint32_t m[GP][2];
+    int ctot, G;
+
+    // issues the loads of the lane's query material
+    __device__ __forceinline__ void fetch(const ScoreArgs& a, int b, int w0)
+    {
+        G = a.G;
+        if (DIRECT) {
+            const uint32_t* qp = a.q + b * a.q_stride_b + w0;
+#pragma unroll
+            for (int g = 0; g < GP; ++g) {
+                m[g][0] = qp[g * a.q_stride_h];
+                m[g][1] = qp[g * a.q_stride_h + 1];
+            }
+        } else {
+            const uint32_t* pl = a.planes + (int64_t)b * GP * a.Wd + w0;
+#pragma unroll
+            for (int p = 0; p < GP; ++p) {
+                m[p][0] = pl[p * a.Wd];
+                m[p][1] = pl[p * a.Wd + 1];
+            }
+        }
+    }
+
+    // first use of the material: call after the code loads are out
+    __device__ __forceinline__ void finish()
+    {
+        ctot = 0;
+        if (!DIRECT) {
+#pragma unroll
+            for (int p = 0; p < GP; ++p) ctot += (__popc(m[p][0]) + __popc(m[p][1])) << p;
+        }
+    }
+
+    // group-summed distance of one 8-byte piece
+    __device__ __forceinline__ int dist(u32x2 k) const
+    {
+        int d = 0;
+        if (DIRECT) {
+#pragma unroll
+            for (int g = 0; g < GP; ++g) d += __popc(k.x ^ m[g][0]) + __popc(k.y ^ m[g][1]);
+            return d;
+        }
+#pragma unroll
+        for (int p = 0; p < GP; ++p) d += (__popc(k.x & m[p][0]) + __popc(k.y & m[p][1])) << p;
+        return ctot + G * (__popc(k.x) + __popc(k.y)) - 2 * d;
+    }
+};
+
+// Sum of a value over the L lanes of a code, valid in the code's first lane (p = 0): a shuffle
+// tree clipped at the code's end.
+__device__ __forceinline__ int pair_code_sum(int d, int p, int L)
+{
+    for (int o = 1; o < L; o <<= 1) {
+        const int t = __shfl_down(d, o);
+        d += (p + o < L) ? t : 0;
+    }
+    return d;
+}
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kPairPasses = 10;  // passes a wave keeps in flight (64 tokens of 18 words: all)
+
+// Block scores: a wave owns one block, a workgroup four consecutive ones.  The pieces of a code
+// are summed over its L lanes by a shuffle tree clipped at the code's end, the block minimum is
+// taken over the passes in registers and over the wave by shuffles: no LDS, no barrier.
+template <bool DIRECT, int GP>
+__global__ __launch_bounds__(kThreads) void block_score_pairs(ScoreArgs a, int L, int TP)
+{
+    const int b = blockIdx.y;
+    const int lane = lane_id();
+    const int j = blockIdx.x * (kThreads / kWave) + wave_id();
+    const int slot = lane / L, p = lane - slot * L;
+    const bool lane_ok = slot < TP;
+    // the table entry, the length and the query material are independent reads: all are out
+    // before the first of them is waited for
+    const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+    const int entry = a.table ? a.table[(int64_t)b * a.table_stride + jc] : 0;
+    const int len = a.lens[b];
+    PairQuery<DIRECT, GP> qm;
+    qm.fetch(a, b, lane_ok ? 2 * p : 0);
+    const int pos0 = j * a.BS;
+    if (j >= a.max_blocks || pos0 >= len) return;
+    int64_t pb = a.table ? (int64_t)entry : (int64_t)b * a.max_blocks + j;
+    if (pb < 0 || pb >= a.NB) pb = -1;
+
+    const u32x2* base = reinterpret_cast<const u32x2*>(a.kc + (pb < 0 ? 0 : pb) * a.ks_block);
+    const int ntok = (a.BS < len - pos0) ? a.BS : len - pos0;
+    int m = kInf;
+    for (int t0 = 0; t0 < ntok; t0 += kPairPasses * TP) {
+        u32x2 kv[kPairPasses];
+#pragma unroll
+        for (int u = 0; u < kPairPasses; ++u) {
+            if (t0 + u * TP < ntok) {
+                // idle lanes and lanes past the block re-read the pass's first piece
+                const int tok = t0 + u * TP + slot;
+                kv[u] = __builtin_nontemporal_load(
+                    base + ((tok < a.BS && lane_ok) ? tok * L + p : (t0 + u * TP) * L));
+            }
+        }
+        if (t0 == 0) qm.finish();
+#pragma unroll
+        for (int u = 0; u < kPairPasses; ++u) {
+            if (t0 + u * TP < ntok) {
+                int d = qm.dist(kv[u]);
+                d = pair_code_sum(d, p, L);
+                if (lane_ok && p == 0 && t0 + u * TP + slot < ntok && d < m) m = d;
+            }
+        }
+    }
+#pragma unroll
+    for (int st = 1; st < kWave; st <<= 1) {
+        const int o = __shfl_xor(m, st);
+        m = o < m ? o : m;
+    }
+    if (lane == 0) {
+        const int full = a.G * 32 * a.Wd;
+        const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
+        const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
+        a.scores[(int64_t)b * a.max_blocks + j] = pb < 0 ? -1 : (forced ? full : full - m);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Generic block scorer: any strides, code width, head count and group size.  One thread per
 // (token, head) code, word-by-word loads; query codes staged in LDS.
 // ---------------------------------------------------------------------------------------
@@ -1082,8 +1235,8 @@ Workspace carve(void* base, int B, int Hkv, int max_blocks)
     w.reduced = (int32_t*)((char*)base + off);
     off += align_up((size_t)B * max_blocks * 4, 256);
     w.planes = (uint32_t*)((char*)base + off);
-    // worst case: 8 planes, widest code handled by the plane path (16 words)
-    off += align_up((size_t)B * Hkv * 8 * 16 * 4, 256);
+    // worst case: 8 planes, widest code handled by a plane path (kMaxPlaneWords words)
+    off += align_up((size_t)B * Hkv * 8 * kMaxPlaneWords * 4, 256);
     w.bytes = off;
     return w;
 }
@@ -1219,6 +1372,14 @@ bool dispatch_one(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 
 bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
+// Layout the 8-byte-piece kernels take: one KV head, an even code width of at most
+// kMaxPlaneWords words, the tokens of a block back to back, 8-byte aligned blocks.
+bool pairs_layout(const ScoreArgs& a, const uint32_t* k_cache)
+{
+    return a.Hkv == 1 && a.Wd % 2 == 0 && a.Wd <= kMaxPlaneWords && a.ks_token == a.Wd &&
+           a.ks_block % 2 == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 7) == 0;
+}
+
 int common_checks(const uint32_t* q, const uint32_t* kc, const int32_t* lens, int64_t NB, int BS,
                   int Hkv, int Wd, int B, int Hq, int max_blocks)
 {
@@ -1297,7 +1458,7 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
         const int pmax = planes_for_group(a.G);
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
         if (!direct) {
-            hipLaunchKernelGGL(plane_kernel, dim3(B * Hkv), dim3(kThreads), 0, st, q_codes,
+            hipLaunchKernelGGL(plane_kernel, dim3(B * Hkv * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
                                q_stride_b, q_stride_h, Hkv, a.G, Wd, pmax, ws.planes);
             rc = ucm::launch_status("plane_kernel");
             if (rc != UCM_OK) return rc;
@@ -1339,6 +1500,27 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             else if (cpu == 2) dispatch_fast<2>(a, pmax, split, u, grid, st);
             else dispatch_fast<4>(a, pmax, split, u, grid, st);
         }
+    } else if (pairs_layout(a, k_cache)) {
+        const int L = Wd / 2, TP = kWave / L;
+        int pmax = 0;
+        while ((1 << pmax) <= a.G) ++pmax;  // bit planes that hold the counts 0..G
+        if (pmax < 4) pmax = 4;
+        const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
+        if (!direct) {
+            hipLaunchKernelGGL(plane_kernel, dim3(B * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
+                               q_stride_b, q_stride_h, 1, a.G, Wd, pmax, ws.planes);
+            rc = ucm::launch_status("plane_kernel");
+            if (rc != UCM_OK) return rc;
+        }
+        const dim3 pgrid((unsigned)ucm::ceil_div(max_blocks, kThreads / kWave), (unsigned)B);
+        if (a.G == 1) launch_score(block_score_pairs<true, 1>, pgrid, 0, st, a, L, TP);
+        else if (a.G == 2) launch_score(block_score_pairs<true, 2>, pgrid, 0, st, a, L, TP);
+        else if (a.G == 4) launch_score(block_score_pairs<true, 4>, pgrid, 0, st, a, L, TP);
+        else if (pmax == 4) launch_score(block_score_pairs<false, 4>, pgrid, 0, st, a, L, TP);
+        else if (pmax == 5) launch_score(block_score_pairs<false, 5>, pgrid, 0, st, a, L, TP);
+        else if (pmax == 6) launch_score(block_score_pairs<false, 6>, pgrid, 0, st, a, L, TP);
+        else if (pmax == 7) launch_score(block_score_pairs<false, 7>, pgrid, 0, st, a, L, TP);
+        else launch_score(block_score_pairs<false, 8>, pgrid, 0, st, a, L, TP);
     } else {
         launch_score(block_score_generic, grid, (size_t)Hq * Wd * 4, st, a);
     }
@@ -1471,7 +1653,131 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t)
     }
 }
 
+// Per-token scores for the 8-byte-piece layout (one KV head, even code width).  A lane's piece
+// is exactly one step of the reference's half-precision accumulation, so the first lane of a
+// code collects the piece sums of its L lanes in order and adds them as the reference does; any
+// group size is exact (bit planes from the workspace above 8 query heads).  A wave owns one
+// logical block and writes every position of it below max_seq_len.
+template <bool DIRECT, int GP, bool F16>
+__global__ __launch_bounds__(kThreads) void token_score_pairs(TokenArgs t, int L, int TP)
+{
+    const ScoreArgs& a = t.s;
+    const int b = blockIdx.y;
+    const int lane = lane_id();
+    const int j = blockIdx.x * (kThreads / kWave) + wave_id();
+    const int pos0 = j * a.BS;
+    if (pos0 >= t.max_seq_len) return;
+    const int slot = lane / L, p = lane - slot * L;
+    const bool lane_ok = slot < TP;
+    const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+    const int entry = a.table ? a.table[(int64_t)b * a.table_stride + jc] : 0;
+    const int len = a.lens[b];
+    PairQuery<DIRECT, GP> qm;
+    qm.fetch(a, b, lane_ok ? 2 * p : 0);
+    int64_t pb = a.table ? (int64_t)entry : (int64_t)b * a.max_blocks + j;
+    if (j >= a.max_blocks || pb < 0 || pb >= a.NB) pb = -1;
+    const int nout = (a.BS < t.max_seq_len - pos0) ? a.BS : t.max_seq_len - pos0;
+    int ntok = len - pos0;  // tokens whose codes are read
+    ntok = pb < 0 ? 0 : (ntok < 0 ? 0 : (ntok > nout ? nout : ntok));
+
+    const u32x2* base = reinterpret_cast<const u32x2*>(a.kc + (pb < 0 ? 0 : pb) * a.ks_block);
+    const int64_t obase = (int64_t)b * t.max_seq_len + pos0;
+    const bool writer = lane_ok && p == 0;
+    // what a position holds when it has no distance of its own
+    auto fixed = [&](int pos, bool& none, bool& keep) {
+        keep = (pos < a.sink) || (pos >= len - a.recent && pos < len);
+        none = pos >= len || (!keep && pb < 0);
+    };
+    for (int t0 = 0; t0 < nout; t0 += kPairPasses * TP) {
+        u32x2 kv[kPairPasses];
+#pragma unroll
+        for (int u = 0; u < kPairPasses; ++u) {
+            if (t0 + u * TP < ntok) {
+                const int tok = t0 + u * TP + slot;
+                kv[u] = __builtin_nontemporal_load(
+                    base + ((tok < a.BS && lane_ok) ? tok * L + p : (t0 + u * TP) * L));
+            }
+        }
+        if (t0 == 0) qm.finish();
+        if (F16) {
+            // two passes share every shuffle and every (packed) half add: the halves of a
+            // register are the piece sums of token `tok` and of token `tok + TP`
+#pragma unroll
+            for (int u = 0; u < kPairPasses; u += 2) {
+                if (t0 + u * TP >= nout) continue;
+                f16x2 acc = {(_Float16)0.0f, (_Float16)0.0f};
+                if (t0 + u * TP < ntok) {
+                    const int d0 = qm.dist(kv[u]);
+                    const int d1 = (t0 + (u + 1) * TP < ntok) ? qm.dist(kv[u + 1]) : 0;
+                    acc.x = (_Float16)(float)d0;
+                    acc.y = (_Float16)(float)d1;
+                    uint32_t mine;
+                    __builtin_memcpy(&mine, &acc, 4);
+                    for (int o = 1; o < L; ++o) {
+                        const uint32_t x = (uint32_t)__shfl_down((int)mine, o);
+                        f16x2 xv;
+                        __builtin_memcpy(&xv, &x, 4);
+                        acc = acc + xv;
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const int tok = t0 + (u + e) * TP + slot;
+                    if (writer && tok < nout) {
+                        bool none, keep;
+                        fixed(pos0 + tok, none, keep);
+                        const _Float16 d = e ? acc.y : acc.x;
+                        const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : d);
+                        uint16_t bits;
+                        __builtin_memcpy(&bits, &v, 2);
+                        ((uint16_t*)t.out)[obase + tok] = bits;
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kPairPasses; ++u) {
+                if (t0 + u * TP >= nout) continue;
+                int di = 0;
+                if (t0 + u * TP < ntok) di = pair_code_sum(qm.dist(kv[u]), p, L);
+                const int tok = t0 + u * TP + slot;
+                if (writer && tok < nout) {
+                    bool none, keep;
+                    fixed(pos0 + tok, none, keep);
+                    ((int32_t*)t.out)[obase + tok] = none ? kInf : (keep ? 0 : di);
+                }
+            }
+        }
+    }
+}
+
+template <bool DIRECT, int GP>
+void launch_token_pairs(const TokenArgs& t, int L, int TP, dim3 grid, hipStream_t st)
+{
+    if (t.out_is_f16)
+        hipLaunchKernelGGL((token_score_pairs<DIRECT, GP, true>), grid, dim3(kThreads), 0, st, t, L, TP);
+    else
+        hipLaunchKernelGGL((token_score_pairs<DIRECT, GP, false>), grid, dim3(kThreads), 0, st, t, L, TP);
+}
+
+// bit planes that hold the counts 0..G
+int exact_planes(int G)
+{
+    int p = 0;
+    while ((1 << p) <= G) ++p;
+    return p < 4 ? 4 : p;
+}
+
+size_t score_plane_bytes(int B, int Wd) { return align_up((size_t)B * 8 * Wd * 4, 256); }
+
 }  // namespace
+
+extern "C" size_t ucm_hamming_score_workspace_bytes(int32_t B, int32_t Hq, int32_t Wd)
+{
+    (void)Hq;
+    if (B <= 0 || Wd <= 0) return 256;
+    return score_plane_bytes(B, Wd);
+}
 
 extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
                                  const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
@@ -1480,7 +1786,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
                                  int32_t max_blocks, const int32_t* seq_lens, int32_t B,
                                  int32_t Hq, int32_t max_seq_len, int32_t sink_tok,
                                  int32_t recent_tok, int reduce_heads, void* out, int out_is_f16,
-                                 ucm_stream_t stream)
+                                 void* workspace, size_t workspace_bytes, ucm_stream_t stream)
 {
     ucm::clear_error();
     int rc = common_checks(q_codes, k_cache, seq_lens, NB, BS, Hkv, Wd, B, Hq, max_blocks);
@@ -1515,6 +1821,36 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
         else if (G == 4) hipLaunchKernelGGL(token_score_fast<4>, fgrid, dim3(kThreads), lds, st, t);
         else hipLaunchKernelGGL(token_score_fast<8>, fgrid, dim3(kThreads), lds, st, t);
         return ucm::launch_status("token_score_fast");
+    }
+    const bool direct = G == 1 || G == 2 || G == 4 || G == 8;
+    const bool have_planes = workspace && workspace_bytes >= score_plane_bytes(B, Wd) &&
+                             (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
+    if (pairs_layout(a, k_cache) && (direct || have_planes)) {
+        hipStream_t st = (hipStream_t)stream;
+        const int L = Wd / 2, TP = kWave / L;
+        const int nblk = ucm::ceil_div(max_seq_len, BS);
+        const dim3 pgrid((unsigned)ucm::ceil_div(nblk, kThreads / kWave), (unsigned)B);
+        if (direct) {
+            if (G == 1) launch_token_pairs<true, 1>(t, L, TP, pgrid, st);
+            else if (G == 2) launch_token_pairs<true, 2>(t, L, TP, pgrid, st);
+            else if (G == 4) launch_token_pairs<true, 4>(t, L, TP, pgrid, st);
+            else launch_token_pairs<true, 8>(t, L, TP, pgrid, st);
+        } else {
+            const int pmax = exact_planes(G);
+            a.planes = static_cast<uint32_t*>(workspace);
+            hipLaunchKernelGGL(plane_kernel, dim3(B * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
+                               q_stride_b, q_stride_h, 1, G, Wd, pmax, static_cast<uint32_t*>(workspace));
+            rc = ucm::launch_status("plane_kernel");
+            if (rc != UCM_OK) return rc;
+            switch (pmax) {
+                case 4: launch_token_pairs<false, 4>(t, L, TP, pgrid, st); break;
+                case 5: launch_token_pairs<false, 5>(t, L, TP, pgrid, st); break;
+                case 6: launch_token_pairs<false, 6>(t, L, TP, pgrid, st); break;
+                case 7: launch_token_pairs<false, 7>(t, L, TP, pgrid, st); break;
+                default: launch_token_pairs<false, 8>(t, L, TP, pgrid, st); break;
+            }
+        }
+        return ucm::launch_status("token_score_pairs");
     }
     const dim3 grid((unsigned)ucm::ceil_div(max_seq_len, kThreads), (unsigned)B);
     hipLaunchKernelGGL(token_score_kernel, grid, dim3(kThreads), (size_t)Hq * Wd * 4,

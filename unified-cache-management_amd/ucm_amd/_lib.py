@@ -40,7 +40,8 @@ _SIGNATURES = {
                                     vp, i64, i32, i32, i64, i64, i64, vp, i32, i32, vp, i32, i32, i32,
                                     i32, i32, u32, vp, vp, vp, vp, sz, vp]),
     "ucm_hamming_score": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
-                               vp, i32, i32, i32, i32, i32, ci, vp, ci, vp]),
+                               vp, i32, i32, i32, i32, i32, ci, vp, ci, vp, sz, vp]),
+    "ucm_hamming_score_workspace_bytes": (sz, [i32, i32, i32]),
     "ucm_update_seq_lens": (ci, [vp, i32, i32, i32, vp, vp]),
     "ucm_trans_setup": (ci, [i32]),
     "ucm_trans_stream_create": (ci, [ci, C.POINTER(vp)]),

@@ -148,12 +148,14 @@ def hamming_score(key_codes, query_code, block_table, seq_len, max_seq_len, sink
     Ho = 1 if reduce_kvhead else Hkv
     out = torch.empty((B, Ho, int(max_seq_len)),
                       dtype=torch.int32 if out_int32 else torch.float16, device=q.device)
+    ws = torch.empty(_lib.lib().ucm_hamming_score_workspace_bytes(B, Hq, Wd), dtype=torch.uint8,
+                     device=q.device)
     _lib.check(_lib.lib().ucm_hamming_score(
         q.data_ptr(), _lib.stride(q, 0), _lib.stride(q, 1), k.data_ptr(), NB, BS, Hkv, Wd, ks[0], ks[1], ks[2],
         block_table.data_ptr(), max(_lib.stride(block_table, 0), block_table.shape[1]),
         block_table.shape[1], seq_len.data_ptr(),
         B, Hq, int(max_seq_len), int(sink), int(recent), int(bool(reduce_kvhead)), out.data_ptr(),
-        int(not out_int32), _lib.stream_ptr(q.device)))
+        int(not out_int32), ws.data_ptr(), ws.numel(), _lib.stream_ptr(q.device)))
     return out
 
 
