@@ -53,3 +53,27 @@ def assert_topk_matches_unordered_ties(idx, score, ref_idx, ref_score, all_score
         for i, s in zip(idx.tolist(), score.tolist()):
             assert all_scores[i] == s
     del boundary
+
+
+def half_piece_sums(q, kc, table, lens, msl):
+    """The reference's per-token accumulation (paged_ham_dist_mla.cu:235-241) for one KV head and
+    an even code width: per 64-bit piece the integer group-summed popcount is converted to half
+    and added in half precision, piece 0 first."""
+    B = q.shape[0]
+    BS = kc.shape[1]
+    kp = np.ascontiguousarray(kc).view(np.uint64)  # [NB,BS,1,L]
+    qp = np.ascontiguousarray(q).view(np.uint64)   # [B,G,L]
+    cnt = np.array([bin(i).count("1") for i in range(256)], np.int64)
+    out = np.full((B, 1, msl), np.inf, np.float16)
+    for b in range(B):
+        for p in range(min(int(lens[b]), msl)):
+            pb = table[b, p // BS]
+            if pb < 0 or pb >= kp.shape[0]:
+                continue  # unusable entry: infinity
+            x = kp[pb, p % BS, 0][None, :] ^ qp[b]          # [G,L]
+            parts = cnt[x.view(np.uint8).reshape(x.shape[0], x.shape[1], 8)].sum(axis=(0, 2))
+            acc = np.float16(0)
+            for part in parts:
+                acc = np.float16(acc + np.float16(part))
+            out[b, 0, p] = acc
+    return out

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import make_paged_case, random_codes, rng_for
+from helpers import half_piece_sums, make_paged_case, random_codes, rng_for
 from oracle import c_api
 
 pytestmark = pytest.mark.gpu
@@ -234,30 +234,6 @@ def test_f16_scores_round_like_sequential_half_adds():
     assert np.array_equal(h, expect)
 
 
-def _half_piece_sums(q, kc, table, lens, msl):
-    """The reference's per-token accumulation (paged_ham_dist_mla.cu:235-241) for one KV head and
-    an even code width: per 64-bit piece the integer group-summed popcount is converted to half
-    and added in half precision, piece 0 first."""
-    B = q.shape[0]
-    BS = kc.shape[1]
-    kp = np.ascontiguousarray(kc).view(np.uint64)  # [NB,BS,1,L]
-    qp = np.ascontiguousarray(q).view(np.uint64)   # [B,G,L]
-    cnt = np.array([bin(i).count("1") for i in range(256)], np.int64)
-    out = np.full((B, 1, msl), np.inf, np.float16)
-    for b in range(B):
-        for p in range(min(int(lens[b]), msl)):
-            pb = table[b, p // BS]
-            if pb < 0 or pb >= kp.shape[0]:
-                continue  # unusable entry: infinity
-            x = kp[pb, p % BS, 0][None, :] ^ qp[b]          # [G,L]
-            parts = cnt[x.view(np.uint8).reshape(x.shape[0], x.shape[1], 8)].sum(axis=(0, 2))
-            acc = np.float16(0)
-            for part in parts:
-                acc = np.float16(acc + np.float16(part))
-            out[b, 0, p] = acc
-    return out
-
-
 @pytest.mark.parametrize("G", [1, 2, 4, 5, 8, 16, 128])
 @pytest.mark.parametrize("Wd,BS", [(18, 64), (18, 128), (18, 16), (18, 1), (6, 32), (2, 64), (34, 8), (64, 4)])
 def test_one_kv_head_even_code_widths(G, Wd, BS):
@@ -280,7 +256,7 @@ def test_one_kv_head_even_code_widths(G, Wd, BS):
         g = hamming_score(*args, sink, recent, False, out_int32=True).cpu().numpy()
         assert np.array_equal(g, o)
     h = hamming_score(*args, 0, 0, False).cpu().numpy()
-    expect = _half_piece_sums(q, kc, table, lens, msl)
+    expect = half_piece_sums(q, kc, table, lens, msl)
     assert np.array_equal(h, expect)
 
 

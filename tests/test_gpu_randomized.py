@@ -256,3 +256,50 @@ def test_per_token_scores_random_configurations(seed):
             h = hamming_score(*args).cpu().numpy()
             expect = np.where(o == c_api.INF, np.inf, o.astype(np.float64)).astype(np.float16)
             assert np.array_equal(h, expect), what
+
+
+@pytest.mark.parametrize("seed", [61, 62])
+def test_one_kv_head_random_configurations(seed):
+    """One KV head (the latent-attention layout) with even and odd code widths and up to 255 query
+    heads: block top-k, exact per-token distances, and the half-precision output against the
+    reference's piecewise accumulation (paged_ham_dist_mla.cu:235-241)."""
+    from helpers import half_piece_sums
+    from ucm_amd.sparse import hamming_score, hamming_topk
+
+    rng = rng_for(seed)
+    for _ in range(60):
+        B = int(rng.integers(1, 5))
+        G = int(rng.choice([1, 2, 3, 4, 8, 16, 64, 128, 255]))
+        Wd = int(rng.choice([2, 3, 6, 8, 10, 16, 18, 34]))
+        BS = int(rng.choice([1, 4, 16, 64, 128]))
+        mb = int(rng.integers(1, 30))
+        NB = B * mb + 3
+        kc = rng.integers(0, 2**32, size=(NB, BS, 1, Wd), dtype=np.uint32)
+        if rng.integers(0, 4) == 0:
+            kc &= np.uint32(0x00010001)  # low-entropy codes: many equal scores
+        q = rng.integers(0, 2**32, size=(B, G, Wd), dtype=np.uint32)
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32)
+        if rng.integers(0, 4) == 0:
+            table[rng.integers(0, B), rng.integers(0, mb)] = NB + 7  # unusable entry
+        lens = rng.integers(0, mb * BS + 1, size=B).astype(np.int32)
+        if rng.integers(0, 3) == 0:
+            lens[rng.integers(0, B)] = mb * BS
+        k = int(rng.integers(1, mb + 3))
+        sink, recent = int(rng.integers(0, 2 * BS)), int(rng.integers(0, 2 * BS))
+        score_order, distance = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        flags = (c_api.F_SCORE_ORDER if score_order else 0) | (c_api.F_DISTANCE if distance else 0)
+        what = dict(B=B, G=G, Wd=Wd, BS=BS, mb=mb, k=k, sink=sink, recent=recent, flags=flags)
+        dq, dk = torch.from_numpy(q.view(np.int32)).cuda(), torch.from_numpy(kc.view(np.int32)).cuda()
+        dt, dl = torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda()
+        oi, osc = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, flags, max_blocks=mb)
+        gi, gs = hamming_topk(dq, dk, dt, dl, k, sink, recent, score_order=score_order, distance=distance,
+                              max_blocks=mb)
+        assert np.array_equal(gi.cpu().numpy(), oi), what
+        assert np.array_equal(gs.cpu().numpy(), osc), what
+        msl = max(mb * BS - int(rng.integers(0, BS)), 1)
+        o = c_api.hamming_score(q, kc, table, lens, msl, sink, recent, False)
+        g = hamming_score(dk, dq[:, None], dt, dl, msl, sink, recent, False, out_int32=True).cpu().numpy()
+        assert np.array_equal(g, o), what
+        if Wd % 2 == 0:
+            h = hamming_score(dk, dq[:, None], dt, dl, msl, 0, 0, False).cpu().numpy()
+            assert np.array_equal(h, half_piece_sums(q, kc, table, lens, msl)), what

@@ -696,20 +696,29 @@ struct PairQuery {
     }
 };
 
-// Sum of a value over the L lanes of a code, valid in the code's first lane (p = 0): a shuffle
-// tree clipped at the code's end.
-__device__ __forceinline__ int pair_code_sum(int d, int p, int L)
-{
-    for (int o = 1; o < L; o <<= 1) {
-        const int t = __shfl_down(d, o);
-        d += (p + o < L) ? t : 0;
-    }
-    return d;
-}
-
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kPairPasses = 10;  // passes a wave keeps in flight (64 tokens of 18 words: all)
+constexpr int kPairGroup = 5;  // passes whose shuffles are issued together
+
+// Distances of the codes of kPairGroup passes, each summed over its code's lanes (valid in the
+// code's first lane).  The shuffles of one tree step go out for all passes before the first
+// result is used, so their latencies overlap.
+template <class Q>
+__device__ __forceinline__ void pair_group_sums(const Q& qm, const u32x2* kv, int* d, int p, int L)
+{
+#pragma unroll
+    for (int u = 0; u < kPairGroup; ++u) d[u] = qm.dist(kv[u]);
+    for (int o = 1; o < L; o <<= 1) {
+        const int keep = (p + o < L) ? -1 : 0;
+        int t[kPairGroup];
+#pragma unroll
+        for (int u = 0; u < kPairGroup; ++u) t[u] = __shfl_down(d[u], o);
+#pragma unroll
+        for (int u = 0; u < kPairGroup; ++u) d[u] += t[u] & keep;
+    }
+}
+
+constexpr int kPairPasses = 2 * kPairGroup;  // passes a wave keeps in flight (64 tokens of 18 words: all)
 
 // Block scores: a wave owns one block, a workgroup four consecutive ones.  The pieces of a code
 // are summed over its L lanes by a shuffle tree clipped at the code's end, the block minimum is
@@ -746,15 +755,19 @@ __global__ __launch_bounds__(kThreads) void block_score_pairs(ScoreArgs a, int L
                 const int tok = t0 + u * TP + slot;
                 kv[u] = __builtin_nontemporal_load(
                     base + ((tok < a.BS && lane_ok) ? tok * L + p : (t0 + u * TP) * L));
+            } else {
+                kv[u] = u32x2{0u, 0u};
             }
         }
         if (t0 == 0) qm.finish();
 #pragma unroll
-        for (int u = 0; u < kPairPasses; ++u) {
-            if (t0 + u * TP < ntok) {
-                int d = qm.dist(kv[u]);
-                d = pair_code_sum(d, p, L);
-                if (lane_ok && p == 0 && t0 + u * TP + slot < ntok && d < m) m = d;
+        for (int g = 0; g < kPairPasses; g += kPairGroup) {
+            if (t0 + g * TP < ntok) {
+                int d[kPairGroup];
+                pair_group_sums(qm, kv + g, d, p, L);
+#pragma unroll
+                for (int u = 0; u < kPairGroup; ++u)
+                    if (lane_ok && p == 0 && t0 + (g + u) * TP + slot < ntok && d[u] < m) m = d[u];
             }
         }
     }
@@ -1454,7 +1467,10 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     a.TB = TB;
     const dim3 grid((unsigned)ucm::ceil_div(max_blocks, TB), (unsigned)B);
 
-    if (fast) {
+    // one KV head, 16-word codes and bit planes: a wave per block of 8-byte pieces beats a
+    // workgroup per 4 KiB block of 16-byte pieces (37 against 68 us at 16 x 65,536 tokens)
+    const bool direct_g = a.G == 1 || a.G == 2 || a.G == 4;
+    if (fast && !(Hkv == 1 && Wd >= 16 && !direct_g && pairs_layout(a, k_cache))) {
         const int pmax = planes_for_group(a.G);
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
         if (!direct) {
@@ -1696,55 +1712,64 @@ __global__ __launch_bounds__(kThreads) void token_score_pairs(TokenArgs t, int L
                 const int tok = t0 + u * TP + slot;
                 kv[u] = __builtin_nontemporal_load(
                     base + ((tok < a.BS && lane_ok) ? tok * L + p : (t0 + u * TP) * L));
+            } else {
+                kv[u] = u32x2{0u, 0u};
             }
         }
         if (t0 == 0) qm.finish();
         if (F16) {
             // two passes share every shuffle and every (packed) half add: the halves of a
-            // register are the piece sums of token `tok` and of token `tok + TP`
+            // register are the piece sums of token `tok` and of token `tok + TP`; the shuffles of
+            // all pass pairs go out together
+            constexpr int NP = kPairPasses / 2;
+            f16x2 acc[NP];
+            uint32_t mine[NP];
 #pragma unroll
-            for (int u = 0; u < kPairPasses; u += 2) {
-                if (t0 + u * TP >= nout) continue;
-                f16x2 acc = {(_Float16)0.0f, (_Float16)0.0f};
-                if (t0 + u * TP < ntok) {
-                    const int d0 = qm.dist(kv[u]);
-                    const int d1 = (t0 + (u + 1) * TP < ntok) ? qm.dist(kv[u + 1]) : 0;
-                    acc.x = (_Float16)(float)d0;
-                    acc.y = (_Float16)(float)d1;
-                    uint32_t mine;
-                    __builtin_memcpy(&mine, &acc, 4);
-                    for (int o = 1; o < L; ++o) {
-                        const uint32_t x = (uint32_t)__shfl_down((int)mine, o);
+            for (int v = 0; v < NP; ++v) {
+                acc[v].x = (_Float16)(float)qm.dist(kv[2 * v]);
+                acc[v].y = (_Float16)(float)qm.dist(kv[2 * v + 1]);
+                __builtin_memcpy(&mine[v], &acc[v], 4);
+            }
+            if (t0 < ntok) {
+                for (int o = 1; o < L; ++o) {
+                    uint32_t x[NP];
+#pragma unroll
+                    for (int v = 0; v < NP; ++v) x[v] = (uint32_t)__shfl_down((int)mine[v], o);
+#pragma unroll
+                    for (int v = 0; v < NP; ++v) {
                         f16x2 xv;
-                        __builtin_memcpy(&xv, &x, 4);
-                        acc = acc + xv;
+                        __builtin_memcpy(&xv, &x[v], 4);
+                        acc[v] = acc[v] + xv;
                     }
                 }
+            }
 #pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const int tok = t0 + (u + e) * TP + slot;
-                    if (writer && tok < nout) {
-                        bool none, keep;
-                        fixed(pos0 + tok, none, keep);
-                        const _Float16 d = e ? acc.y : acc.x;
-                        const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : d);
-                        uint16_t bits;
-                        __builtin_memcpy(&bits, &v, 2);
-                        ((uint16_t*)t.out)[obase + tok] = bits;
-                    }
+            for (int u = 0; u < kPairPasses; ++u) {
+                const int tok = t0 + u * TP + slot;
+                if (t0 + u * TP < nout && writer && tok < nout) {
+                    bool none, keep;
+                    fixed(pos0 + tok, none, keep);
+                    const _Float16 d = (u & 1) ? acc[u >> 1].y : acc[u >> 1].x;
+                    const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : d);
+                    uint16_t bits;
+                    __builtin_memcpy(&bits, &v, 2);
+                    ((uint16_t*)t.out)[obase + tok] = bits;
                 }
             }
         } else {
 #pragma unroll
-            for (int u = 0; u < kPairPasses; ++u) {
-                if (t0 + u * TP >= nout) continue;
-                int di = 0;
-                if (t0 + u * TP < ntok) di = pair_code_sum(qm.dist(kv[u]), p, L);
-                const int tok = t0 + u * TP + slot;
-                if (writer && tok < nout) {
-                    bool none, keep;
-                    fixed(pos0 + tok, none, keep);
-                    ((int32_t*)t.out)[obase + tok] = none ? kInf : (keep ? 0 : di);
+            for (int g = 0; g < kPairPasses; g += kPairGroup) {
+                if (t0 + g * TP >= nout) continue;
+                int d[kPairGroup];
+                pair_group_sums(qm, kv + g, d, p, L);
+#pragma unroll
+                for (int u = 0; u < kPairGroup; ++u) {
+                    const int tok = t0 + (g + u) * TP + slot;
+                    if (writer && tok < nout) {
+                        bool none, keep;
+                        fixed(pos0 + tok, none, keep);
+                        ((int32_t*)t.out)[obase + tok] = none ? kInf : (keep ? 0 : d[u]);
+                    }
                 }
             }
         }
