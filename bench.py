@@ -354,6 +354,18 @@ def extras(torch, enc_k, gen):
     out["config5_mla_topk128"] = {"tokens": b5 * ctx5, "ms": ms, "tokens_per_s": b5 * ctx5 / ms * 1e3,
                                   "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6}
     del cache5, table5
+    # the reference's own latent-attention setting: 18-word codes (512 nope + 64 rope bits), 64 query
+    # heads after its head reduction (128 heads, reduction 2), same 16 x 65536 tokens
+    wd6 = 18
+    cache6 = codes((b5 * ctx5 // bs5, bs5, 1, wd6))
+    table6 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
+    q6 = codes((b5, 64, wd6))
+    ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6, table6, lens5, 128))
+    ms_tok = graph_ms(torch, lambda i: hamming_score(cache6, q6, table6, lens5, ctx5, 0, 0, False), reps=5)
+    out["mla_576bit_64heads"] = {"tokens": b5 * ctx5, "topk128_ms": ms, "token_scores_ms": ms_tok,
+                                 "tokens_per_s": b5 * ctx5 / ms * 1e3,
+                                 "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6}
+    del cache6, table6
     # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
     cache2 = codes((NB, BS, HKV, WD))
     table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, NBLK)
