@@ -155,6 +155,73 @@ def test_plugin_rehashes_a_prefix_cache_hit_from_the_key_cache():
     assert torch.equal(plugin.prefix_slot_mapping[: 8 * BS], allslots[: 8 * BS])
 
 
+def test_plugin_latent_attention_mode():
+    """MLA: nope (512) and rope (64) parts hashed by two encoders into 18-word codes
+    (gsa_on_device.py:210-232,426-455), decode query heads averaged down by
+    reduction_head_num and compared as 8 query codes against the one latent head (:667-709)."""
+    from ucm_amd.sparse.base import UcmSparseFactory, UcmSparseRole
+
+    B, Hq, BS, nblk, topk_tok, red = 3, 16, 64, 20, 512, 2
+    cfg = {"ucm_sparse_config": {"GSAOnDevice": {
+        "num_q_heads": Hq, "num_kv_heads": 1, "head_dim": 576, "block_size": BS, "is_mla": True,
+        "kv_lora_rank": 512, "qk_rope_head_dim": 64, "vllm_hash_attention_reduction_head_num": red,
+        "vllm_hash_attention_topk": topk_tok, "seed": 9}}}
+    plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+    rng = rng_for(79)
+    NB = B * nblk + 2
+    name = "model.layers.1.self_attn.attn"
+    k_hash = torch.zeros((NB, BS, 36), dtype=torch.bfloat16, device="cuda")  # 72 bytes per token
+    kv_cache = torch.from_numpy(rng.standard_normal((NB, BS, 576)).astype(np.float32)).to(torch.bfloat16).cuda()
+    table = torch.from_numpy(rng.permutation(NB)[: B * nblk].astype(np.int32).reshape(B, nblk)).cuda()
+    lens = torch.tensor([nblk * BS, nblk * BS - 100, 9 * BS + 1], dtype=torch.int32, device="cuda")
+    # request 0 and 2: prefill through the hook; request 1: first 6 blocks are a prefix-cache hit
+    for b in range(B):
+        L = int(lens[b])
+        first = 6 * BS if b == 1 else 0
+        pos = torch.arange(first, L, device="cuda")
+        slots = table[b, pos // BS].long() * BS + pos % BS
+        lat = kv_cache.view(NB * BS, 576)[slots]
+        plugin.set_prefix_cache_hits([(table[b], L, L - first)] if first else [])
+        meta = types.SimpleNamespace(slot_mapping=slots)
+        layer = types.SimpleNamespace(kv_cache=[kv_cache])
+        ctx = types.SimpleNamespace(attn_metadata={name: meta}, no_compile_layers={name: layer}, virtual_engine=0)
+        plugin.attention_begin(None, lat[:, :512].contiguous(), lat[:, 512:].contiguous(), name, ctx,
+                               phase="prefill", k_hash=k_hash)
+    plugin.set_prefix_cache_hits([])
+    # every cached token's code = nope code followed by rope code of its latent vector
+    codes = k_hash.view(torch.uint8).view(NB * BS, 72)
+    flat = kv_cache.view(NB * BS, 576)
+    for b in range(B):
+        pos = torch.arange(int(lens[b]), device="cuda")
+        slots = table[b, pos // BS].long() * BS + pos % BS
+        cn, cr = plugin.hash_code(nope=flat[slots, :512].contiguous(), rope=flat[slots, 512:].contiguous())
+        assert torch.equal(codes[slots], torch.cat([cn, cr], dim=-1))
+    # decode
+    ql = torch.from_numpy(rng.standard_normal((B, Hq, 512)).astype(np.float32)).to(torch.bfloat16).cuda()
+    qp = torch.from_numpy(rng.standard_normal((B, Hq, 64)).astype(np.float32)).to(torch.bfloat16).cuda()
+    pos = lens.long() - 1
+    slots = table[torch.arange(B), pos // BS].long() * BS + pos % BS
+    lat = flat[slots]
+    dec = types.SimpleNamespace(block_table=table.clone(), seq_lens=lens.clone())
+    meta = types.SimpleNamespace(slot_mapping=slots, decode=dec)
+    ctx = types.SimpleNamespace(attn_metadata={name: meta})
+    plugin.attention_begin(None, lat[:, :512].contiguous(), lat[:, 512:].contiguous(), name, ctx,
+                           phase="decode", k_hash=k_hash, decode_ql_nope=ql, decode_q_pe=qp)
+    kblk = topk_tok // BS
+    qn, qr = plugin.hash_code(nope=ql, rope=qp, reduction_head_num=red)
+    qc = torch.cat([qn, qr], dim=-1).cpu().numpy().view(np.uint32)          # [B, Hq/red, 18]
+    assert qc.shape == (B, Hq // red, 18)
+    kc = k_hash.view(torch.uint8).cpu().numpy().view(np.uint32).reshape(NB, BS, 1, 18)
+    oi, _ = c_api.hamming_topk(qc, kc, table.cpu().numpy(), lens.cpu().numpy(), kblk, BS, 4 * BS,
+                               flags=c_api.F_REDUCE_HEADS | c_api.F_PHYSICAL)
+    got = dec.block_table.cpu().numpy()
+    assert np.array_equal(got[:, :kblk], np.maximum(oi[:, 0], 0))
+    assert not got[:, kblk:].any()
+    assert np.array_equal(dec.seq_lens.cpu().numpy(), c_api.update_seq_lens(lens.cpu().numpy(), topk_tok, BS))
+    plugin.attention_finished(None, None, None, None, name, ctx, phase="decode")
+    assert torch.equal(dec.block_table, table) and torch.equal(dec.seq_lens, lens)
+
+
 def test_host_memory_store_dump_lookup_load_roundtrip():
     """The store contract of the reference's e2e test (ucm/store/test/e2e/cache_on_empty_test.py:
     46-79): dump -> lookup -> load -> bit-exact."""

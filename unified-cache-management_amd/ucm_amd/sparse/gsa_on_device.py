@@ -1,4 +1,4 @@
-"""GSAOnDevice-shaped driver of the MI355X operators (GQA decode path).
+"""GSAOnDevice-shaped driver of the MI355X operators (GQA and latent-attention decode paths).
 
 A thin counterpart of the reference plugin's worker-side hot path
 (ucm/sparse/gsa_on_device/gsa_on_device.py): `attention_begin` stores the hash codes of the
@@ -8,15 +8,21 @@ and seq_lens with the top-k blocks (update_decode_topk_gqa_cuda, :773-811);
 layer's `attn_metadata` needs `slot_mapping`, `block_table` and `seq_lens` attributes.
 After a prefix-cache hit (`set_prefix_cache_hits`, the bookkeeping of build_sparse_meta,
 :1322-1366) the keys that were loaded into the paged KV cache are re-encoded in place
-(cache_k_hash_gqa_cuda's `has_pc_hit` branch, :574-588).  The scheduler-side hooks, MLA
-metadata surgery and layer-skip profiling of the reference are outside this build.
+(cache_k_hash_gqa_cuda's `has_pc_hit` branch, :574-588).  With `is_mla` the keys are the latent
+vector (nope, kv_lora_rank values) and the rope part (qk_rope_head_dim values) of one KV head:
+two encoders write their codes side by side into 18-word cache rows (cache_k_hash_mla_cuda,
+:426-455 — the fused encode-and-store takes the place of hash + vLLM's concat_and_cache_mla),
+and the decode query codes of the, optionally head-reduced, q_nope / q_pe are compared against
+them (update_decode_topk_mla_cuda, :667-709).  The scheduler-side hooks, the FlashMLA tile
+metadata swap and layer-skip profiling of the reference are outside this build.
 
 Configuration (`ucm_sparse_config["GSAOnDevice"]`), names from
 gsa_on_device_config.py:36-98 where they exist:
     num_q_heads, num_kv_heads, head_dim, block_size, hash_bits (default head_dim),
     vllm_hash_attention_topk (tokens kept), sink_tokens (default block_size),
     recent_tokens (default 4 * block_size), vllm_hash_attention_rollback_layers,
-    gpu_seq_len_threshold, dtype ("bfloat16"|"float16"|"float32"), device, seed
+    gpu_seq_len_threshold, dtype ("bfloat16"|"float16"|"float32"), device, seed;
+    is_mla, kv_lora_rank (512), qk_rope_head_dim (64), vllm_hash_attention_reduction_head_num
 """
 from typing import List, Optional, Union
 
@@ -54,9 +60,20 @@ class GSAOnDevice(UcmSparseBase):
         self.dtype = _DTYPES[cfg.get("dtype", "bfloat16")]
         if "seed" in cfg:
             torch.manual_seed(int(cfg["seed"]))
-        self.is_mla = False
+        self.is_mla = bool(cfg.get("is_mla", False))
         self.gsa_enabled = True
-        self.hash_encoder = HashEncoder(self.head_dim, self.hash_bits, self.dtype, self.device)
+        if self.is_mla:
+            # gsa_on_device.py:210-232: one encoder per part, as many bits as dimensions
+            self.hash_reduction_head_num = cfg.get("vllm_hash_attention_reduction_head_num") or 1
+            self.kv_lora_rank = int(cfg.get("kv_lora_rank", 512))
+            self.qk_rope_head_dim = int(cfg.get("qk_rope_head_dim", 64))
+            self.hash_encoder_nope = HashEncoder(self.kv_lora_rank, self.kv_lora_rank, self.dtype,
+                                                 self.device)
+            self.hash_encoder_rope = HashEncoder(self.qk_rope_head_dim, self.qk_rope_head_dim,
+                                                 self.dtype, self.device)
+            self.hash_encoder = None
+        else:
+            self.hash_encoder = HashEncoder(self.head_dim, self.hash_bits, self.dtype, self.device)
         self._saved = {}
         self.has_pc_hit = False
         self.prefix_block_ids = None      # int32 [sum of prefix blocks], all hit requests
@@ -72,8 +89,23 @@ class GSAOnDevice(UcmSparseBase):
         layer_id = int(layer_name.split(".")[2])
         return layer_id in self.hash_rollback_layers, False
 
-    def hash_code(self, query: torch.Tensor) -> torch.Tensor:
-        """Group-mean query -> one code per KV head (gsa_on_device.py:396-412)."""
+    def hash_code(self, query: Optional[torch.Tensor] = None, nope: Optional[torch.Tensor] = None,
+                  rope: Optional[torch.Tensor] = None, reduction_head_num: int = 1):
+        """GQA: group-mean query -> one code per KV head (gsa_on_device.py:396-412).
+        MLA: (nope codes, rope codes) of [T, H, D] or [T, D] inputs; with reduction_head_num > 1
+        the H heads are first averaged down to H / reduction_head_num (:376-393)."""
+        if self.is_mla:
+            if nope is None or rope is None:
+                raise ValueError("MLA mode requires `nope` and `rope`.")
+            if reduction_head_num > 1:
+                nope = nope.view(nope.shape[0], reduction_head_num, nope.shape[1] // reduction_head_num,
+                                 nope.shape[2]).mean(dim=1)
+                rope = rope.view(rope.shape[0], reduction_head_num, rope.shape[1] // reduction_head_num,
+                                 rope.shape[2]).mean(dim=1)
+            return (self.hash_encoder_nope.compute_hash(nope),
+                    self.hash_encoder_rope.compute_hash(rope))
+        if query is None:
+            raise ValueError("GQA mode requires `query`.")
         if self.num_q_heads > self.num_key_heads:
             query = query.view(query.shape[0], self.num_key_heads,
                                self.num_q_heads // self.num_key_heads, query.shape[2]).mean(2)
@@ -132,6 +164,58 @@ class GSAOnDevice(UcmSparseBase):
                     k_cache, self.prefix_block_ids[first:first + n_blk], n_tok, k_hash,
                     block_size=self.block_size)
 
+    def _mla_code_views(self, k_hash):
+        """The nope and rope byte ranges of a latent code cache [NB, BS, code] (any element type
+        whose rows are (kv_lora_rank + qk_rope_head_dim) / 8 bytes) as rank-4 uint8 views."""
+        u8 = k_hash if k_hash.dtype == torch.uint8 else k_hash.view(torch.uint8)
+        if u8.ndim == 3:
+            u8 = u8.unsqueeze(2)
+        nb, rb = self.kv_lora_rank // 8, self.qk_rope_head_dim // 8
+        if u8.ndim != 4 or u8.shape[2] != 1 or u8.shape[3] != nb + rb:
+            raise ValueError(f"latent code cache must be [NB, BS, {nb + rb} bytes], got {tuple(k_hash.shape)}")
+        return u8[..., :nb], u8[..., nb:]
+
+    def cache_k_hash_mla(self, nope, rope, k_hash, attn_metadata, kv_cache=None):
+        """Encode the step's latent keys and store the 18-word codes by slot
+        (cache_k_hash_mla_cuda, gsa_on_device.py:426-455)."""
+        slots = attn_metadata.slot_mapping.flatten()
+        n = slots.numel()
+        c_nope, c_rope = self._mla_code_views(k_hash)
+        self.hash_encoder_nope.compute_hash_and_cache(
+            nope[:n].reshape(n, 1, self.kv_lora_rank), slots, c_nope, block_size=self.block_size)
+        self.hash_encoder_rope.compute_hash_and_cache(
+            rope[:n].reshape(n, 1, self.qk_rope_head_dim), slots, c_rope, block_size=self.block_size)
+        if self.has_pc_hit:
+            # kv_cache [NB, BS, kv_lora_rank + qk_rope_head_dim]: both parts are read in place
+            if kv_cache is None:
+                raise ValueError("a prefix-cache hit needs the layer's latent cache")
+            kc = kv_cache if kv_cache.ndim == 4 else kv_cache.unsqueeze(2)
+            k_nope, k_rope = kc[..., :self.kv_lora_rank], kc[..., self.kv_lora_rank:]
+            for first, n_blk, n_tok in self._prefix_segments:
+                ids = self.prefix_block_ids[first:first + n_blk]
+                self.hash_encoder_nope.compute_hash_from_paged_cache(k_nope, ids, n_tok, c_nope,
+                                                                     block_size=self.block_size)
+                self.hash_encoder_rope.compute_hash_from_paged_cache(k_rope, ids, n_tok, c_rope,
+                                                                     block_size=self.block_size)
+
+    def update_decode_topk_mla(self, layer_name, attn_metadata, decode_ql_nope, decode_q_pe, k_hash):
+        """Top-k block table of a latent-attention decode step
+        (update_decode_topk_mla_cuda, gsa_on_device.py:667-709)."""
+        q_nope_hash, q_rope_hash = self.hash_code(nope=decode_ql_nope, rope=decode_q_pe,
+                                                  reduction_head_num=self.hash_reduction_head_num)
+        q_hash = torch.cat([q_nope_hash, q_rope_hash], dim=-1)
+        u8 = k_hash if k_hash.dtype == torch.uint8 else k_hash.view(torch.uint8)
+        meta = getattr(attn_metadata, "decode", attn_metadata)
+        topk_table = cuda_hamming_topk(
+            q_hash.unsqueeze(1), u8.unsqueeze(2) if u8.ndim == 3 else u8, meta.block_table,
+            meta.seq_lens, topk_token=self.hash_topk_tokens, sink_token=self.block_size,
+            recent_token=self.block_size * 4, is_mla=True)
+        self._saved[layer_name] = (meta.block_table, meta.seq_lens)
+        new_table = torch.zeros_like(meta.block_table)
+        new_table[:, :topk_table.shape[1]] = topk_table
+        meta.block_table = new_table
+        meta.seq_lens = update_seq_lens(meta.seq_lens, self.hash_topk_tokens, self.block_size)
+
     # ---- hooks ----
     def attention_begin(self, query, key, value, layer_name: str, forward_context, output=None,
                         phase: Optional[str] = None, k_hash=None, decode_ql_nope=None,
@@ -139,6 +223,18 @@ class GSAOnDevice(UcmSparseBase):
         if not self.gsa_enabled or k_hash is None:
             return query, key, value, output
         attn_metadata = self.get_layer_attn_metadata(forward_context, layer_name)
+        if self.is_mla:
+            # key / value carry the latent vector and its rope part (gsa_on_device.py:872-880)
+            kv_cache = None
+            if self.has_pc_hit:
+                attn = forward_context.no_compile_layers[layer_name]
+                kv_cache = attn.kv_cache[forward_context.virtual_engine]
+            self.cache_k_hash_mla(key, value, k_hash, attn_metadata, kv_cache)
+            is_rollback_layer, _ = self.get_layer_state(layer_name)
+            if phase == "decode" and not is_rollback_layer:
+                self.update_decode_topk_mla(layer_name, attn_metadata, decode_ql_nope, decode_q_pe,
+                                            k_hash)
+            return query, key, value, output
         k_cache = None
         if self.has_pc_hit:
             # kv_cache[0] is the key cache [NB, BS, Hkv, D] (gsa_on_device.py:576-579)
@@ -172,6 +268,8 @@ class GSAOnDevice(UcmSparseBase):
         saved = self._saved.pop(layer_name, None)
         if saved is not None:
             attn_metadata = self.get_layer_attn_metadata(forward_context, layer_name)
+            if self.is_mla:
+                attn_metadata = getattr(attn_metadata, "decode", attn_metadata)
             attn_metadata.block_table, attn_metadata.seq_lens = saved
 
     def request_begin(self, request_id: Union[int, str], prompt_token_ids: List[int]):
