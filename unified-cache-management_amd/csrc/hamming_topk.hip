@@ -785,6 +785,154 @@ __global__ __launch_bounds__(kThreads) void block_score_pairs(ScoreArgs a, int L
 }
 
 // ---------------------------------------------------------------------------------------
+// Token-per-lane kernels for the latent-attention layout (one KV head, WD = 2 * LC words per
+// code, token-major, 16-byte aligned blocks) at block sizes that are multiples of 64 tokens.
+// A wave owns one block and walks it in rounds of 64 tokens: the round's 64 * WD * 4 contiguous
+// bytes are fetched with 16-byte loads (the next round's loads are issued before the current
+// round is computed), written to a wave-private LDS strip as they lie, and read back one whole
+// code per lane (8-byte reads at a stride of WD words: every bank is hit once per 16 lanes).
+// With a complete code in the lane there is no cross-lane sum, no idle lane and one popcount
+// accumulator per bit plane for the whole code, which halves the integer work of the
+// piece-per-lane kernels; the bit planes are the same for all lanes and are read from LDS as
+// broadcasts (padded to 8 words per code word).
+// ---------------------------------------------------------------------------------------
+template <int LC, bool DIRECT, int GP>
+struct LaneCode {
+    static constexpr int WD = 2 * LC;
+    static constexpr int kRoundWords = 64 * WD;
+    static constexpr int kVec = kRoundWords / 4;     // 16-byte pieces per round
+    static constexpr int kLoads = (kVec + 63) / 64;  // loads per lane and round
+
+    // Planes of request b into LDS as pl[word][8] and the per-piece constants
+    // ctot[piece] = sum over the piece's two words and all planes of popc(plane word) << plane.
+    // Every thread of the workgroup calls this; the caller synchronises afterwards.
+    static __device__ __forceinline__ void stage_planes(const ScoreArgs& a, int b, uint32_t* pl, int* ctot)
+    {
+        if (DIRECT) return;
+        const uint32_t* src = a.planes + (int64_t)b * GP * WD;
+        for (int i = threadIdx.x; i < GP * WD; i += kThreads) {
+            const int p = i / WD, w = i - p * WD;
+            pl[w * 8 + p] = src[i];
+        }
+        if ((int)threadIdx.x >= kThreads - LC) {  // the last LC threads: one piece each
+            const int piece = kThreads - 1 - threadIdx.x;
+            int c = 0;
+#pragma unroll
+            for (int p = 0; p < GP; ++p)
+                c += (__popc(src[p * WD + 2 * piece]) + __popc(src[p * WD + 2 * piece + 1])) << p;
+            ctot[piece] = c;
+        }
+    }
+
+    static __device__ __forceinline__ void load_round(const u32x4* src, int round, int lane, u32x4 (&v)[kLoads])
+    {
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int i = u * 64 + lane;
+            // lanes past the round's end re-read the load's first piece
+            v[u] = __builtin_nontemporal_load(src + round * kVec + (i < kVec ? i : u * 64));
+        }
+    }
+
+    static __device__ __forceinline__ void store_round(u32x4* strip, int lane, const u32x4 (&v)[kLoads])
+    {
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int i = u * 64 + lane;
+            if (i < kVec) strip[i] = v[u];
+        }
+    }
+};
+
+template <int LC, bool DIRECT, int GP>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void block_score_lanes(ScoreArgs a)
+{
+    using LCd = LaneCode<LC, DIRECT, GP>;
+    constexpr int WD = LCd::WD;
+    __shared__ __align__(16) uint32_t strip[kThreads / kWave][LCd::kRoundWords];
+    __shared__ __align__(16) uint32_t pl[DIRECT ? 8 : WD * 8];
+    __shared__ int ctot[LC];
+    const int b = blockIdx.y;
+    const int lane = lane_id(), wid = wave_id();
+    const int j = blockIdx.x * (kThreads / kWave) + wid;
+    const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+    const int entry = a.table ? a.table[(int64_t)b * a.table_stride + jc] : 0;
+    const int len = a.lens[b];
+    LCd::stage_planes(a, b, pl, ctot);
+    if (!DIRECT) __syncthreads();
+    const int pos0 = j * a.BS;
+    if (j >= a.max_blocks || pos0 >= len) return;
+    int64_t pb = a.table ? (int64_t)entry : (int64_t)b * a.max_blocks + j;
+    if (pb < 0 || pb >= a.NB) pb = -1;
+    const int ntok = (a.BS < len - pos0) ? a.BS : len - pos0;
+    const int rounds = (ntok + 63) >> 6;
+    const u32x4* src = reinterpret_cast<const u32x4*>(a.kc + (pb < 0 ? 0 : pb) * a.ks_block);
+    u32x4* mine = reinterpret_cast<u32x4*>(strip[wid]);
+    const uint32_t* row = strip[wid] + lane * WD;
+
+    u32x4 cur[LCd::kLoads], nxt[LCd::kLoads];
+    LCd::load_round(src, 0, lane, cur);
+#pragma unroll
+    for (int u = 0; u < LCd::kLoads; ++u) nxt[u] = cur[u];
+    // wave-uniform query words (scalar registers) when the codes are compared directly
+    const uint32_t* qp = a.q + b * a.q_stride_b;
+    int base = 0;
+    if (!DIRECT) {
+#pragma unroll
+        for (int i = 0; i < LC; ++i) base += ctot[i];
+    }
+    int m = kInf;
+    for (int r = 0; r < rounds; ++r) {
+        if (r + 1 < rounds) LCd::load_round(src, r + 1, lane, nxt);
+        LCd::store_round(mine, lane, cur);
+        // the planes are re-read from LDS every round: kept in registers across rounds they
+        // would cost the kernel half of its resident waves
+        asm volatile("" ::: "memory");
+        int d = 0;
+        if (DIRECT) {
+#pragma unroll
+            for (int i = 0; i < LC; ++i) {
+                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
+#pragma unroll
+                for (int g = 0; g < GP; ++g)
+                    d += __popc(k.x ^ qp[g * a.q_stride_h + 2 * i]) +
+                         __popc(k.y ^ qp[g * a.q_stride_h + 2 * i + 1]);
+            }
+        } else {
+            int acc[GP], pk = 0;
+#pragma unroll
+            for (int p = 0; p < GP; ++p) acc[p] = 0;
+#pragma unroll
+            for (int i = 0; i < LC; ++i) {
+                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
+                pk += __popc(k.x) + __popc(k.y);
+#pragma unroll
+                for (int p = 0; p < GP; ++p)
+                    acc[p] += __popc(k.x & pl[(2 * i) * 8 + p]) + __popc(k.y & pl[(2 * i + 1) * 8 + p]);
+            }
+            int x = 0;
+#pragma unroll
+            for (int p = 0; p < GP; ++p) x += acc[p] << p;
+            d = base + a.G * pk - 2 * x;
+        }
+        if (r * 64 + lane < ntok && d < m) m = d;
+#pragma unroll
+        for (int u = 0; u < LCd::kLoads; ++u) cur[u] = nxt[u];
+    }
+#pragma unroll
+    for (int st = 1; st < kWave; st <<= 1) {
+        const int o = __shfl_xor(m, st);
+        m = o < m ? o : m;
+    }
+    if (lane == 0) {
+        const int full = a.G * 32 * a.Wd;
+        const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
+        const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
+        a.scores[(int64_t)b * a.max_blocks + j] = pb < 0 ? -1 : (forced ? full : full - m);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Generic block scorer: any strides, code width, head count and group size.  One thread per
 // (token, head) code, word-by-word loads; query codes staged in LDS.
 // ---------------------------------------------------------------------------------------
@@ -1054,6 +1202,21 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
             raw[e] = r0[j < a.max_blocks ? j : 0];
         }
     }
+    // physical block ids of the whole row, fetched alongside the scores: the output loop then
+    // has no load (and no round trip to memory) per selected element
+    const bool physical = (a.flags & UCM_TOPK_RETURN_PHYSICAL) != 0;
+    int tab[EL];
+    if (physical && a.table) {
+        const int32_t* t0 = a.table + (int64_t)b * a.table_stride;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int j = lane * EL + e;
+            tab[e] = t0[j < a.max_blocks ? j : 0];
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < EL; ++e) tab[e] = physical ? b * a.max_blocks + lane * EL + e : lane * EL + e;
+    }
     const int len = a.lens[b];
     int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
     if (n > a.max_blocks) n = a.max_blocks;
@@ -1088,7 +1251,22 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
         for (int e = 0; e < EL; ++e) c += __popcll(__ballot(v[e] >= t));
         return c;
     };
-    int lo = -1, hi = a.full;  // count_ge(lo) >= kk always holds
+    // the search runs between the row's smallest and largest score (count_ge(lo) >= kk always
+    // holds: every one of the n >= kk real scores is >= the smallest)
+    int lo = 0x7fffffff, hi = -0x7fffffff;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        if (lane * EL + e < n) lo = v[e] < lo ? v[e] : lo;
+        hi = v[e] > hi ? v[e] : hi;
+    }
+#pragma unroll
+    for (int st = 1; st < kWave; st <<= 1) {
+        const int l2 = __shfl_xor(lo, st), h2 = __shfl_xor(hi, st);
+        lo = l2 < lo ? l2 : lo;
+        hi = h2 > hi ? h2 : hi;
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    hi = __builtin_amdgcn_readfirstlane(hi);
     while (lo < hi) {
         const int mid = lo + ((hi - lo + 1) >> 1);
         if (count_ge(mid) >= kk) lo = mid;
@@ -1116,10 +1294,7 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
             ++eq_seen;
         }
         if (take && pos < a.k) {
-            const int j = lane * EL + e;
-            oi[pos] = (a.flags & UCM_TOPK_RETURN_PHYSICAL)
-                          ? (a.table ? a.table[(int64_t)b * a.table_stride + j] : b * a.max_blocks + j)
-                          : j;
+            oi[pos] = tab[e];
             if (os) os[pos] = (a.flags & UCM_TOPK_DISTANCE) ? a.full - v[e] : v[e];
             ++pos;
         }
@@ -1385,6 +1560,29 @@ bool dispatch_one(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 
 bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
+// Layout and shapes the code-per-lane kernels take (on top of pairs_layout): 18-word codes
+// with any group size, 8- and 16-word codes with bit planes (directly compared codes of those
+// widths have the 16-byte-piece kernels).
+bool lanes_layout(const ScoreArgs& a, const uint32_t* k_cache, bool direct)
+{
+    const bool width = a.Wd == 18 || (!direct && (a.Wd == 16 || a.Wd == 8));
+    return width && a.BS % 64 == 0 && a.ks_block % 4 == 0 &&
+           (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0;
+}
+
+template <int LC>
+void dispatch_lanes(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+{
+    if (LC == 9 && a.G == 1) launch_score(block_score_lanes<9, true, 1>, grid, 0, st, a);
+    else if (LC == 9 && a.G == 2) launch_score(block_score_lanes<9, true, 2>, grid, 0, st, a);
+    else if (LC == 9 && a.G == 4) launch_score(block_score_lanes<9, true, 4>, grid, 0, st, a);
+    else if (pmax == 4) launch_score(block_score_lanes<LC, false, 4>, grid, 0, st, a);
+    else if (pmax == 5) launch_score(block_score_lanes<LC, false, 5>, grid, 0, st, a);
+    else if (pmax == 6) launch_score(block_score_lanes<LC, false, 6>, grid, 0, st, a);
+    else if (pmax == 7) launch_score(block_score_lanes<LC, false, 7>, grid, 0, st, a);
+    else launch_score(block_score_lanes<LC, false, 8>, grid, 0, st, a);
+}
+
 // Layout the 8-byte-piece kernels take: one KV head, an even code width of at most
 // kMaxPlaneWords words, the tokens of a block back to back, 8-byte aligned blocks.
 bool pairs_layout(const ScoreArgs& a, const uint32_t* k_cache)
@@ -1470,7 +1668,9 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     // one KV head, 16-word codes and bit planes: a wave per block of 8-byte pieces beats a
     // workgroup per 4 KiB block of 16-byte pieces (37 against 68 us at 16 x 65,536 tokens)
     const bool direct_g = a.G == 1 || a.G == 2 || a.G == 4;
-    if (fast && !(Hkv == 1 && Wd >= 16 && !direct_g && pairs_layout(a, k_cache))) {
+    const bool one_head_planes = Hkv == 1 && !direct_g && pairs_layout(a, k_cache) &&
+                                 (Wd >= 16 || lanes_layout(a, k_cache, false));
+    if (fast && !one_head_planes) {
         const int pmax = planes_for_group(a.G);
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
         if (!direct) {
@@ -1529,6 +1729,13 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             if (rc != UCM_OK) return rc;
         }
         const dim3 pgrid((unsigned)ucm::ceil_div(max_blocks, kThreads / kWave), (unsigned)B);
+        // 18-word codes (and 8- or 16-word codes with bit planes) in blocks of 64, 128, ...
+        // tokens: a whole code per lane
+        if (lanes_layout(a, k_cache, direct)) {
+            if (Wd == 18) dispatch_lanes<9>(a, pmax, pgrid, st);
+            else if (Wd == 16) dispatch_lanes<8>(a, pmax, pgrid, st);
+            else dispatch_lanes<4>(a, pmax, pgrid, st);
+        } else
         if (a.G == 1) launch_score(block_score_pairs<true, 1>, pgrid, 0, st, a, L, TP);
         else if (a.G == 2) launch_score(block_score_pairs<true, 2>, pgrid, 0, st, a, L, TP);
         else if (a.G == 4) launch_score(block_score_pairs<true, 4>, pgrid, 0, st, a, L, TP);
@@ -1776,6 +1983,111 @@ __global__ __launch_bounds__(kThreads) void token_score_pairs(TokenArgs t, int L
     }
 }
 
+// Per-token scores, a whole code per lane (see block_score_lanes): the lane adds its code's
+// 8-byte piece sums in half precision in the reference's order without any cross-lane step, and
+// the 64 results of a round leave as one contiguous run.
+template <int LC, bool DIRECT, int GP, bool F16>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void token_score_lanes(TokenArgs t)
+{
+    using LCd = LaneCode<LC, DIRECT, GP>;
+    constexpr int WD = LCd::WD;
+    __shared__ __align__(16) uint32_t strip[kThreads / kWave][LCd::kRoundWords];
+    __shared__ __align__(16) uint32_t pl[DIRECT ? 8 : WD * 8];
+    __shared__ int ctot[LC];
+    const ScoreArgs& a = t.s;
+    const int b = blockIdx.y;
+    const int lane = lane_id(), wid = wave_id();
+    const int j = blockIdx.x * (kThreads / kWave) + wid;
+    const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+    const int entry = a.table ? a.table[(int64_t)b * a.table_stride + jc] : 0;
+    const int len = a.lens[b];
+    LCd::stage_planes(a, b, pl, ctot);
+    if (!DIRECT) __syncthreads();
+    const int pos0 = j * a.BS;
+    if (pos0 >= t.max_seq_len) return;
+    int64_t pb = a.table ? (int64_t)entry : (int64_t)b * a.max_blocks + j;
+    if (j >= a.max_blocks || pb < 0 || pb >= a.NB) pb = -1;
+    const int nout = (a.BS < t.max_seq_len - pos0) ? a.BS : t.max_seq_len - pos0;
+    int ntok = len - pos0;  // tokens whose codes are read
+    ntok = pb < 0 ? 0 : (ntok < 0 ? 0 : (ntok > nout ? nout : ntok));
+    const int rounds_in = (ntok + 63) >> 6, rounds_out = (nout + 63) >> 6;
+    const u32x4* src = reinterpret_cast<const u32x4*>(a.kc + (pb < 0 ? 0 : pb) * a.ks_block);
+    u32x4* mine = reinterpret_cast<u32x4*>(strip[wid]);
+    const uint32_t* row = strip[wid] + lane * WD;
+    const uint32_t* qp = a.q + b * a.q_stride_b;
+    const int64_t obase = (int64_t)b * t.max_seq_len + pos0;
+
+    u32x4 cur[LCd::kLoads], nxt[LCd::kLoads];
+    LCd::load_round(src, 0, lane, cur);  // block 0 when there is nothing to read: harmless
+#pragma unroll
+    for (int u = 0; u < LCd::kLoads; ++u) nxt[u] = cur[u];
+    for (int r = 0; r < rounds_out; ++r) {
+        int di = 0;
+        _Float16 dh = (_Float16)0.0f;
+        if (r < rounds_in) {
+            if (r + 1 < rounds_in) LCd::load_round(src, r + 1, lane, nxt);
+            LCd::store_round(mine, lane, cur);
+            asm volatile("" ::: "memory");  // planes re-read per round, see block_score_lanes
+#pragma unroll
+            for (int i = 0; i < LC; ++i) {
+                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
+                int part = 0;
+                if (DIRECT) {
+#pragma unroll
+                    for (int g = 0; g < GP; ++g)
+                        part += __popc(k.x ^ qp[g * a.q_stride_h + 2 * i]) +
+                                __popc(k.y ^ qp[g * a.q_stride_h + 2 * i + 1]);
+                } else {
+                    int x = 0;
+#pragma unroll
+                    for (int p = 0; p < GP; ++p)
+                        x += (__popc(k.x & pl[(2 * i) * 8 + p]) + __popc(k.y & pl[(2 * i + 1) * 8 + p])) << p;
+                    part = ctot[i] + a.G * (__popc(k.x) + __popc(k.y)) - 2 * x;
+                }
+                di += part;
+                if (F16) dh = dh + (_Float16)(float)part;
+            }
+#pragma unroll
+            for (int u = 0; u < LCd::kLoads; ++u) cur[u] = nxt[u];
+        }
+        const int tok = r * 64 + lane;
+        if (tok < nout) {
+            const int pos = pos0 + tok;
+            const bool keep = (pos < a.sink) || (pos >= len - a.recent && pos < len);
+            const bool none = pos >= len || (!keep && pb < 0);
+            if (F16) {
+                const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : dh);
+                uint16_t bits;
+                __builtin_memcpy(&bits, &v, 2);
+                ((uint16_t*)t.out)[obase + tok] = bits;
+            } else {
+                ((int32_t*)t.out)[obase + tok] = none ? kInf : (keep ? 0 : di);
+            }
+        }
+    }
+}
+
+template <int LC, bool DIRECT, int GP>
+void launch_token_lanes(const TokenArgs& t, dim3 grid, hipStream_t st)
+{
+    if (t.out_is_f16)
+        hipLaunchKernelGGL((token_score_lanes<LC, DIRECT, GP, true>), grid, dim3(kThreads), 0, st, t);
+    else
+        hipLaunchKernelGGL((token_score_lanes<LC, DIRECT, GP, false>), grid, dim3(kThreads), 0, st, t);
+}
+
+template <int LC>
+void dispatch_token_lanes_planes(const TokenArgs& t, int pmax, dim3 grid, hipStream_t st)
+{
+    switch (pmax) {
+        case 4: launch_token_lanes<LC, false, 4>(t, grid, st); break;
+        case 5: launch_token_lanes<LC, false, 5>(t, grid, st); break;
+        case 6: launch_token_lanes<LC, false, 6>(t, grid, st); break;
+        case 7: launch_token_lanes<LC, false, 7>(t, grid, st); break;
+        default: launch_token_lanes<LC, false, 8>(t, grid, st); break;
+    }
+}
+
 template <bool DIRECT, int GP>
 void launch_token_pairs(const TokenArgs& t, int L, int TP, dim3 grid, hipStream_t st)
 {
@@ -1855,7 +2167,16 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
         const int L = Wd / 2, TP = kWave / L;
         const int nblk = ucm::ceil_div(max_seq_len, BS);
         const dim3 pgrid((unsigned)ucm::ceil_div(nblk, kThreads / kWave), (unsigned)B);
-        if (direct) {
+        // 18-word codes in blocks of 64, 128, ... tokens: a whole code per lane
+        const bool lanes = lanes_layout(a, k_cache, G <= 4 && direct);
+        if (lanes && G <= 4 && direct) {
+            if (G == 1) launch_token_lanes<9, true, 1>(t, pgrid, st);
+            else if (G == 2) launch_token_lanes<9, true, 2>(t, pgrid, st);
+            else launch_token_lanes<9, true, 4>(t, pgrid, st);
+            return ucm::launch_status("token_score_lanes");
+        }
+        // 8 query heads: bit planes when the caller brought the workspace for them
+        if (direct && !(lanes && have_planes)) {
             if (G == 1) launch_token_pairs<true, 1>(t, L, TP, pgrid, st);
             else if (G == 2) launch_token_pairs<true, 2>(t, L, TP, pgrid, st);
             else if (G == 4) launch_token_pairs<true, 4>(t, L, TP, pgrid, st);
@@ -1867,6 +2188,12 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
                                q_stride_b, q_stride_h, 1, G, Wd, pmax, static_cast<uint32_t*>(workspace));
             rc = ucm::launch_status("plane_kernel");
             if (rc != UCM_OK) return rc;
+            if (lanes) {
+                if (Wd == 18) dispatch_token_lanes_planes<9>(t, pmax, pgrid, st);
+                else if (Wd == 16) dispatch_token_lanes_planes<8>(t, pmax, pgrid, st);
+                else dispatch_token_lanes_planes<4>(t, pmax, pgrid, st);
+                return ucm::launch_status("token_score_lanes");
+            }
             switch (pmax) {
                 case 4: launch_token_pairs<false, 4>(t, L, TP, pgrid, st); break;
                 case 5: launch_token_pairs<false, 5>(t, L, TP, pgrid, st); break;
