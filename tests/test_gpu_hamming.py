@@ -260,6 +260,21 @@ def test_one_kv_head_even_code_widths(G, Wd, BS):
     assert np.array_equal(h, expect)
 
 
+@pytest.mark.parametrize("G,Wd,BS", [(1, 18, 64), (64, 18, 64), (128, 18, 128), (16, 16, 64), (5, 6, 16)])
+def test_one_kv_head_contiguous_cache_without_table(G, Wd, BS):
+    """The one-KV-head kernels with block j of request b at b * max_blocks + j (no table)."""
+    rng = rng_for(450 + G + Wd)
+    B, mb = 3, 9
+    kc = random_codes(rng, (B * mb, BS, 1, Wd))
+    q = random_codes(rng, (B, G, Wd))
+    lens = np.array([mb * BS, 4 * BS + 3, 1], np.int32)
+    table = np.arange(B * mb, dtype=np.int32).reshape(B, mb)
+    for kw in ({}, {"return_physical": True}, {"score_order": True, "distance": True}):
+        gi, gs = run_gpu(q, kc, None, lens, 4, max_blocks=mb, **kw)
+        oi, os_ = run_oracle(q, kc, table, lens, 4, **kw)
+        assert np.array_equal(gi, oi) and np.array_equal(gs, os_)
+
+
 def test_update_seq_lens():
     from ucm_amd.sparse import update_seq_lens
 
