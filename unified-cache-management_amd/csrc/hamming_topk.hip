@@ -1823,15 +1823,28 @@ namespace {
 // head.  Used when G * bits <= 2048, where every partial sum is an integer that fp16 holds
 // exactly, so the reference's piecewise half-precision accumulation equals the exact sum.
 template <int G>
-__global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t)
+__global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t, int tb_shift)
 {
-    extern __shared__ uint32_t dyn[];  // [Hkv][BS] distances
+    extern __shared__ uint32_t dyn[];  // [Hkv][tile tokens] distances
+    __shared__ int64_t pbs[32];        // physical block of each of the tile's blocks, or -1
     const ScoreArgs& a = t.s;
-    const int b = blockIdx.y, j = blockIdx.x;
+    // the tile: 1 << tb_shift consecutive logical blocks (more than one only for power-of-two
+    // block sizes below 128 tokens, so that a workgroup still has ~16 KiB of codes to read)
+    const int TBK = 1 << tb_shift, TT = a.BS << tb_shift;
+    const int bs_shift = tb_shift ? __builtin_ctz((unsigned)a.BS) : 31;  // 31: every token -> block 0
+    const int b = blockIdx.y, j0 = blockIdx.x << tb_shift;
     const int P = a.Wd >> 2, HP = a.Hkv * P;
     const int sub = threadIdx.x & (HP - 1);
     const int p_shift = __builtin_ctz(P), hp_shift = __builtin_ctz(HP);
     const int h = sub >> p_shift, part = sub & (P - 1);
+    // one block per workgroup: its table entry is a scalar read, no LDS and no extra barrier
+    int64_t pb0 = -1;
+    if (tb_shift == 0) {
+        pb0 = j0 < a.max_blocks ? physical_block(a, b, j0) : -1;
+    } else if ((int)threadIdx.x < TBK) {
+        const int j = j0 + threadIdx.x;
+        pbs[threadIdx.x] = j < a.max_blocks ? physical_block(a, b, j) : -1;
+    }
     uint32_t qw[G][4];
 #pragma unroll
     for (int g = 0; g < G; ++g)
@@ -1839,38 +1852,51 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t)
         for (int i = 0; i < 4; ++i)
             qw[g][i] = a.q[b * a.q_stride_b + (int64_t)(h * G + g) * a.q_stride_h + part * 4 + i];
     const int len = a.lens[b];
-    const int64_t pb = j < a.max_blocks ? physical_block(a, b, j) : -1;
-    const uint32_t* base = a.kc + (pb < 0 ? 0 : pb) * a.ks_block + sub * 4;
+    if (tb_shift) __syncthreads();
     const int step = kThreads >> hp_shift;
-    for (int tok = threadIdx.x >> hp_shift; tok < a.BS; tok += step) {
-        int d = 0;
-        if (pb >= 0) {
-            const uint4 kw = *reinterpret_cast<const uint4*>(base + (int64_t)tok * a.ks_token);
+    // four passes of loads go out together (tokens past the tile re-read its last token; an
+    // unusable block reads block 0 and is masked at the output)
+    for (int tt0 = threadIdx.x >> hp_shift; tt0 < TT; tt0 += 4 * step) {
+        u32x4 kw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            int tt = tt0 + u * step;
+            tt = tt < TT ? tt : TT - 1;
+            const int64_t pb = tb_shift ? pbs[tt >> bs_shift] : pb0;
+            const int tok = tb_shift ? (tt & (a.BS - 1)) : tt;
+            kw[u] = *reinterpret_cast<const u32x4*>(
+                a.kc + (pb < 0 ? 0 : pb) * a.ks_block + (int64_t)tok * a.ks_token + sub * 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int tt = tt0 + u * step;
+            int d = 0;
 #pragma unroll
             for (int g = 0; g < G; ++g)
-                d += __popc(kw.x ^ qw[g][0]) + __popc(kw.y ^ qw[g][1]) + __popc(kw.z ^ qw[g][2]) +
-                     __popc(kw.w ^ qw[g][3]);
+                d += __popc(kw[u].x ^ qw[g][0]) + __popc(kw[u].y ^ qw[g][1]) +
+                     __popc(kw[u].z ^ qw[g][2]) + __popc(kw[u].w ^ qw[g][3]);
+            for (int o = 1; o < P; o <<= 1) d += __shfl_xor(d, o);
+            if (part == 0 && tt < TT) dyn[h * TT + tt] = (uint32_t)d;
         }
-        for (int o = 1; o < P; o <<= 1) d += __shfl_xor(d, o);
-        if (part == 0) dyn[h * a.BS + tok] = (uint32_t)d;
     }
     __syncthreads();
     for (int hh = 0; hh < a.Hkv; ++hh) {
-        for (int tok = threadIdx.x; tok < a.BS; tok += kThreads) {
-            const int pos = j * a.BS + tok;
+        for (int tt = threadIdx.x; tt < TT; tt += kThreads) {
+            const int pos = j0 * a.BS + tt;
             if (pos >= t.max_seq_len) continue;
             const bool is_inf = pos >= len;
             const bool keep = (pos < a.sink) || (pos >= len - a.recent && pos < len);
-            const int d = (int)dyn[hh * a.BS + tok];
+            const bool have = (tb_shift ? pbs[tt >> bs_shift] : pb0) >= 0;
+            const int d = (int)dyn[hh * TT + tt];
             const int64_t o = ((int64_t)b * a.Hkv + hh) * t.max_seq_len + pos;
             if (t.out_is_f16) {
                 const _Float16 v = is_inf ? (_Float16)__builtin_inff()
-                                          : (keep ? (_Float16)0.0f : (pb >= 0 ? (_Float16)(float)d : (_Float16)__builtin_inff()));
+                                          : (keep ? (_Float16)0.0f : (have ? (_Float16)(float)d : (_Float16)__builtin_inff()));
                 uint16_t u;
                 __builtin_memcpy(&u, &v, 2);
                 ((uint16_t*)t.out)[o] = u;
             } else {
-                ((int32_t*)t.out)[o] = is_inf ? kInf : (keep ? 0 : (pb >= 0 ? d : kInf));
+                ((int32_t*)t.out)[o] = is_inf ? kInf : (keep ? 0 : (have ? d : kInf));
             }
         }
     }
@@ -2150,13 +2176,18 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
                       (G == 1 || G == 2 || G == 4 || G == 8) && (int64_t)G * Wd * 32 <= 2048 &&
                       (int64_t)BS * Hkv * 4 <= 48 * 1024 && ucm::ceil_div(max_seq_len, BS) <= 0x7fffffff;
     if (fast) {
-        const dim3 fgrid((unsigned)ucm::ceil_div(max_seq_len, BS), (unsigned)B);
-        const size_t lds = (size_t)BS * Hkv * 4;
+        // blocks below 128 tokens (power-of-two sizes): several per workgroup, 128 tokens in all
+        int tbs = 0;
+        if (is_pow2(BS))
+            while ((BS << tbs) < 128 && tbs < 5) ++tbs;
+        while (tbs > 0 && ((size_t)BS << tbs) * Hkv * 4 > 48 * 1024) --tbs;
+        const dim3 fgrid((unsigned)ucm::ceil_div(ucm::ceil_div(max_seq_len, BS), 1 << tbs), (unsigned)B);
+        const size_t lds = ((size_t)BS << tbs) * Hkv * 4;
         hipStream_t st = (hipStream_t)stream;
-        if (G == 1) hipLaunchKernelGGL(token_score_fast<1>, fgrid, dim3(kThreads), lds, st, t);
-        else if (G == 2) hipLaunchKernelGGL(token_score_fast<2>, fgrid, dim3(kThreads), lds, st, t);
-        else if (G == 4) hipLaunchKernelGGL(token_score_fast<4>, fgrid, dim3(kThreads), lds, st, t);
-        else hipLaunchKernelGGL(token_score_fast<8>, fgrid, dim3(kThreads), lds, st, t);
+        if (G == 1) hipLaunchKernelGGL(token_score_fast<1>, fgrid, dim3(kThreads), lds, st, t, tbs);
+        else if (G == 2) hipLaunchKernelGGL(token_score_fast<2>, fgrid, dim3(kThreads), lds, st, t, tbs);
+        else if (G == 4) hipLaunchKernelGGL(token_score_fast<4>, fgrid, dim3(kThreads), lds, st, t, tbs);
+        else hipLaunchKernelGGL(token_score_fast<8>, fgrid, dim3(kThreads), lds, st, t, tbs);
         return ucm::launch_status("token_score_fast");
     }
     const bool direct = G == 1 || G == 2 || G == 4 || G == 8;
