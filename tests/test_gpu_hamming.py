@@ -235,7 +235,8 @@ def test_f16_scores_round_like_sequential_half_adds():
 
 
 @pytest.mark.parametrize("G", [1, 2, 4, 5, 8, 16, 128])
-@pytest.mark.parametrize("Wd,BS", [(18, 64), (18, 128), (18, 16), (18, 1), (6, 32), (2, 64), (34, 8), (64, 4)])
+@pytest.mark.parametrize("Wd,BS", [(18, 64), (18, 128), (18, 192), (18, 16), (18, 1), (16, 256), (8, 192),
+                                   (6, 32), (2, 64), (34, 8), (64, 4)])
 def test_one_kv_head_even_code_widths(G, Wd, BS):
     """One KV head with codes that are not a whole number of 16-byte pieces per token — the
     18-word (512 + 64 bit) codes of the reference's latent-attention path
