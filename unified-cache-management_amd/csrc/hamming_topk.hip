@@ -52,6 +52,17 @@ struct ScoreArgs {
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 
+// Every read of cached codes goes through here.
+template <class T>
+__device__ __forceinline__ T code_load(const T* p)
+{
+#ifdef UCM_PLAIN_CODE_LOADS
+    return *p;
+#else
+    return __builtin_nontemporal_load(p);
+#endif
+}
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -218,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void block_score_fast(ScoreArgs a, int sp
                 const int run = run_first + k * run_step;
                 const u32x4* src =
                     reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + (run << 6) + lane;
-                kv[u] = __builtin_nontemporal_load(src);
+                kv[u] = code_load(src);
             }
         }
     };
@@ -357,11 +368,11 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
     if (pb >= 0) {
         if (EXACT || rpw >= 4) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * u) << 6));
+            for (int u = 0; u < 4; ++u) kv[u] = code_load(base + ((wid + 4 * u) << 6));
         } else {
 #pragma unroll
             for (int u = 0; u < 4; ++u)
-                if (u < rpw) kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * u) << 6));
+                if (u < rpw) kv[u] = code_load(base + ((wid + 4 * u) << 6));
         }
     }
     if (!DIRECT) {
@@ -403,7 +414,7 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
                 for (int u = 0; u < 4; ++u) {
                     kv[u] = (u32x4)(0u);
                     if (k0 + 4 + u < rpw)
-                        kv[u] = __builtin_nontemporal_load(base + ((wid + 4 * (k0 + 4 + u)) << 6));
+                        kv[u] = code_load(base + ((wid + 4 * (k0 + 4 + u)) << 6));
                 }
             }
         }
@@ -488,7 +499,7 @@ __global__ __launch_bounds__(kThreads) void block_score_small(ScoreArgs a)
             for (int r = 0; r < RPB; ++r) {
                 kv[ub * RPB + r] = (u32x4)(0u);
                 if (ok[ub])
-                    kv[ub * RPB + r] = __builtin_nontemporal_load(
+                    kv[ub * RPB + r] = code_load(
                         reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + (r << 6) + lane);
             }
         }
@@ -600,7 +611,7 @@ __global__ __launch_bounds__(kThreads) void block_score_rows(ScoreArgs a)
         pb[bi] = v;
         const u32x4* base = reinterpret_cast<const u32x4*>(a.kc + (v < 0 ? 0 : v) * a.ks_block) + lane;
 #pragma unroll
-        for (int r = 0; r < RPB; ++r) kv[bi * RPB + r] = __builtin_nontemporal_load(base + (r << 6));
+        for (int r = 0; r < RPB; ++r) kv[bi * RPB + r] = code_load(base + (r << 6));
     }
 
     const int full = a.G * 32 * a.Wd;
@@ -753,7 +764,7 @@ __global__ __launch_bounds__(kThreads) void block_score_pairs(ScoreArgs a, int L
             if (t0 + u * TP < ntok) {
                 // idle lanes and lanes past the block re-read the pass's first piece
                 const int tok = t0 + u * TP + slot;
-                kv[u] = __builtin_nontemporal_load(
+                kv[u] = code_load(
                     base + ((tok < a.BS && lane_ok) ? tok * L + p : (t0 + u * TP) * L));
             } else {
                 kv[u] = u32x2{0u, 0u};
@@ -830,7 +841,7 @@ struct LaneCode {
         for (int u = 0; u < kLoads; ++u) {
             const int i = u * 64 + lane;
             // lanes past the round's end re-read the load's first piece
-            v[u] = __builtin_nontemporal_load(src + round * kVec + (i < kVec ? i : u * 64));
+            v[u] = code_load(src + round * kVec + (i < kVec ? i : u * 64));
         }
     }
 
@@ -1829,7 +1840,7 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t, int tb
     __shared__ int64_t pbs[32];        // physical block of each of the tile's blocks, or -1
     const ScoreArgs& a = t.s;
     // the tile: 1 << tb_shift consecutive logical blocks (more than one only for power-of-two
-    // block sizes below 128 tokens, so that a workgroup still has ~16 KiB of codes to read)
+    // block sizes, so that a workgroup has at least 128 tokens and ~16 KiB of codes to read)
     const int TBK = 1 << tb_shift, TT = a.BS << tb_shift;
     const int bs_shift = tb_shift ? __builtin_ctz((unsigned)a.BS) : 31;  // 31: every token -> block 0
     const int b = blockIdx.y, j0 = blockIdx.x << tb_shift;
@@ -1943,7 +1954,7 @@ __global__ __launch_bounds__(kThreads) void token_score_pairs(TokenArgs t, int L
         for (int u = 0; u < kPairPasses; ++u) {
             if (t0 + u * TP < ntok) {
                 const int tok = t0 + u * TP + slot;
-                kv[u] = __builtin_nontemporal_load(
+                kv[u] = code_load(
                     base + ((tok < a.BS && lane_ok) ? tok * L + p : (t0 + u * TP) * L));
             } else {
                 kv[u] = u32x2{0u, 0u};
@@ -2176,10 +2187,11 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
                       (G == 1 || G == 2 || G == 4 || G == 8) && (int64_t)G * Wd * 32 <= 2048 &&
                       (int64_t)BS * Hkv * 4 <= 48 * 1024 && ucm::ceil_div(max_seq_len, BS) <= 0x7fffffff;
     if (fast) {
-        // blocks below 128 tokens (power-of-two sizes): several per workgroup, 128 tokens in all
+        // small blocks (power-of-two sizes): several per workgroup, until it has at least 128
+        // tokens and 16 KiB of codes to read
         int tbs = 0;
         if (is_pow2(BS))
-            while ((BS << tbs) < 128 && tbs < 5) ++tbs;
+            while (tbs < 5 && ((BS << tbs) < 128 || ((int64_t)BS << tbs) * Hkv * Wd * 4 < 16384)) ++tbs;
         while (tbs > 0 && ((size_t)BS << tbs) * Hkv * 4 > 48 * 1024) --tbs;
         const dim3 fgrid((unsigned)ucm::ceil_div(ucm::ceil_div(max_seq_len, BS), 1 << tbs), (unsigned)B);
         const size_t lds = ((size_t)BS << tbs) * Hkv * 4;
