@@ -701,7 +701,6 @@ int dispatch_mfma(const EncArgs& a, hipStream_t st)
 }
 
 constexpr int64_t kSmallRows = 256;  // at most this many rows per head take the latency path
-constexpr int64_t kSmallRowsWide = 4096;  // the same for K = 512 with >= 256 hash columns
 
 bool mfma_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 {
@@ -865,12 +864,24 @@ int launch_tiled(const EncArgs& a, hipStream_t st)
     return ucm::launch_status("encode_tiled_kernel");
 }
 
+// Which matrix-core kernel: the wave-per-tile kernel costs about 4 us plus 12.5 ps per wave and
+// k value (each wave gathers its own operand columns from L2); the LDS kernel has a floor of
+// about 6 us plus 0.13 us per KiB of projection slice that every workgroup stages before its
+// first tile (7 us at 64 x 64, 10 us at 128 x 128, 23-24 us for a 133 KiB slice), after which it
+// streams rows at HBM rate.  Measured crossovers this reproduces: 128 -> 128 bits with 8 heads at
+// ~4000 rows, 256 -> 256 with 4 heads and 512 -> 512 at ~5000-6000 rows, 64 -> 64 never below
+// 16,384 rows.
 bool small_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 {
-    // K = 512 with 512 hash columns leaves the LDS kernel four column slices and few workgroups:
-    // up to kSmallRowsWide rows the wave-per-tile kernel is faster there
-    const int64_t cap = (a.K == 512 && a.N >= 256) ? kSmallRowsWide : kSmallRows;
-    return mfma_eligible(a, x_dtype, w_dtype) && a.T <= cap && small_waves(a) <= 0x7fffffff;
+    if (!mfma_eligible(a, x_dtype, w_dtype) || small_waves(a) > 0x7fffffff) return false;
+    if (a.T <= kSmallRows && a.K <= 256) return true;
+    constexpr size_t kStage = (size_t)kMfmaWaves * kStageBytes;
+    const int bn = pick_slice(a.N, a.K, (size_t)160 * 1024 - kStage);
+    if (bn == 0) return true;
+    const double slice_kib = (double)bn * (a.K + kPad) * 2 / 1024.0;
+    const double lds_floor_us = 6.0 + 0.13 * slice_kib;
+    const double small_us = 4.0 + (double)small_waves(a) * a.K * 12.5e-6;
+    return small_us < lds_floor_us;
 }
 
 int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
