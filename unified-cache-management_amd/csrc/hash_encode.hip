@@ -528,12 +528,10 @@ struct EncJobs {
     int waves0;  // waves of job 0; waves >= waves0 belong to job 1
 };
 
-// NCH: K is walked in NCH chunks of KS k-steps (K = 512: two chunks of 256, which keeps the
-// operand registers of one chunk within the budget of two waves per SIMD).
-template <typename V, int KS, int NCH = 1>
+template <typename V, int KS>
 __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
 {
-    constexpr int K = KS * 16 * NCH;
+    constexpr int K = KS * 16;
     const bool second = (int)blockIdx.x >= js.waves0;
     const EncArgs& a = second ? js.job[1] : js.job[0];
     int wv = second ? blockIdx.x - js.waves0 : blockIdx.x;
@@ -552,25 +550,23 @@ __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
     if (!row_ok) t = a.T - 1;
     const uint16_t* xr = (const uint16_t*)a.x + src_offset(a, t, h) + kb * 8;
 
+    // K = 512 holds 128 + 256 operand registers: one wave per SIMD, which is all a launch of
+    // this kernel has anyway
+    V av[KS];
+    uint16_t bw[KS][8];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bw[ks][i] = wsrc[(int64_t)(ks * 16 + kb * 8 + i) * a.N];
+
     f32x16 acc = {0};
-#pragma unroll 1
-    for (int ch = 0; ch < NCH; ++ch) {
-        V av[KS];
-        uint16_t bw[KS][8];
-        const int k0 = ch * KS * 16;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + k0 + ks * 16);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                bw[ks][i] = wsrc[(int64_t)(k0 + ks * 16 + kb * 8 + i) * a.N];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            V bv;
-            __builtin_memcpy(&bv, bw[ks], 16);
-            acc = Mfma<V>::run(bv, av[ks], acc);
-        }
+    for (int ks = 0; ks < KS; ++ks) {
+        V bv;
+        __builtin_memcpy(&bv, bw[ks], 16);
+        acc = Mfma<V>::run(bv, av[ks], acc);
     }
     const uint32_t half = pack_half(acc);
     const uint32_t word = join_halves(kb ? half << 4 : half);
@@ -728,7 +724,7 @@ int launch_small(const EncJobs& js, int64_t waves, int K, hipStream_t st)
         case 64: hipLaunchKernelGGL((encode_small_kernel<V, 4>), grid, dim3(64), 0, st, js); break;
         case 128: hipLaunchKernelGGL((encode_small_kernel<V, 8>), grid, dim3(64), 0, st, js); break;
         case 256: hipLaunchKernelGGL((encode_small_kernel<V, 16>), grid, dim3(64), 0, st, js); break;
-        case 512: hipLaunchKernelGGL((encode_small_kernel<V, 16, 2>), grid, dim3(64), 0, st, js); break;
+        case 512: hipLaunchKernelGGL((encode_small_kernel<V, 32>), grid, dim3(64), 0, st, js); break;
         default: return ucm::fail(UCM_ERROR, "internal: K %d has no small-row kernel", K);
     }
     return ucm::launch_status("encode_small_kernel");
