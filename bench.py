@@ -373,8 +373,13 @@ def extras(torch, enc_k, gen):
     q2 = codes((B, HQ, WD))
     ms = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, False), reps=10)
     byt = B * CTX * HKV * (WD * 4 + 2)
+    # the reference's own GQA call reduces over the KV heads (hamming_topk.py:33): one fp16 row per request
+    ms_red = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, True), reps=10)
+    byt_red = B * CTX * (HKV * WD * 4 + 2)
     out["token_scores_config2"] = {"tokens": B * CTX, "ms": ms, "tokens_per_s": B * CTX / ms * 1e3,
-                                   "hbm_GBps": byt / ms / 1e6, "hbm_frac": byt / ms / 1e6 / HBM_PEAK_GBPS}
+                                   "hbm_GBps": byt / ms / 1e6, "hbm_frac": byt / ms / 1e6 / HBM_PEAK_GBPS,
+                                   "reduce_kvhead_ms": ms_red,
+                                   "reduce_kvhead_hbm_frac": byt_red / ms_red / 1e6 / HBM_PEAK_GBPS}
     del cache2, table2
 
     # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---

@@ -1891,15 +1891,24 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t, int tb
         }
     }
     __syncthreads();
-    for (int hh = 0; hh < a.Hkv; ++hh) {
+    // with the KV-head reduction (the reference's GQA call, hamming_topk.py:33) one row per
+    // request holds the minimum over the heads; the sums are exact here, so the minimum of
+    // the integers is the minimum of the reference's half values
+    const int rows_out = t.reduce_heads ? 1 : a.Hkv;
+    for (int hh = 0; hh < rows_out; ++hh) {
         for (int tt = threadIdx.x; tt < TT; tt += kThreads) {
             const int pos = j0 * a.BS + tt;
             if (pos >= t.max_seq_len) continue;
             const bool is_inf = pos >= len;
             const bool keep = (pos < a.sink) || (pos >= len - a.recent && pos < len);
             const bool have = (tb_shift ? pbs[tt >> bs_shift] : pb0) >= 0;
-            const int d = (int)dyn[hh * TT + tt];
-            const int64_t o = ((int64_t)b * a.Hkv + hh) * t.max_seq_len + pos;
+            int d = (int)dyn[hh * TT + tt];
+            if (t.reduce_heads)
+                for (int h2 = 1; h2 < a.Hkv; ++h2) {
+                    const int o2 = (int)dyn[h2 * TT + tt];
+                    d = o2 < d ? o2 : d;
+                }
+            const int64_t o = ((int64_t)b * rows_out + hh) * t.max_seq_len + pos;
             if (t.out_is_f16) {
                 const _Float16 v = is_inf ? (_Float16)__builtin_inff()
                                           : (keep ? (_Float16)0.0f : (have ? (_Float16)(float)d : (_Float16)__builtin_inff()));
@@ -2181,7 +2190,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
     t.max_seq_len = max_seq_len; t.reduce_heads = reduce_heads; t.out_is_f16 = out_is_f16;
     t.out = out;
     const int G = a.G;
-    const bool fast = !reduce_heads && Wd % 4 == 0 && is_pow2(Wd / 4) && is_pow2(Hkv * (Wd / 4)) &&
+    const bool fast = Wd % 4 == 0 && is_pow2(Wd / 4) && is_pow2(Hkv * (Wd / 4)) &&
                       Hkv * (Wd / 4) <= kThreads && ks_head == Wd && ks_token == (int64_t)Hkv * Wd &&
                       ks_block % 4 == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 &&
                       (G == 1 || G == 2 || G == 4 || G == 8) && (int64_t)G * Wd * 32 <= 2048 &&
