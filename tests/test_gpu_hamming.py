@@ -276,6 +276,26 @@ def test_one_kv_head_contiguous_cache_without_table(G, Wd, BS):
         assert np.array_equal(gi, oi) and np.array_equal(gs, os_)
 
 
+@pytest.mark.parametrize("S,Hkv,G,Wd", [(1024, 8, 1, 4), (1000, 4, 2, 8), (333, 1, 64, 18), (640, 1, 1, 18)])
+def test_per_token_scores_contiguous_form(S, Hkv, G, Wd):
+    """block_table=None: key_codes [B, S, Hkv, C], position p of request b at key_codes[b, p]
+    (the reference's non-block mode, paged_ham_dist_mla.cu:345,444-)."""
+    from ucm_amd.sparse import hamming_score
+
+    rng = rng_for(460 + S)
+    B = 3
+    kc = random_codes(rng, (B, S, Hkv, Wd))
+    q = random_codes(rng, (B, Hkv * G, Wd))
+    lens = np.array([S, S // 2 + 1, 0], np.int32)
+    # checker: one block of S tokens per request
+    table = np.arange(B, dtype=np.int32).reshape(B, 1)
+    for red in ((False, True) if Hkv > 1 else (False,)):
+        o = c_api.hamming_score(q, kc, table, lens, S, 3, 5, red)
+        g = hamming_score(dev(as_i32(kc)), dev(as_i32(q))[:, None], None, dev(lens), S, 3, 5, red,
+                          out_int32=True).cpu().numpy()
+        assert np.array_equal(g, o)
+
+
 def test_update_seq_lens():
     from ucm_amd.sparse import update_seq_lens
 

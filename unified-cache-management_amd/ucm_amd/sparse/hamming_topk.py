@@ -140,11 +140,33 @@ def hamming_score(key_codes, query_code, block_table, seq_len, max_seq_len, sink
     """Per-token group-summed Hamming distance, the output of the reference's scorer
     (kvlib::HammingScoreContiCUDA, csrc/cuda/ham_dist/paged_ham_dist_mla.cu:332-443):
     float16 [B, Hkv or 1, max_seq_len]; 0 at sink/recent positions, +inf past seq_len.
-    out_int32=True returns exact int32 distances (inf = int32 max) instead."""
+    out_int32=True returns exact int32 distances (inf = int32 max) instead.
+
+    block_table=None is the reference's contiguous form (paged_ham_dist_mla.cu:345,444-):
+    key_codes is [B, S, Hkv, C] and position p of request b is key_codes[b, p].  The codes are
+    then read as blocks of the largest power of two up to 128 that divides S, block j of request b
+    at b * (S / block) + j, which is the library's table-free addressing."""
     if block_table is None:
-        raise ValueError("the paged form needs a block table")
+        kw = _as_words(key_codes, "key_codes")
+        if kw.ndim != 4:
+            raise ValueError(f"key_codes must be [B,S,Hkv,C], got {tuple(kw.shape)}")
+        kw = kw.contiguous()
+        Bk, S, Hk, C = kw.shape
+        bsv = 128
+        while S % bsv:
+            bsv //= 2
+        key_codes = kw.view(Bk * (S // bsv), bsv, Hk, C)
+        n_table_blocks = S // bsv
     q, k, block_table, seq_len, (NB, BS, Hkv, Wd, ks, B, Hq) = _common(
         query_code, key_codes, block_table, seq_len, False)
+    if block_table is None:
+        if NB != B * n_table_blocks:
+            raise ValueError("batch size mismatch between query_code and key_codes")
+        table_ptr, table_stride, max_blocks = None, 0, n_table_blocks
+    else:
+        table_ptr = block_table.data_ptr()
+        table_stride = max(_lib.stride(block_table, 0), block_table.shape[1])
+        max_blocks = block_table.shape[1]
     Ho = 1 if reduce_kvhead else Hkv
     out = torch.empty((B, Ho, int(max_seq_len)),
                       dtype=torch.int32 if out_int32 else torch.float16, device=q.device)
@@ -152,8 +174,7 @@ def hamming_score(key_codes, query_code, block_table, seq_len, max_seq_len, sink
                      device=q.device)
     _lib.check(_lib.lib().ucm_hamming_score(
         q.data_ptr(), _lib.stride(q, 0), _lib.stride(q, 1), k.data_ptr(), NB, BS, Hkv, Wd, ks[0], ks[1], ks[2],
-        block_table.data_ptr(), max(_lib.stride(block_table, 0), block_table.shape[1]),
-        block_table.shape[1], seq_len.data_ptr(),
+        table_ptr, table_stride, max_blocks, seq_len.data_ptr(),
         B, Hq, int(max_seq_len), int(sink), int(recent), int(bool(reduce_kvhead)), out.data_ptr(),
         int(not out_int32), ws.data_ptr(), ws.numel(), _lib.stream_ptr(q.device)))
     return out
