@@ -1243,19 +1243,31 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
     const int32_t* row = a.scores + ((int64_t)b * a.Hkv + (reduce ? 0 : ho)) * a.max_blocks;
     int v[EL];
 #pragma unroll
-    for (int e = 0; e < EL; ++e) {
-        const int j = lane * EL + e;
-        int x = -0x7fffffff;  // below every real score (>= -1): never selected
-        if (j < n) {
-            x = raw[e];
-            if (reduce)
-                for (int h = 1; h < a.Hkv; ++h) {
-                    const int o = row[(int64_t)h * a.max_blocks + j];
-                    x = o > x ? o : x;
+    for (int e = 0; e < EL; ++e) v[e] = raw[e];
+    if (reduce) {
+        // maximum over the KV heads, CH heads at a time with all of their loads in flight
+        // (heads past the last re-read head 0, which changes nothing)
+        constexpr int CH = EL <= 4 ? 8 : 2;
+        for (int h0 = 1; h0 < a.Hkv; h0 += CH) {
+            int o[CH][EL];
+#pragma unroll
+            for (int u = 0; u < CH; ++u) {
+                const int hh = h0 + u < a.Hkv ? h0 + u : 0;
+#pragma unroll
+                for (int e = 0; e < EL; ++e) {
+                    const int j = lane * EL + e;
+                    o[u][e] = row[(int64_t)hh * a.max_blocks + (j < a.max_blocks ? j : 0)];
                 }
+            }
+#pragma unroll
+            for (int u = 0; u < CH; ++u)
+#pragma unroll
+                for (int e = 0; e < EL; ++e) v[e] = o[u][e] > v[e] ? o[u][e] : v[e];
         }
-        v[e] = x;
     }
+#pragma unroll
+    for (int e = 0; e < EL; ++e)
+        if (lane * EL + e >= n) v[e] = -0x7fffffff;  // below every real score (>= -1): never selected
     auto count_ge = [&](int t) {
         int c = 0;
 #pragma unroll
