@@ -45,6 +45,8 @@ struct ScoreArgs {
     const int32_t* lens;
     int B, Hq, G, sink, recent;
     int TB;                  // logical blocks per workgroup
+    int reduce_out;          // block_score_one only: write the maximum over the KV heads,
+                             // scores then is [B][1][max_blocks]
     const uint32_t* planes;  // [B][Hkv][PMAX][Wd], planes mode only
     int32_t* scores;         // [B][Hkv][max_blocks]
 };
@@ -433,6 +435,17 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
         const int full = a.G * 32 * a.Wd;
         const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
         const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
+        if (a.reduce_out) {
+            // one list per request: the best head, i.e. the smallest distance over the heads
+#pragma unroll
+            for (int st = 1; st < HKV; st <<= 1) {
+                const int o = __shfl_xor(dmin, st);
+                dmin = o < dmin ? o : dmin;
+            }
+            if (threadIdx.x == 0)
+                a.scores[(int64_t)b * a.max_blocks + j] = pb < 0 ? -1 : (forced ? full : full - dmin);
+            return;
+        }
         const int sc = pb < 0 ? -1 : (forced ? full : full - dmin);
         a.scores[((int64_t)b * HKV + threadIdx.x) * a.max_blocks + j] = sc;
     }
@@ -1669,7 +1682,8 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     a.ks_block = ks_block; a.ks_token = ks_token; a.ks_head = ks_head;
     a.table = block_table; a.table_stride = table_stride; a.max_blocks = max_blocks;
     a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
-    a.recent = recent_tok; a.planes = ws.planes; a.scores = ws.scores;
+    a.recent = recent_tok; a.planes = ws.planes; a.scores = ws.scores; a.reduce_out = 0;
+    bool reduced_scores = false;  // the score kernel already took the maximum over the heads
 
     // fast path eligibility
     const int cpu = Wd / 4;
@@ -1716,10 +1730,13 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
         }
         if (!done && split && Hkv <= 16) {
             a.TB = 1;
+            a.reduce_out = ((flags & UCM_TOPK_REDUCE_HEADS) && Hkv > 1) ? 1 : 0;
             const dim3 grid1((unsigned)max_blocks, (unsigned)B);
             if (cpu == 1) done = dispatch_one<1>(a, pmax, grid1, st);
             else if (cpu == 2) done = dispatch_one<2>(a, pmax, grid1, st);
             else done = dispatch_one<4>(a, pmax, grid1, st);
+            reduced_scores = done && a.reduce_out;
+            a.reduce_out = 0;
         }
         if (!done) a.TB = TB;
         if (!done && !split) {
@@ -1776,7 +1793,7 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     SelectArgs s;
     s.scores = ws.scores; s.reduced = ws.reduced; s.table = block_table;
     s.table_stride = table_stride; s.max_blocks = max_blocks; s.lens = seq_lens; s.BS = BS;
-    s.Hkv = Hkv; s.Ho = (flags & UCM_TOPK_REDUCE_HEADS) ? 1 : Hkv; s.k = k;
+    s.Hkv = reduced_scores ? 1 : Hkv; s.Ho = (flags & UCM_TOPK_REDUCE_HEADS) ? 1 : Hkv; s.k = k;
     s.full = a.G * 32 * Wd;
     s.key_bits = 1;
     while ((1ll << s.key_bits) <= (int64_t)s.full + 1) ++s.key_bits;
@@ -2198,7 +2215,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
     a.ks_block = ks_block; a.ks_token = ks_token; a.ks_head = ks_head;
     a.table = block_table; a.table_stride = table_stride; a.max_blocks = max_blocks;
     a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
-    a.recent = recent_tok; a.TB = 1; a.planes = nullptr; a.scores = nullptr;
+    a.recent = recent_tok; a.TB = 1; a.reduce_out = 0; a.planes = nullptr; a.scores = nullptr;
     t.max_seq_len = max_seq_len; t.reduce_heads = reduce_heads; t.out_is_f16 = out_is_f16;
     t.out = out;
     const int G = a.G;
