@@ -45,8 +45,8 @@ struct ScoreArgs {
     const int32_t* lens;
     int B, Hq, G, sink, recent;
     int TB;                  // logical blocks per workgroup
-    int reduce_out;          // block_score_one only: write the maximum over the KV heads,
-                             // scores then is [B][1][max_blocks]
+    int reduce_out;          // block_score_one / block_score_rows: write the maximum over the
+                             // KV heads, scores then is [B][1][max_blocks]
     const uint32_t* planes;  // [B][Hkv][PMAX][Wd], planes mode only
     int32_t* scores;         // [B][Hkv][max_blocks]
 };
@@ -650,6 +650,20 @@ __global__ __launch_bounds__(kThreads) void block_score_rows(ScoreArgs a)
         for (int st = PERIOD; st < kWave; st <<= 1) {
             const int o = __shfl_xor(m, st);
             m = o < m ? o : m;
+        }
+        if (a.reduce_out) {
+            // one list per request: the smallest distance over the heads, one score per block
+#pragma unroll
+            for (int st = CPU; st < PERIOD; st <<= 1) {
+                const int o = __shfl_xor(m, st);
+                m = o < m ? o : m;
+            }
+            if (lane == 0 && j < a.max_blocks && pos0 < len) {
+                const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
+                const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
+                a.scores[(int64_t)b * a.max_blocks + j] = pb[bi] < 0 ? -1 : (forced ? full : full - m);
+            }
+            continue;
         }
         if (lane < PERIOD && part == 0 && j < a.max_blocks && pos0 < len) {
             const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
@@ -1724,9 +1738,12 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
         bool done = false;
         // blocks of at most 8 KiB with directly compared query codes: whole blocks per wave
         if (direct && rpb <= 8) {
+            a.reduce_out = ((flags & UCM_TOPK_REDUCE_HEADS) && Hkv > 1) ? 1 : 0;
             if (cpu == 1) done = dispatch_rows<1>(a, rpb, B, st);
             else if (cpu == 2) done = dispatch_rows<2>(a, rpb, B, st);
             else done = dispatch_rows<4>(a, rpb, B, st);
+            reduced_scores = done && a.reduce_out;
+            a.reduce_out = 0;
         }
         if (!done && split && Hkv <= 16) {
             a.TB = 1;
