@@ -303,3 +303,43 @@ def test_one_kv_head_random_configurations(seed):
         if Wd % 2 == 0:
             h = hamming_score(dk, dq[:, None], dt, dl, msl, 0, 0, False).cpu().numpy()
             assert np.array_equal(h, half_piece_sums(q, kc, table, lens, msl)), what
+
+
+@pytest.mark.parametrize("seed", [71, 72])
+def test_topk_rows_of_257_to_1024_blocks(seed):
+    """Rows of 257 to 1024 blocks take the workgroup-per-row selection: ragged lengths, ties
+    (low-entropy codes), every output flag, head reduction, k up to the row length."""
+    from ucm_amd.sparse import hamming_topk
+
+    rng = rng_for(seed)
+    for _ in range(40):
+        B = int(rng.integers(1, 4))
+        Hkv = int(rng.choice([1, 2, 8]))
+        G = int(rng.choice([1, 4, 16]))
+        Wd = int(rng.choice([2, 4, 18])) if Hkv == 1 else 4
+        BS = int(rng.choice([4, 8, 16]))
+        mb = int(rng.choice([257, 300, 511, 512, 513, 777, 1000, 1023, 1024]))
+        NB = B * mb + 2
+        kc = rng.integers(0, 2**32, size=(NB, BS, Hkv, Wd), dtype=np.uint32)
+        if rng.integers(0, 2) == 0:
+            kc &= np.uint32(0x00000101)  # many equal scores
+        q = rng.integers(0, 2**32, size=(B, Hkv * G, Wd), dtype=np.uint32)
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32)
+        if rng.integers(0, 3) == 0:
+            table[rng.integers(0, B), rng.integers(0, mb)] = -5  # unusable entry
+        lens = rng.integers(0, mb * BS + 1, size=B).astype(np.int32)
+        lens[rng.integers(0, B)] = mb * BS - int(rng.integers(0, BS))
+        k = int(rng.choice([1, 7, 64, 128, 300, mb, mb + 5]))
+        sink, recent = int(rng.integers(0, 3)) * BS, int(rng.integers(0, 5)) * BS
+        reduce_heads, physical = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        distance = bool(rng.integers(0, 2))
+        flags = (c_api.F_REDUCE_HEADS if reduce_heads else 0) | (c_api.F_PHYSICAL if physical else 0) | \
+                (c_api.F_DISTANCE if distance else 0)
+        what = dict(B=B, Hkv=Hkv, G=G, Wd=Wd, BS=BS, mb=mb, k=k, sink=sink, recent=recent, flags=flags)
+        oi, osc = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, flags, max_blocks=mb)
+        gi, gs = hamming_topk(torch.from_numpy(q.view(np.int32)).cuda(), torch.from_numpy(kc.view(np.int32)).cuda(),
+                              torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda(), k, sink, recent,
+                              reduce_heads=reduce_heads, return_physical=physical, distance=distance,
+                              max_blocks=mb)
+        assert np.array_equal(gi.cpu().numpy(), oi), what
+        assert np.array_equal(gs.cpu().numpy(), osc), what

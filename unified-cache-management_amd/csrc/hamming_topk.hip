@@ -1351,6 +1351,140 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
     }
 }
 
+// Rows of 257 to 1024 block scores, index-ordered output: one workgroup per row, four scores
+// per thread.  Same algorithm as select_wave_kernel<16>, but a wave there runs some 2000
+// instructions back to back for its row (7 us, however few rows there are); here each wave has
+// a quarter of the row and the four partial counts of a search step meet in LDS (two buffers
+// in turn, one barrier per step).
+template <int EL>
+__global__ __launch_bounds__(kThreads) void select_group_kernel(SelectArgs a)
+{
+    constexpr int kWaves = kThreads / kWave;
+    __shared__ int cnt[2][kWaves];
+    __shared__ int ext[2][kWaves];
+    __shared__ int wsum[kWaves];
+    const int b = blockIdx.x / a.Ho, ho = blockIdx.x % a.Ho;
+    const int tid = threadIdx.x, lane = lane_id(), wid = wave_id();
+    const bool reduce = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
+    const int32_t* row = a.scores + ((int64_t)b * a.Hkv + (reduce ? 0 : ho)) * a.max_blocks;
+    int v[EL], tab[EL];
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        const int j = tid * EL + e;
+        v[e] = row[j < a.max_blocks ? j : 0];
+    }
+    const bool physical = (a.flags & UCM_TOPK_RETURN_PHYSICAL) != 0;
+    if (physical && a.table) {
+        const int32_t* t0 = a.table + (int64_t)b * a.table_stride;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int j = tid * EL + e;
+            tab[e] = t0[j < a.max_blocks ? j : 0];
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < EL; ++e) tab[e] = physical ? b * a.max_blocks + tid * EL + e : tid * EL + e;
+    }
+    const int len = a.lens[b];
+    int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
+    if (n > a.max_blocks) n = a.max_blocks;
+    int32_t* oi = a.out_idx + ((int64_t)b * a.Ho + ho) * a.k;
+    int32_t* os = a.out_score ? a.out_score + ((int64_t)b * a.Ho + ho) * a.k : nullptr;
+    const int kk = a.k < n ? a.k : n;
+    for (int i = kk + tid; i < a.k; i += kThreads) {
+        oi[i] = -1;
+        if (os) os[i] = 0;
+    }
+    if (n == 0) return;  // the same for every thread of the row
+    if (reduce) {
+        for (int h0 = 1; h0 < a.Hkv; h0 += 8) {
+            int o[8][EL];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int hh = h0 + u < a.Hkv ? h0 + u : 0;
+#pragma unroll
+                for (int e = 0; e < EL; ++e) {
+                    const int j = tid * EL + e;
+                    o[u][e] = row[(int64_t)hh * a.max_blocks + (j < a.max_blocks ? j : 0)];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int e = 0; e < EL; ++e) v[e] = o[u][e] > v[e] ? o[u][e] : v[e];
+        }
+    }
+    int lo = 0x7fffffff, hi = -0x7fffffff;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        if (tid * EL + e >= n) v[e] = -0x7fffffff;  // below every real score (>= -1): never selected
+        else lo = v[e] < lo ? v[e] : lo;
+        hi = v[e] > hi ? v[e] : hi;
+    }
+#pragma unroll
+    for (int st = 1; st < kWave; st <<= 1) {
+        const int l2 = __shfl_xor(lo, st), h2 = __shfl_xor(hi, st);
+        lo = l2 < lo ? l2 : lo;
+        hi = h2 > hi ? h2 : hi;
+    }
+    if (lane == 0) {
+        ext[0][wid] = lo;
+        ext[1][wid] = hi;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        lo = ext[0][w] < lo ? ext[0][w] : lo;
+        hi = ext[1][w] > hi ? ext[1][w] : hi;
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    hi = __builtin_amdgcn_readfirstlane(hi);
+    // count of scores >= t over the whole row; `step` alternates the LDS buffer
+    int step = 0;
+    auto count_ge = [&](int t) {
+        int c = 0;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) c += __popcll(__ballot(v[e] >= t));
+        int* buf = cnt[step & 1];
+        ++step;
+        if (lane == 0) buf[wid] = c;
+        __syncthreads();
+        return buf[0] + buf[1] + buf[2] + buf[3];
+    };
+    while (lo < hi) {  // count_ge(lo) >= kk always holds
+        const int mid = lo + ((hi - lo + 1) >> 1);
+        if (count_ge(mid) >= kk) lo = mid;
+        else hi = mid - 1;
+    }
+    const int thr = lo;
+    const int need = kk - count_ge(thr + 1);  // ties at thr to take, lowest indices first
+    int eq = 0, gt = 0;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        eq += (v[e] == thr);
+        gt += (v[e] > thr);
+    }
+    int tot;
+    const int eq_before = block_exclusive_scan(eq, wsum, &tot);
+    int eq_take = need - eq_before;
+    eq_take = eq_take < 0 ? 0 : (eq_take > eq ? eq : eq_take);
+    int pos = block_exclusive_scan(gt + eq_take, wsum, &tot);
+    int eq_seen = 0;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+        bool take = v[e] > thr;
+        if (v[e] == thr) {
+            take = eq_seen < eq_take;
+            ++eq_seen;
+        }
+        if (take && pos < a.k) {
+            oi[pos] = tab[e];
+            if (os) os[pos] = (a.flags & UCM_TOPK_DISTANCE) ? a.full - v[e] : v[e];
+            ++pos;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // Per-token scores in the reference scorer's output shape.
 // ---------------------------------------------------------------------------------------
@@ -1818,12 +1952,17 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     const int rows_total = B * s.Ho;
     const dim3 wgrid((unsigned)ucm::ceil_div(rows_total, kThreads / kWave));
     if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256) {
+        // up to 256 blocks a wave per row stays ahead of a workgroup per row (config 2 step:
+        // 32.7 against 33.3 us)
         hipLaunchKernelGGL(select_wave_kernel<4>, wgrid, dim3(kThreads), 0, st, s, rows_total);
         return ucm::launch_status("select_wave_kernel");
     }
     if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 1024) {
-        hipLaunchKernelGGL(select_wave_kernel<16>, wgrid, dim3(kThreads), 0, st, s, rows_total);
-        return ucm::launch_status("select_wave_kernel");
+        if (max_blocks <= 512)
+            hipLaunchKernelGGL(select_group_kernel<2>, dim3((unsigned)rows_total), dim3(kThreads), 0, st, s);
+        else
+            hipLaunchKernelGGL(select_group_kernel<4>, dim3((unsigned)rows_total), dim3(kThreads), 0, st, s);
+        return ucm::launch_status("select_group_kernel");
     }
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
     return ucm::launch_status("select_kernel");
