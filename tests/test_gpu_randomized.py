@@ -306,8 +306,8 @@ def test_one_kv_head_random_configurations(seed):
 
 
 @pytest.mark.parametrize("seed", [71, 72])
-def test_topk_rows_of_257_to_1024_blocks(seed):
-    """Rows of 257 to 1024 blocks take the workgroup-per-row selection: ragged lengths, ties
+def test_topk_rows_of_257_to_4096_blocks(seed):
+    """Rows of 257 to 4096 blocks take the workgroup-per-row selection: ragged lengths, ties
     (low-entropy codes), every output flag, head reduction, k up to the row length."""
     from ucm_amd.sparse import hamming_topk
 
@@ -318,7 +318,7 @@ def test_topk_rows_of_257_to_1024_blocks(seed):
         G = int(rng.choice([1, 4, 16]))
         Wd = int(rng.choice([2, 4, 18])) if Hkv == 1 else 4
         BS = int(rng.choice([4, 8, 16]))
-        mb = int(rng.choice([257, 300, 511, 512, 513, 777, 1000, 1023, 1024]))
+        mb = int(rng.choice([257, 300, 511, 512, 513, 777, 1000, 1023, 1024, 1025, 2048, 2500, 4096]))
         NB = B * mb + 2
         kc = rng.integers(0, 2**32, size=(NB, BS, Hkv, Wd), dtype=np.uint32)
         if rng.integers(0, 2) == 0:

@@ -1351,8 +1351,8 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
     }
 }
 
-// Rows of 257 to 1024 block scores, index-ordered output: one workgroup per row, four scores
-// per thread.  Same algorithm as select_wave_kernel<16>, but a wave there runs some 2000
+// Rows of 257 to 4096 block scores, index-ordered output: one workgroup per row, EL = 2 to 16
+// scores per thread.  Same algorithm as select_wave_kernel<16>, but a wave there runs some 2000
 // instructions back to back for its row (7 us, however few rows there are); here each wave has
 // a quarter of the row and the four partial counts of a search step meet in LDS (two buffers
 // in turn, one barrier per step).
@@ -1957,11 +1957,16 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
         hipLaunchKernelGGL(select_wave_kernel<4>, wgrid, dim3(kThreads), 0, st, s, rows_total);
         return ucm::launch_status("select_wave_kernel");
     }
-    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 1024) {
+    if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 4096) {
+        const dim3 rgrid((unsigned)rows_total);
         if (max_blocks <= 512)
-            hipLaunchKernelGGL(select_group_kernel<2>, dim3((unsigned)rows_total), dim3(kThreads), 0, st, s);
+            hipLaunchKernelGGL(select_group_kernel<2>, rgrid, dim3(kThreads), 0, st, s);
+        else if (max_blocks <= 1024)
+            hipLaunchKernelGGL(select_group_kernel<4>, rgrid, dim3(kThreads), 0, st, s);
+        else if (max_blocks <= 2048)
+            hipLaunchKernelGGL(select_group_kernel<8>, rgrid, dim3(kThreads), 0, st, s);
         else
-            hipLaunchKernelGGL(select_group_kernel<4>, dim3((unsigned)rows_total), dim3(kThreads), 0, st, s);
+            hipLaunchKernelGGL(select_group_kernel<16>, rgrid, dim3(kThreads), 0, st, s);
         return ucm::launch_status("select_group_kernel");
     }
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
