@@ -362,7 +362,18 @@ def extras(torch, enc_k, gen):
     q6 = codes((b5, 64, wd6))
     ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6, table6, lens5, 128))
     ms_tok = graph_ms(torch, lambda i: hamming_score(cache6, q6, table6, lens5, ctx5, 0, 0, False), reps=5)
+    # the whole decode step of that layout in one native call: both parts of 16 new keys into the cache,
+    # both parts of the 16 x 64 query rows hashed, score, select
+    from ucm_amd.sparse import SparseDecodeStepMLA
+    bf = lambda *shape: torch.randn(*shape, device="cuda", dtype=torch.bfloat16, generator=gen)
+    stm = SparseDecodeStepMLA(bf(512, 512), bf(64, 64), 64, b5, ctx5 // bs5, 128, block_size=bs5,
+                              sink_token=bs5, recent_token=4 * bs5, return_physical=True)
+    kn6, kr6, qn6, qr6 = bf(b5, 512), bf(b5, 64), bf(b5, 64, 512), bf(b5, 64, 64)
+    slots6 = (table6[:, -1].to(torch.int64) * bs5 + bs5 - 1)
+    cache6v = cache6.view(cache6.shape[0], bs5, wd6)
+    ms_step = graph_ms(torch, lambda i: stm.step(kn6, kr6, slots6, qn6, qr6, cache6v, table6, lens5))
     out["mla_576bit_64heads"] = {"tokens": b5 * ctx5, "topk128_ms": ms, "token_scores_ms": ms_tok,
+                                 "decode_step_ms": ms_step,
                                  "tokens_per_s": b5 * ctx5 / ms * 1e3,
                                  "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6}
     del cache6, table6

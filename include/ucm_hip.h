@@ -235,6 +235,37 @@ int ucm_sparse_decode_step(const void* new_keys, int64_t T, int64_t k_stride_t, 
                            uint32_t* q_codes, int32_t* out_idx, int32_t* out_score,
                            void* workspace, size_t workspace_bytes, ucm_stream_t stream);
 
+/*
+ * The same single call for the latent-attention (MLA) layout: one KV head whose code is the
+ * nope part's hash followed by the rope part's hash (GSAOnDevice with is_mla,
+ * ucm/sparse/gsa_on_device/gsa_on_device.py:426-455 cache_k_hash_mla_cuda — hash_code followed by
+ * vLLM's concat_and_cache_mla — and :667-709 update_decode_topk_mla_cuda).  Each part has its own
+ * projection matrix; both parts of the step's new keys go to the paged code cache, both parts
+ * of the (already head-reduced, :376-393) queries to q_codes, then score and select.
+ *
+ * new_nope [T, K_nope], new_rope [T, K_rope] (row strides in elements), slot_mapping [T];
+ * T = 0 skips the cache update.  q_nope [B, Hq, K_nope], q_rope [B, Hq, K_rope].
+ * w_nope [K_nope, N_nope_bits], w_rope [K_rope, N_rope_bits].
+ * k_cache  uint32 [NB, BS, Wd] with Wd = (N_nope_bits + N_rope_bits) / 32, strides in words.
+ * q_codes  uint32 [B, Hq, Wd] contiguous scratch.  Remaining arguments as in ucm_hamming_topk
+ * with Hkv = 1.
+ */
+int ucm_sparse_decode_step_mla(const void* new_nope, int64_t nope_stride_t,
+                               const void* new_rope, int64_t rope_stride_t, int64_t T,
+                               const void* slot_mapping, int slot_is_i64,
+                               const void* q_nope, int64_t qn_stride_b, int64_t qn_stride_h,
+                               const void* q_rope, int64_t qr_stride_b, int64_t qr_stride_h,
+                               int x_dtype, int32_t K_nope, int32_t K_rope,
+                               const void* w_nope, const void* w_rope, int w_dtype,
+                               int32_t N_nope_bits, int32_t N_rope_bits,
+                               uint32_t* k_cache, int64_t NB, int32_t BS,
+                               int64_t ks_block, int64_t ks_token,
+                               const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                               const int32_t* seq_lens, int32_t B, int32_t Hq, int32_t k,
+                               int32_t sink_tok, int32_t recent_tok, uint32_t flags,
+                               uint32_t* q_codes, int32_t* out_idx, int32_t* out_score,
+                               void* workspace, size_t workspace_bytes, ucm_stream_t stream);
+
 /* Replaces update_seq_lens (hamming_topk.py:7-12):
  * out[b] = len[b] - ceil(max(len[b] - topk_tok, 0) / BS) * BS. */
 int ucm_update_seq_lens(const int32_t* seq_lens, int32_t B, int32_t topk_tok, int32_t BS,

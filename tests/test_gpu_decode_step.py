@@ -135,3 +135,57 @@ def test_argument_errors():
         st.step(keys, slots, qs, cache, table.to(torch.int64), lens)
     with pytest.raises(ValueError):
         SparseDecodeStep(W[:3], 32, 8, 4, 6, 3)
+
+
+@pytest.mark.parametrize("Hq,T", [(64, 4), (8, 4), (1, 0), (128, 4)])
+def test_fused_latent_attention_step_equals_separate_operators_and_oracle(Hq, T):
+    """MLA: nope (512) + rope (64) encoders, 18-word codes, one KV head; the fused call must
+    leave the same codes in the cache and return the same blocks as the separate operators;
+    the replayed HIP graph of it must agree with the eager call."""
+    from ucm_amd.sparse import HashEncoder, SparseDecodeStepMLA, hamming_topk
+
+    rng = rng_for(91 + Hq)
+    B, BS, nblk, K = 4, 64, 20, 5
+    NB = B * nblk + 3
+    dev = torch.device("cuda:0")
+    en = HashEncoder(512, 512, torch.bfloat16, dev)
+    er = HashEncoder(64, 64, torch.bfloat16, dev)
+    cache = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=(NB, BS, 18), dtype=np.int64)
+                             .astype(np.int32)).cuda()
+    table = torch.from_numpy(rng.permutation(NB)[: B * nblk].astype(np.int32).reshape(B, nblk)).cuda()
+    lens = torch.from_numpy(rng.integers((nblk - 1) * BS + 1, nblk * BS + 1, size=B).astype(np.int32)).cuda()
+    bf = lambda shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(torch.bfloat16).cuda()
+    kn, kr, qn, qr = bf((B, 512)), bf((B, 64)), bf((B, Hq, 512)), bf((B, Hq, 64))
+    pos = lens.to(torch.int64) - 1
+    slots = table[torch.arange(B), (pos // BS)].to(torch.int64) * BS + pos % BS
+    cache2 = cache.clone()
+    st = SparseDecodeStepMLA(en.hash_weights, er.hash_weights, Hq, B, nblk, K, block_size=BS,
+                             sink_token=BS, recent_token=4 * BS, return_physical=True)
+    args = (kn[:T] if T else None, kr[:T] if T else None, slots[:T] if T else None, qn, qr, cache, table, lens)
+    idx, sc = st.step(*args)
+    torch.cuda.synchronize()
+    idx, sc = idx.clone(), sc.clone()
+    # separate operators
+    u8 = cache2.view(torch.uint8).unsqueeze(2)
+    if T:
+        en.compute_hash_and_cache(kn[:T, None], slots[:T], u8[..., :64], BS)
+        er.compute_hash_and_cache(kr[:T, None], slots[:T], u8[..., 64:], BS)
+    qc = torch.cat([en.compute_hash(qn), er.compute_hash(qr)], dim=-1).view(torch.int32)
+    i2, s2 = hamming_topk(qc, cache2.unsqueeze(2), table, lens, K, BS, 4 * BS, return_physical=True)
+    assert torch.equal(cache, cache2)
+    assert torch.equal(st.q_codes, qc)
+    assert torch.equal(idx, i2) and torch.equal(sc, s2)
+    oi, osc = c_api.hamming_topk(qc.cpu().numpy().view(np.uint32),
+                                 cache.cpu().numpy().view(np.uint32).reshape(NB, BS, 1, 18),
+                                 table.cpu().numpy(), lens.cpu().numpy(), K, BS, 4 * BS, flags=c_api.F_PHYSICAL)
+    assert np.array_equal(idx.cpu().numpy(), oi) and np.array_equal(sc.cpu().numpy(), osc)
+    # graph replays (the step allocates nothing)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        st.step(*args)
+    for _ in range(3):
+        st.out_idx.fill_(-7)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(st.out_idx, idx) and torch.equal(st.out_score, sc)

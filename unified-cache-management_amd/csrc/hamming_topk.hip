@@ -1995,12 +1995,47 @@ extern "C" int ucm_sparse_decode_step(const void* new_keys, int64_t T, int64_t k
     const int32_t Wd = N_bits / 32;
     int rc = ucm::encode_pair(new_keys, T, Hkv, k_stride_t, k_stride_h, slot_mapping, slot_is_i64,
                               k_cache, NB, BS, ks_block, ks_token, ks_head, queries, B, Hq,
-                              q_stride_b, q_stride_h, q_codes, x_dtype, K, w, w_dtype, n_w, N_bits,
-                              (hipStream_t)stream);
+                              q_stride_b, q_stride_h, q_codes, (int64_t)Hq * Wd, Wd, x_dtype, K, w,
+                              w_dtype, n_w, N_bits, (hipStream_t)stream);
     if (rc != UCM_OK) return rc;
     return ucm_hamming_topk(q_codes, (int64_t)Hq * Wd, Wd, k_cache, NB, BS, Hkv, Wd, ks_block,
                             ks_token, ks_head, block_table, table_stride, max_blocks, seq_lens, B,
                             Hq, k, sink_tok, recent_tok, flags, out_idx, out_score, workspace,
+                            workspace_bytes, stream);
+}
+
+extern "C" int ucm_sparse_decode_step_mla(
+    const void* new_nope, int64_t nope_stride_t, const void* new_rope, int64_t rope_stride_t, int64_t T,
+    const void* slot_mapping, int slot_is_i64, const void* q_nope, int64_t qn_stride_b,
+    int64_t qn_stride_h, const void* q_rope, int64_t qr_stride_b, int64_t qr_stride_h, int x_dtype,
+    int32_t K_nope, int32_t K_rope, const void* w_nope, const void* w_rope, int w_dtype,
+    int32_t N_nope_bits, int32_t N_rope_bits, uint32_t* k_cache, int64_t NB, int32_t BS,
+    int64_t ks_block, int64_t ks_token, const int32_t* block_table, int32_t table_stride,
+    int32_t max_blocks, const int32_t* seq_lens, int32_t B, int32_t Hq, int32_t k, int32_t sink_tok,
+    int32_t recent_tok, uint32_t flags, uint32_t* q_codes, int32_t* out_idx, int32_t* out_score,
+    void* workspace, size_t workspace_bytes, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(Hq > 0, "bad head count");
+    UCM_REQUIRE(N_nope_bits > 0 && N_nope_bits % 32 == 0 && N_rope_bits > 0 && N_rope_bits % 32 == 0,
+                "hash_bits of both parts must be multiples of 32");
+    UCM_REQUIRE(q_codes && k_cache, "q_codes or k_cache is null");
+    const int32_t Wn = N_nope_bits / 32, Wd = Wn + N_rope_bits / 32;
+    UCM_REQUIRE(ks_token >= Wd, "cache rows of %lld words do not hold %d-word codes", (long long)ks_token, Wd);
+    // nope part: words [0, Wn) of every code; rope part: words [Wn, Wd)
+    int rc = ucm::encode_pair(new_nope, T, 1, nope_stride_t, 0, slot_mapping, slot_is_i64, k_cache, NB,
+                              BS, ks_block, ks_token, ks_token, q_nope, B, Hq, qn_stride_b, qn_stride_h,
+                              q_codes, (int64_t)Hq * Wd, Wd, x_dtype, K_nope, w_nope, w_dtype, 1,
+                              N_nope_bits, (hipStream_t)stream);
+    if (rc != UCM_OK) return rc;
+    rc = ucm::encode_pair(new_rope, T, 1, rope_stride_t, 0, slot_mapping, slot_is_i64, k_cache + Wn, NB,
+                          BS, ks_block, ks_token, ks_token, q_rope, B, Hq, qr_stride_b, qr_stride_h,
+                          q_codes + Wn, (int64_t)Hq * Wd, Wd, x_dtype, K_rope, w_rope, w_dtype, 1,
+                          N_rope_bits, (hipStream_t)stream);
+    if (rc != UCM_OK) return rc;
+    return ucm_hamming_topk(q_codes, (int64_t)Hq * Wd, Wd, k_cache, NB, BS, 1, Wd, ks_block, ks_token,
+                            ks_token, block_table, table_stride, max_blocks, seq_lens, B, Hq, k,
+                            sink_tok, recent_tok, flags, out_idx, out_score, workspace,
                             workspace_bytes, stream);
 }
 

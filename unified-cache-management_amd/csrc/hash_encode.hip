@@ -1006,14 +1006,14 @@ namespace ucm {
 int encode_pair(const void* keys, int64_t T, int Hkv, int64_t k_stride_t, int64_t k_stride_h,
                 const void* slot, int slot_is_i64, uint32_t* cache, int64_t NB, int BS,
                 int64_t cs_block, int64_t cs_token, int64_t cs_head, const void* queries, int64_t B,
-                int Hq, int64_t q_stride_b, int64_t q_stride_h, uint32_t* q_codes, int x_dtype,
+                int Hq, int64_t q_stride_b, int64_t q_stride_h, uint32_t* q_codes,
+                int64_t qc_stride_b, int64_t qc_stride_h, int x_dtype,
                 int K, const void* w, int w_dtype, int n_w, int N_bits, hipStream_t st)
 {
-    const int Wd = N_bits / 32;
     EncArgs kq{};
     kq.x = queries; kq.T = B; kq.H = Hq; kq.K = K; kq.x_stride_t = q_stride_b; kq.x_stride_h = q_stride_h;
     kq.w = w; kq.n_w = n_w; kq.heads_per_w = n_w > 1 ? Hq / Hkv : 0; kq.N = N_bits;
-    kq.out = q_codes; kq.out_stride_t = (int64_t)Hq * Wd; kq.out_stride_h = Wd;
+    kq.out = q_codes; kq.out_stride_t = qc_stride_b; kq.out_stride_h = qc_stride_h;
     int rc = check_shape(kq, x_dtype, w_dtype);
     if (rc != UCM_OK) return rc;
     if (T <= 0) return encode_common(kq, x_dtype, w_dtype, st);

@@ -97,3 +97,74 @@ class SparseDecodeStep:
             return result
 
         return run
+
+
+class SparseDecodeStepMLA:
+    """One latent-attention (MLA) decode step of the retrieval path in a single native call:
+    cache_k_hash_mla_cuda (gsa_on_device.py:426-455) followed by update_decode_topk_mla_cuda
+    (:667-709).  The code of a token is the hash of its latent vector (nope) followed by the hash
+    of its rope part; the queries are the already head-reduced q_nope / q_pe.  All buffers are
+    allocated in the constructor; `step` allocates nothing."""
+
+    def __init__(self, w_nope, w_rope, num_q_heads, batch, max_blocks, topk_blocks, block_size=64,
+                 sink_token=0, recent_token=0, return_physical=False):
+        """w_nope [K_nope, N_nope], w_rope [K_rope, N_rope]: the two encoders' projections."""
+        if w_nope.dtype != w_rope.dtype or w_nope.dtype not in _DT:
+            raise ValueError("both projections must share one supported dtype")
+        if w_nope.dim() != 2 or w_rope.dim() != 2:
+            raise ValueError("projections must be [K, N]")
+        self.wn, self.wr = w_nope.contiguous(), w_rope.contiguous()
+        self.Kn, self.Nn = (int(v) for v in w_nope.shape)
+        self.Kr, self.Nr = (int(v) for v in w_rope.shape)
+        if self.Nn % 32 or self.Nr % 32:
+            raise ValueError("hash_bits of both parts must be multiples of 32")
+        self.Wd = (self.Nn + self.Nr) // 32
+        self.Hq, self.B = int(num_q_heads), int(batch)
+        self.max_blocks, self.k, self.BS = int(max_blocks), int(topk_blocks), int(block_size)
+        self.sink, self.recent = int(sink_token), int(recent_token)
+        self.flags = _lib.TOPK_RETURN_PHYSICAL if return_physical else 0
+        dev = w_nope.device
+        self.q_codes = torch.empty((self.B, self.Hq, self.Wd), dtype=torch.int32, device=dev)
+        self.out_idx = torch.empty((self.B, 1, self.k), dtype=torch.int32, device=dev)
+        self.out_score = torch.empty_like(self.out_idx)
+        nbytes = _lib.lib().ucm_hamming_topk_workspace_bytes(self.B, 1, self.max_blocks)
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+    def step(self, new_nope, new_rope, slot_mapping, q_nope, q_rope, k_hash_cache, block_table,
+             seq_lens):
+        """new_nope [T,K_nope], new_rope [T,K_rope] + slot_mapping [T] (T may be 0);
+        q_nope [B,Hq,K_nope], q_rope [B,Hq,K_rope]; k_hash_cache int32 [NB,BS,Wd];
+        block_table int32 [B,max_blocks]; seq_lens int32 [B].
+        Returns (indices, scores) int32 [B, 1, k]: views of buffers reused by every call."""
+        dt = self.wn.dtype
+        T = 0 if new_nope is None else int(new_nope.shape[0])
+        for t in (q_nope, q_rope) + ((new_nope, new_rope) if T else ()):
+            if t.dtype != dt or t.stride(-1) != 1:
+                raise ValueError("keys, queries and weights must share one dtype and have contiguous rows")
+        if tuple(q_nope.shape) != (self.B, self.Hq, self.Kn) or tuple(q_rope.shape) != (self.B, self.Hq, self.Kr):
+            raise ValueError("queries must be [B,Hq,K_nope] and [B,Hq,K_rope]")
+        if k_hash_cache.dtype != torch.int32 or k_hash_cache.dim() != 3 or k_hash_cache.shape[1] != self.BS \
+                or k_hash_cache.shape[2] != self.Wd or k_hash_cache.stride(-1) != 1:
+            raise ValueError(f"k_hash_cache must be int32 [NB,{self.BS},{self.Wd}]")
+        if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
+            raise ValueError("block_table and seq_lens must be int32")
+        if block_table.shape[0] != self.B or block_table.shape[1] < self.max_blocks or block_table.stride(-1) != 1:
+            raise ValueError("block_table must be [B, >= max_blocks]")
+        if T:
+            if tuple(new_nope.shape) != (T, self.Kn) or tuple(new_rope.shape) != (T, self.Kr):
+                raise ValueError("new keys must be [T,K_nope] and [T,K_rope]")
+            if slot_mapping.dtype not in (torch.int32, torch.int64) or slot_mapping.numel() != T:
+                raise ValueError("slot_mapping must be int32/int64 [T]")
+        s = _lib.stride
+        _lib.check(_lib.lib().ucm_sparse_decode_step_mla(
+            new_nope.data_ptr() if T else None, s(new_nope, 0) if T else 0,
+            new_rope.data_ptr() if T else None, s(new_rope, 0) if T else 0, T,
+            slot_mapping.data_ptr() if T else None, int(T > 0 and slot_mapping.dtype == torch.int64),
+            q_nope.data_ptr(), s(q_nope, 0), s(q_nope, 1), q_rope.data_ptr(), s(q_rope, 0), s(q_rope, 1),
+            _DT[dt], self.Kn, self.Kr, self.wn.data_ptr(), self.wr.data_ptr(), _DT[dt], self.Nn, self.Nr,
+            k_hash_cache.data_ptr(), k_hash_cache.shape[0], self.BS, s(k_hash_cache, 0), s(k_hash_cache, 1),
+            block_table.data_ptr(), max(s(block_table, 0), self.max_blocks), self.max_blocks,
+            seq_lens.data_ptr(), self.B, self.Hq, self.k, self.sink, self.recent, self.flags,
+            self.q_codes.data_ptr(), self.out_idx.data_ptr(), self.out_score.data_ptr(),
+            self.workspace.data_ptr(), self.workspace.numel(), _lib.stream_ptr(q_nope.device)))
+        return self.out_idx, self.out_score
