@@ -197,20 +197,44 @@ __device__ __forceinline__ uint32_t* row_dst(const EncArgs& a, int64_t t, int h)
 // between a compare and the use of its mask, are inserted by the compiler only for
 // instructions it can see.
 //
-// Half of the row's word: bit 8g + j is the sign of accumulator 4g + j (g, j in 0..3).  Two
+// The matrix-core kernels start every accumulator at the smallest negative normal number
+// instead of zero.  A projection that is exactly zero (an all-zero row) then stays negative,
+// any other projection keeps its sign (|p| would have to be below 1.2e-38 to lose it), and
+// "projection > 0" becomes "sign bit clear": one funnel shift per accumulator instead of a
+// compare, a select and an or.  NaN is the one value whose sign bit says nothing; a row with a
+// NaN input has NaN in every accumulator, so one accumulator per row is tested and the row's
+// bits are cleared, as `NaN > 0` is false.
+constexpr float kAccStart = -1.17549435e-38f;
+
+__device__ __forceinline__ f32x16 acc_start()
+{
+    f32x16 a;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = kAccStart;
+    return a;
+}
+
+// Half of the row's word: bit 8g + j is "accumulator 4g + j is positive" (g, j in 0..3).  Two
 // independent chains (g = 3,2 and g = 1,0) halve the dependent-instruction latency.
 __device__ __forceinline__ uint32_t pack_half(const f32x16& acc)
 {
-    uint32_t hi = 0, lo = 0;
+    uint32_t hi = 0, lo = 0;  // collect the sign bits: x = (x << 1) | sign
 #pragma unroll
     for (int g = 1; g >= 0; --g) {
+        if (g == 0) {
+            hi <<= 4;
+            lo <<= 4;
+        }
 #pragma unroll
         for (int j = 3; j >= 0; --j) {
-            hi |= (acc[4 * (g + 2) + j] > 0.0f ? 1u : 0u) << (8 * g + j);
-            lo |= (acc[4 * g + j] > 0.0f ? 1u : 0u) << (8 * g + j);
+            hi = __builtin_amdgcn_alignbit(hi, __float_as_uint(acc[4 * (g + 2) + j]), 31);
+            lo = __builtin_amdgcn_alignbit(lo, __float_as_uint(acc[4 * g + j]), 31);
         }
     }
-    return (hi << 16) | lo;
+    // positive = sign bit clear: flip the 16 collected bits
+    const uint32_t neg = (hi << 16) | lo;
+    const uint32_t word = neg ^ 0x0F0F0F0Fu;
+    return acc[0] != acc[0] ? 0u : word;
 }
 
 // Lanes l and l+32 hold the two interleaved halves (nibbles 0,2,4,6 and 1,3,5,7) of row l%32's
@@ -427,7 +451,7 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
 
     // 32 hash columns x 32 rows: K/16 MFMAs into one accumulator tile
     auto project = [&](int nt) {
-        f32x16 acc = {0};
+        f32x16 acc = acc_start();
         const uint16_t* bp = wt + (nt * 32 + r) * KP + kb * 8;
 #pragma unroll
         for (int k0 = 0; k0 < KS; k0 += 4) {
@@ -561,7 +585,7 @@ __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
 #pragma unroll
         for (int i = 0; i < 8; ++i) bw[ks][i] = wsrc[(int64_t)(ks * 16 + kb * 8 + i) * a.N];
 
-    f32x16 acc = {0};
+    f32x16 acc = acc_start();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         V bv;
