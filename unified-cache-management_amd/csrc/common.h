@@ -45,13 +45,19 @@ inline int launch_status(const char* kernel)
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// hash_encode.hip: new keys -> paged cache and queries -> codes at q_codes + b * qc_stride_b +
-// h * qc_stride_h (32-bit words), one launch when small
-int encode_pair(const void* keys, int64_t T, int Hkv, int64_t k_stride_t, int64_t k_stride_h,
-                const void* slot, int slot_is_i64, uint32_t* cache, int64_t NB, int BS,
-                int64_t cs_block, int64_t cs_token, int64_t cs_head, const void* queries, int64_t B,
-                int Hq, int64_t q_stride_b, int64_t q_stride_h, uint32_t* q_codes,
-                int64_t qc_stride_b, int64_t qc_stride_h, int x_dtype,
-                int K, const void* w, int w_dtype, int n_w, int N_bits, hipStream_t st);
+// hash_encode.hip: one (new keys -> paged cache, queries -> codes) pair of a decode step.
+// Strides of keys and queries in elements, of the cache and of q_codes in 32-bit words.
+struct PairSpec {
+    const void* keys; int64_t T; int Hkv; int64_t k_stride_t, k_stride_h;
+    const void* slot; int slot_is_i64;
+    uint32_t* cache; int64_t NB; int BS; int64_t cs_block, cs_token, cs_head;
+    const void* queries; int64_t B; int Hq; int64_t q_stride_b, q_stride_h;
+    uint32_t* q_codes; int64_t qc_stride_b, qc_stride_h;
+    int x_dtype; int K; const void* w; int w_dtype; int n_w; int N_bits;
+};
+// one launch when both jobs are small
+int encode_pair(const PairSpec& p, hipStream_t st);
+// two pairs; one launch when all four jobs are small and the input widths are 512 and 64
+int encode_two_pairs(const PairSpec& a, const PairSpec& b, hipStream_t st);
 
 }  // namespace ucm

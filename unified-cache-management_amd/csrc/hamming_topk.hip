@@ -1993,10 +1993,11 @@ extern "C" int ucm_sparse_decode_step(const void* new_keys, int64_t T, int64_t k
     UCM_REQUIRE(n_w == 1 || n_w == Hkv, "n_w must be 1 or the number of KV heads");
     UCM_REQUIRE(q_codes, "q_codes is null");
     const int32_t Wd = N_bits / 32;
-    int rc = ucm::encode_pair(new_keys, T, Hkv, k_stride_t, k_stride_h, slot_mapping, slot_is_i64,
-                              k_cache, NB, BS, ks_block, ks_token, ks_head, queries, B, Hq,
-                              q_stride_b, q_stride_h, q_codes, (int64_t)Hq * Wd, Wd, x_dtype, K, w,
-                              w_dtype, n_w, N_bits, (hipStream_t)stream);
+    const ucm::PairSpec spec{new_keys, T, Hkv, k_stride_t, k_stride_h, slot_mapping, slot_is_i64,
+                             k_cache, NB, BS, ks_block, ks_token, ks_head, queries, B, Hq,
+                             q_stride_b, q_stride_h, q_codes, (int64_t)Hq * Wd, Wd, x_dtype, K, w,
+                             w_dtype, n_w, N_bits};
+    int rc = ucm::encode_pair(spec, (hipStream_t)stream);
     if (rc != UCM_OK) return rc;
     return ucm_hamming_topk(q_codes, (int64_t)Hq * Wd, Wd, k_cache, NB, BS, Hkv, Wd, ks_block,
                             ks_token, ks_head, block_table, table_stride, max_blocks, seq_lens, B,
@@ -2023,15 +2024,15 @@ extern "C" int ucm_sparse_decode_step_mla(
     const int32_t Wn = N_nope_bits / 32, Wd = Wn + N_rope_bits / 32;
     UCM_REQUIRE(ks_token >= Wd, "cache rows of %lld words do not hold %d-word codes", (long long)ks_token, Wd);
     // nope part: words [0, Wn) of every code; rope part: words [Wn, Wd)
-    int rc = ucm::encode_pair(new_nope, T, 1, nope_stride_t, 0, slot_mapping, slot_is_i64, k_cache, NB,
-                              BS, ks_block, ks_token, ks_token, q_nope, B, Hq, qn_stride_b, qn_stride_h,
-                              q_codes, (int64_t)Hq * Wd, Wd, x_dtype, K_nope, w_nope, w_dtype, 1,
-                              N_nope_bits, (hipStream_t)stream);
-    if (rc != UCM_OK) return rc;
-    rc = ucm::encode_pair(new_rope, T, 1, rope_stride_t, 0, slot_mapping, slot_is_i64, k_cache + Wn, NB,
-                          BS, ks_block, ks_token, ks_token, q_rope, B, Hq, qr_stride_b, qr_stride_h,
-                          q_codes + Wn, (int64_t)Hq * Wd, Wd, x_dtype, K_rope, w_rope, w_dtype, 1,
-                          N_rope_bits, (hipStream_t)stream);
+    const ucm::PairSpec nope{new_nope, T, 1, nope_stride_t, 0, slot_mapping, slot_is_i64, k_cache, NB, BS,
+                             ks_block, ks_token, ks_token, q_nope, B, Hq, qn_stride_b, qn_stride_h,
+                             q_codes, (int64_t)Hq * Wd, Wd, x_dtype, K_nope, w_nope, w_dtype, 1,
+                             N_nope_bits};
+    const ucm::PairSpec rope{new_rope, T, 1, rope_stride_t, 0, slot_mapping, slot_is_i64, k_cache + Wn, NB,
+                             BS, ks_block, ks_token, ks_token, q_rope, B, Hq, qr_stride_b, qr_stride_h,
+                             q_codes + Wn, (int64_t)Hq * Wd, Wd, x_dtype, K_rope, w_rope, w_dtype, 1,
+                             N_rope_bits};
+    const int rc = ucm::encode_two_pairs(nope, rope, (hipStream_t)stream);
     if (rc != UCM_OK) return rc;
     return ucm_hamming_topk(q_codes, (int64_t)Hq * Wd, Wd, k_cache, NB, BS, 1, Wd, ks_block, ks_token,
                             ks_token, block_table, table_stride, max_blocks, seq_lens, B, Hq, k,

@@ -552,13 +552,11 @@ struct EncJobs {
     int waves0;  // waves of job 0; waves >= waves0 belong to job 1
 };
 
+// One wave's tile of job `a`: wave index wv counts (row tile, head, 32-column tile), columns fastest.
 template <typename V, int KS>
-__global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
+__device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
 {
     constexpr int K = KS * 16;
-    const bool second = (int)blockIdx.x >= js.waves0;
-    const EncArgs& a = second ? js.job[1] : js.job[0];
-    int wv = second ? blockIdx.x - js.waves0 : blockIdx.x;
     const int ntiles = a.N / 32;
     const int nt = wv % ntiles;
     wv /= ntiles;
@@ -597,6 +595,34 @@ __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
     if (row_ok && lane < 32) {
         uint32_t* dst = row_dst(a, t, h);
         if (dst) dst[nt] = word;
+    }
+}
+
+template <typename V, int KS>
+__global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
+{
+    const bool second = (int)blockIdx.x >= js.waves0;
+    encode_small_body<V, KS>(second ? js.job[1] : js.job[0],
+                             second ? blockIdx.x - js.waves0 : blockIdx.x);
+}
+
+// Four jobs in one launch, two of input width 16 * KSA and two of 16 * KSB (the two parts of a
+// latent-attention step: new keys and queries of the nope and of the rope encoder).
+struct EncJobs4 {
+    EncArgs job[4];
+    int end[4];  // first wave index past job i
+};
+
+template <typename V, int KSA, int KSB>
+__global__ __launch_bounds__(64) void encode_small_mixed_kernel(EncJobs4 js)
+{
+    const int w = blockIdx.x;
+    if (w < js.end[1]) {
+        const int j = w >= js.end[0] ? 1 : 0;
+        encode_small_body<V, KSA>(js.job[j], j ? w - js.end[0] : w);
+    } else {
+        const int j = w >= js.end[2] ? 3 : 2;
+        encode_small_body<V, KSB>(js.job[j], w - js.end[j - 1]);
     }
 }
 
@@ -1024,34 +1050,44 @@ extern "C" int ucm_code_scatter(const uint32_t* codes, int64_t T, int32_t H, int
     return ucm::launch_status("code_scatter_kernel");
 }
 
-// Encodes the step's new keys into the paged cache and the step's queries into a dense
-// tensor.  When both are small enough for the latency path they share one launch.
+// Encodes a step's new keys into the paged cache and its queries into a code tensor.  When both
+// are small enough for the latency path they share one launch; two such pairs of input widths
+// 512 and 64 (a latent-attention step) share one launch as well.
 namespace ucm {
-int encode_pair(const void* keys, int64_t T, int Hkv, int64_t k_stride_t, int64_t k_stride_h,
-                const void* slot, int slot_is_i64, uint32_t* cache, int64_t NB, int BS,
-                int64_t cs_block, int64_t cs_token, int64_t cs_head, const void* queries, int64_t B,
-                int Hq, int64_t q_stride_b, int64_t q_stride_h, uint32_t* q_codes,
-                int64_t qc_stride_b, int64_t qc_stride_h, int x_dtype,
-                int K, const void* w, int w_dtype, int n_w, int N_bits, hipStream_t st)
+namespace {
+// Fills the two jobs of a pair; has_keys = false when there are no new keys.
+int build_pair(const PairSpec& p, EncArgs& kk, EncArgs& kq, bool& has_keys)
 {
-    EncArgs kq{};
-    kq.x = queries; kq.T = B; kq.H = Hq; kq.K = K; kq.x_stride_t = q_stride_b; kq.x_stride_h = q_stride_h;
-    kq.w = w; kq.n_w = n_w; kq.heads_per_w = n_w > 1 ? Hq / Hkv : 0; kq.N = N_bits;
-    kq.out = q_codes; kq.out_stride_t = qc_stride_b; kq.out_stride_h = qc_stride_h;
-    int rc = check_shape(kq, x_dtype, w_dtype);
+    kq = EncArgs{};
+    kq.x = p.queries; kq.T = p.B; kq.H = p.Hq; kq.K = p.K; kq.x_stride_t = p.q_stride_b;
+    kq.x_stride_h = p.q_stride_h; kq.w = p.w; kq.n_w = p.n_w;
+    kq.heads_per_w = p.n_w > 1 ? p.Hq / p.Hkv : 0; kq.N = p.N_bits;
+    kq.out = p.q_codes; kq.out_stride_t = p.qc_stride_b; kq.out_stride_h = p.qc_stride_h;
+    int rc = check_shape(kq, p.x_dtype, p.w_dtype);
     if (rc != UCM_OK) return rc;
-    if (T <= 0) return encode_common(kq, x_dtype, w_dtype, st);
+    has_keys = p.T > 0;
+    if (!has_keys) return UCM_OK;
+    kk = EncArgs{};
+    kk.x = p.keys; kk.T = p.T; kk.H = p.Hkv; kk.K = p.K; kk.x_stride_t = p.k_stride_t;
+    kk.x_stride_h = p.k_stride_h; kk.w = p.w; kk.n_w = p.n_w; kk.heads_per_w = p.n_w > 1 ? 1 : 0;
+    kk.N = p.N_bits; kk.slot = p.slot; kk.slot_is_i64 = p.slot_is_i64; kk.cache = p.cache;
+    kk.NB = p.NB; kk.BS = p.BS; kk.cs_block = p.cs_block; kk.cs_token = p.cs_token;
+    kk.cs_head = p.cs_head;
+    rc = check_shape(kk, p.x_dtype, p.w_dtype);
+    if (rc != UCM_OK) return rc;
+    return check_cache(p.slot, p.cache, p.NB, p.BS);
+}
 
-    EncArgs kk{};
-    kk.x = keys; kk.T = T; kk.H = Hkv; kk.K = K; kk.x_stride_t = k_stride_t; kk.x_stride_h = k_stride_h;
-    kk.w = w; kk.n_w = n_w; kk.heads_per_w = n_w > 1 ? 1 : 0; kk.N = N_bits;
-    kk.slot = slot; kk.slot_is_i64 = slot_is_i64; kk.cache = cache; kk.NB = NB; kk.BS = BS;
-    kk.cs_block = cs_block; kk.cs_token = cs_token; kk.cs_head = cs_head;
-    rc = check_shape(kk, x_dtype, w_dtype);
-    if (rc != UCM_OK) return rc;
-    rc = check_cache(slot, cache, NB, BS);
-    if (rc != UCM_OK) return rc;
-    if (B > 0 && small_eligible(kk, x_dtype, w_dtype) && small_eligible(kq, x_dtype, w_dtype)) {
+bool pair_is_small(const PairSpec& p, const EncArgs& kk, const EncArgs& kq, bool has_keys)
+{
+    return has_keys && p.B > 0 && small_eligible(kk, p.x_dtype, p.w_dtype) &&
+           small_eligible(kq, p.x_dtype, p.w_dtype);
+}
+
+int launch_pair(const PairSpec& p, EncArgs& kk, EncArgs& kq, bool has_keys, hipStream_t st)
+{
+    if (!has_keys) return encode_common(kq, p.x_dtype, p.w_dtype, st);
+    if (pair_is_small(p, kk, kq, has_keys)) {
         EncJobs js{};
         set_block_shift(kk);
         set_block_shift(kq);
@@ -1059,11 +1095,53 @@ int encode_pair(const void* keys, int64_t T, int Hkv, int64_t k_stride_t, int64_
         js.job[1] = kq;
         js.waves0 = (int)small_waves(kk);
         const int64_t waves = js.waves0 + small_waves(kq);
-        return x_dtype == UCM_DT_BF16 ? launch_small<bf16x8>(js, waves, K, st)
-                                      : launch_small<f16x8>(js, waves, K, st);
+        return p.x_dtype == UCM_DT_BF16 ? launch_small<bf16x8>(js, waves, p.K, st)
+                                        : launch_small<f16x8>(js, waves, p.K, st);
     }
-    rc = encode_common(kk, x_dtype, w_dtype, st);
+    const int rc = encode_common(kk, p.x_dtype, p.w_dtype, st);
     if (rc != UCM_OK) return rc;
-    return encode_common(kq, x_dtype, w_dtype, st);
+    return encode_common(kq, p.x_dtype, p.w_dtype, st);
+}
+}  // namespace
+
+int encode_pair(const PairSpec& p, hipStream_t st)
+{
+    EncArgs kk, kq;
+    bool has_keys;
+    const int rc = build_pair(p, kk, kq, has_keys);
+    if (rc != UCM_OK) return rc;
+    return launch_pair(p, kk, kq, has_keys, st);
+}
+
+int encode_two_pairs(const PairSpec& pa, const PairSpec& pb, hipStream_t st)
+{
+    EncArgs ka, qa, kb, qb;
+    bool ha, hb;
+    int rc = build_pair(pa, ka, qa, ha);
+    if (rc != UCM_OK) return rc;
+    rc = build_pair(pb, kb, qb, hb);
+    if (rc != UCM_OK) return rc;
+    if (pa.K == 512 && pb.K == 64 && pa.x_dtype == pb.x_dtype && pair_is_small(pa, ka, qa, ha) &&
+        pair_is_small(pb, kb, qb, hb)) {
+        EncJobs4 js{};
+        EncArgs* jobs[4] = {&ka, &qa, &kb, &qb};
+        int64_t end = 0;
+        for (int i = 0; i < 4; ++i) {
+            set_block_shift(*jobs[i]);
+            js.job[i] = *jobs[i];
+            end += small_waves(*jobs[i]);
+            js.end[i] = (int)end;
+        }
+        if (end <= 0x7fffffff) {
+            if (pa.x_dtype == UCM_DT_BF16)
+                hipLaunchKernelGGL((encode_small_mixed_kernel<bf16x8, 32, 4>), dim3((unsigned)end), dim3(64), 0, st, js);
+            else
+                hipLaunchKernelGGL((encode_small_mixed_kernel<f16x8, 32, 4>), dim3((unsigned)end), dim3(64), 0, st, js);
+            return ucm::launch_status("encode_small_mixed_kernel");
+        }
+    }
+    rc = launch_pair(pa, ka, qa, ha, st);
+    if (rc != UCM_OK) return rc;
+    return launch_pair(pb, kb, qb, hb, st);
 }
 }  // namespace ucm
