@@ -675,6 +675,87 @@ __global__ __launch_bounds__(kThreads) void block_score_rows(ScoreArgs a)
 }
 
 // ---------------------------------------------------------------------------------------
+// Blocks smaller than one 1 KiB run (e.g. 16-token blocks of one or two KV heads, the shape a
+// tensor-parallel rank sees with the serving engine's default block size): a run of 64 pieces
+// covers BPR = 2, 4 or 8 blocks, each read through its own table entry, and a wave owns four
+// runs.  Directly compared query codes only (G = 1, 2, 4).  The lanes of one block reduce among
+// themselves; no LDS, no barrier, no loop.
+// ---------------------------------------------------------------------------------------
+template <int CPU, int GP>
+__global__ __launch_bounds__(kThreads) void block_score_tiny(ScoreArgs a, int bpr_shift)
+{
+    const int b = blockIdx.y;
+    const int lane = lane_id();
+    const int BPR = 1 << bpr_shift;
+    const int LPB = kWave >> bpr_shift;      // pieces of one block
+    const int PERIOD = a.Hkv * CPU;          // pieces of one token (a power of two <= LPB)
+    const int sub = lane >> (6 - bpr_shift);  // the lane's block within a run
+    const int lb = lane & (LPB - 1);          // its piece within that block
+    const int pshift = __builtin_ctz((unsigned)PERIOD);
+    const int h = (lb & (PERIOD - 1)) / CPU, part = lb % CPU;
+    const int jw = (blockIdx.x * (kThreads / kWave) + wave_id()) * (4 * BPR);  // the wave's first block
+
+    int entry[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int j = jw + u * BPR + sub;
+        entry[u] = a.table ? a.table[(int64_t)b * a.table_stride + (j < a.max_blocks ? j : a.max_blocks - 1)] : 0;
+    }
+    const int len = a.lens[b];
+    uint32_t qr[GP][4];
+    {
+        const uint32_t* qp = a.q + b * a.q_stride_b + (int64_t)h * GP * a.q_stride_h + part * 4;
+#pragma unroll
+        for (int g = 0; g < GP; ++g)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[g][w] = qp[g * a.q_stride_h + w];
+    }
+    if ((int64_t)jw * a.BS >= len) return;  // the whole wave lies past the request's last block
+
+    int64_t pb[4];
+    u32x4 kv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int j = jw + u * BPR + sub;
+        int64_t v = a.table ? (int64_t)entry[u] : (int64_t)b * a.max_blocks + j;
+        if (j >= a.max_blocks || v < 0 || v >= a.NB) v = -1;
+        pb[u] = v;
+        kv[u] = code_load(reinterpret_cast<const u32x4*>(a.kc + (v < 0 ? 0 : v) * a.ks_block) + lb);
+    }
+    const int full = a.G * 32 * a.Wd;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int j = jw + u * BPR + sub;
+        const int pos0 = j * a.BS;
+        int d = 0;
+#pragma unroll
+        for (int g = 0; g < GP; ++g)
+            d += __popc(kv[u].x ^ qr[g][0]) + __popc(kv[u].y ^ qr[g][1]) + __popc(kv[u].z ^ qr[g][2]) +
+                 __popc(kv[u].w ^ qr[g][3]);
+        if (CPU >= 2) d += __shfl_xor(d, 1);
+        if (CPU >= 4) d += __shfl_xor(d, 2);
+        int m = (pos0 + (lb >> pshift) < len) ? d : kInf;
+        for (int st = PERIOD; st < LPB; st <<= 1) {  // over the block's tokens
+            const int o = __shfl_xor(m, st);
+            m = o < m ? o : m;
+        }
+        const int p1 = (pos0 + a.BS < len) ? pos0 + a.BS : len;
+        const bool forced = (pos0 < a.sink) || (p1 > len - a.recent);
+        const bool live = j < a.max_blocks && pos0 < len;
+        if (a.reduce_out) {
+            for (int st = CPU; st < PERIOD; st <<= 1) {  // over the heads
+                const int o = __shfl_xor(m, st);
+                m = o < m ? o : m;
+            }
+            if (lb == 0 && live)
+                a.scores[(int64_t)b * a.max_blocks + j] = pb[u] < 0 ? -1 : (forced ? full : full - m);
+        } else if (lb < PERIOD && part == 0 && live) {
+            a.scores[((int64_t)b * a.Hkv + h) * a.max_blocks + j] = pb[u] < 0 ? -1 : (forced ? full : full - m);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // One KV head and codes of an even number of words that the 16-byte kernels above cannot take
 // — above all the 18-word codes of a latent-attention cache (512 + 64 hash bits), where a
 // 16-byte piece would straddle two tokens.  The unit is the 8-byte piece: L = Wd / 2 consecutive
@@ -1744,6 +1825,26 @@ bool dispatch_one(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 
 bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
+// Blocks of 128, 256 or 512 bytes in the layout of the 16-byte-piece kernels, query codes
+// compared directly.
+bool tiny_layout(const ScoreArgs& a, const uint32_t* k_cache, bool direct)
+{
+    const int cpu = a.Wd / 4;
+    if (!direct || a.Wd % 4 || !(cpu == 1 || cpu == 2 || cpu == 4)) return false;
+    const int64_t pieces = (int64_t)a.BS * a.Hkv * cpu;
+    return a.ks_head == a.Wd && a.ks_token == (int64_t)a.Hkv * a.Wd && a.ks_block % 4 == 0 &&
+           (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 && is_pow2(a.Hkv * cpu) &&
+           is_pow2((int)pieces) && pieces >= 8 && pieces < kWave && a.Hkv * cpu <= pieces;
+}
+
+template <int CPU>
+void launch_tiny(const ScoreArgs& a, int bshift, dim3 grid, hipStream_t st)
+{
+    if (a.G == 1) launch_score(block_score_tiny<CPU, 1>, grid, 0, st, a, bshift);
+    else if (a.G == 2) launch_score(block_score_tiny<CPU, 2>, grid, 0, st, a, bshift);
+    else launch_score(block_score_tiny<CPU, 4>, grid, 0, st, a, bshift);
+}
+
 // Layout and shapes the code-per-lane kernels take (on top of pairs_layout): 18-word codes
 // with any group size, 8- and 16-word codes with bit planes (directly compared codes of those
 // widths have the 16-byte-piece kernels).
@@ -1907,6 +2008,18 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
             else if (cpu == 2) dispatch_fast<2>(a, pmax, split, u, grid, st);
             else dispatch_fast<4>(a, pmax, split, u, grid, st);
         }
+    } else if (tiny_layout(a, k_cache, direct_g)) {
+        // blocks below 1 KiB with directly compared query codes: several blocks per run of 64 pieces
+        const int pieces = BS * Hkv * cpu;
+        int bshift = 0;
+        while ((pieces << bshift) < kWave) ++bshift;
+        a.reduce_out = ((flags & UCM_TOPK_REDUCE_HEADS) && Hkv > 1) ? 1 : 0;
+        reduced_scores = a.reduce_out != 0;
+        const dim3 tgrid((unsigned)ucm::ceil_div(max_blocks, (kThreads / kWave) * (4 << bshift)), (unsigned)B);
+        if (cpu == 1) launch_tiny<1>(a, bshift, tgrid, st);
+        else if (cpu == 2) launch_tiny<2>(a, bshift, tgrid, st);
+        else launch_tiny<4>(a, bshift, tgrid, st);
+        a.reduce_out = 0;
     } else if (pairs_layout(a, k_cache)) {
         const int L = Wd / 2, TP = kWave / L;
         int pmax = 0;
