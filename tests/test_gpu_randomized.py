@@ -343,3 +343,51 @@ def test_topk_rows_of_257_to_4096_blocks(seed):
                               max_blocks=mb)
         assert np.array_equal(gi.cpu().numpy(), oi), what
         assert np.array_equal(gs.cpu().numpy(), osc), what
+
+
+@pytest.mark.parametrize("seed", [81, 82])
+def test_topk_blocks_below_one_kib(seed):
+    """Blocks of 128 to 512 bytes of codes (e.g. 16-token blocks of one or two KV heads, what a
+    tensor-parallel rank sees with small serving blocks): several blocks share a wave's run of 64
+    pieces, each read through its own table entry.  Rows long enough for several workgroups,
+    ragged ends inside a run, unusable table entries, every output flag."""
+    from ucm_amd.sparse import hamming_topk
+
+    rng = rng_for(seed)
+    for _ in range(60):
+        Wd = int(rng.choice([4, 8, 16]))
+        cpu = Wd // 4
+        Hkv = int(rng.choice([h for h in (1, 2, 4, 8) if h * cpu <= 32]))
+        # 8 <= BS * Hkv * cpu < 64 sixteen-byte pieces per block
+        BS = int(rng.choice([bs for bs in (1, 2, 4, 8, 16, 32) if 8 <= bs * Hkv * cpu < 64]))
+        G = int(rng.choice([1, 2, 4]))
+        B = int(rng.integers(1, 5))
+        mb = int(rng.choice([1, 3, 15, 16, 17, 63, 64, 65, 127, 129, 255, 300, 700, 1500]))
+        NB = B * mb + 3
+        kc = rng.integers(0, 2**32, size=(NB, BS, Hkv, Wd), dtype=np.uint32)
+        if rng.integers(0, 3) == 0:
+            kc &= np.uint32(0x00010001)  # many equal scores
+        q = rng.integers(0, 2**32, size=(B, Hkv * G, Wd), dtype=np.uint32)
+        use_table = bool(rng.integers(0, 4))
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32) if use_table else None
+        if use_table and rng.integers(0, 3) == 0:
+            table[rng.integers(0, B), rng.integers(0, mb)] = int(rng.choice([-3, NB, NB + 9]))  # unusable entry
+        if not use_table:
+            kc = kc[:B * mb]
+        lens = rng.integers(0, mb * BS + 1, size=B).astype(np.int32)
+        lens[rng.integers(0, B)] = mb * BS - int(rng.integers(0, BS))
+        k = int(rng.choice([1, 5, 64, mb, mb + 2]))
+        sink, recent = int(rng.integers(0, 3)) * BS, int(rng.integers(0, 5)) * BS
+        reduce_heads, physical = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        distance = bool(rng.integers(0, 2))
+        flags = (c_api.F_REDUCE_HEADS if reduce_heads else 0) | (c_api.F_PHYSICAL if physical else 0) | \
+                (c_api.F_DISTANCE if distance else 0)
+        what = dict(B=B, Hkv=Hkv, G=G, Wd=Wd, BS=BS, mb=mb, k=k, table=use_table, sink=sink, recent=recent,
+                    flags=flags)
+        oi, osc = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, flags, max_blocks=mb)
+        gi, gs = hamming_topk(torch.from_numpy(q.view(np.int32)).cuda(), torch.from_numpy(kc.view(np.int32)).cuda(),
+                              torch.from_numpy(table).cuda() if use_table else None, torch.from_numpy(lens).cuda(),
+                              k, sink, recent, reduce_heads=reduce_heads, return_physical=physical,
+                              distance=distance, max_blocks=mb)
+        assert np.array_equal(gi.cpu().numpy(), oi), what
+        assert np.array_equal(gs.cpu().numpy(), osc), what
