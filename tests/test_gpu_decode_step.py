@@ -189,3 +189,58 @@ def test_fused_latent_attention_step_equals_separate_operators_and_oracle(Hq, T)
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(st.out_idx, idx) and torch.equal(st.out_score, sc)
+
+
+@pytest.mark.parametrize("G", [4, 8])
+def test_separate_operators_under_graph_capture(G):
+    """The operators a serving engine captures one by one (encode-and-cache, query hash, block
+    top-k, per-token scores) in one HIP graph: every replay, with new inputs written in place and
+    eager work between the replays, must equal the eager calls and the CPU checker.  G = 8 takes
+    the bit-plane path (an extra kernel and its workspace inside the graph)."""
+    from ucm_amd.sparse import hamming_score, hamming_topk
+
+    Hkv, K = 8, 3
+    W, cache, table, lens, keys, qs, slots, enc_k, enc_q = build(5, Hq=Hkv * G)
+    from ucm_amd.sparse import HashEncoder
+
+    enc_q = HashEncoder(128, 128, torch.bfloat16, torch.device("cuda:0"), num_weights=Hkv, heads_per_weight=G)
+    enc_q.set_hash_weight(W)
+    msl = table.shape[1] * 128
+
+    def ops():
+        enc_k.compute_hash_and_cache(keys, slots, cache, 128)
+        qc = enc_q.compute_hash(qs, per_head=True).view(torch.int32)
+        idx, sc = hamming_topk(qc, cache, table, lens, K)
+        tok = hamming_score(cache, qc[:, None], table, lens, msl, 128, 256, False, out_int32=True)
+        return qc, idx, sc, tok
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        g_out = ops()
+    rng = rng_for(55 + G)
+    for rep in range(3):
+        qs.copy_(torch.from_numpy(rng.standard_normal(tuple(qs.shape)).astype(np.float32)).to(torch.bfloat16))
+        keys.copy_(torch.from_numpy(rng.standard_normal(tuple(keys.shape)).astype(np.float32)).to(torch.bfloat16))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in g_out]
+        gc = cache.clone()
+        want = ops()
+        torch.cuda.synchronize()
+        assert torch.equal(gc, cache)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        oi, osc = c_api.hamming_topk(got[0].cpu().numpy().view(np.uint32), gc.cpu().numpy().view(np.uint32),
+                                     table.cpu().numpy(), lens.cpu().numpy(), K)
+        assert np.array_equal(got[1].cpu().numpy(), oi) and np.array_equal(got[2].cpu().numpy(), osc)
+        ot = c_api.hamming_score(got[0].cpu().numpy().view(np.uint32), gc.cpu().numpy().view(np.uint32),
+                                 table.cpu().numpy(), lens.cpu().numpy(), msl, 128, 256, False)
+        assert np.array_equal(got[3].cpu().numpy(), ot)
+        _ = (qs.float() @ qs.float().transpose(1, 2)).sum().item()  # unrelated eager work
