@@ -28,7 +28,7 @@ for p in (ROOT, os.path.join(ROOT, "unified-cache-management_amd")):
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per block-score launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # what the counter reads for a 1 GiB copy (profiles/decode_step_config2_hbm_traffic_pmc.txt)
-HBM_TRAFFIC_PER_LAUNCH = 136946880
+HBM_TRAFFIC_PER_LAUNCH = 135122716
 
 B, CTX, HQ, HKV, D, BS, TOPK = 32, 32768, 32, 8, 128, 128, 64
 NBLK = CTX // BS          # 256 logical blocks per request

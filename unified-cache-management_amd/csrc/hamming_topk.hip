@@ -49,6 +49,11 @@ struct ScoreArgs {
                              // KV heads, scores then is [B][1][max_blocks]
     const uint32_t* planes;  // [B][Hkv][PMAX][Wd], planes mode only
     int32_t* scores;         // [B][Hkv][max_blocks]
+    int sc_h, sc_j;          // block_score_one only: strides of head and block inside a request's
+                             // Hkv * max_blocks scores (max_blocks, 1), or (1, Hkv) when the
+                             // wave-per-row selection follows: the 8 scores of a block are then
+                             // one 32-byte store instead of eight 4-byte stores into lines that
+                             // other workgroups write too
 };
 
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
@@ -447,7 +452,7 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
             return;
         }
         const int sc = pb < 0 ? -1 : (forced ? full : full - dmin);
-        a.scores[((int64_t)b * HKV + threadIdx.x) * a.max_blocks + j] = sc;
+        a.scores[(int64_t)b * HKV * a.max_blocks + (int64_t)threadIdx.x * a.sc_h + (int64_t)j * a.sc_j] = sc;
     }
 }
 
@@ -1098,6 +1103,7 @@ __global__ __launch_bounds__(kThreads) void block_score_generic(ScoreArgs a)
 // ---------------------------------------------------------------------------------------
 struct SelectArgs {
     const int32_t* scores;  // [B][Hkv][max_blocks]
+    int sc_h, sc_j;         // select_wave_kernel only: head / block strides inside a request's scores
     int32_t* reduced;       // [B][max_blocks] scratch for head-reduced rows beyond the LDS cap
     const int32_t* table;
     int table_stride, max_blocks;
@@ -1314,11 +1320,11 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
     int raw[EL];
     {
         const bool red = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
-        const int32_t* r0 = a.scores + ((int64_t)b * a.Hkv + (red ? 0 : ho)) * a.max_blocks;
+        const int32_t* r0 = a.scores + (int64_t)b * a.Hkv * a.max_blocks + (int64_t)(red ? 0 : ho) * a.sc_h;
 #pragma unroll
         for (int e = 0; e < EL; ++e) {
             const int j = lane * EL + e;
-            raw[e] = r0[j < a.max_blocks ? j : 0];
+            raw[e] = r0[(int64_t)(j < a.max_blocks ? j : 0) * a.sc_j];
         }
     }
     // physical block ids of the whole row, fetched alongside the scores: the output loop then
@@ -1348,7 +1354,7 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
     }
     if (n == 0) return;
     const bool reduce = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
-    const int32_t* row = a.scores + ((int64_t)b * a.Hkv + (reduce ? 0 : ho)) * a.max_blocks;
+    const int32_t* row = a.scores + (int64_t)b * a.Hkv * a.max_blocks + (int64_t)(reduce ? 0 : ho) * a.sc_h;
     int v[EL];
 #pragma unroll
     for (int e = 0; e < EL; ++e) v[e] = raw[e];
@@ -1364,7 +1370,7 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
 #pragma unroll
                 for (int e = 0; e < EL; ++e) {
                     const int j = lane * EL + e;
-                    o[u][e] = row[(int64_t)hh * a.max_blocks + (j < a.max_blocks ? j : 0)];
+                    o[u][e] = row[(int64_t)hh * a.sc_h + (int64_t)(j < a.max_blocks ? j : 0) * a.sc_j];
                 }
             }
 #pragma unroll
@@ -1932,6 +1938,9 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     a.table = block_table; a.table_stride = table_stride; a.max_blocks = max_blocks;
     a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
     a.recent = recent_tok; a.planes = ws.planes; a.scores = ws.scores; a.reduce_out = 0;
+    a.sc_h = max_blocks; a.sc_j = 1;
+    // the wave-per-row selection (same test as at its launch below) reads either layout
+    const bool wave_select = !(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256;
     bool reduced_scores = false;  // the score kernel already took the maximum over the heads
 
     // fast path eligibility
@@ -1983,12 +1992,20 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
         if (!done && split && Hkv <= 16) {
             a.TB = 1;
             a.reduce_out = ((flags & UCM_TOPK_REDUCE_HEADS) && Hkv > 1) ? 1 : 0;
+            if (wave_select && !a.reduce_out && Hkv > 1) {
+                a.sc_h = 1;
+                a.sc_j = Hkv;
+            }
             const dim3 grid1((unsigned)max_blocks, (unsigned)B);
             if (cpu == 1) done = dispatch_one<1>(a, pmax, grid1, st);
             else if (cpu == 2) done = dispatch_one<2>(a, pmax, grid1, st);
             else done = dispatch_one<4>(a, pmax, grid1, st);
             reduced_scores = done && a.reduce_out;
             a.reduce_out = 0;
+            if (!done) {
+                a.sc_h = max_blocks;
+                a.sc_j = 1;
+            }
         }
         if (!done) a.TB = TB;
         if (!done && !split) {
@@ -2055,7 +2072,7 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     if (rc != UCM_OK) return rc;
 
     SelectArgs s;
-    s.scores = ws.scores; s.reduced = ws.reduced; s.table = block_table;
+    s.scores = ws.scores; s.sc_h = a.sc_h; s.sc_j = a.sc_j; s.reduced = ws.reduced; s.table = block_table;
     s.table_stride = table_stride; s.max_blocks = max_blocks; s.lens = seq_lens; s.BS = BS;
     s.Hkv = reduced_scores ? 1 : Hkv; s.Ho = (flags & UCM_TOPK_REDUCE_HEADS) ? 1 : Hkv; s.k = k;
     s.full = a.G * 32 * Wd;
