@@ -391,3 +391,48 @@ def test_topk_blocks_below_one_kib(seed):
                               distance=distance, max_blocks=mb)
         assert np.array_equal(gi.cpu().numpy(), oi), what
         assert np.array_equal(gs.cpu().numpy(), osc), what
+
+
+@pytest.mark.parametrize("seed", [91])
+def test_blocks_of_4_kib_and_more_in_rows_of_over_256_blocks(seed):
+    """Blocks of at least 4 KiB (one workgroup per block) in rows of 257 to 1100 blocks (one
+    workgroup per row in the selection): the pair that passes the block scores block-major.
+    Ragged lengths, ties, unusable entries, every index-ordered flag combination."""
+    from ucm_amd.sparse import hamming_topk
+
+    rng = rng_for(seed)
+    for _ in range(16):
+        Hkv = int(rng.choice([2, 4, 8]))
+        Wd, G = 4, int(rng.choice([1, 4, 8]))
+        BS = int(rng.choice([bs for bs in (32, 64, 128, 256) if bs * Hkv * 16 >= 4096]))
+        B = int(rng.integers(1, 3))
+        mb = int(rng.choice([257, 300, 512, 600, 1025, 1100]))
+        while B * mb * BS * Hkv * 16 > (48 << 20):
+            mb = 257 if mb > 300 else mb
+            BS //= 2
+        if BS * Hkv * 16 < 4096:
+            continue
+        NB = B * mb + 2
+        kc = rng.integers(0, 2**32, size=(NB, BS, Hkv, Wd), dtype=np.uint32)
+        if rng.integers(0, 2) == 0:
+            kc &= np.uint32(0x00000101)  # many equal scores
+        q = rng.integers(0, 2**32, size=(B, Hkv * G, Wd), dtype=np.uint32)
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32)
+        if rng.integers(0, 2) == 0:
+            table[rng.integers(0, B), rng.integers(0, mb)] = NB + 3  # unusable entry
+        lens = rng.integers(0, mb * BS + 1, size=B).astype(np.int32)
+        lens[rng.integers(0, B)] = mb * BS - int(rng.integers(0, BS))
+        k = int(rng.choice([1, 64, 128, 300, mb]))
+        sink, recent = int(rng.integers(0, 3)) * BS, int(rng.integers(0, 5)) * BS
+        reduce_heads, physical = bool(rng.integers(0, 3) == 0), bool(rng.integers(0, 2))
+        distance = bool(rng.integers(0, 2))
+        flags = (c_api.F_REDUCE_HEADS if reduce_heads else 0) | (c_api.F_PHYSICAL if physical else 0) | \
+                (c_api.F_DISTANCE if distance else 0)
+        what = dict(B=B, Hkv=Hkv, G=G, BS=BS, mb=mb, k=k, sink=sink, recent=recent, flags=flags)
+        oi, osc = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, flags, max_blocks=mb)
+        gi, gs = hamming_topk(torch.from_numpy(q.view(np.int32)).cuda(), torch.from_numpy(kc.view(np.int32)).cuda(),
+                              torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda(), k, sink, recent,
+                              reduce_heads=reduce_heads, return_physical=physical, distance=distance,
+                              max_blocks=mb)
+        assert np.array_equal(gi.cpu().numpy(), oi), what
+        assert np.array_equal(gs.cpu().numpy(), osc), what
