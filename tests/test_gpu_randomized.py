@@ -396,8 +396,7 @@ def test_topk_blocks_below_one_kib(seed):
 @pytest.mark.parametrize("seed", [91])
 def test_blocks_of_4_kib_and_more_in_rows_of_over_256_blocks(seed):
     """Blocks of at least 4 KiB (one workgroup per block) in rows of 257 to 1100 blocks (one
-    workgroup per row in the selection): the pair that passes the block scores block-major.
-    Ragged lengths, ties, unusable entries, every index-ordered flag combination."""
+    workgroup per row in the selection).  Ragged lengths, ties, unusable entries, every index-ordered flag combination."""
     from ucm_amd.sparse import hamming_topk
 
     rng = rng_for(seed)

@@ -51,7 +51,7 @@ struct ScoreArgs {
     int32_t* scores;         // [B][Hkv][max_blocks]
     int sc_h, sc_j;          // block_score_one only: strides of head and block inside a request's
                              // Hkv * max_blocks scores (max_blocks, 1), or (1, Hkv) when the
-                             // wave- or workgroup-per-row selection follows: the 8 scores of a block are then
+                             // wave-per-row selection follows: the 8 scores of a block are then
                              // one 32-byte store instead of eight 4-byte stores into lines that
                              // other workgroups write too
 };
@@ -1103,8 +1103,7 @@ __global__ __launch_bounds__(kThreads) void block_score_generic(ScoreArgs a)
 // ---------------------------------------------------------------------------------------
 struct SelectArgs {
     const int32_t* scores;  // [B][Hkv][max_blocks]
-    int sc_h, sc_j;         // select_wave_kernel, select_group_kernel: head / block strides inside a
-                            // request's scores (select_kernel reads [Hkv][max_blocks] only)
+    int sc_h, sc_j;         // select_wave_kernel only: head / block strides inside a request's scores
     int32_t* reduced;       // [B][max_blocks] scratch for head-reduced rows beyond the LDS cap
     const int32_t* table;
     int table_stride, max_blocks;
@@ -1454,12 +1453,12 @@ __global__ __launch_bounds__(kThreads) void select_group_kernel(SelectArgs a)
     const int b = blockIdx.x / a.Ho, ho = blockIdx.x % a.Ho;
     const int tid = threadIdx.x, lane = lane_id(), wid = wave_id();
     const bool reduce = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
-    const int32_t* row = a.scores + (int64_t)b * a.Hkv * a.max_blocks + (int64_t)(reduce ? 0 : ho) * a.sc_h;
+    const int32_t* row = a.scores + ((int64_t)b * a.Hkv + (reduce ? 0 : ho)) * a.max_blocks;
     int v[EL], tab[EL];
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
         const int j = tid * EL + e;
-        v[e] = row[(int64_t)(j < a.max_blocks ? j : 0) * a.sc_j];
+        v[e] = row[j < a.max_blocks ? j : 0];
     }
     const bool physical = (a.flags & UCM_TOPK_RETURN_PHYSICAL) != 0;
     if (physical && a.table) {
@@ -1493,7 +1492,7 @@ __global__ __launch_bounds__(kThreads) void select_group_kernel(SelectArgs a)
 #pragma unroll
                 for (int e = 0; e < EL; ++e) {
                     const int j = tid * EL + e;
-                    o[u][e] = row[(int64_t)hh * a.sc_h + (int64_t)(j < a.max_blocks ? j : 0) * a.sc_j];
+                    o[u][e] = row[(int64_t)hh * a.max_blocks + (j < a.max_blocks ? j : 0)];
                 }
             }
 #pragma unroll
@@ -1940,9 +1939,8 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
     a.recent = recent_tok; a.planes = ws.planes; a.scores = ws.scores; a.reduce_out = 0;
     a.sc_h = max_blocks; a.sc_j = 1;
-    // the wave-per-row and workgroup-per-row selections (same test as at their launch below)
-    // read either layout
-    const bool wave_select = !(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 4096;
+    // the wave-per-row selection (same test as at its launch below) reads either layout
+    const bool wave_select = !(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256;
     bool reduced_scores = false;  // the score kernel already took the maximum over the heads
 
     // fast path eligibility
