@@ -3,8 +3,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# UCM_HIP_LIBRARY overrides the in-tree build (e.g. to try a differently compiled library)
-LIB_PATH = os.environ.get("UCM_HIP_LIBRARY") or os.path.join(os.path.dirname(_HERE), "lib", "libucm_hip.so")
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libucm_hip.so")
 
 UCM_OK = 0
 UCM_ERROR = -1
