@@ -173,6 +173,29 @@ int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
                      ucm_stream_t stream);
 
 /*
+ * ucm_hamming_topk for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Arguments and results are those of ucm_hamming_topk without the workspace: block
+ * scores and bit planes live in a fixed array of UCM_TOPK_STATIC_SCRATCH_BYTES that every GPU the
+ * library runs on holds until the process ends.  Shapes whose
+ * ucm_hamming_topk_workspace_bytes(B, Hkv, max_blocks) exceeds that size are rejected with
+ * UCM_EPARAM.  The call allocates nothing; the array's address on the current device is looked
+ * up on the first call on that device (make that call outside a graph capture).  All calls on
+ * one GPU share the array: calls that overlap in time on one GPU (two streams, two threads)
+ * race; calls on one stream are ordered and safe.
+ */
+#define UCM_TOPK_STATIC_SCRATCH_BYTES (4u << 20)
+int ucm_hamming_topk_static(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                            const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
+                            int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                            const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                            const int32_t* seq_lens,
+                            int32_t B, int32_t Hq, int32_t k,
+                            int32_t sink_tok, int32_t recent_tok, uint32_t flags,
+                            int32_t* out_idx, int32_t* out_score,
+                            ucm_stream_t stream);
+
+/*
  * Replaces kvlib::HammingScoreContiCUDA (csrc/cuda/ham_dist/operator.h:10-13,
  * paged_ham_dist_mla.cu:332-443) for callers that want its per-token output:
  * out[b, h, p] for p < max_seq_len is the group-summed Hamming distance of position p,

@@ -20,6 +20,8 @@
 // its NPU op (csrc/ascend/hamming_dist_top_k/op_kernel/hamming_dist_top_k_base.h:150-347).
 #include <hip/hip_ext.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -2101,6 +2103,64 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     }
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
     return ucm::launch_status("select_kernel");
+}
+
+// ---------------------------------------------------------------------------------------
+// ucm_hamming_topk_static: the same operator for callers that cannot allocate.  Its block
+// scores, head-reduced rows and bit planes live in a fixed device array instead of a caller's
+// workspace.  The array's name is only a host-side handle: each GPU holds its own copy, whose
+// address is resolved once per device and passed to the kernels like any workspace.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[UCM_TOPK_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the calling thread's current device.
+int static_scratch(void** out)
+{
+    int dev = -1;
+    UCM_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return ucm::fail(UCM_EUNSUPPORTED, "device %d out of range", dev);
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return ucm::hip_fail(e, "hipGetSymbolAddress(scratch)");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return UCM_OK;
+}
+}  // namespace
+
+extern "C" int ucm_hamming_topk_static(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                                       const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
+                                       int32_t Wd, int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                                       const int32_t* block_table, int32_t table_stride,
+                                       int32_t max_blocks, const int32_t* seq_lens, int32_t B,
+                                       int32_t Hq, int32_t k, int32_t sink_tok, int32_t recent_tok,
+                                       uint32_t flags, int32_t* out_idx, int32_t* out_score,
+                                       ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(B >= 0 && Hkv > 0 && max_blocks > 0, "non-positive shape");
+    const size_t need = B > 0 ? carve(nullptr, B, Hkv, max_blocks).bytes : 0;
+    if (need > (size_t)UCM_TOPK_STATIC_SCRATCH_BYTES)
+        return ucm::fail(UCM_EPARAM,
+                         "B=%d x Hkv=%d x max_blocks=%d needs %zu bytes of scratch, the static "
+                         "entry point holds %zu: use ucm_hamming_topk with a workspace",
+                         B, Hkv, max_blocks, need, (size_t)UCM_TOPK_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != UCM_OK) return rc;
+    // Nothing in the scratch has to start at zero: every kernel writes the cells it later reads.
+    return ucm_hamming_topk(q_codes, q_stride_b, q_stride_h, k_cache, NB, BS, Hkv, Wd, ks_block, ks_token,
+                            ks_head, block_table, table_stride, max_blocks, seq_lens, B, Hq, k, sink_tok,
+                            recent_tok, flags, out_idx, out_score, ws, (size_t)UCM_TOPK_STATIC_SCRATCH_BYTES,
+                            stream);
 }
 
 extern "C" int ucm_sparse_decode_step(const void* new_keys, int64_t T, int64_t k_stride_t,
