@@ -354,11 +354,13 @@ int ucm_trans_batch(ucm_trans_stream_t* s, const void* const* src, void* const* 
  * The flat buffer is laid out (block, col) row-major, column c of a block at the running
  * sum of col_bytes (dump_queue.cc:145-161).  base / col_bytes are host arrays of n_cols
  * entries; block_ids is a host array of n_blocks entries.  to_cache = 0 gathers cache ->
- * flat, 1 scatters flat -> cache.  SM streams only.
+ * flat, 1 scatters flat -> cache.  SM streams only.  Ids that are negative, or not below
+ * n_cache_blocks (the number of blocks every column holds; 0 = unknown, only the sign is
+ * checked), are refused with UCM_EPARAM before anything is launched.
  */
 int ucm_trans_paged_copy(ucm_trans_stream_t* s, const uint64_t* base, const uint64_t* col_bytes,
                          int32_t n_cols, const int32_t* block_ids, int64_t n_blocks,
-                         void* flat, int to_cache, int sync);
+                         int64_t n_cache_blocks, void* flat, int to_cache, int sync);
 
 /* Buffer::MakeHostBuffer / MakeDeviceBuffer / RegisterHostBuffer
  * (ucm/shared/trans/buffer.h:32-47, cuda/cuda_buffer.cc:29-56). */

@@ -73,7 +73,10 @@ def half_piece_sums(q, kc, table, lens, msl):
             x = kp[pb, p % BS, 0][None, :] ^ qp[b]          # [G,L]
             parts = cnt[x.view(np.uint8).reshape(x.shape[0], x.shape[1], 8)].sum(axis=(0, 2))
             acc = np.float16(0)
-            for part in parts:
-                acc = np.float16(acc + np.float16(part))
+            # sums above 65,504 (128 query heads x 576 bits) overflow to infinity in half
+            # precision: that is the reference's own result, not an accident of this helper
+            with np.errstate(over="ignore"):
+                for part in parts:
+                    acc = np.float16(acc + np.float16(part))
             out[b, 0, p] = acc
     return out

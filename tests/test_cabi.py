@@ -62,6 +62,13 @@ def test_parameter_errors_need_no_gpu():
     rc = lib.ucm_hash_encode(None, 0, 1, 1, 128, 128, 128, None, 0, 1, 0, 128, None, 4, 4, None)
     assert rc == _lib.UCM_EPARAM
     assert lib.ucm_hamming_topk_workspace_bytes(32, 8, 256) >= 32 * 8 * 256 * 4
+    # block ids that would turn into wild device addresses are refused before any launch
+    base = (ctypes.c_uint64 * 1)(4096)
+    size = (ctypes.c_uint64 * 1)(64)
+    flat = ctypes.c_void_p(4096)
+    for ids, n_cache in (((ctypes.c_int32 * 2)(0, -1), 0), ((ctypes.c_int32 * 2)(1, 9), 9)):
+        rc2 = lib.ucm_trans_paged_copy(None, base, size, 1, ids, 2, n_cache, flat, 0, 0)
+        assert rc2 == _lib.UCM_EPARAM and "block_ids[1]" in _lib.last_error()
     with pytest.raises(ValueError):
         _lib.check(rc)
 

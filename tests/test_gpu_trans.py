@@ -209,3 +209,8 @@ def test_errors(device):
         ce.DeviceToHostGather(t.data_ptr(), t.data_ptr(), 8, 2)
     with pytest.raises(ValueError):
         ce.PagedGatherAsync([t.data_ptr()], [8], [0], t.data_ptr())
+    sm = device.MakeSMStream()
+    with pytest.raises(ValueError):  # a negative id would be a wild address
+        sm.PagedGatherAsync([t.data_ptr()], [8], [0, -1], t.data_ptr())
+    with pytest.raises(ValueError):  # beyond the cache's extent
+        sm.PagedScatterAsync(t.data_ptr(), [t.data_ptr()], [8], [0, 8], num_cache_blocks=8)

@@ -200,6 +200,7 @@ struct ucm_cache_store {
     BoundedQueue<LoadCtx> load_running;
     BoundedQueue<DumpCtx> dumping;
     std::atomic<bool> stop{false};
+    std::atomic<bool> stop_backend{false};  // set after the dump dispatcher has been joined
     ucm_trans_stream_t* dump_stream = nullptr;
     ucm_trans_stream_t* load_stream = nullptr;
     std::thread dump_dispatcher, dump_backend, load_dispatcher, load_transfer;
@@ -327,7 +328,7 @@ void dump_dispatch_stage(ucm_cache_store* st)
 void dump_backend_stage(ucm_cache_store* st)
 {
     DumpCtx ctx;
-    while (st->dumping.pop(ctx, st->stop)) {
+    while (st->dumping.pop(ctx, st->stop_backend)) {
         if (ctx.backend > 0 && st->backend.wait) (void)st->backend.wait(st->backend.ctx, ctx.backend);
         for (size_t p : ctx.held) st->buffer.release(p);
         ctx = {};
@@ -374,8 +375,14 @@ void load_dispatch_stage(ucm_cache_store* st)
         }
         if (!ok) {
             for (size_t i = 0; i < ctx.pos.size(); ++i) {
-                if (ctx.backend[i] > 0) st->buffer.discard(ctx.pos[i]);
-                else st->buffer.release(ctx.pos[i]);
+                if (ctx.backend[i] > 0) {
+                    // the backend may still be writing into the node: it goes back to the ring
+                    // only after that load has ended, whatever its outcome
+                    if (st->backend.wait) (void)st->backend.wait(st->backend.ctx, ctx.backend[i]);
+                    st->buffer.discard(ctx.pos[i]);
+                } else {
+                    st->buffer.release(ctx.pos[i]);
+                }
             }
             st->fail(task->id);
             pr.second->done();
@@ -394,9 +401,11 @@ void load_transfer_stage(ucm_cache_store* st)
         const int64_t id = ctx.task->id;
         bool ok = !st->failed(id);
         const auto deadline = Clock::now() + std::chrono::milliseconds(st->timeout_ms);
+        std::vector<char> waited(ctx.pos.size(), 0);
         for (size_t i = 0; ok && i < ctx.pos.size(); ++i) {
             if (ctx.backend[i] > 0) {
                 ok = !st->backend.wait || st->backend.wait(st->backend.ctx, ctx.backend[i]) == UCM_OK;
+                waited[i] = 1;
                 if (ok) st->buffer.mark_ready(ctx.pos[i]);
             } else {
                 // another task is filling this node (load_queue.cc:168-174)
@@ -416,6 +425,11 @@ void load_transfer_stage(ucm_cache_store* st)
                  ucm_trans_stream_sync(st->load_stream) == UCM_OK;
         }
         for (size_t i = 0; i < ctx.pos.size(); ++i) {
+            // a load the loop above never reached (an earlier shard failed, the task was marked
+            // failed or timed out) may still be writing into its node: wait before the node can
+            // be handed to another key
+            if (ctx.backend[i] > 0 && !waited[i] && st->backend.wait)
+                (void)st->backend.wait(st->backend.ctx, ctx.backend[i]);
             if (!ok && ctx.backend[i] > 0 && !st->buffer.ready(ctx.pos[i])) st->buffer.discard(ctx.pos[i]);
             else st->buffer.release(ctx.pos[i]);
         }
@@ -513,8 +527,12 @@ extern "C" int ucm_cache_store_destroy(ucm_cache_store_t* st)
     ucm::clear_error();
     if (!st) return UCM_OK;
     st->stop.store(true);
-    for (std::thread* t : {&st->dump_dispatcher, &st->load_dispatcher, &st->load_transfer, &st->dump_backend})
+    for (std::thread* t : {&st->dump_dispatcher, &st->load_dispatcher, &st->load_transfer})
         if (t->joinable()) t->join();
+    // only now can no new backend dump appear: let the backend stage wait for the ones in flight
+    // (their source is the pinned slab, freed below) and exit
+    st->stop_backend.store(true);
+    if (st->dump_backend.joinable()) st->dump_backend.join();
     (void)ucm_trans_stream_destroy(st->dump_stream);
     (void)ucm_trans_stream_destroy(st->load_stream);
     delete st;

@@ -65,11 +65,7 @@ __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 template <class T>
 __device__ __forceinline__ T code_load(const T* p)
 {
-#ifdef UCM_PLAIN_CODE_LOADS
-    return *p;
-#else
     return __builtin_nontemporal_load(p);
-#endif
 }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

@@ -708,15 +708,22 @@ extern "C" int ucm_posix_store_wait(ucm_posix_store_t* st, int64_t task)
         w = it->second;
     }
     const bool done = w->wait_for(st->timeout_ms);
+    if (!done) {
+        {
+            std::lock_guard<std::mutex> lock(st->tasks_mu);
+            st->failures.insert(task);  // shards still queued are skipped
+        }
+        // the caller's buffers are free to reuse once this returns, so the units that are queued
+        // (now skipped) or in the middle of their read / write must have drained first
+        while (!w->wait_for(1000)) {
+        }
+    }
     bool failed;
     {
         std::lock_guard<std::mutex> lock(st->tasks_mu);
-        if (!done) st->failures.insert(task);  // shards still queued are skipped
         failed = st->failures.count(task) != 0;
-        if (done) {
-            st->tasks.erase(task);
-            st->failures.erase(task);
-        }
+        st->tasks.erase(task);
+        st->failures.erase(task);
     }
     if (!done) return ucm::fail(UCM_ETIMEOUT, "task %lld timed out after %zu ms", (long long)task, st->timeout_ms);
     if (failed) return ucm::fail(UCM_ERROR, "task %lld failed", (long long)task);

@@ -355,14 +355,19 @@ extern "C" int ucm_trans_batch(ucm_trans_stream_t* s, const void* const* src, vo
 
 extern "C" int ucm_trans_paged_copy(ucm_trans_stream_t* s, const uint64_t* base,
                                     const uint64_t* col_bytes, int32_t n_cols,
-                                    const int32_t* block_ids, int64_t n_blocks, void* flat,
-                                    int to_cache, int sync)
+                                    const int32_t* block_ids, int64_t n_blocks,
+                                    int64_t n_cache_blocks, void* flat, int to_cache, int sync)
 {
     ucm::clear_error();
+    UCM_REQUIRE(n_cols > 0 && n_blocks >= 0 && n_cache_blocks >= 0, "bad sizes");
+    UCM_REQUIRE(base && col_bytes && flat && (block_ids || n_blocks == 0), "null argument");
+    // an id outside the cache would become a wild device address inside the kernel
+    for (int64_t i = 0; i < n_blocks; ++i)
+        UCM_REQUIRE(block_ids[i] >= 0 && (n_cache_blocks == 0 || block_ids[i] < n_cache_blocks),
+                    "block_ids[%lld] = %d outside the cache's %lld blocks", (long long)i, block_ids[i],
+                    (long long)n_cache_blocks);
     UCM_REQUIRE(s, "null stream");
     UCM_REQUIRE(s->kind == UCM_TRANS_SM, "paged copy needs an SM stream");
-    UCM_REQUIRE(n_cols > 0 && n_blocks >= 0, "bad sizes");
-    UCM_REQUIRE(base && col_bytes && flat && (block_ids || n_blocks == 0), "null argument");
     if (n_blocks == 0) return finish(s, sync);
     std::lock_guard<std::mutex> lock(s->mu);
 

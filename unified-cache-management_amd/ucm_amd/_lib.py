@@ -59,7 +59,7 @@ _SIGNATURES = {
     "ucm_trans_gather": (ci, [vp, vp, ci, vp, sz, sz, ci]),
     "ucm_trans_scatter": (ci, [vp, vp, vp, ci, sz, sz, ci]),
     "ucm_trans_batch": (ci, [vp, vp, vp, ci, sz, sz, ci]),
-    "ucm_trans_paged_copy": (ci, [vp, vp, vp, i32, vp, i64, vp, ci, ci]),
+    "ucm_trans_paged_copy": (ci, [vp, vp, vp, i32, vp, i64, i64, vp, ci, ci]),
     "ucm_trans_host_alloc": (ci, [sz, C.POINTER(vp)]),
     "ucm_trans_host_free": (ci, [vp]),
     "ucm_trans_device_alloc": (ci, [sz, C.POINTER(vp)]),

@@ -10,13 +10,24 @@ import torch
 from .. import _lib
 
 _workspaces = {}
+_retired = []
 
 
 def _workspace(device, nbytes):
-    key = (device.type, device.index)
+    """Scratch of the calling stream.  One buffer per (device, stream): calls on different
+    streams (a retrieval worker's side stream beside the plugin on the main stream) may be in
+    flight together and must not share block scores.  A buffer that is outgrown stays alive
+    (kernels already enqueued, or a captured graph, may still use it); sizes double, so the
+    retired ones add up to less than the live one."""
+    stream = torch.cuda.current_stream(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device(),
+           stream.cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        if ws is not None:
+            _retired.append(ws)
+        size = max(nbytes, 1 << 20, 2 * ws.numel() if ws is not None else 0)
+        ws = torch.empty(size, dtype=torch.uint8, device=device)  # allocated on `stream`
         _workspaces[key] = ws
     return ws
 

@@ -102,13 +102,15 @@ class Stream:
 
     # ---- table-free paged form (address rule of KVCacheLayout.extract_block_addrs,
     #      ucm/integration/vllm/ucm_connector.py:135-148) ----
-    def PagedGatherAsync(self, base_ptrs, col_bytes, block_ids, dst, sync=False):
-        self._paged(base_ptrs, col_bytes, block_ids, dst, 0, sync)
+    def PagedGatherAsync(self, base_ptrs, col_bytes, block_ids, dst, sync=False, num_cache_blocks=0):
+        self._paged(base_ptrs, col_bytes, block_ids, dst, 0, sync, num_cache_blocks)
 
-    def PagedScatterAsync(self, src, base_ptrs, col_bytes, block_ids, sync=False):
-        self._paged(base_ptrs, col_bytes, block_ids, src, 1, sync)
+    def PagedScatterAsync(self, src, base_ptrs, col_bytes, block_ids, sync=False, num_cache_blocks=0):
+        self._paged(base_ptrs, col_bytes, block_ids, src, 1, sync, num_cache_blocks)
 
-    def _paged(self, base_ptrs, col_bytes, block_ids, flat, to_cache, sync):
+    def _paged(self, base_ptrs, col_bytes, block_ids, flat, to_cache, sync, num_cache_blocks=0):
+        """num_cache_blocks: blocks every column holds; ids outside [0, num_cache_blocks) are
+        refused (0 = unknown: only negative ids are)."""
         base = np.ascontiguousarray(base_ptrs, dtype=np.uint64).reshape(-1)
         cb = np.ascontiguousarray(col_bytes, dtype=np.uint64).reshape(-1)
         ids = np.ascontiguousarray(block_ids, dtype=np.int32).reshape(-1)
@@ -116,7 +118,8 @@ class Stream:
             raise ValueError("base_ptrs and col_bytes must have the same length")
         _lib.check(_lib.lib().ucm_trans_paged_copy(self._h, base.ctypes.data, cb.ctypes.data,
                                                    base.shape[0], ids.ctypes.data, ids.shape[0],
-                                                   int(flat), to_cache, int(bool(sync))))
+                                                   int(num_cache_blocks), int(flat), to_cache,
+                                                   int(bool(sync))))
 
     # ---- ordering ----
     def Synchronized(self):
