@@ -85,6 +85,14 @@ int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int3
                           ucm_stream_t stream);
 
 /*
+ * Tuning and test hook, no counterpart in the reference.  Inputs of at least `rows` rows (tokens x
+ * heads) with 64 or 128 input dimensions and 64 or 128 hash bits take the streaming kernel
+ * (persistent waves, projection matrix in registers, rows loaded straight into LDS); smaller ones
+ * take the tiled kernel.  Both give identical codes.  rows <= 0 restores the default (2^20).
+ */
+int ucm_hash_encode_set_stream_threshold(int64_t rows);
+
+/*
  * Re-encodes keys that already sit in the paged KV cache (prefix-cache hit): replaces the
  * gather `kv_cache[0][0][prefix_block_ids]` followed by compute_hash_and_cache with the
  * prefix slot mapping (ucm/sparse/gsa_on_device/gsa_on_device.py:574-588; the slot rule is

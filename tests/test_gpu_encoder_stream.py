@@ -1,0 +1,155 @@
+"""GPU parity of the streaming encoder kernel (the cache-build path: persistent waves, projection
+matrix in registers, rows loaded straight into LDS) against the CPU oracle under the margin rule
+(a bit may differ only where |projection| < 1e-2 * ||x||), and against the tiled kernel, whose
+MFMA sequence it shares (identical codes expected).  The threshold hook sends small shapes to the
+streaming kernel, so that the oracle stays cheap."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import rng_for
+from oracle import brute
+
+pytestmark = pytest.mark.gpu
+
+MARGIN_TOL = 1e-2
+_DT = {torch.bfloat16: 0, torch.float16: 1}
+
+
+@pytest.fixture
+def stream_everything():
+    from ucm_amd import _lib
+
+    L = _lib.lib()
+    L.ucm_hash_encode_set_stream_threshold(1)
+    yield L
+    L.ucm_hash_encode_set_stream_threshold(0)
+
+
+def _encode_cache(L, x, W, slots, cache, BS, n_w, hpw):
+    from ucm_amd import _lib
+
+    T, H, K = x.shape
+    N = W.shape[-1]
+    _lib.check(L.ucm_hash_encode_cache(
+        x.data_ptr(), _DT[x.dtype], T, H, K, x.stride(0), x.stride(1), W.data_ptr(), _DT[W.dtype], n_w, hpw, N,
+        slots.data_ptr(), int(slots.dtype == torch.int64), cache.data_ptr(), cache.shape[0], BS,
+        cache.stride(0), cache.stride(1), cache.stride(2), torch.cuda.current_stream().cuda_stream))
+
+
+def _check_against_oracle(cache_np, x, W, slots_np, BS, hpw, rows):
+    """Margin rule on the sampled token rows."""
+    H = x.shape[1]
+    xs = x.float().cpu().numpy()
+    Ws = W.float().cpu().numpy()
+    flat = cache_np.reshape(-1, H, cache_np.shape[-1])
+    flips = 0
+    for h in range(H):
+        w = Ws[min(h // hpw, Ws.shape[0] - 1)] if hpw > 0 else Ws[0]
+        ref = brute.hash_encode(xs[rows, h], w)
+        got = flat[slots_np[rows], h]
+        diff = np.unpackbits((got ^ ref).view(np.uint8), axis=-1, bitorder="little").astype(bool)
+        marg = brute.margins(xs[rows, h], w)
+        assert not np.any(diff & (marg >= MARGIN_TOL)), "bit flipped outside the margin"
+        flips += int(diff.sum())
+    return flips
+
+
+# (seed, T, H, K, N, dtype, slot dtype, shared W)
+CASES = [
+    (1, 4096, 8, 128, 128, torch.bfloat16, torch.int64, False),
+    (2, 4096 + 37, 8, 128, 128, torch.bfloat16, torch.int32, False),   # ragged last tile
+    (3, 31, 8, 128, 128, torch.bfloat16, torch.int64, True),           # fewer rows than one tile
+    (4, 3000, 4, 128, 64, torch.float16, torch.int64, False),
+    (5, 5000, 2, 64, 128, torch.bfloat16, torch.int32, True),
+    (6, 2048 + 1, 1, 64, 64, torch.float16, torch.int64, True),
+    (7, 1500, 12, 128, 128, torch.bfloat16, torch.int64, False),       # head count that is no power of two
+    (8, 70000, 8, 128, 128, torch.bfloat16, torch.int64, False),       # several tiles per wave
+]
+
+
+@pytest.mark.parametrize("seed,T,H,K,N,dtype,sdt,shared", CASES)
+def test_streaming_kernel_matches_oracle_and_tiled_kernel(stream_everything, seed, T, H, K, N, dtype, sdt, shared):
+    L = stream_everything
+    rng = rng_for(seed)
+    BS = 16
+    NB = -(-T // BS) + 3
+    x = torch.from_numpy(rng.standard_normal((T, H, K)).astype(np.float32)).to(dtype).cuda()
+    n_w, hpw = (1, 0) if shared else (H, 1)
+    W = torch.from_numpy(rng.standard_normal((n_w, K, N)).astype(np.float32)).to(dtype).cuda()
+    perm = rng.permutation(NB)
+    slots_np = (np.repeat(perm, BS)[:T] * BS + np.tile(np.arange(BS), NB)[:T]).astype(np.int64)
+    drop = rng.choice(T, size=min(5, T), replace=False)
+    slots_in = slots_np.copy()
+    slots_in[drop[0]] = -1
+    if len(drop) > 1:
+        slots_in[drop[1]] = NB * BS + 4
+    slots = torch.from_numpy(slots_in).to(sdt).cuda()
+    canary = 0x5A5A5A5A
+    got = torch.full((NB, BS, H, N // 32), canary, dtype=torch.int32, device="cuda")
+    _encode_cache(L, x, W, slots, got, BS, n_w, hpw)
+    torch.cuda.synchronize()
+    # the tiled kernel on the same input
+    L.ucm_hash_encode_set_stream_threshold(1 << 62)
+    ref = torch.full_like(got, canary)
+    _encode_cache(L, x, W, slots, ref, BS, n_w, hpw)
+    torch.cuda.synchronize()
+    L.ucm_hash_encode_set_stream_threshold(1)
+    assert torch.equal(got, ref), "streaming and tiled kernels disagree"
+    g = got.cpu().numpy().view(np.uint32)
+    # dropped rows and unused slots keep the canary
+    flat = g.reshape(-1, H, N // 32)
+    used = np.zeros(NB * BS, bool)
+    keep = np.ones(T, bool)
+    keep[drop[:2]] = False
+    used[slots_np[keep]] = True
+    assert np.all(flat[~used] == canary)
+    rows = np.flatnonzero(keep)
+    if len(rows) > 600:
+        rows = np.sort(rng.choice(rows, size=600, replace=False))
+    _check_against_oracle(g, x, W, slots_np, BS, hpw, rows)
+
+
+def test_streaming_kernel_dense_output(stream_everything):
+    from ucm_amd import _lib
+
+    L = stream_everything
+    rng = rng_for(21)
+    T, H, K, N = 2500, 8, 128, 128
+    x = torch.from_numpy(rng.standard_normal((T, H, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    W = torch.from_numpy(rng.standard_normal((H, K, N)).astype(np.float32)).to(torch.bfloat16).cuda()
+    out = torch.zeros((T, H, N // 32), dtype=torch.int32, device="cuda")
+    _lib.check(L.ucm_hash_encode(x.data_ptr(), 0, T, H, K, x.stride(0), x.stride(1), W.data_ptr(), 0, H, 1, N,
+                                 out.data_ptr(), out.stride(0), out.stride(1),
+                                 torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    o = out.cpu().numpy().view(np.uint32)
+    rows = np.sort(rng.choice(T, size=500, replace=False))
+    _check_against_oracle(o[:, None].reshape(T, 1, H, N // 32), x, W, np.arange(T), 1, 1, rows)
+
+
+def test_cache_build_size_takes_the_streaming_kernel_by_default():
+    """2^20 rows (131,072 tokens x 8 KV heads of 128 -> 128 bits): the default threshold; sampled
+    rows against the oracle, everything against the tiled kernel."""
+    from ucm_amd import _lib
+
+    L = _lib.lib()
+    L.ucm_hash_encode_set_stream_threshold(0)
+    rng = rng_for(33)
+    T, H, K, N, BS = 131072, 8, 128, 128, 128
+    NB = T // BS
+    x = torch.randn((T, H, K), device="cuda", dtype=torch.bfloat16, generator=torch.Generator("cuda").manual_seed(33))
+    W = torch.randn((H, K, N), device="cuda", dtype=torch.bfloat16, generator=torch.Generator("cuda").manual_seed(34))
+    perm = rng.permutation(NB)
+    slots_np = (np.repeat(perm, BS) * BS + np.tile(np.arange(BS), NB)).astype(np.int64)
+    slots = torch.from_numpy(slots_np).cuda()
+    got = torch.zeros((NB, BS, H, N // 32), dtype=torch.int32, device="cuda")
+    _encode_cache(L, x, W, slots, got, BS, H, 1)
+    L.ucm_hash_encode_set_stream_threshold(1 << 62)
+    ref = torch.zeros_like(got)
+    _encode_cache(L, x, W, slots, ref, BS, H, 1)
+    L.ucm_hash_encode_set_stream_threshold(0)
+    torch.cuda.synchronize()
+    assert torch.equal(got, ref)
+    rows = np.sort(rng.choice(T, size=400, replace=False))
+    _check_against_oracle(got.cpu().numpy().view(np.uint32), x, W, slots_np, BS, 1, rows)

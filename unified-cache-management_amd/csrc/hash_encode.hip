@@ -20,6 +20,8 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <atomic>
+
 #include "common.h"
 
 namespace {
@@ -542,6 +544,286 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2,
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Streaming kernel for cache-build sizes (millions of rows, K * N <= 128 * 128).
+//
+// A wave owns one head and keeps that head's whole projection matrix in registers, already in
+// MFMA operand layout (N/32 * K/16 operands of 4 registers: 128 at 128 x 128), so the inner loop
+// reads nothing but rows.  Rows never pass through registers on their way in: every lane issues
+// 16-byte loads that the memory pipeline writes straight into LDS (lane l of an instruction
+// lands at byte 16 * l of that instruction's 1 KiB window), two 32-row tiles ahead of the tile
+// being computed.  The lane -> (row, 16-byte chunk) assignment of a load instruction is free as
+// long as 8 consecutive lanes cover one 128-byte line, so lane l fetches chunk (l % 8) ^ swz(row):
+// the rows arrive in LDS already swizzled for the conflict-free operand reads
+// (one 16-byte read per lane and MFMA k-step).  The slot-mapping entries of a tile travel the
+// same way (one 4-byte load per lane into the 256 bytes behind the tile).
+//
+// The loads are inline assembly on purpose: the wave waits with an explicit count for "all but
+// the newest tile's loads", which the compiler cannot express for loads whose destination is
+// LDS (it waits for every outstanding one before any LDS read).  Loads and stores of a wave
+// complete in issue order, and a wait for "at most n outstanding" only errs on the side of
+// waiting when more operations were issued behind the awaited one than n — so the count names
+// only the loads this code issues itself (a fixed number per tile; the last tile of a wave is
+// awaited with a full drain) and the compiler's own stores and reads merely make it wait a
+// little more.
+//
+// grid = persistent workgroups of 8 waves; global wave g: head g % H, tile stream g / H of
+// `nstreams` (tiles stream, stream + nstreams, ...).  LDS per wave: 2 x (tile + 256 bytes).
+// ---------------------------------------------------------------------------------------
+constexpr int kStreamWaves = 8;
+constexpr int kStreamThreads = kStreamWaves * 64;
+
+// One row group J (8 rows x 128 bytes) of a tile's line 0 or 1.  The instruction's immediate
+// offset moves the memory address AND the LDS address, so the window base of a line-1 load
+// (LDS bytes 4096 + 1024 J) is given 128 bytes low.
+#define UCM_DMA(J, WIN, OFF)                                            \
+    "s_add_u32 m0, %[lds], " #WIN "\n\ts_nop 0\n\t"                     \
+    "global_load_lds_dwordx4 %[o" #J "], %[base] offset:" #OFF " nt\n\t"
+
+// m0 (the LDS window of a load-to-LDS instruction) is put back as it was: the compiler treats
+// it as reserved and does not expect inline assembly to change it.
+template <int LN>
+__device__ __forceinline__ void stream_issue_rows(uint32_t lds, uint64_t base, const uint32_t (&off)[4])
+{
+    uint32_t keep;
+    if constexpr (LN == 2) {
+        asm volatile("s_mov_b32 %[keep], m0\n\t"
+                     UCM_DMA(0, 0, 0) UCM_DMA(1, 1024, 0) UCM_DMA(2, 2048, 0) UCM_DMA(3, 3072, 0)
+                     UCM_DMA(0, 3968, 128) UCM_DMA(1, 4992, 128) UCM_DMA(2, 6016, 128) UCM_DMA(3, 7040, 128)
+                     "s_mov_b32 m0, %[keep]\n\t"
+                     : [keep] "=&s"(keep)
+                     : [lds] "s"(lds), [base] "s"(base), [o0] "v"(off[0]), [o1] "v"(off[1]),
+                       [o2] "v"(off[2]), [o3] "v"(off[3])
+                     : "memory", "scc");
+    } else {
+        asm volatile("s_mov_b32 %[keep], m0\n\t"
+                     UCM_DMA(0, 0, 0) UCM_DMA(1, 1024, 0) UCM_DMA(2, 2048, 0) UCM_DMA(3, 3072, 0)
+                     "s_mov_b32 m0, %[keep]\n\t"
+                     : [keep] "=&s"(keep)
+                     : [lds] "s"(lds), [base] "s"(base), [o0] "v"(off[0]), [o1] "v"(off[1]),
+                       [o2] "v"(off[2]), [o3] "v"(off[3])
+                     : "memory", "scc");
+    }
+}
+
+__device__ __forceinline__ void stream_issue_slots(uint32_t lds, uint64_t base, uint32_t off)
+{
+    uint32_t keep;
+    asm volatile("s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[lds]\n\ts_nop 0\n\t"
+                 "global_load_lds_dword %[o], %[base]\n\ts_mov_b32 m0, %[keep]\n\t"
+                 : [keep] "=&s"(keep)
+                 : [lds] "s"(lds), [base] "s"(base), [o] "v"(off)
+                 : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void stream_wait_loads()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void stream_wait_lds()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
+// SLOT: 0 = identity slots (dense output), 1 = int32 slot mapping, 2 = int64 slot mapping.
+// ACCS: accumulator tiles in flight (the MFMAs of ACCS column tiles are interleaved, so that a
+// wave's consecutive MFMAs do not depend on each other).
+//
+// Stores: one 16-byte store per row and head.  Handing the codes of neighbouring heads to one
+// wave through LDS, which then writes whole 128-byte runs, was built and measured: the writes
+// got cheaper and the arrival counters, the extra LDS traffic and the waves waiting for each
+// other cost more than that (2.1 GB of keys: 476-520 us against 446 us).  What the stores cost
+// is not their size: on this part a read stream slows down by a fifth as soon as ANY write
+// stream runs beside it (2 GiB of plain 16-byte loads: 304 us alone, 350 us with 1.6 % writes,
+// 400 us with 6.25 % writes in 1 KiB runs, whatever the store's cache policy).
+template <typename V, int KS, int NT, int SLOT, int ACCS>
+__global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void encode_stream_kernel(
+    EncArgs a, int64_t ntiles, int nstreams)
+{
+    extern __shared__ __attribute__((aligned(1024))) uint8_t stream_lds[];
+    constexpr int K = KS * 16;
+    constexpr int LN = KS / 4;                      // 128-byte lines per row
+    constexpr int kTileBytes = kRowsPerWave * K * 2;
+    constexpr int kBufBytes = kTileBytes + 256;     // the tile's 32 slots behind its rows
+    constexpr int kLoads = 4 * LN + (SLOT ? 1 : 0);  // load instructions per tile
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int gw = blockIdx.x * kStreamWaves + wave;
+    const int h = gw % a.H;
+    const int stream = gw / a.H;
+    const int r = lane & 31, kb = lane >> 5;
+
+    uint8_t* mybuf = stream_lds + (size_t)wave * 2 * kBufBytes;
+
+    // ---- the head's projection matrix, in operand layout, for the kernel's lifetime ----
+    // 32 hash columns at a time are transposed through the wave's own (still unused) LDS: a lane
+    // fetches one 8 x 8 patch of W (eight 16-byte rows), transposes it in registers and writes the
+    // eight columns as LDS rows of K values; then every lane reads its K/16 operands.
+    V wreg[NT][KS];
+    {
+        constexpr int KP = K + kPad;
+        constexpr int kPatches = (K / 8) * 4;  // per 32 columns
+        uint16_t* wt = reinterpret_cast<uint16_t*>(mybuf);
+        const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N;
+        const int idx = lane % kPatches;
+        const int kq = idx >> 2, j = idx & 3;
+        // all patches of the head are requested before the first one is used: one round trip
+        u32x4 row[NT][8];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint16_t* src = wsrc + (int64_t)(kq * 8) * a.N + nt * 32 + 8 * j;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) row[nt][i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * a.N);
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                u32x4 o;
+                o.x = __builtin_amdgcn_perm(row[nt][1][c >> 1], row[nt][0][c >> 1], sel);
+                o.y = __builtin_amdgcn_perm(row[nt][3][c >> 1], row[nt][2][c >> 1], sel);
+                o.z = __builtin_amdgcn_perm(row[nt][5][c >> 1], row[nt][4][c >> 1], sel);
+                o.w = __builtin_amdgcn_perm(row[nt][7][c >> 1], row[nt][6][c >> 1], sel);
+                *reinterpret_cast<u32x4*>(wt + (8 * j + c) * KP + kq * 8) = o;
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                wreg[nt][ks] = *reinterpret_cast<const V*>(wt + r * KP + ks * 16 + kb * 8);
+            __builtin_amdgcn_wave_barrier();
+        }
+        stream_wait_lds();  // the staging area becomes the row buffers from here on
+    }
+
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)mybuf);
+    const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)h * a.x_stride_h;
+    const int slot_sz = SLOT == 2 ? 8 : 4;
+    const uint32_t row_bytes = (uint32_t)(a.x_stride_t * 2);
+
+    // lane's share of a tile's loads: row 8 j + lane / 8 of the tile, chunk (lane % 8) ^ swz(row);
+    // rows past the end of the input re-read its last row
+    uint32_t off_full[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t q = 8 * j + (lane >> 3);
+        off_full[j] = q * row_bytes + ((((uint32_t)lane & 7) ^ ((q ^ (q >> 3)) & 7)) << 4);
+    }
+    const uint32_t slot_e = SLOT == 2 ? (uint32_t)lane >> 1 : (uint32_t)lane & 31;
+    const uint32_t slot_full = slot_e * slot_sz + (SLOT == 2 ? ((uint32_t)lane & 1) * 4 : 0);
+    auto issue = [&](int64_t tile, int b) {
+        const int64_t t0 = tile * kRowsPerWave;
+        const int64_t left64 = a.T - 1 - t0;
+        const uint64_t base = (uint64_t)(uintptr_t)(xbase + t0 * a.x_stride_t);
+        const uint32_t lds = lds0 + b * kBufBytes;
+        uint32_t so = slot_full;
+        if (left64 >= 31) {
+            stream_issue_rows<LN>(lds, base, off_full);
+        } else {
+            const uint32_t left = (uint32_t)left64;
+            uint32_t off[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t q = 8 * j + (lane >> 3);
+                const uint32_t qq = q > left ? left : q;
+                off[j] = qq * row_bytes + ((((uint32_t)lane & 7) ^ ((q ^ (q >> 3)) & 7)) << 4);
+            }
+            stream_issue_rows<LN>(lds, base, off);
+            const uint32_t ee = slot_e > left ? left : slot_e;
+            so = ee * slot_sz + (SLOT == 2 ? ((uint32_t)lane & 1) * 4 : 0);
+        }
+        if constexpr (SLOT != 0)
+            // 4 bytes per lane: the tile's 32 slots (int64: lane l = half l % 2 of slot l / 2)
+            stream_issue_slots(lds + kTileBytes, (uint64_t)(uintptr_t)((const char*)a.slot + t0 * slot_sz), so);
+    };
+
+    // operand read offsets (conflict-free with the swizzle above)
+    uint32_t r_off[4];
+#pragma unroll
+    for (int c2 = 0; c2 < 4; ++c2) r_off[c2] = r * 128 + (((2 * c2 + kb) ^ ((r ^ (r >> 3)) & 7)) << 4);
+
+    // The host only sends shapes here whose block size is a power of two, whose code rows are
+    // 16-byte aligned when they are four words, and whose cache spans less than 2^31 words:
+    // one shift, two 32-bit multiplications, one store.
+    uint32_t words_prev[NT];
+    uint32_t* dst_prev = nullptr;
+#pragma unroll
+    for (int q = 0; q < NT; ++q) words_prev[q] = 0;
+    const int64_t n_slots = a.NB << a.bs_shift;
+    uint32_t* const cache_h = a.cache + (int64_t)h * a.cs_head;
+    const uint32_t csb = (uint32_t)a.cs_block, cst = (uint32_t)a.cs_token;
+
+    auto store_prev = [&]() {
+        if (dst_prev) {
+            if constexpr (NT == 4) {
+                u32x4 v = {words_prev[0], words_prev[1 % NT], words_prev[2 % NT], words_prev[3 % NT]};
+                *reinterpret_cast<u32x4*>(dst_prev) = v;
+            } else {
+#pragma unroll
+                for (int q = 0; q < NT; ++q) dst_prev[q] = words_prev[q];
+            }
+        }
+    };
+
+    // newer: the next tile's loads are in flight behind this tile's; more: a tile two ahead exists
+    auto step = [&](int64_t tile, int b, bool newer, bool more) {
+        const uint8_t* buf = mybuf + b * kBufBytes;
+        if (newer) stream_wait_loads<kLoads>();  // everything but the newest tile's loads has landed
+        else stream_wait_loads<0>();
+        V av[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            av[ks] = *reinterpret_cast<const V*>(buf + (ks >> 2) * 4096 + r_off[ks & 3]);
+        const int64_t t = tile * kRowsPerWave + r;
+        int64_t sv = t;
+        if constexpr (SLOT == 2) sv = *reinterpret_cast<const int64_t*>(buf + kTileBytes + r * 8);
+        if constexpr (SLOT == 1) sv = *reinterpret_cast<const int32_t*>(buf + kTileBytes + r * 4);
+        stream_wait_lds();  // the buffer may be overwritten from here on
+        store_prev();
+        if (more) issue(tile + 2 * (int64_t)nstreams, b);
+
+        const bool ok = t < a.T && lane < 32 && sv >= 0 && sv < n_slots;
+        const uint32_t svl = (uint32_t)sv;  // below 2^31 when ok
+        dst_prev = ok ? cache_h + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) : nullptr;
+
+#pragma unroll
+        for (int n0 = 0; n0 < NT; n0 += ACCS) {
+            f32x16 acc[ACCS];
+#pragma unroll
+            for (int q = 0; q < ACCS; ++q) acc[q] = acc_start();
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int q = 0; q < ACCS; ++q) acc[q] = Mfma<V>::run(wreg[n0 + q][ks], av[ks], acc[q]);
+#pragma unroll
+            for (int q = 0; q < ACCS; ++q) {
+                const uint32_t half = pack_half(acc[q]);
+                words_prev[n0 + q] = join_halves(kb ? half << 4 : half);
+            }
+        }
+    };
+
+    // tiles stream, stream + nstreams, ... : n of them
+    const int64_t n = stream < ntiles ? (ntiles - 1 - stream) / nstreams + 1 : 0;
+    int64_t tile = stream;
+    if (n > 0) issue(tile, 0);
+    if (n > 1) issue(tile + nstreams, 1);
+    for (int64_t i = 0; i < n; i += 2) {
+        step(tile, 0, i + 1 < n, i + 2 < n);
+        tile += nstreams;
+        if (i + 1 >= n) break;
+        step(tile, 1, i + 2 < n, i + 3 < n);
+        tile += nstreams;
+    }
+    store_prev();
+    // no load may still be writing into this workgroup's LDS when the wave ends
+    stream_wait_loads<0>();
+}
+
 // Latency path for a handful of rows (decode): one wave per (job, head, 32 hash columns,
 // 32 rows).  No LDS and no persistent loop: the B operand is assembled straight from the
 // row-major projection matrix with eight 2-byte loads per k-step, all issued up front, so the
@@ -761,6 +1043,90 @@ bool mfma_eligible(const EncArgs& a, int x_dtype, int w_dtype)
     return same16 && k_ok && aligned && paged_ok;
 }
 
+// ---- streaming kernel: eligibility and launch ----
+// rows x heads from which the streaming kernel is used: below about a million rows its fixed
+// cost (every wave stages a projection matrix of its own, 256 persistent workgroups) loses against
+// the tiled kernel (65,536 rows: 14.8 against 12.4 us; 1M rows: 67.6 against 71.8 us; 4M rows: 225
+// against 262 us)
+constexpr int64_t kStreamMinRows = (int64_t)1 << 20;
+std::atomic<int64_t> g_stream_min_rows{kStreamMinRows};
+
+int stream_workgroups()
+{
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        cus = n;
+    }
+    return cus;
+}
+
+bool stream_eligible(const EncArgs& a, int x_dtype, int w_dtype)
+{
+    if (!mfma_eligible(a, x_dtype, w_dtype) || a.src_blocks) return false;
+    if (!((a.K == 128 && (a.N == 128 || a.N == 64)) || (a.K == 64 && (a.N == 128 || a.N == 64)))) return false;
+    if (a.T * a.H < g_stream_min_rows.load(std::memory_order_relaxed)) return false;
+    if (a.slot && ((uintptr_t)a.slot & 3)) return false;
+    // one shift per slot, one 16-byte store per four-word code (set_block_shift() has run)
+    if (a.bs_shift < 0) return false;
+    if (a.N == 128 && ((((uintptr_t)a.cache) & 15) || a.cs_block % 4 || a.cs_token % 4 || a.cs_head % 4)) return false;
+    // 32-bit offsets into the cache: non-negative strides, the last slot below 2^31 words
+    if (a.cs_block < 0 || a.cs_token < 0 || a.cs_head < 0) return false;
+    if ((double)a.NB * (double)a.cs_block + (double)a.BS * (double)a.cs_token >= 2147483648.0) return false;
+    if ((double)a.NB * (double)a.BS >= 2147483648.0) return false;
+    // every head needs at least one wave, and the heads must share the waves evenly
+    const int waves = stream_workgroups() * kStreamWaves;
+    return a.H <= waves;
+}
+
+template <typename V, int KS, int NT, int SLOT, int ACCS>
+int launch_stream_a(const EncArgs& a, hipStream_t st)
+{
+    constexpr size_t lds = (size_t)kStreamWaves * 2 * (kRowsPerWave * KS * 32 + 256);
+    static int opted = 0;  // 0 = not tried, 1 = allowed, -1 = refused by the runtime
+    if (opted == 0) {
+        const hipError_t e = hipFuncSetAttribute((const void*)encode_stream_kernel<V, KS, NT, SLOT, ACCS>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) (void)hipGetLastError();
+        opted = (e == hipSuccess) ? 1 : -1;
+    }
+    if (opted < 0) return UCM_EUNSUPPORTED;
+    int wgs = stream_workgroups();
+    // total waves a multiple of the head count: lower the workgroup count until it is
+    while (wgs > 1 && (wgs * kStreamWaves) % a.H) --wgs;
+    if ((wgs * kStreamWaves) % a.H) return UCM_EUNSUPPORTED;
+    const int nstreams = wgs * kStreamWaves / a.H;
+    const int64_t ntiles = ucm::ceil_div(a.T, kRowsPerWave);
+    hipLaunchKernelGGL((encode_stream_kernel<V, KS, NT, SLOT, ACCS>), dim3((unsigned)wgs), dim3(kStreamThreads),
+                       lds, st, a, ntiles, nstreams);
+    return ucm::launch_status("encode_stream_kernel");
+}
+
+template <typename V, int KS, int NT, int SLOT>
+int launch_stream_i(const EncArgs& a, hipStream_t st)
+{
+    return launch_stream_a<V, KS, NT, SLOT, (NT == 4 ? 4 : 2)>(a, st);
+}
+
+template <typename V, int KS, int NT>
+int launch_stream_s(const EncArgs& a, hipStream_t st)
+{
+    if (!a.slot) return launch_stream_i<V, KS, NT, 0>(a, st);
+    return a.slot_is_i64 ? launch_stream_i<V, KS, NT, 2>(a, st) : launch_stream_i<V, KS, NT, 1>(a, st);
+}
+
+template <typename V>
+int launch_stream(const EncArgs& a, hipStream_t st)
+{
+    if (a.K == 128) return a.N == 128 ? launch_stream_s<V, 8, 4>(a, st) : launch_stream_s<V, 8, 2>(a, st);
+    return a.N == 128 ? launch_stream_s<V, 4, 4>(a, st) : launch_stream_s<V, 4, 2>(a, st);
+}
+
 int64_t small_waves(const EncArgs& a)
 {
     return ucm::ceil_div(a.T, kRowsPerWave) * a.H * (a.N / 32);
@@ -945,6 +1311,11 @@ int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
         return x_dtype == UCM_DT_BF16 ? launch_small<bf16x8>(js, js.waves0, a.K, st)
                                       : launch_small<f16x8>(js, js.waves0, a.K, st);
     }
+    if (stream_eligible(a, x_dtype, w_dtype)) {
+        rc = x_dtype == UCM_DT_BF16 ? launch_stream<bf16x8>(a, st) : launch_stream<f16x8>(a, st);
+        if (rc != UCM_EUNSUPPORTED) return rc;  // no large-LDS opt-in: the tiled kernel below
+        ucm::clear_error();
+    }
     if (mfma_eligible(a, x_dtype, w_dtype))
         return x_dtype == UCM_DT_BF16 ? dispatch_mfma<bf16x8>(a, st) : dispatch_mfma<f16x8>(a, st);
     // same element type on both sides, enough rows to fill a tile, grid within limits
@@ -982,6 +1353,13 @@ extern "C" int ucm_hash_encode(const void* x, int x_dtype, int64_t T, int32_t H,
     a.w = w; a.n_w = n_w; a.heads_per_w = heads_per_w; a.N = N_bits;
     a.out = out; a.out_stride_t = out_stride_t; a.out_stride_h = out_stride_h;
     return encode_common(a, x_dtype, w_dtype, (hipStream_t)stream);
+}
+
+extern "C" int ucm_hash_encode_set_stream_threshold(int64_t rows)
+{
+    ucm::clear_error();
+    g_stream_min_rows.store(rows > 0 ? rows : kStreamMinRows, std::memory_order_relaxed);
+    return UCM_OK;
 }
 
 extern "C" int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int32_t K,
