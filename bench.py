@@ -284,6 +284,81 @@ def encoder_cache_build(torch, enc_k, gen, launches=9):
                     "the published peak; the same reads alone take 304 us"}
 
 
+def plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots):
+    """The same decode step at the reference's plugin surface: GSAOnDevice.attention_begin +
+    attention_finished per layer (group-mean query, best KV head per block, sink = one block,
+    recent = four blocks, physical ids, replacement table and lengths), once as the single
+    native call and once as the separate operators, eager and as HIP-graph replays."""
+    import types
+
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa_on_device import GSAOnDevice
+
+    name = "model.layers.1.self_attn.attn"
+    cfg = {"ucm_sparse_config": {"GSAOnDevice": {
+        "num_q_heads": HQ, "num_kv_heads": HKV, "head_dim": D, "block_size": BS,
+        "vllm_hash_attention_topk": TOPK * BS, "seed": 3}}}
+    plugin = GSAOnDevice(cfg, UcmSparseRole.WORKER)
+    R = len(caches)
+    q2 = queries.reshape(B, HQ * D)
+    k2 = new_keys.reshape(B, HKV * D)
+    metas = [types.SimpleNamespace(slot_mapping=new_slots[r], block_table=tables[r], seq_lens=lens)
+             for r in range(R)]
+    ctxs = [types.SimpleNamespace(attn_metadata={name: m}) for m in metas]
+
+    def call(i):
+        r = i % R
+        plugin.attention_begin(q2, k2, None, name, ctxs[r], phase="decode", k_hash=caches[r])
+        plugin.attention_finished(q2, k2, None, None, name, ctxs[r], phase="decode")
+
+    out = {"shape": "configs[1]: batch 32 x 32768 tokens, top-64 blocks per request (best KV head), "
+                    "sink 128 + recent 512 tokens kept", "cache_rotation": R}
+    for mode in ("single_call", "separate_operators"):
+        plugin.fused_decode = mode == "single_call"
+        for i in range(2 * R):
+            call(i)
+        torch.cuda.synchronize()
+        n = 100
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+        t0 = time.perf_counter()
+        for i in range(n):
+            ev[i].record()
+            call(i)
+        ev[n].record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / n * 1e6
+        gaps = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(n))
+        res = {"eager_p50_us": gaps[n // 2], "eager_p90_us": gaps[int(n * 0.9)], "eager_wall_us_per_call": wall}
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for i in range(R):
+                    call(i)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for i in range(R):
+                    call(i)
+            g.replay()
+            torch.cuda.synchronize()
+            m = 50
+            ge = [torch.cuda.Event(enable_timing=True) for _ in range(m + 1)]
+            for i in range(m):
+                ge[i].record()
+                g.replay()
+            ge[m].record()
+            torch.cuda.synchronize()
+            gg = sorted(ge[i].elapsed_time(ge[i + 1]) * 1e3 / R for i in range(m))
+            res["graph_p50_us"] = gg[m // 2]
+            res["graph_p90_us"] = gg[int(m * 0.9)]
+        except Exception as e:  # noqa: BLE001
+            res["graph_error"] = str(e)[:200]
+        out[mode] = res
+    return out
+
+
 def extras(torch, enc_k, gen):
     """Side figures: encoder at cache-build shape, device gather, pinned-host dump."""
     import numpy as np
@@ -717,9 +792,16 @@ def main():
         line["cpu_baseline"] = cpu_baseline(torch, caches[0], tables[0], qc, lens)
         line["gpu_over_cpu"] = line["value"] / line["cpu_baseline"]["value"]
     if not args.skip_extras:
+        plug = plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots)
+        line["plugin_attention_begin_p50_us"] = {
+            "single_call_graph": plug["single_call"].get("graph_p50_us"),
+            "single_call_eager": plug["single_call"]["eager_p50_us"],
+            "separate_operators_graph": plug["separate_operators"].get("graph_p50_us"),
+            "separate_operators_eager": plug["separate_operators"]["eager_p50_us"]}
         del caches[1:], tables[1:]
         torch.cuda.empty_cache()
         line["extras"] = extras(torch, enc_k, gen)
+        line["extras"]["plugin_surface"] = plug
         if not args.skip_cpu:
             line["extras"].update(cpu_side_baselines(torch))
     print(json.dumps(line))

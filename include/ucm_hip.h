@@ -297,6 +297,44 @@ int ucm_sparse_decode_step_mla(const void* new_nope, int64_t nope_stride_t,
                                uint32_t* q_codes, int32_t* out_idx, int32_t* out_score,
                                void* workspace, size_t workspace_bytes, ucm_stream_t stream);
 
+/*
+ * The per-layer decode work of the reference's GQA plugin in one call, with the outputs in the
+ * form its attention backend reads: replaces GSAOnDevice.attention_begin at decode
+ * (ucm/sparse/gsa_on_device/gsa_on_device.py:564-572 cache_k_hash_gqa_cuda, :396-412 hash_code,
+ * :773-811 update_decode_topk_gqa_cuda) and cuda_hamming_topk / update_seq_lens
+ * (hamming_topk.py:7-54) — a dozen framework launches there, three kernel launches here.
+ *
+ *   1. the codes of the step's new keys go to the paged code cache (as ucm_hash_encode_cache);
+ *   2. the queries of every KV head's group are averaged (fp32 sum, times 1/G, rounded to the
+ *      input type — what `query.view(B, Hkv, G, D).mean(2)` gives, gsa_on_device.py:400-406) and
+ *      hashed: q_codes uint32 [B, Hkv, N_bits/32], contiguous scratch;
+ *   3. blocks are scored against their KV head's code, the best head counts
+ *      (UCM_TOPK_REDUCE_HEADS, hamming_topk.py:33), blocks holding a position < sink_tok or
+ *      >= len - recent_tok are always kept, and the topk_tok / BS best blocks are selected;
+ *   4. new_block_table[b, 0 .. max_blocks) = the selected physical ids in logical order, 0 in
+ *      every other entry (gsa_on_device.py:789-791); new_seq_lens[b] = len - ceil(max(len -
+ *      topk_tok, 0) / BS) * BS (hamming_topk.py:7-12).  A request with len < seq_len_threshold
+ *      (threshold > 0) keeps its own table row and length.
+ *
+ * Arguments as in ucm_sparse_decode_step; new_block_table int32 [B, new_table_stride] with
+ * new_table_stride >= max_blocks <= 4096, new_seq_lens int32 [B].  Requires topk_tok % BS == 0,
+ * recent_tok > 0 and topk_tok > sink_tok + recent_tok (hamming_topk.py:30-31); bf16 / fp16 inputs
+ * of 64, 128, 256 or 512 dimensions.  Allocates nothing.
+ */
+int ucm_gsa_decode_step(const void* new_keys, int64_t T, int64_t k_stride_t, int64_t k_stride_h,
+                        const void* slot_mapping, int slot_is_i64,
+                        const void* queries, int64_t q_stride_b, int64_t q_stride_h,
+                        int x_dtype, int32_t K,
+                        const void* w, int w_dtype, int32_t n_w, int32_t N_bits,
+                        uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
+                        int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                        const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                        const int32_t* seq_lens, int32_t B, int32_t Hq, int32_t topk_tok,
+                        int32_t sink_tok, int32_t recent_tok, int32_t seq_len_threshold,
+                        uint32_t* q_codes, int32_t* new_block_table, int32_t new_table_stride,
+                        int32_t* new_seq_lens, void* workspace, size_t workspace_bytes,
+                        ucm_stream_t stream);
+
 /* Replaces update_seq_lens (hamming_topk.py:7-12):
  * out[b] = len[b] - ceil(max(len[b] - topk_tok, 0) / BS) * BS. */
 int ucm_update_seq_lens(const int32_t* seq_lens, int32_t B, int32_t topk_tok, int32_t BS,

@@ -116,6 +116,110 @@ def test_plugin_hooks_swap_and_restore_the_block_table():
     assert torch.equal(meta0.block_table, table)
 
 
+@pytest.mark.parametrize("threshold", [0, 2000])
+def test_plugin_single_call_decode_equals_separate_operators_and_oracle(threshold):
+    """attention_begin at decode as ONE native call (ucm_gsa_decode_step) against the same hook
+    running the separate operators (encode-and-cache, mean-query hash, top-k, torch table swap)
+    and against the CPU checker: identical code cache, replacement table and lengths.  Lengths
+    include a request shorter than the top-k budget, one shorter than the threshold and a ragged
+    last block."""
+    from ucm_amd.sparse.base import UcmSparseFactory, UcmSparseRole
+
+    B, Hq, Hkv, D, BS, nblk, topk_tok = 5, 32, 8, 128, 128, 40, 2048
+    name = "model.layers.3.self_attn.attn"
+    rng = rng_for(91)
+    NB = B * nblk + 3
+    base_codes = torch.from_numpy(rng.integers(0, 256, size=(NB, BS, Hkv, D // 8), dtype=np.uint8)).cuda()
+    table = torch.from_numpy(rng.permutation(NB)[: B * nblk].astype(np.int32).reshape(B, nblk)).cuda()
+    lens = torch.tensor([nblk * BS, nblk * BS - 300, 9 * BS + 1, 1500, 17 * BS], dtype=torch.int32, device="cuda")
+    q = torch.from_numpy(rng.standard_normal((B, Hq * D)).astype(np.float32)).to(torch.bfloat16).cuda()
+    newk = torch.from_numpy(rng.standard_normal((B, Hkv * D)).astype(np.float32)).to(torch.bfloat16).cuda()
+    pos = lens.long() - 1
+    slots = table[torch.arange(B), pos // BS].long() * BS + pos % BS
+    results = []
+    for fused in (True, False):
+        cfg = {"ucm_sparse_config": {"GSAOnDevice": {
+            "num_q_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "block_size": BS,
+            "vllm_hash_attention_topk": topk_tok, "gpu_seq_len_threshold": threshold,
+            "fused_decode": fused, "seed": 11}}}
+        plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+        k_hash = base_codes.clone()
+        meta = types.SimpleNamespace(slot_mapping=slots, block_table=table.clone(), seq_lens=lens.clone())
+        ctx = types.SimpleNamespace(attn_metadata={name: meta})
+        for _ in range(2):  # twice: the step's buffers are reused
+            plugin.attention_begin(q, newk, None, name, ctx, phase="decode", k_hash=k_hash)
+            torch.cuda.synchronize()
+            out = (k_hash.clone(), meta.block_table.clone(), meta.seq_lens.clone())
+            plugin.attention_finished(q, newk, None, None, name, ctx, phase="decode")
+            assert torch.equal(meta.block_table, table) and torch.equal(meta.seq_lens, lens)
+        results.append((plugin, out))
+    (pf, (kh_f, bt_f, sl_f)), (ps, (kh_s, bt_s, sl_s)) = results
+    assert torch.equal(pf.hash_encoder.hash_weights, ps.hash_encoder.hash_weights)
+    assert torch.equal(kh_f, kh_s), "code cache differs between the single call and the separate operators"
+    assert torch.equal(bt_f, bt_s) and torch.equal(sl_f, sl_s)
+    # the query codes of the single call are the codes of torch's group mean
+    step = next(iter(pf._fused_steps.values()))
+    qc_sep = ps.hash_code(q.view(B, Hq, D)).view(torch.int32)
+    assert torch.equal(step.q_codes, qc_sep)
+    # and the CPU checker on the codes now in the cache
+    kblk = topk_tok // BS
+    oi, _ = c_api.hamming_topk(step.q_codes.cpu().numpy().view(np.uint32),
+                               kh_f.cpu().numpy().view(np.uint32).reshape(NB, BS, Hkv, D // 32),
+                               table.cpu().numpy(), lens.cpu().numpy(), kblk, BS, 4 * BS,
+                               flags=c_api.F_REDUCE_HEADS | c_api.F_PHYSICAL)
+    exp_t = np.zeros((B, nblk), np.int32)
+    exp_t[:, :kblk] = np.maximum(oi[:, 0], 0)
+    exp_l = c_api.update_seq_lens(lens.cpu().numpy(), topk_tok, BS)
+    if threshold:
+        short = lens.cpu().numpy() < threshold
+        exp_t[short] = table.cpu().numpy()[short]
+        exp_l[short] = lens.cpu().numpy()[short]
+        assert short.any() and not short.all()
+    assert np.array_equal(bt_f.cpu().numpy(), exp_t)
+    assert np.array_equal(sl_f.cpu().numpy(), exp_l)
+
+
+def test_single_call_decode_step_in_a_hip_graph():
+    """GSADecodeStep allocates nothing: captured once, replayed with changing inputs, every replay
+    checked against an eager call."""
+    from ucm_amd.sparse import GSADecodeStep
+
+    B, Hq, Hkv, D, BS, nblk, topk_tok = 4, 32, 8, 128, 128, 32, 1024
+    rng = rng_for(92)
+    NB = B * nblk
+    W = torch.from_numpy(rng.standard_normal((D, D)).astype(np.float32)).to(torch.bfloat16).cuda()
+    cache = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=(NB, BS, Hkv, D // 32), dtype=np.int64)
+                             .astype(np.int32)).cuda()
+    table = torch.from_numpy(rng.permutation(NB).astype(np.int32).reshape(B, nblk)).cuda()
+    lens = torch.full((B,), nblk * BS, dtype=torch.int32, device="cuda")
+    q = torch.empty((B, Hq, D), dtype=torch.bfloat16, device="cuda")
+    newk = torch.empty((B, Hkv, D), dtype=torch.bfloat16, device="cuda")
+    slots = (table[:, -1].long() * BS + BS - 1)
+    step = GSADecodeStep(W, Hq, Hkv, B, nblk, topk_tok, block_size=BS)
+    eager = GSADecodeStep(W, Hq, Hkv, B, nblk, topk_tok, block_size=BS)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        q.normal_(); newk.normal_()
+        step.step(newk, slots, q, cache, table, lens)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step.step(newk, slots, q, cache, table, lens)
+    for it in range(4):
+        q.normal_(); newk.normal_()
+        lens[it % B] -= 37 * (it + 1)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = (step.new_table.clone(), step.new_lens.clone(), step.q_codes.clone())
+        eager.step(newk, slots, q, cache, table, lens)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], eager.new_table) and torch.equal(got[1], eager.new_lens)
+        assert torch.equal(got[2], eager.q_codes)
+
+
 def test_plugin_rehashes_a_prefix_cache_hit_from_the_key_cache():
     """Two requests whose prompt prefixes were loaded from the store into the paged KV cache:
     the hook must produce, for the prefix tokens, the codes a full prefill of the same keys

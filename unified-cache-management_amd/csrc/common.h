@@ -54,6 +54,7 @@ struct PairSpec {
     const void* queries; int64_t B; int Hq; int64_t q_stride_b, q_stride_h;
     uint32_t* q_codes; int64_t qc_stride_b, qc_stride_h;
     int x_dtype; int K; const void* w; int w_dtype; int n_w; int N_bits;
+    int q_group_mean = 0;  // hash the mean of every KV head's query group: q_codes is [B, Hkv, Wd]
 };
 // one launch when both jobs are small
 int encode_pair(const PairSpec& p, hipStream_t st);

@@ -1110,7 +1110,38 @@ struct SelectArgs {
     uint32_t flags;
     int32_t* out_idx;    // [B][Ho][k]
     int32_t* out_score;  // may be null
+    // Replacement block table and sequence lengths of a decode step (null = not asked for; needs
+    // Ho == 1 and physical ids): row b of new_table gets the selected ids in its first k entries
+    // and 0 in all others up to max_blocks; a request shorter than thr_len keeps its own row and
+    // length; new_lens[b] = len - ceil(max(len - topk_tok, 0) / BS) * BS otherwise.
+    int32_t* new_table;
+    int new_table_stride;
+    int32_t* new_lens;
+    int thr_len, topk_tok;
 };
+
+// The first part of that epilogue, shared by the selection kernels: `tid` of `nthreads` threads
+// own a row.  Returns true when the row is complete (short request or no blocks) and the
+// selection can be skipped; otherwise entries [kk, max_blocks) are zeroed and the caller
+// fills [0, kk).
+__device__ __forceinline__ bool plugin_row_prologue(const SelectArgs& a, int b, int len, int kk, int tid,
+                                                    int nthreads)
+{
+    int32_t* row = a.new_table + (int64_t)b * a.new_table_stride;
+    const bool keep = a.thr_len > 0 && len < a.thr_len;
+    if (tid == 0) {
+        int over = len - a.topk_tok;
+        over = over < 0 ? 0 : over;
+        a.new_lens[b] = keep ? len : len - ((over + a.BS - 1) / a.BS) * a.BS;
+    }
+    if (keep) {
+        const int32_t* src = a.table + (int64_t)b * a.table_stride;
+        for (int j = tid; j < a.max_blocks; j += nthreads) row[j] = src[j];
+        return true;
+    }
+    for (int j = kk + tid; j < a.max_blocks; j += nthreads) row[j] = 0;
+    return kk == 0;
+}
 
 // Exclusive prefix sum of one int per thread over the 256-thread workgroup; *total gets the
 // sum.  `wsum` is a 4-entry LDS array.
@@ -1346,11 +1377,17 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
     int32_t* oi = a.out_idx + ((int64_t)b * a.Ho + ho) * a.k;
     int32_t* os = a.out_score ? a.out_score + ((int64_t)b * a.Ho + ho) * a.k : nullptr;
     const int kk = a.k < n ? a.k : n;
-    for (int i = kk + lane; i < a.k; i += kWave) {
-        oi[i] = -1;
-        if (os) os[i] = 0;
+    if (a.new_table) {
+        if (plugin_row_prologue(a, b, len, kk, lane, kWave)) return;
+        oi = a.new_table + (int64_t)b * a.new_table_stride;
+        os = nullptr;
+    } else {
+        for (int i = kk + lane; i < a.k; i += kWave) {
+            oi[i] = -1;
+            if (os) os[i] = 0;
+        }
+        if (n == 0) return;
     }
-    if (n == 0) return;
     const bool reduce = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
     const int32_t* row = a.scores + (int64_t)b * a.Hkv * a.max_blocks + (int64_t)(reduce ? 0 : ho) * a.sc_h;
     int v[EL];
@@ -1476,11 +1513,17 @@ __global__ __launch_bounds__(kThreads) void select_group_kernel(SelectArgs a)
     int32_t* oi = a.out_idx + ((int64_t)b * a.Ho + ho) * a.k;
     int32_t* os = a.out_score ? a.out_score + ((int64_t)b * a.Ho + ho) * a.k : nullptr;
     const int kk = a.k < n ? a.k : n;
-    for (int i = kk + tid; i < a.k; i += kThreads) {
-        oi[i] = -1;
-        if (os) os[i] = 0;
+    if (a.new_table) {
+        if (plugin_row_prologue(a, b, len, kk, tid, kThreads)) return;  // the same for every thread
+        oi = a.new_table + (int64_t)b * a.new_table_stride;
+        os = nullptr;
+    } else {
+        for (int i = kk + tid; i < a.k; i += kThreads) {
+            oi[i] = -1;
+            if (os) os[i] = 0;
+        }
+        if (n == 0) return;  // the same for every thread of the row
     }
-    if (n == 0) return;  // the same for every thread of the row
     if (reduce) {
         for (int h0 = 1; h0 < a.Hkv; h0 += 8) {
             int o[8][EL];
@@ -1902,19 +1945,39 @@ extern "C" size_t ucm_hamming_topk_workspace_bytes(int32_t B, int32_t Hkv, int32
     return carve(nullptr, B, Hkv, max_blocks).bytes;
 }
 
-extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
-                                const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
-                                int32_t Wd, int64_t ks_block, int64_t ks_token, int64_t ks_head,
-                                const int32_t* block_table, int32_t table_stride,
-                                int32_t max_blocks, const int32_t* seq_lens, int32_t B,
-                                int32_t Hq, int32_t k, int32_t sink_tok, int32_t recent_tok,
-                                uint32_t flags, int32_t* out_idx, int32_t* out_score,
-                                void* workspace, size_t workspace_bytes, ucm_stream_t stream)
+namespace {
+
+// Outputs of a decode step in the form the serving engine's attention reads them (see
+// SelectArgs): replaces out_idx / out_score when given.
+struct StepOut {
+    int32_t* new_table;
+    int32_t new_table_stride;
+    int32_t* new_lens;
+    int32_t thr_len, topk_tok;
+};
+
+int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                     const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
+                     int64_t ks_block, int64_t ks_token, int64_t ks_head, const int32_t* block_table,
+                     int32_t table_stride, int32_t max_blocks, const int32_t* seq_lens, int32_t B,
+                     int32_t Hq, int32_t k, int32_t sink_tok, int32_t recent_tok, uint32_t flags,
+                     int32_t* out_idx, int32_t* out_score, void* workspace, size_t workspace_bytes,
+                     ucm_stream_t stream, const StepOut* step_out)
 {
-    ucm::clear_error();
     int rc = common_checks(q_codes, k_cache, seq_lens, NB, BS, Hkv, Wd, B, Hq, max_blocks);
     if (rc != UCM_OK) return rc;
-    UCM_REQUIRE(out_idx, "out_idx is null");
+    if (step_out) {
+        UCM_REQUIRE(step_out->new_table && step_out->new_lens && block_table, "null table or length output");
+        UCM_REQUIRE(step_out->new_table_stride >= max_blocks, "new table rows of %d entries for %d blocks",
+                    step_out->new_table_stride, max_blocks);
+        UCM_REQUIRE((flags & UCM_TOPK_RETURN_PHYSICAL) && !(flags & UCM_TOPK_SCORE_ORDER) &&
+                        ((flags & UCM_TOPK_REDUCE_HEADS) || Hkv == 1),
+                    "a replacement table is one list of physical ids per request");
+        if (max_blocks > 4096)
+            return ucm::fail(UCM_EUNSUPPORTED, "replacement tables support at most 4096 blocks per request");
+    } else {
+        UCM_REQUIRE(out_idx, "out_idx is null");
+    }
     UCM_REQUIRE(k > 0, "k must be positive");
     UCM_REQUIRE(!block_table || table_stride >= max_blocks, "table_stride %d < max_blocks %d",
                 table_stride, max_blocks);
@@ -2077,6 +2140,11 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     s.key_bits = 1;
     while ((1ll << s.key_bits) <= (int64_t)s.full + 1) ++s.key_bits;
     s.flags = flags; s.out_idx = out_idx; s.out_score = out_score;
+    s.new_table = step_out ? step_out->new_table : nullptr;
+    s.new_table_stride = step_out ? step_out->new_table_stride : 0;
+    s.new_lens = step_out ? step_out->new_lens : nullptr;
+    s.thr_len = step_out ? step_out->thr_len : 0;
+    s.topk_tok = step_out ? step_out->topk_tok : 0;
     const int rows_total = B * s.Ho;
     const dim3 wgrid((unsigned)ucm::ceil_div(rows_total, kThreads / kWave));
     if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256) {
@@ -2099,6 +2167,62 @@ extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int
     }
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
     return ucm::launch_status("select_kernel");
+}
+
+}  // namespace
+
+extern "C" int ucm_hamming_topk(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
+                                const uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
+                                int32_t Wd, int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                                const int32_t* block_table, int32_t table_stride,
+                                int32_t max_blocks, const int32_t* seq_lens, int32_t B,
+                                int32_t Hq, int32_t k, int32_t sink_tok, int32_t recent_tok,
+                                uint32_t flags, int32_t* out_idx, int32_t* out_score,
+                                void* workspace, size_t workspace_bytes, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    return hamming_topk_run(q_codes, q_stride_b, q_stride_h, k_cache, NB, BS, Hkv, Wd, ks_block, ks_token,
+                            ks_head, block_table, table_stride, max_blocks, seq_lens, B, Hq, k, sink_tok,
+                            recent_tok, flags, out_idx, out_score, workspace, workspace_bytes, stream,
+                            nullptr);
+}
+
+/* One GQA decode step as the reference's plugin performs it, see ucm_hip.h. */
+extern "C" int ucm_gsa_decode_step(const void* new_keys, int64_t T, int64_t k_stride_t, int64_t k_stride_h,
+                                   const void* slot_mapping, int slot_is_i64, const void* queries,
+                                   int64_t q_stride_b, int64_t q_stride_h, int x_dtype, int32_t K,
+                                   const void* w, int w_dtype, int32_t n_w, int32_t N_bits,
+                                   uint32_t* k_cache, int64_t NB, int32_t BS, int32_t Hkv,
+                                   int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                                   const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                                   const int32_t* seq_lens, int32_t B, int32_t Hq, int32_t topk_tok,
+                                   int32_t sink_tok, int32_t recent_tok, int32_t seq_len_threshold,
+                                   uint32_t* q_codes, int32_t* new_block_table, int32_t new_table_stride,
+                                   int32_t* new_seq_lens, void* workspace, size_t workspace_bytes,
+                                   ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(Hkv > 0 && Hq > 0 && Hq % Hkv == 0, "bad head counts");
+    UCM_REQUIRE(N_bits > 0 && N_bits % 32 == 0, "hash_bits must be a multiple of 32");
+    UCM_REQUIRE(n_w == 1 || n_w == Hkv, "n_w must be 1 or the number of KV heads");
+    UCM_REQUIRE(q_codes, "q_codes is null");
+    // the reference's own checks (hamming_topk.py:30-31)
+    UCM_REQUIRE(BS > 0 && topk_tok > 0 && topk_tok % BS == 0, "topk_token %d is no multiple of the block size %d",
+                topk_tok, BS);
+    UCM_REQUIRE(recent_tok > 0 && topk_tok > sink_tok + recent_tok, "topk_token must exceed sink + recent > 0");
+    const int32_t Wd = N_bits / 32;
+    ucm::PairSpec spec{new_keys, T, Hkv, k_stride_t, k_stride_h, slot_mapping, slot_is_i64,
+                       k_cache, NB, BS, ks_block, ks_token, ks_head, queries, B, Hq,
+                       q_stride_b, q_stride_h, q_codes, (int64_t)Hkv * Wd, Wd, x_dtype, K, w,
+                       w_dtype, n_w, N_bits};
+    spec.q_group_mean = 1;
+    int rc = ucm::encode_pair(spec, (hipStream_t)stream);
+    if (rc != UCM_OK) return rc;
+    const StepOut so{new_block_table, new_table_stride, new_seq_lens, seq_len_threshold, topk_tok};
+    return hamming_topk_run(q_codes, (int64_t)Hkv * Wd, Wd, k_cache, NB, BS, Hkv, Wd, ks_block, ks_token,
+                            ks_head, block_table, table_stride, max_blocks, seq_lens, B, Hkv, topk_tok / BS,
+                            sink_tok, recent_tok, UCM_TOPK_REDUCE_HEADS | UCM_TOPK_RETURN_PHYSICAL, nullptr,
+                            nullptr, workspace, workspace_bytes, stream, &so);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -63,6 +63,11 @@ struct EncArgs {
     int BS;
     int64_t cs_block, cs_token, cs_head;
     int BN;        // hash columns per workgroup slice
+    // group mean (small-row kernel only): row (t, h) is the mean of the gmean source rows
+    // (t, h * gmean + g) at x_stride_g elements from one another, rounded to the input type as
+    // a framework's mean over the group would be; 0 or 1 = plain rows
+    int gmean;
+    int64_t x_stride_g;
     int bs_shift;  // log2(BS) when BS is a power of two, else -1
 };
 
@@ -251,6 +256,7 @@ template <typename V>
 struct Mfma;
 template <>
 struct Mfma<bf16x8> {
+    typedef __bf16 elem;
     static __device__ __forceinline__ f32x16 run(bf16x8 a, bf16x8 b, f32x16 c)
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
@@ -258,6 +264,7 @@ struct Mfma<bf16x8> {
 };
 template <>
 struct Mfma<f16x8> {
+    typedef _Float16 elem;
     static __device__ __forceinline__ f32x16 run(f16x8 a, f16x8 b, f32x16 c)
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
@@ -858,8 +865,28 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
     // this kernel has anyway
     V av[KS];
     uint16_t bw[KS][8];
+    if (a.gmean > 1) {
+        // fp32 sum of the group's rows in order, times 1/G, rounded to the input type
+        const float inv = 1.0f / (float)a.gmean;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
+        for (int ks = 0; ks < KS; ++ks) {
+            float sum[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum[i] = 0.0f;
+            for (int g = 0; g < a.gmean; ++g) {
+                const V v = *reinterpret_cast<const V*>(xr + (int64_t)g * a.x_stride_g + ks * 16);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sum[i] += (float)v[i];
+            }
+            V m;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) m[i] = (typename Mfma<V>::elem)(sum[i] * inv);  // round to nearest even
+            av[ks] = m;
+        }
+    } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -1440,6 +1467,14 @@ int build_pair(const PairSpec& p, EncArgs& kk, EncArgs& kq, bool& has_keys)
     kq.x = p.queries; kq.T = p.B; kq.H = p.Hq; kq.K = p.K; kq.x_stride_t = p.q_stride_b;
     kq.x_stride_h = p.q_stride_h; kq.w = p.w; kq.n_w = p.n_w;
     kq.heads_per_w = p.n_w > 1 ? p.Hq / p.Hkv : 0; kq.N = p.N_bits;
+    if (p.q_group_mean && p.Hq > p.Hkv) {
+        // one row per KV head: the mean of its Hq / Hkv query heads
+        kq.H = p.Hkv;
+        kq.gmean = p.Hq / p.Hkv;
+        kq.x_stride_g = p.q_stride_h;
+        kq.x_stride_h = p.q_stride_h * kq.gmean;
+        kq.heads_per_w = p.n_w > 1 ? 1 : 0;
+    }
     kq.out = p.q_codes; kq.out_stride_t = p.qc_stride_b; kq.out_stride_h = p.qc_stride_h;
     int rc = check_shape(kq, p.x_dtype, p.w_dtype);
     if (rc != UCM_OK) return rc;
@@ -1462,8 +1497,31 @@ bool pair_is_small(const PairSpec& p, const EncArgs& kk, const EncArgs& kq, bool
            small_eligible(kq, p.x_dtype, p.w_dtype);
 }
 
+// The queries alone through the small-row kernel (the only one that averages query groups).
+int launch_queries_small(const PairSpec& p, EncArgs& kq, hipStream_t st)
+{
+    set_block_shift(kq);
+    if (!mfma_eligible(kq, p.x_dtype, p.w_dtype) || small_waves(kq) > 0x7fffffff)
+        return ucm::fail(UCM_EUNSUPPORTED,
+                         "group-mean queries need bf16 / fp16 inputs of 64, 128, 256 or 512 dimensions, 16-byte aligned");
+    if (kq.T == 0) return UCM_OK;
+    EncJobs js{};
+    js.job[0] = kq;
+    js.job[1] = kq;
+    js.waves0 = (int)small_waves(kq);
+    return p.x_dtype == UCM_DT_BF16 ? launch_small<bf16x8>(js, js.waves0, p.K, st)
+                                    : launch_small<f16x8>(js, js.waves0, p.K, st);
+}
+
 int launch_pair(const PairSpec& p, EncArgs& kk, EncArgs& kq, bool has_keys, hipStream_t st)
 {
+    if (kq.gmean > 1 && !(has_keys && pair_is_small(p, kk, kq, has_keys))) {
+        if (has_keys) {
+            const int rc = encode_common(kk, p.x_dtype, p.w_dtype, st);
+            if (rc != UCM_OK) return rc;
+        }
+        return launch_queries_small(p, kq, st);
+    }
     if (!has_keys) return encode_common(kq, p.x_dtype, p.w_dtype, st);
     if (pair_is_small(p, kk, kq, has_keys)) {
         EncJobs js{};

@@ -168,3 +168,91 @@ class SparseDecodeStepMLA:
             self.q_codes.data_ptr(), self.out_idx.data_ptr(), self.out_score.data_ptr(),
             self.workspace.data_ptr(), self.workspace.numel(), _lib.stream_ptr(q_nope.device)))
         return self.out_idx, self.out_score
+
+
+class GSADecodeStep:
+    """The GQA plugin's per-layer decode work in one native call (ucm_gsa_decode_step): codes of
+    the step's new keys into the paged cache, hash of every KV head's mean query
+    (gsa_on_device.py:396-412), block scores with the best KV head counting and sink / recent
+    blocks kept (hamming_topk.py:15-54), and the replacement block table and sequence lengths
+    the attention backend reads (gsa_on_device.py:786-811).  Buffers are allocated once here;
+    `step` allocates nothing and can be captured in a HIP graph."""
+
+    def __init__(self, weights, num_q_heads, num_kv_heads, batch, table_width, topk_tokens,
+                 block_size=128, sink_token=None, recent_token=None, seq_len_threshold=0):
+        w = weights if weights.dim() == 3 else weights.unsqueeze(0)
+        if w.shape[0] not in (1, num_kv_heads):
+            raise ValueError("weights must be [K,N] or [Hkv,K,N]")
+        if w.dtype not in _DT or w.dtype == torch.float32:
+            raise ValueError("the fused step needs bfloat16 or float16 weights")
+        self.w = w.contiguous()
+        self.K, self.N = int(w.shape[1]), int(w.shape[2])
+        self.Hq, self.Hkv, self.B = int(num_q_heads), int(num_kv_heads), int(batch)
+        self.width, self.BS = int(table_width), int(block_size)
+        self.topk = int(topk_tokens)
+        self.sink = self.BS if sink_token is None else int(sink_token)
+        self.recent = 4 * self.BS if recent_token is None else int(recent_token)
+        self.threshold = int(seq_len_threshold)
+        assert self.topk % self.BS == 0
+        assert self.recent > 0 and self.topk > self.sink + self.recent
+        dev = w.device
+        self.q_codes = torch.empty((self.B, self.Hkv, self.N // 32), dtype=torch.int32, device=dev)
+        self.new_table = torch.empty((self.B, self.width), dtype=torch.int32, device=dev)
+        self.new_lens = torch.empty((self.B,), dtype=torch.int32, device=dev)
+        nbytes = _lib.lib().ucm_hamming_topk_workspace_bytes(self.B, self.Hkv, self.width)
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+    def _arguments(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
+        if queries.dtype != self.w.dtype or (new_keys is not None and new_keys.dtype != self.w.dtype):
+            raise ValueError("keys, queries and weights must share one dtype")
+        if tuple(queries.shape) != (self.B, self.Hq, self.K) or queries.stride(-1) != 1:
+            raise ValueError(f"queries must be {(self.B, self.Hq, self.K)} with contiguous rows")
+        if k_hash_cache.dtype != torch.int32 or k_hash_cache.dim() != 4 or k_hash_cache.stride(-1) != 1:
+            raise ValueError("k_hash_cache must be int32 [NB,BS,Hkv,W]")
+        NB, BS, Hkv, Wd = k_hash_cache.shape
+        if BS != self.BS or Hkv != self.Hkv or Wd != self.N // 32:
+            raise ValueError("k_hash_cache shape does not match this step's configuration")
+        if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
+            raise ValueError("block_table and seq_lens must be int32")
+        if tuple(block_table.shape) != (self.B, self.width) or block_table.stride(-1) != 1:
+            raise ValueError(f"block_table must be {(self.B, self.width)}")
+        if seq_lens.numel() != self.B or not seq_lens.is_contiguous():
+            raise ValueError("seq_lens must be a contiguous [B] tensor")
+        T = 0 if new_keys is None else int(new_keys.shape[0])
+        if T:
+            if tuple(new_keys.shape[1:]) != (self.Hkv, self.K) or new_keys.stride(-1) != 1:
+                raise ValueError(f"new_keys must be [T,{self.Hkv},{self.K}] with contiguous rows")
+            if slot_mapping.dtype not in (torch.int32, torch.int64) or slot_mapping.numel() != T \
+                    or not slot_mapping.is_contiguous():
+                raise ValueError("slot_mapping must be a contiguous int32/int64 [T] tensor")
+        s = _lib.stride
+        return (
+            new_keys.data_ptr() if T else None, T, s(new_keys, 0) if T else 0,
+            s(new_keys, 1) if T else 0, slot_mapping.data_ptr() if T else None,
+            int(T > 0 and slot_mapping.dtype == torch.int64),
+            queries.data_ptr(), s(queries, 0), s(queries, 1), _DT[self.w.dtype], self.K,
+            self.w.data_ptr(), _DT[self.w.dtype], self.w.shape[0], self.N,
+            k_hash_cache.data_ptr(), NB, BS, Hkv, s(k_hash_cache, 0), s(k_hash_cache, 1),
+            s(k_hash_cache, 2), block_table.data_ptr(), max(s(block_table, 0), self.width),
+            self.width, seq_lens.data_ptr(), self.B, self.Hq, self.topk, self.sink, self.recent,
+            self.threshold, self.q_codes.data_ptr(), self.new_table.data_ptr(), self.width,
+            self.new_lens.data_ptr(), self.workspace.data_ptr(), self.workspace.numel())
+
+    def step(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
+        """Returns (new_block_table [B, width], new_seq_lens [B]): buffers reused by every call."""
+        args = self._arguments(new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens)
+        _lib.check(_lib.lib().ucm_gsa_decode_step(*args, _lib.stream_ptr(queries.device)))
+        return self.new_table, self.new_lens
+
+    def bind(self, new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens):
+        """Validates once; the returned `run()` reissues the step with the same tensors."""
+        args = self._arguments(new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens)
+        keep = (new_keys, slot_mapping, queries, k_hash_cache, block_table, seq_lens)
+        fn, dev, stream_ptr, check = _lib.lib().ucm_gsa_decode_step, queries.device, _lib.stream_ptr, _lib.check
+        result = (self.new_table, self.new_lens)
+
+        def run(_keep=keep):
+            check(fn(*args, stream_ptr(dev)))
+            return result
+
+        return run

@@ -29,7 +29,8 @@ from typing import List, Optional, Union
 import torch
 
 from .base import UcmSparseBase, UcmSparseMetadata, UcmSparseRole
-from .hamming_topk import cuda_hamming_topk, update_seq_lens
+from .decode_step import GSADecodeStep
+from .hamming_topk import _as_words, cuda_hamming_topk, update_seq_lens
 from .hash_encoder import HashEncoder
 
 _DTYPES = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}
@@ -75,6 +76,9 @@ class GSAOnDevice(UcmSparseBase):
         else:
             self.hash_encoder = HashEncoder(self.head_dim, self.hash_bits, self.dtype, self.device)
         self._saved = {}
+        self._fused_steps = {}  # (requests, table width) -> GSADecodeStep
+        # one native call per layer at decode; False keeps the separate operators (same results)
+        self.fused_decode = bool(cfg.get("fused_decode", True))
         self.has_pc_hit = False
         self.prefix_block_ids = None      # int32 [sum of prefix blocks], all hit requests
         self.prefix_slot_mapping = None   # int64 [sum of prefix tokens]
@@ -240,9 +244,13 @@ class GSAOnDevice(UcmSparseBase):
             # kv_cache[0] is the key cache [NB, BS, Hkv, D] (gsa_on_device.py:576-579)
             attn = forward_context.no_compile_layers[layer_name]
             k_cache = attn.kv_cache[forward_context.virtual_engine][0]
-        self.cache_k_hash_gqa(key, attn_metadata, k_hash, k_cache)
         is_rollback_layer, _ = self.get_layer_state(layer_name)
-        if phase == "decode" and not is_rollback_layer:
+        decode = phase == "decode" and not is_rollback_layer
+        if decode and self._fused_decode_ok(attn_metadata):
+            self._fused_decode_step(query, key, attn_metadata, k_hash, k_cache, layer_name)
+            return query, key, value, output
+        self.cache_k_hash_gqa(key, attn_metadata, k_hash, k_cache)
+        if decode:
             num_reqs = attn_metadata.seq_lens.shape[0]
             q = query[:num_reqs].view(num_reqs, self.num_q_heads, self.head_dim)
             q_hash = self.hash_code(q)
@@ -262,6 +270,48 @@ class GSAOnDevice(UcmSparseBase):
             attn_metadata.block_table = new_table
             attn_metadata.seq_lens = new_lens
         return query, key, value, output
+
+    def _fused_decode_ok(self, attn_metadata):
+        """The single-call decode step takes 16-bit inputs with one projection, int32 metadata
+        and tables of at most 4096 blocks per request; anything else runs the separate operators."""
+        bt, sl = attn_metadata.block_table, attn_metadata.seq_lens
+        return (self.fused_decode and self.dtype in (torch.bfloat16, torch.float16)
+                and self.head_dim in (64, 128, 256, 512) and self.hash_bits % 32 == 0
+                and self.num_q_heads >= self.num_key_heads
+                and bt.dtype == torch.int32 and sl.dtype == torch.int32 and bt.shape[1] <= 4096
+                and bt.stride(-1) == 1 and sl.is_contiguous()
+                and self.hash_topk_tokens % self.block_size == 0
+                and self.recent_tokens > 0 and self.hash_topk_tokens > self.sink_tokens + self.recent_tokens)
+
+    def _fused_decode_step(self, query, key, attn_metadata, k_hash, k_cache, layer_name):
+        """cache_k_hash_gqa + hash_code + cuda_hamming_topk + the table / length swap of
+        update_decode_topk_gqa_cuda (gsa_on_device.py:564-572, 773-811) as one native call."""
+        bt, sl = attn_metadata.block_table, attn_metadata.seq_lens
+        num_reqs = sl.shape[0]
+        w = self.hash_encoder.hash_weights
+        key_ = (num_reqs, bt.shape[1], w.data_ptr())
+        step = self._fused_steps.get(key_)
+        if step is None:
+            step = GSADecodeStep(w, self.num_q_heads, self.num_key_heads, num_reqs,
+                                 bt.shape[1], self.hash_topk_tokens, block_size=self.block_size,
+                                 sink_token=self.sink_tokens, recent_token=self.recent_tokens,
+                                 seq_len_threshold=self.seq_len_threshold)
+            self._fused_steps[key_] = step
+        slots = attn_metadata.slot_mapping.flatten()
+        n = slots.numel()
+        keys = key[:n].view(n, self.num_key_heads, self.head_dim)
+        q = query[:num_reqs].view(num_reqs, self.num_q_heads, self.head_dim)
+        if self.has_pc_hit:  # prefix keys are re-encoded where they lie (gsa_on_device.py:574-588)
+            if k_cache is None:
+                raise ValueError("a prefix-cache hit needs the layer's key cache")
+            for first, n_blk, n_tok in self._prefix_segments:
+                self.hash_encoder.compute_hash_from_paged_cache(
+                    k_cache, self.prefix_block_ids[first:first + n_blk], n_tok, k_hash,
+                    block_size=self.block_size)
+        new_table, new_lens = step.step(keys, slots, q, _as_words(k_hash, "k_hash"), bt, sl)
+        self._saved[layer_name] = (bt, sl)
+        attn_metadata.block_table = new_table
+        attn_metadata.seq_lens = new_lens
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context,
                            phase: Optional[str] = None) -> None:
