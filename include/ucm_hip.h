@@ -239,6 +239,17 @@ int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_str
 int ucm_hamming_topk_set_profile_events(void* before, void* after);
 
 /*
+ * Test hook, no counterpart in the reference.  Writes the names of the kernels that the last
+ * ucm_hamming_topk / ucm_hamming_topk_static / ucm_sparse_decode_step* / ucm_gsa_decode_step /
+ * ucm_hamming_score call on the calling thread launched, e.g.
+ * "block_score_one<1,8,1,4,1>+select_wave_kernel<4>" or
+ * "plane_kernel+block_score_lanes<4,0,8>+select_group_kernel<4>" (family, then its template
+ * arguments), cut to cap - 1 characters.  Returns the full length.  Several kernel families give
+ * the same results at very different speeds; this lets a test pin which one a shape takes.
+ */
+int64_t ucm_hamming_last_dispatch(char* buf, size_t cap);
+
+/*
  * One decode step of the GQA retrieval path in a single call: store the hash codes of the
  * step's new keys in the paged code cache, hash the step's queries, then score and select.
  * Replaces the call sequence of GSAOnDevice.attention_begin at decode

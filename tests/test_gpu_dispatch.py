@@ -1,0 +1,99 @@
+"""GPU: which kernels a shape takes.  Several kernel families compute the same block scores at
+very different speeds, so a dispatch regression to a general kernel would pass every parity test
+and only show up as time.  Every family is reached here by a shape of its own, checked
+bit-exactly against the CPU checker, and the BASELINE.json shapes are pinned to the kernels
+that were tuned for them."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_paged_case
+from oracle import c_api
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if t.dtype == torch.uint32:
+        t = t.view(torch.int32)
+    return t.cuda()
+
+
+# (B, Hq, Hkv, Wd, BS, lens, k, kwargs, kernels launched)
+TOPK_SHAPES = {
+    "config1": (1, 32, 8, 4, 128, [8192], 16, {}, "block_score_one<1,8,1,4,1>+select_wave_kernel<4>"),
+    "config2_two_requests": (2, 32, 8, 4, 128, [32768, 32768], 64, {},
+                             "block_score_one<1,8,1,4,1>+select_wave_kernel<4>"),
+    "config3_one_long_request": (1, 32, 8, 4, 128, [70001], 128, {},
+                                 "block_score_one<1,8,1,4,1>+select_group_kernel<4>"),
+    "config5_two_requests": (2, 128, 1, 8, 64, [65536, 700], 128, {},
+                             "plane_kernel+block_score_lanes<4,0,8>+select_group_kernel<4>"),
+    "plugin_reduced_physical": (2, 8, 8, 4, 128, [4096, 3000], 8,
+                                {"reduce_heads": True, "return_physical": True},
+                                "block_score_one<1,8,1,1,1>+select_wave_kernel<4>"),
+    "blocks_of_32_KiB": (2, 32, 8, 4, 256, [4096, 3000], 4, {}, "block_score_one<1,8,1,4,0>+select_wave_kernel<4>"),
+    "eight_query_heads_per_kv_head": (2, 64, 8, 4, 128, [4096, 3000], 8, {},
+                                      "plane_kernel+block_score_one<1,8,0,4,1>+select_wave_kernel<4>"),
+    "blocks_of_64_tokens": (2, 32, 8, 4, 64, [4096, 3000], 8, {}, "block_score_rows<1,8,4,8>+select_wave_kernel<4>"),
+    "blocks_of_16_tokens": (2, 32, 8, 4, 16, [1024, 700], 8, {}, "block_score_rows<1,8,4,2>+select_wave_kernel<4>"),
+    "small_blocks_bit_planes": (2, 16, 2, 4, 32, [2048, 700], 8, {},
+                                "plane_kernel+block_score_small<1,2,0,4,1>+select_wave_kernel<4>"),
+    "odd_block_size_bit_planes": (2, 64, 8, 4, 48, [2048, 700], 8, {},
+                                  "plane_kernel+block_score_fast<1,0,4,4>+select_wave_kernel<4>"),
+    "blocks_below_1_KiB": (2, 1, 1, 4, 16, [2048, 700], 8, {}, "block_score_tiny<1,1>+select_wave_kernel<4>"),
+    "one_head_6_words": (2, 1, 1, 6, 32, [2048, 700], 8, {}, "block_score_pairs<1,1>+select_wave_kernel<4>"),
+    "one_head_6_words_16_query_heads": (2, 16, 1, 6, 32, [2048, 700], 8, {},
+                                        "plane_kernel+block_score_pairs<0,5>+select_wave_kernel<4>"),
+    "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], 8, {}, "block_score_lanes<9,1,1>+select_wave_kernel<4>"),
+    "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], 8, {},
+                                       "plane_kernel+block_score_lanes<9,0,7>+select_wave_kernel<4>"),
+    "odd_code_width": (2, 6, 2, 3, 16, [1024, 300], 8, {}, "block_score_generic+select_wave_kernel<4>"),
+    "more_than_4096_blocks": (1, 4, 1, 4, 16, [70000], 16, {}, "block_score_tiny<1,4>+select_kernel"),
+    "score_order": (2, 32, 8, 4, 128, [4096, 3000], 8, {"score_order": True},
+                    "block_score_one<1,8,1,4,1>+select_kernel"),
+}
+
+
+@pytest.mark.parametrize("name", list(TOPK_SHAPES))
+def test_topk_shape_takes_its_kernels_and_matches_the_checker(name):
+    from ucm_amd import _lib
+    from ucm_amd.sparse import hamming_topk
+
+    B, Hq, Hkv, Wd, BS, lens, k, kw, expect = TOPK_SHAPES[name]
+    q, kc, table, lens = make_paged_case(1234, B, Hq, Hkv, Wd, BS, lens)
+    idx, sc = hamming_topk(_dev(q), _dev(kc), _dev(table), _dev(lens), k, **kw)
+    assert _lib.last_dispatch() == expect
+    torch.cuda.synchronize()
+    flags = ((c_api.F_REDUCE_HEADS if kw.get("reduce_heads") else 0)
+             | (c_api.F_PHYSICAL if kw.get("return_physical") else 0)
+             | (c_api.F_SCORE_ORDER if kw.get("score_order") else 0))
+    oi, os_ = c_api.hamming_topk(q, kc, table, lens, k, 0, 0, flags)
+    assert np.array_equal(idx.cpu().numpy(), oi)
+    assert np.array_equal(sc.cpu().numpy(), os_)
+
+
+# (B, Hq, Hkv, Wd, BS, lens, kernels launched)
+SCORE_SHAPES = {
+    "config2_two_requests": (2, 32, 8, 4, 128, [32768, 30000], "token_score_fast<4>"),
+    "one_head_6_words": (2, 2, 1, 6, 32, [2048, 700], "token_score_pairs<1,2>"),
+    "one_head_6_words_16_query_heads": (2, 16, 1, 6, 32, [2048, 700], "plane_kernel+token_score_pairs<0,5>"),
+    "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], "token_score_lanes<9,1,1>"),
+    "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], "plane_kernel+token_score_lanes<9,0,7>"),
+    "odd_code_width": (2, 6, 2, 3, 16, [1024, 300], "token_score_kernel"),
+}
+
+
+@pytest.mark.parametrize("name", list(SCORE_SHAPES))
+def test_per_token_scorer_takes_its_kernels_and_matches_the_checker(name):
+    from ucm_amd import _lib
+    from ucm_amd.sparse import hamming_score
+
+    B, Hq, Hkv, Wd, BS, lens, expect = SCORE_SHAPES[name]
+    q, kc, table, lens = make_paged_case(4321, B, Hq, Hkv, Wd, BS, lens)
+    msl = int(max(lens))
+    out = hamming_score(_dev(kc), _dev(q), _dev(table), _dev(lens), msl, 0, 0, False, out_int32=True)
+    assert _lib.last_dispatch() == expect
+    torch.cuda.synchronize()
+    ref = c_api.hamming_score(q, kc, table, lens, msl)
+    assert np.array_equal(out.cpu().numpy(), ref)

@@ -1747,6 +1747,29 @@ Workspace carve(void* base, int B, int Hkv, int max_blocks)
 thread_local hipEvent_t g_prof_before = nullptr;
 thread_local hipEvent_t g_prof_after = nullptr;
 
+// Which kernels the last call on this thread launched (ucm_hamming_last_dispatch): a dispatch
+// regression to a general kernel gives the same results and would otherwise only show as time.
+struct DispatchNote {
+    const char* planes;   // "plane_kernel" when the bit planes were built
+    const char* score;    // scoring kernel family
+    int sp[5];            // its template arguments, -1 = unused
+    const char* select;   // selection kernel family
+    int sel_el;
+};
+thread_local DispatchNote g_note = {nullptr, nullptr, {-1, -1, -1, -1, -1}, nullptr, -1};
+
+void note_reset() { g_note = DispatchNote{nullptr, nullptr, {-1, -1, -1, -1, -1}, nullptr, -1}; }
+void note_score(const char* family, int a = -1, int b = -1, int c = -1, int d = -1, int e = -1)
+{
+    g_note.score = family;
+    g_note.sp[0] = a; g_note.sp[1] = b; g_note.sp[2] = c; g_note.sp[3] = d; g_note.sp[4] = e;
+}
+void note_select(const char* family, int el = -1)
+{
+    g_note.select = family;
+    g_note.sel_el = el;
+}
+
 template <typename K, typename... Args>
 void launch_score(K kernel, dim3 grid, size_t lds, hipStream_t st, Args... args)
 {
@@ -1760,6 +1783,7 @@ void launch_score(K kernel, dim3 grid, size_t lds, hipStream_t st, Args... args)
 template <int CPU, bool DIRECT, int GP>
 void launch_fast(const ScoreArgs& a, int split, int u, dim3 grid, hipStream_t st)
 {
+    note_score("block_score_fast", CPU, DIRECT, GP, u >= 4 ? 4 : (u >= 2 ? 2 : 1));
     if (u >= 4)
         launch_score(block_score_fast<CPU, DIRECT, GP, 4>, grid, 0, st, a, split);
     else if (u >= 2)
@@ -1782,6 +1806,8 @@ bool dispatch_fast(const ScoreArgs& a, int pmax, int split, int u, dim3 grid, hi
 template <int CPU, int HKV, bool EXACT>
 void dispatch_one_e(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
+    const bool dir = a.G == 1 || a.G == 2 || a.G == 4;
+    note_score("block_score_one", CPU, HKV, dir, dir ? a.G : (pmax == 4 ? 4 : 8), EXACT);
     if (a.G == 1) launch_score(block_score_one<CPU, HKV, true, 1, EXACT>, grid, 0, st, a);
     else if (a.G == 2) launch_score(block_score_one<CPU, HKV, true, 2, EXACT>, grid, 0, st, a);
     else if (a.G == 4) launch_score(block_score_one<CPU, HKV, true, 4, EXACT>, grid, 0, st, a);
@@ -1799,6 +1825,8 @@ void dispatch_one_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 template <int CPU, int HKV, int RPB>
 void dispatch_small_g(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
+    const bool dir = a.G == 1 || a.G == 2 || a.G == 4;
+    note_score("block_score_small", CPU, HKV, dir, dir ? a.G : (pmax == 4 ? 4 : 8), RPB);
     if (a.G == 1) launch_score(block_score_small<CPU, HKV, true, 1, RPB>, grid, 0, st, a);
     else if (a.G == 2) launch_score(block_score_small<CPU, HKV, true, 2, RPB>, grid, 0, st, a);
     else if (a.G == 4) launch_score(block_score_small<CPU, HKV, true, 4, RPB>, grid, 0, st, a);
@@ -1822,6 +1850,7 @@ bool dispatch_small(const ScoreArgs& a, int rpb, int pmax, dim3 grid, hipStream_
 template <int CPU, int HKV, int RPB>
 void dispatch_rows_g(const ScoreArgs& a, dim3 grid, hipStream_t st)
 {
+    note_score("block_score_rows", CPU, HKV, a.G, RPB);
     if (a.G == 1) launch_score(block_score_rows<CPU, HKV, 1, RPB>, grid, 0, st, a);
     else if (a.G == 2) launch_score(block_score_rows<CPU, HKV, 2, RPB>, grid, 0, st, a);
     else launch_score(block_score_rows<CPU, HKV, 4, RPB>, grid, 0, st, a);
@@ -1887,6 +1916,7 @@ bool tiny_layout(const ScoreArgs& a, const uint32_t* k_cache, bool direct)
 template <int CPU>
 void launch_tiny(const ScoreArgs& a, int bshift, dim3 grid, hipStream_t st)
 {
+    note_score("block_score_tiny", CPU, a.G == 1 || a.G == 2 ? a.G : 4);
     if (a.G == 1) launch_score(block_score_tiny<CPU, 1>, grid, 0, st, a, bshift);
     else if (a.G == 2) launch_score(block_score_tiny<CPU, 2>, grid, 0, st, a, bshift);
     else launch_score(block_score_tiny<CPU, 4>, grid, 0, st, a, bshift);
@@ -1905,6 +1935,8 @@ bool lanes_layout(const ScoreArgs& a, const uint32_t* k_cache, bool direct)
 template <int LC>
 void dispatch_lanes(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
+    const bool dir = LC == 9 && (a.G == 1 || a.G == 2 || a.G == 4);
+    note_score("block_score_lanes", LC, dir, dir ? a.G : (pmax < 4 ? 4 : (pmax > 8 ? 8 : pmax)));
     if (LC == 9 && a.G == 1) launch_score(block_score_lanes<9, true, 1>, grid, 0, st, a);
     else if (LC == 9 && a.G == 2) launch_score(block_score_lanes<9, true, 2>, grid, 0, st, a);
     else if (LC == 9 && a.G == 4) launch_score(block_score_lanes<9, true, 4>, grid, 0, st, a);
@@ -1964,6 +1996,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
                      int32_t* out_idx, int32_t* out_score, void* workspace, size_t workspace_bytes,
                      ucm_stream_t stream, const StepOut* step_out)
 {
+    note_reset();
     int rc = common_checks(q_codes, k_cache, seq_lens, NB, BS, Hkv, Wd, B, Hq, max_blocks);
     if (rc != UCM_OK) return rc;
     if (step_out) {
@@ -2030,6 +2063,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         const int pmax = planes_for_group(a.G);
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
         if (!direct) {
+            g_note.planes = "plane_kernel";
             hipLaunchKernelGGL(plane_kernel, dim3(B * Hkv * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
                                q_stride_b, q_stride_h, Hkv, a.G, Wd, pmax, ws.planes);
             rc = ucm::launch_status("plane_kernel");
@@ -2105,6 +2139,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         if (pmax < 4) pmax = 4;
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
         if (!direct) {
+            g_note.planes = "plane_kernel";
             hipLaunchKernelGGL(plane_kernel, dim3(B * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
                                q_stride_b, q_stride_h, 1, a.G, Wd, pmax, ws.planes);
             rc = ucm::launch_status("plane_kernel");
@@ -2118,6 +2153,8 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
             else if (Wd == 16) dispatch_lanes<8>(a, pmax, pgrid, st);
             else dispatch_lanes<4>(a, pmax, pgrid, st);
         } else
+        if (!lanes_layout(a, k_cache, direct))
+            note_score("block_score_pairs", direct, direct ? a.G : (pmax > 8 ? 8 : pmax));
         if (a.G == 1) launch_score(block_score_pairs<true, 1>, pgrid, 0, st, a, L, TP);
         else if (a.G == 2) launch_score(block_score_pairs<true, 2>, pgrid, 0, st, a, L, TP);
         else if (a.G == 4) launch_score(block_score_pairs<true, 4>, pgrid, 0, st, a, L, TP);
@@ -2127,6 +2164,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         else if (pmax == 7) launch_score(block_score_pairs<false, 7>, pgrid, 0, st, a, L, TP);
         else launch_score(block_score_pairs<false, 8>, pgrid, 0, st, a, L, TP);
     } else {
+        note_score("block_score_generic");
         launch_score(block_score_generic, grid, (size_t)Hq * Wd * 4, st, a);
     }
     rc = ucm::launch_status("block_score");
@@ -2150,11 +2188,13 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
     if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256) {
         // up to 256 blocks a wave per row stays ahead of a workgroup per row (config 2 step:
         // 32.7 against 33.3 us)
+        note_select("select_wave_kernel", 4);
         hipLaunchKernelGGL(select_wave_kernel<4>, wgrid, dim3(kThreads), 0, st, s, rows_total);
         return ucm::launch_status("select_wave_kernel");
     }
     if (!(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 4096) {
         const dim3 rgrid((unsigned)rows_total);
+        note_select("select_group_kernel", max_blocks <= 512 ? 2 : (max_blocks <= 1024 ? 4 : (max_blocks <= 2048 ? 8 : 16)));
         if (max_blocks <= 512)
             hipLaunchKernelGGL(select_group_kernel<2>, rgrid, dim3(kThreads), 0, st, s);
         else if (max_blocks <= 1024)
@@ -2165,6 +2205,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
             hipLaunchKernelGGL(select_group_kernel<16>, rgrid, dim3(kThreads), 0, st, s);
         return ucm::launch_status("select_group_kernel");
     }
+    note_select("select_kernel");
     hipLaunchKernelGGL(select_kernel, dim3(B * s.Ho), dim3(kThreads), 0, st, s);
     return ucm::launch_status("select_kernel");
 }
@@ -2348,6 +2389,28 @@ extern "C" int ucm_sparse_decode_step_mla(
                             ks_token, block_table, table_stride, max_blocks, seq_lens, B, Hq, k,
                             sink_tok, recent_tok, flags, out_idx, out_score, workspace,
                             workspace_bytes, stream);
+}
+
+extern "C" int64_t ucm_hamming_last_dispatch(char* buf, size_t cap)
+{
+    char tmp[256];
+    int n = 0;
+    if (g_note.planes) n += snprintf(tmp + n, sizeof(tmp) - n, "%s+", g_note.planes);
+    if (g_note.score) {
+        n += snprintf(tmp + n, sizeof(tmp) - n, "%s", g_note.score);
+        for (int i = 0; i < 5 && g_note.sp[i] >= 0; ++i)
+            n += snprintf(tmp + n, sizeof(tmp) - n, "%c%d", i == 0 ? '<' : ',', g_note.sp[i]);
+        if (g_note.sp[0] >= 0) n += snprintf(tmp + n, sizeof(tmp) - n, ">");
+    }
+    if (g_note.select) {
+        n += snprintf(tmp + n, sizeof(tmp) - n, "+%s", g_note.select);
+        if (g_note.sel_el >= 0) n += snprintf(tmp + n, sizeof(tmp) - n, "<%d>", g_note.sel_el);
+    }
+    tmp[n] = 0;
+    if (buf && cap) {
+        snprintf(buf, cap, "%s", tmp);
+    }
+    return n;
 }
 
 extern "C" int ucm_hamming_topk_set_profile_events(void* before, void* after)
@@ -2708,6 +2771,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
                                  void* workspace, size_t workspace_bytes, ucm_stream_t stream)
 {
     ucm::clear_error();
+    note_reset();
     int rc = common_checks(q_codes, k_cache, seq_lens, NB, BS, Hkv, Wd, B, Hq, max_blocks);
     if (rc != UCM_OK) return rc;
     UCM_REQUIRE(out, "out is null");
@@ -2741,6 +2805,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
         const dim3 fgrid((unsigned)ucm::ceil_div(ucm::ceil_div(max_seq_len, BS), 1 << tbs), (unsigned)B);
         const size_t lds = ((size_t)BS << tbs) * Hkv * 4;
         hipStream_t st = (hipStream_t)stream;
+        note_score("token_score_fast", G);
         if (G == 1) hipLaunchKernelGGL(token_score_fast<1>, fgrid, dim3(kThreads), lds, st, t, tbs);
         else if (G == 2) hipLaunchKernelGGL(token_score_fast<2>, fgrid, dim3(kThreads), lds, st, t, tbs);
         else if (G == 4) hipLaunchKernelGGL(token_score_fast<4>, fgrid, dim3(kThreads), lds, st, t, tbs);
@@ -2758,6 +2823,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
         // 18-word codes in blocks of 64, 128, ... tokens: a whole code per lane
         const bool lanes = lanes_layout(a, k_cache, G <= 4 && direct);
         if (lanes && G <= 4 && direct) {
+            note_score("token_score_lanes", 9, 1, G);
             if (G == 1) launch_token_lanes<9, true, 1>(t, pgrid, st);
             else if (G == 2) launch_token_lanes<9, true, 2>(t, pgrid, st);
             else launch_token_lanes<9, true, 4>(t, pgrid, st);
@@ -2765,6 +2831,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
         }
         // 8 query heads: bit planes when the caller brought the workspace for them
         if (direct && !(lanes && have_planes)) {
+            note_score("token_score_pairs", 1, G);
             if (G == 1) launch_token_pairs<true, 1>(t, L, TP, pgrid, st);
             else if (G == 2) launch_token_pairs<true, 2>(t, L, TP, pgrid, st);
             else if (G == 4) launch_token_pairs<true, 4>(t, L, TP, pgrid, st);
@@ -2772,16 +2839,19 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
         } else {
             const int pmax = exact_planes(G);
             a.planes = static_cast<uint32_t*>(workspace);
+            g_note.planes = "plane_kernel";
             hipLaunchKernelGGL(plane_kernel, dim3(B * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
                                q_stride_b, q_stride_h, 1, G, Wd, pmax, static_cast<uint32_t*>(workspace));
             rc = ucm::launch_status("plane_kernel");
             if (rc != UCM_OK) return rc;
             if (lanes) {
+                note_score("token_score_lanes", Wd / 2, 0, pmax > 8 ? 8 : pmax);
                 if (Wd == 18) dispatch_token_lanes_planes<9>(t, pmax, pgrid, st);
                 else if (Wd == 16) dispatch_token_lanes_planes<8>(t, pmax, pgrid, st);
                 else dispatch_token_lanes_planes<4>(t, pmax, pgrid, st);
                 return ucm::launch_status("token_score_lanes");
             }
+            note_score("token_score_pairs", 0, pmax > 8 ? 8 : pmax);
             switch (pmax) {
                 case 4: launch_token_pairs<false, 4>(t, L, TP, pgrid, st); break;
                 case 5: launch_token_pairs<false, 5>(t, L, TP, pgrid, st); break;
@@ -2793,6 +2863,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
         return ucm::launch_status("token_score_pairs");
     }
     const dim3 grid((unsigned)ucm::ceil_div(max_seq_len, kThreads), (unsigned)B);
+    note_score("token_score_kernel");
     hipLaunchKernelGGL(token_score_kernel, grid, dim3(kThreads), (size_t)Hq * Wd * 4,
                        (hipStream_t)stream, t);
     return ucm::launch_status("token_score_kernel");
