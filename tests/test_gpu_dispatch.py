@@ -28,7 +28,7 @@ TOPK_SHAPES = {
     "config3_one_long_request": (1, 32, 8, 4, 128, [70001], 128, {},
                                  "block_score_one<1,8,1,4,1>+select_group_kernel<4>"),
     "config5_two_requests": (2, 128, 1, 8, 64, [65536, 700], 128, {},
-                             "plane_kernel+block_score_lanes<4,0,8>+select_group_kernel<4>"),
+                             "plane_kernel+block_score_lanes64<4,0,8>+select_group_kernel<4>"),
     "plugin_reduced_physical": (2, 8, 8, 4, 128, [4096, 3000], 8,
                                 {"reduce_heads": True, "return_physical": True},
                                 "block_score_one<1,8,1,1,1>+select_wave_kernel<4>"),
@@ -48,6 +48,8 @@ TOPK_SHAPES = {
     "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], 8, {}, "block_score_lanes<9,1,1>+select_wave_kernel<4>"),
     "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], 8, {},
                                        "plane_kernel+block_score_lanes<9,0,7>+select_wave_kernel<4>"),
+    "config5_blocks_of_128": (2, 128, 1, 8, 128, [8192, 700], 8, {},
+                              "plane_kernel+block_score_lanes<4,0,8>+select_wave_kernel<4>"),
     "odd_code_width": (2, 6, 2, 3, 16, [1024, 300], 8, {}, "block_score_generic+select_wave_kernel<4>"),
     "more_than_4096_blocks": (1, 4, 1, 4, 16, [70000], 16, {}, "block_score_tiny<1,4>+select_kernel"),
     "score_order": (2, 32, 8, 4, 128, [4096, 3000], 8, {"score_order": True},

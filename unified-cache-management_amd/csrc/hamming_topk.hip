@@ -1054,6 +1054,109 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     }
 }
 
+// The same walk for 64-token blocks (one round per block), several blocks per wave: with one
+// block per wave a wave's whole life is three dependent round trips to memory (table entry,
+// codes, and the bit planes behind a barrier) around some 250 instructions, and the counters show
+// it (16 x 65,536 tokens of 256-bit codes, 128 query heads: vector ALU busy 11 % of a wave's
+// resident cycles, 82 % spent waiting).  Here a wave owns kLaneRun consecutive logical blocks:
+// their table entries arrive in one load, the codes of all of them are requested together (the
+// whole problem is a few tens of MB: everything should be in flight at once), the planes are
+// staged once per 4 * kLaneRun blocks, and the run's scores leave in one store.
+constexpr int kLaneRun = 4;
+
+template <int LC, bool DIRECT, int GP>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void block_score_lanes64(ScoreArgs a)
+{
+    using LCd = LaneCode<LC, DIRECT, GP>;
+    constexpr int WD = LCd::WD;
+    __shared__ __align__(16) uint32_t strip[kThreads / kWave][LCd::kRoundWords];
+    __shared__ __align__(16) uint32_t pl[DIRECT ? 8 : WD * 8];
+    __shared__ int ctot[LC];
+    const int b = blockIdx.y;
+    const int lane = lane_id(), wid = wave_id();
+    const int j0 = (blockIdx.x * (kThreads / kWave) + wid) * kLaneRun;
+    const int len = a.lens[b];
+    // the run's table entries: lane i holds block j0 + i
+    int my_entry = 0;
+    {
+        const int j = j0 + (lane < kLaneRun ? lane : 0);
+        const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+        if (a.table) my_entry = a.table[(int64_t)b * a.table_stride + (jc < 0 ? 0 : jc)];
+        else my_entry = b * a.max_blocks + jc;
+    }
+    LCd::stage_planes(a, b, pl, ctot);
+    if (!DIRECT) __syncthreads();
+    int nblk = len > 0 ? (len + 63) >> 6 : 0;
+    if (nblk > a.max_blocks) nblk = a.max_blocks;
+    if (j0 >= nblk) return;
+    const int run = (nblk - j0 < kLaneRun) ? nblk - j0 : kLaneRun;
+    u32x4* mine = reinterpret_cast<u32x4*>(strip[wid]);
+    const uint32_t* row = strip[wid] + lane * WD;
+    const uint32_t* qp = a.q + b * a.q_stride_b;
+    int base = 0;
+    if (!DIRECT) {
+#pragma unroll
+        for (int i = 0; i < LC; ++i) base += ctot[i];
+    }
+    auto block_src = [&](int i) -> const u32x4* {
+        int64_t pb = __shfl(my_entry, i);
+        if (pb < 0 || pb >= a.NB) pb = 0;  // scored as -1 below
+        return reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block);
+    };
+    // the codes of the whole run are requested at once (blocks past the run re-read its first)
+    u32x4 v[kLaneRun][LCd::kLoads];
+#pragma unroll
+    for (int i = 0; i < kLaneRun; ++i) LCd::load_round(block_src(i < run ? i : 0), 0, lane, v[i]);
+    int result = 0;  // lane i: score of block j0 + i
+    const int full = a.G * 32 * a.Wd;
+#pragma unroll
+    for (int i = 0; i < kLaneRun; ++i) {
+        if (i >= run) break;
+        LCd::store_round(mine, lane, v[i]);
+        asm volatile("" ::: "memory");  // the planes are re-read from LDS for every block
+        int d = 0;
+        if (DIRECT) {
+#pragma unroll
+            for (int w = 0; w < LC; ++w) {
+                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * w);
+#pragma unroll
+                for (int g = 0; g < GP; ++g)
+                    d += __popc(k.x ^ qp[g * a.q_stride_h + 2 * w]) + __popc(k.y ^ qp[g * a.q_stride_h + 2 * w + 1]);
+            }
+        } else {
+            int acc[GP], pk = 0;
+#pragma unroll
+            for (int p = 0; p < GP; ++p) acc[p] = 0;
+#pragma unroll
+            for (int w = 0; w < LC; ++w) {
+                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * w);
+                pk += __popc(k.x) + __popc(k.y);
+#pragma unroll
+                for (int p = 0; p < GP; ++p)
+                    acc[p] += __popc(k.x & pl[(2 * w) * 8 + p]) + __popc(k.y & pl[(2 * w + 1) * 8 + p]);
+            }
+            int x = 0;
+#pragma unroll
+            for (int p = 0; p < GP; ++p) x += acc[p] << p;
+            d = base + a.G * pk - 2 * x;
+        }
+        asm volatile("" ::: "memory");  // the strip is rewritten by the next block
+        const int pos0 = (j0 + i) << 6;
+        const int ntok = (64 < len - pos0) ? 64 : len - pos0;
+        int m = lane < ntok ? d : kInf;
+#pragma unroll
+        for (int st = 1; st < kWave; st <<= 1) {
+            const int o = __shfl_xor(m, st);
+            m = o < m ? o : m;
+        }
+        const int entry = __shfl(my_entry, i);
+        const bool forced = (pos0 < a.sink) || (pos0 + ntok > len - a.recent);
+        const int sc = (entry < 0 || entry >= a.NB) ? -1 : (forced ? full : full - m);
+        if (lane == i) result = sc;
+    }
+    if (lane < run) a.scores[(int64_t)b * a.max_blocks + j0 + lane] = result;
+}
+
 // ---------------------------------------------------------------------------------------
 // Generic block scorer: any strides, code width, head count and group size.  One thread per
 // (token, head) code, word-by-word loads; query codes staged in LDS.
@@ -1755,10 +1858,11 @@ struct DispatchNote {
     int sp[5];            // its template arguments, -1 = unused
     const char* select;   // selection kernel family
     int sel_el;
+    int score_launches;   // scoring kernels launched (one, unless the dispatch is broken)
 };
-thread_local DispatchNote g_note = {nullptr, nullptr, {-1, -1, -1, -1, -1}, nullptr, -1};
+thread_local DispatchNote g_note = {nullptr, nullptr, {-1, -1, -1, -1, -1}, nullptr, -1, 0};
 
-void note_reset() { g_note = DispatchNote{nullptr, nullptr, {-1, -1, -1, -1, -1}, nullptr, -1}; }
+void note_reset() { g_note = DispatchNote{nullptr, nullptr, {-1, -1, -1, -1, -1}, nullptr, -1, 0}; }
 void note_score(const char* family, int a = -1, int b = -1, int c = -1, int d = -1, int e = -1)
 {
     g_note.score = family;
@@ -1773,6 +1877,7 @@ void note_select(const char* family, int el = -1)
 template <typename K, typename... Args>
 void launch_score(K kernel, dim3 grid, size_t lds, hipStream_t st, Args... args)
 {
+    ++g_note.score_launches;
     if (g_prof_before && g_prof_after)
         hipExtLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, st, g_prof_before, g_prof_after, 0,
                               args...);
@@ -1936,6 +2041,21 @@ template <int LC>
 void dispatch_lanes(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
     const bool dir = LC == 9 && (a.G == 1 || a.G == 2 || a.G == 4);
+    // 64-token blocks of 8-word codes: runs of kLaneRun blocks per wave (wider codes hold too
+    // many registers for the run's loads: 18 words measured 21.9 against 18.4 us)
+    if (a.BS == 64 && LC == 4) {
+        note_score("block_score_lanes64", LC, dir, dir ? a.G : (pmax < 4 ? 4 : (pmax > 8 ? 8 : pmax)));
+        const dim3 g64((unsigned)ucm::ceil_div(a.max_blocks, (kThreads / kWave) * kLaneRun), grid.y);
+        if (LC == 9 && a.G == 1) launch_score(block_score_lanes64<9, true, 1>, g64, 0, st, a);
+        else if (LC == 9 && a.G == 2) launch_score(block_score_lanes64<9, true, 2>, g64, 0, st, a);
+        else if (LC == 9 && a.G == 4) launch_score(block_score_lanes64<9, true, 4>, g64, 0, st, a);
+        else if (pmax == 4) launch_score(block_score_lanes64<LC, false, 4>, g64, 0, st, a);
+        else if (pmax == 5) launch_score(block_score_lanes64<LC, false, 5>, g64, 0, st, a);
+        else if (pmax == 6) launch_score(block_score_lanes64<LC, false, 6>, g64, 0, st, a);
+        else if (pmax == 7) launch_score(block_score_lanes64<LC, false, 7>, g64, 0, st, a);
+        else launch_score(block_score_lanes64<LC, false, 8>, g64, 0, st, a);
+        return;
+    }
     note_score("block_score_lanes", LC, dir, dir ? a.G : (pmax < 4 ? 4 : (pmax > 8 ? 8 : pmax)));
     if (LC == 9 && a.G == 1) launch_score(block_score_lanes<9, true, 1>, grid, 0, st, a);
     else if (LC == 9 && a.G == 2) launch_score(block_score_lanes<9, true, 2>, grid, 0, st, a);
@@ -2152,17 +2272,17 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
             if (Wd == 18) dispatch_lanes<9>(a, pmax, pgrid, st);
             else if (Wd == 16) dispatch_lanes<8>(a, pmax, pgrid, st);
             else dispatch_lanes<4>(a, pmax, pgrid, st);
-        } else
-        if (!lanes_layout(a, k_cache, direct))
+        } else {
             note_score("block_score_pairs", direct, direct ? a.G : (pmax > 8 ? 8 : pmax));
-        if (a.G == 1) launch_score(block_score_pairs<true, 1>, pgrid, 0, st, a, L, TP);
-        else if (a.G == 2) launch_score(block_score_pairs<true, 2>, pgrid, 0, st, a, L, TP);
-        else if (a.G == 4) launch_score(block_score_pairs<true, 4>, pgrid, 0, st, a, L, TP);
-        else if (pmax == 4) launch_score(block_score_pairs<false, 4>, pgrid, 0, st, a, L, TP);
-        else if (pmax == 5) launch_score(block_score_pairs<false, 5>, pgrid, 0, st, a, L, TP);
-        else if (pmax == 6) launch_score(block_score_pairs<false, 6>, pgrid, 0, st, a, L, TP);
-        else if (pmax == 7) launch_score(block_score_pairs<false, 7>, pgrid, 0, st, a, L, TP);
-        else launch_score(block_score_pairs<false, 8>, pgrid, 0, st, a, L, TP);
+            if (a.G == 1) launch_score(block_score_pairs<true, 1>, pgrid, 0, st, a, L, TP);
+            else if (a.G == 2) launch_score(block_score_pairs<true, 2>, pgrid, 0, st, a, L, TP);
+            else if (a.G == 4) launch_score(block_score_pairs<true, 4>, pgrid, 0, st, a, L, TP);
+            else if (pmax == 4) launch_score(block_score_pairs<false, 4>, pgrid, 0, st, a, L, TP);
+            else if (pmax == 5) launch_score(block_score_pairs<false, 5>, pgrid, 0, st, a, L, TP);
+            else if (pmax == 6) launch_score(block_score_pairs<false, 6>, pgrid, 0, st, a, L, TP);
+            else if (pmax == 7) launch_score(block_score_pairs<false, 7>, pgrid, 0, st, a, L, TP);
+            else launch_score(block_score_pairs<false, 8>, pgrid, 0, st, a, L, TP);
+        }
     } else {
         note_score("block_score_generic");
         launch_score(block_score_generic, grid, (size_t)Hq * Wd * 4, st, a);
@@ -2406,6 +2526,7 @@ extern "C" int64_t ucm_hamming_last_dispatch(char* buf, size_t cap)
         n += snprintf(tmp + n, sizeof(tmp) - n, "+%s", g_note.select);
         if (g_note.sel_el >= 0) n += snprintf(tmp + n, sizeof(tmp) - n, "<%d>", g_note.sel_el);
     }
+    if (g_note.score_launches > 1) n += snprintf(tmp + n, sizeof(tmp) - n, " (%d scoring launches)", g_note.score_launches);
     tmp[n] = 0;
     if (buf && cap) {
         snprintf(buf, cap, "%s", tmp);
