@@ -359,6 +359,90 @@ def plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots):
     return out
 
 
+def gather_beside_decode(torch, gen, run_step, steps_per_call):
+    """The decode step while a 1 GiB KV dump to pinned host memory runs on a side stream
+    (north_star: the gather runs beside decode), and the dump's rate while the step loops:
+    64 blocks x 32 layers x {K,V} x 256 KiB, once through the kernel copy of an SM stream
+    (table-free paged form) and once as 4096 copy-engine transfers of a CE stream."""
+    import numpy as np
+    from ucm_amd.trans import Device
+
+    L, NBP, n_sel = 32, 128, 64
+    chunk = BS * HKV * D * 2
+    kv = [torch.empty((2, NBP, BS, HKV, D), dtype=torch.bfloat16, device="cuda").normal_(generator=gen)
+          for _ in range(L)]
+    base = np.array([[t[0].data_ptr(), t[1].data_ptr()] for t in kv], np.uint64).reshape(-1)
+    sizes = np.full(base.shape, chunk, np.uint64)
+    ids = np.random.Generator(np.random.PCG64(2004)).choice(NBP, n_sel, replace=False).astype(np.int32)
+    payload = len(ids) * L * 2 * chunk
+    host = torch.empty(payload, dtype=torch.uint8).pin_memory()
+    addrs = (ids.astype(np.uint64)[:, None] * sizes[None, :] + base[None, :]).reshape(-1)
+    d = Device()
+    d.Setup(0)
+    out = {"payload_GiB": payload / 2**30}
+
+    def steps_alone(n):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+        for i in range(n):
+            ev[i].record()
+            run_step(i)
+        ev[n].record()
+        torch.cuda.synchronize()
+        return sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 / steps_per_call for i in range(n))
+
+    for i in range(10):
+        run_step(i)
+    alone = steps_alone(200)
+    out["step_alone_us"] = {"p50": alone[100], "p90": alone[180]}
+    for kind, make in (("sm_stream_kernel", d.MakeSMStream), ("ce_stream_copy_engine", d.MakeStream)):
+        st = make()
+        side = torch.cuda.ExternalStream(st.handle)
+        if kind == "sm_stream_kernel":
+            dump = lambda: st.PagedGatherAsync(base, sizes, ids, host.data_ptr())  # noqa: E731
+        else:
+            dump = lambda: st.DeviceToHostGatherAsync(addrs, host.data_ptr(), chunk, len(addrs))  # noqa: E731
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        dump()
+        st.Synchronized()
+        e0.record(side)
+        dump()
+        e1.record(side)
+        st.Synchronized()
+        alone_ms = e0.elapsed_time(e1)
+        # the dump in flight, the step looping on the compute stream until the dump has ended
+        torch.cuda.synchronize()
+        gaps = []
+        e0.record(side)
+        dump()
+        e1.record(side)
+        i = 0
+        prev = torch.cuda.Event(enable_timing=True)
+        prev.record()
+        evs = [prev]
+        while not e1.query() and i < 20000:
+            run_step(i)
+            e = torch.cuda.Event(enable_timing=True)
+            e.record()
+            evs.append(e)
+            i += 1
+            if i % 64 == 0:
+                evs[-1].synchronize()  # keep the host a bounded distance ahead of the GPU
+        torch.cuda.synchronize()
+        st.Synchronized()
+        busy_ms = e0.elapsed_time(e1)
+        gaps = sorted(evs[j].elapsed_time(evs[j + 1]) * 1e3 / steps_per_call for j in range(len(evs) - 1))
+        res = {"dump_alone_GBps": payload / alone_ms / 1e6, "dump_beside_steps_GBps": payload / busy_ms / 1e6,
+               "steps_during_dump": len(gaps) * steps_per_call}
+        if gaps:
+            res["step_beside_dump_us"] = {"p50": gaps[len(gaps) // 2], "p90": gaps[int(len(gaps) * 0.9)],
+                                          "max": gaps[-1]}
+            res["steps_ms_total"] = evs[0].elapsed_time(evs[-1])
+            res["dump_ms"] = busy_ms
+        out[kind] = res
+        del st
+    return out
+
+
 def extras(torch, enc_k, gen):
     """Side figures: encoder at cache-build shape, device gather, pinned-host dump."""
     import numpy as np
@@ -543,12 +627,30 @@ def extras(torch, enc_k, gen):
     ms = timed(lambda: st.PagedScatterAsync(dev_flat.data_ptr(), base, sizes, ids), 5)
     out["scatter_device"] = {"ms": ms, "hbm_GBps": 2 * payload / ms / 1e6}
     ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids, host.data_ptr()), 2)
-    out["gather_to_pinned_host_kernel"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
+    out["gather_to_pinned_host"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6,
+                                    "form": "per 64 MiB piece: compaction kernel into device staging, one copy-engine transfer"}
     ms = timed(lambda: st.DeviceToHostAsync(dev_flat.data_ptr(), host.data_ptr(), payload), 2)
     out["d2h_copy_engine_flat"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
     ms = timed(lambda: st.PagedScatterAsync(host.data_ptr(), base, sizes, ids), 2)
-    out["scatter_from_pinned_host_kernel"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
+    out["scatter_from_pinned_host"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
     del host, dev_flat
+
+    # --- config 4 at its full size, device side: 32 requests x 64 blocks x 32 layers x {K,V} x 256 KiB
+    #     = 32 GiB gathered from the 4 GiB cache into one device buffer by one launch, and scattered back ---
+    ids_full = np.concatenate([np.random.Generator(np.random.PCG64(1004 + r)).choice(NBP, n_sel, replace=False)
+                               for r in range(32)]).astype(np.int32)
+    full_payload = len(ids_full) * L * 2 * chunk
+    try:
+        dev_full = torch.empty(full_payload, dtype=torch.uint8, device="cuda")
+        ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids_full, dev_full.data_ptr()), 3)
+        ms_s = timed(lambda: st.PagedScatterAsync(dev_full.data_ptr(), base, sizes, ids_full), 3)
+        out["gather_device_full_config4"] = {"payload_GiB": full_payload / 2**30, "gather_ms": ms, "scatter_ms": ms_s,
+                                             "gather_hbm_GBps": 2 * full_payload / ms / 1e6,
+                                             "gather_hbm_frac": 2 * full_payload / ms / 1e6 / HBM_PEAK_GBPS,
+                                             "scatter_hbm_GBps": 2 * full_payload / ms_s / 1e6}
+        del dev_full
+    except Exception as e:  # noqa: BLE001 - a side figure
+        out["gather_device_full_config4"] = {"error": str(e)[:200]}
 
     # --- the same blocks through the native cache store (task queues + pinned staging nodes):
     #     submit -> wait, one request (64 blocks = 1 GiB) per task, as the connector's
@@ -798,10 +900,12 @@ def main():
             "single_call_eager": plug["single_call"]["eager_p50_us"],
             "separate_operators_graph": plug["separate_operators"].get("graph_p50_us"),
             "separate_operators_eager": plug["separate_operators"]["eager_p50_us"]}
+        beside = gather_beside_decode(torch, gen, run_launch, GS)
         del caches[1:], tables[1:]
         torch.cuda.empty_cache()
         line["extras"] = extras(torch, enc_k, gen)
         line["extras"]["plugin_surface"] = plug
+        line["extras"]["gather_beside_decode"] = beside
         if not args.skip_cpu:
             line["extras"].update(cpu_side_baselines(torch))
     print(json.dumps(line))

@@ -36,6 +36,16 @@ extern "C" int ucm_trans_stream_create(int, ucm_trans_stream_t** out) { *out = n
 extern "C" int ucm_trans_stream_destroy(ucm_trans_stream_t* s) { delete s; return UCM_OK; }
 extern "C" int ucm_trans_stream_sync(ucm_trans_stream_t*) { return UCM_OK; }
 extern "C" int ucm_trans_stream_wait_event(ucm_trans_stream_t*, void*) { return UCM_OK; }
+extern "C" int ucm_trans_gather(ucm_trans_stream_t*, const void* const* src, int, void* dst, size_t size, size_t number, int)
+{
+    for (size_t i = 0; i < number; ++i) std::memcpy((char*)dst + i * size, src[i], size);
+    return UCM_OK;
+}
+extern "C" int ucm_trans_scatter(ucm_trans_stream_t*, const void* src, void* const* dst, int, size_t size, size_t number, int)
+{
+    for (size_t i = 0; i < number; ++i) std::memcpy(dst[i], (const char*)src + i * size, size);
+    return UCM_OK;
+}
 extern "C" int ucm_trans_batch(ucm_trans_stream_t*, const void* const* src, void* const* dst, int, size_t size,
                                size_t number, int)
 {

@@ -224,8 +224,8 @@ struct ucm_cache_store {
 
 namespace {
 
-// One kernel launch per distinct tensor size: (shard, tensor) chunk i moves between
-// dev[i] and host[i].  to_device = false: device -> host.
+// (shard, tensor) chunk i moves between dev[i] and host[i]; to_device = false: device -> host.
+// Mixed tensor sizes: one kernel launch per distinct size over a pointer table.
 int move_chunks(ucm_cache_store* st, ucm_trans_stream_t* stream, const std::vector<size_t>& pos,
                 const std::vector<const Shard*>& shards, bool to_device)
 {
@@ -233,6 +233,20 @@ int move_chunks(ucm_cache_store* st, ucm_trans_stream_t* stream, const std::vect
     std::vector<size_t> sizes(st->tensor_sizes);
     std::sort(sizes.begin(), sizes.end());
     sizes.erase(std::unique(sizes.begin(), sizes.end()), sizes.end());
+    if (sizes.size() == 1) {
+        // equal tensors (the usual KV layout): a shard's node is the flat side of a gather /
+        // scatter, which the copy stream stages through device memory and moves over PCIe with
+        // the copy engine, so that kernels of other streams keep running beside the transfer
+        for (size_t s = 0; s < shards.size(); ++s) {
+            void* node = st->buffer.data(pos[s]);
+            const int rc = to_device
+                               ? ucm_trans_scatter(stream, node, shards[s]->addrs.data(), 0, sizes[0], nt, 0)
+                               : ucm_trans_gather(stream, (const void* const*)shards[s]->addrs.data(), 0, node,
+                                                  sizes[0], nt, 0);
+            if (rc != UCM_OK) return rc;
+        }
+        return UCM_OK;
+    }
     std::vector<const void*> src;
     std::vector<void*> dst;
     for (size_t size : sizes) {

@@ -9,7 +9,17 @@
 //       store per lane and no loop, instead of the reference's fixed 32x256 grid-stride threads.
 //       Many short workgroups let the dispatcher interleave reads and writes across all HBM
 //       channels; on this part that moves 25-30 % more bytes per second than a persistent
-//       grid-stride copy.
+//       grid-stride copy.  A copy with a HOST end is the exception.  Kernel stores into pinned
+//       host memory fill the PCIe link (55 GB/s) but hold up every other kernel on the GPU while
+//       they run: a decode step of 32 us beside such a dump takes 47 us with 8 copy workgroups
+//       (28 GB/s), 72 us with 16 (44 GB/s) and stalls for milliseconds from 32 workgroups on —
+//       bounding the grid, as the reference does (cuda_sm_kernel.cu:29-32), does not help here.
+//       So gather / scatter / paged copies whose flat side is host memory go in two stages per
+//       piece of up to kStageBytes: the kernel compacts between the paged cache and a device
+//       staging buffer at HBM speed, and one copy-engine transfer moves the piece over PCIe
+//       (41-55 GB/s with the decode step running beside it at 33-37 us, no stalls).  Batch copies
+//       (two pointer tables) with a host end keep the direct kernel on kHostCopyGroups
+//       workgroups.
 #include "common.h"
 
 #include <cstring>
@@ -22,6 +32,8 @@ namespace {
 constexpr int kThreads = 256;
 constexpr size_t kSeg = (size_t)kThreads * 16;  // 4 KiB per workgroup
 constexpr int kSlots = 4;
+constexpr size_t kHostCopyGroups = 16;          // workgroups of a batch copy with a host end
+constexpr size_t kStageBytes = (size_t)64 << 20;  // device staging of host-ended copies, per stream
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -53,14 +65,16 @@ __global__ __launch_bounds__(kThreads) void table_copy_kernel(const uint64_t* __
                                                               uint8_t* dst_flat, size_t size,
                                                               size_t number, size_t segs_per_chunk)
 {
-    const size_t seg = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
-    if (seg >= number * segs_per_chunk) return;
-    const size_t i = seg / segs_per_chunk;
-    const size_t off = (seg - i * segs_per_chunk) * kSeg;
-    const size_t bytes = (size - off < kSeg) ? size - off : kSeg;
-    const uint8_t* s = (MODE == 1) ? src_flat + i * size : (const uint8_t*)src_tab[i];
-    uint8_t* d = (MODE == 0) ? dst_flat + i * size : (uint8_t*)dst_tab[i];
-    wg_copy(s + off, d + off, bytes);
+    // one segment per workgroup, or a bounded grid striding over the segments
+    const size_t groups = (size_t)gridDim.y * gridDim.x;
+    for (size_t seg = (size_t)blockIdx.y * gridDim.x + blockIdx.x; seg < number * segs_per_chunk; seg += groups) {
+        const size_t i = seg / segs_per_chunk;
+        const size_t off = (seg - i * segs_per_chunk) * kSeg;
+        const size_t bytes = (size - off < kSeg) ? size - off : kSeg;
+        const uint8_t* s = (MODE == 1) ? src_flat + i * size : (const uint8_t*)src_tab[i];
+        uint8_t* d = (MODE == 0) ? dst_flat + i * size : (uint8_t*)dst_tab[i];
+        wg_copy(s + off, d + off, bytes);
+    }
 }
 
 // Table-free paged copy.  meta: [n_cols] base, [n_cols] col_bytes, [n_cols] col offset in a
@@ -68,25 +82,27 @@ __global__ __launch_bounds__(kThreads) void table_copy_kernel(const uint64_t* __
 __global__ __launch_bounds__(kThreads) void paged_copy_kernel(const uint64_t* __restrict__ meta,
                                                               int n_cols, size_t segs_per_row,
                                                               size_t row_bytes, size_t n_blocks,
-                                                              uint8_t* flat, int to_cache)
+                                                              uint8_t* flat, int to_cache,
+                                                              size_t first_block)
 {
-    const size_t seg = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
-    if (seg >= n_blocks * segs_per_row) return;
     const uint64_t* base = meta;
     const uint64_t* cbytes = meta + n_cols;
     const uint64_t* coff = meta + 2 * n_cols;
     const uint64_t* segmap = meta + 3 * n_cols;
     const int32_t* ids = reinterpret_cast<const int32_t*>(segmap + segs_per_row);
-    const size_t i = seg / segs_per_row;
-    const uint64_t e = segmap[seg - i * segs_per_row];
-    const int c = (int)(e >> 40);
-    const size_t off = (size_t)(e & ((1ull << 40) - 1));
-    const size_t csz = cbytes[c];
-    const size_t bytes = (csz - off < kSeg) ? csz - off : kSeg;
-    uint8_t* cache_p = (uint8_t*)(base[c] + (uint64_t)ids[i] * csz) + off;
-    uint8_t* flat_p = flat + i * row_bytes + coff[c] + off;
-    if (to_cache) wg_copy(flat_p, cache_p, bytes);
-    else wg_copy(cache_p, flat_p, bytes);
+    const size_t groups = (size_t)gridDim.y * gridDim.x;
+    for (size_t seg = (size_t)blockIdx.y * gridDim.x + blockIdx.x; seg < n_blocks * segs_per_row; seg += groups) {
+        const size_t i = seg / segs_per_row;
+        const uint64_t e = segmap[seg - i * segs_per_row];
+        const int c = (int)(e >> 40);
+        const size_t off = (size_t)(e & ((1ull << 40) - 1));
+        const size_t csz = cbytes[c];
+        const size_t bytes = (csz - off < kSeg) ? csz - off : kSeg;
+        uint8_t* cache_p = (uint8_t*)(base[c] + (uint64_t)ids[first_block + i] * csz) + off;
+        uint8_t* flat_p = flat + i * row_bytes + coff[c] + off;
+        if (to_cache) wg_copy(flat_p, cache_p, bytes);
+        else wg_copy(cache_p, flat_p, bytes);
+    }
 }
 
 struct Slot {
@@ -106,6 +122,8 @@ struct ucm_trans_stream {
     Slot slots[kSlots];
     int next = 0;
     int num_cus = 256;
+    void* stage = nullptr;  // device staging buffer of host-ended copies
+    size_t stage_cap = 0;
     std::mutex mu;
 };
 
@@ -143,12 +161,44 @@ int release_slot(ucm_trans_stream* s, Slot* sl)
     return UCM_OK;
 }
 
-// One workgroup per segment, folded over x and y (x <= 2^20) so that any count fits a grid.
-dim3 grid_for(size_t total_segs)
+// True when p lies in host memory the device can address (pinned or registered).
+bool is_host_memory(const void* p)
 {
+    if (!p) return false;
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return attr.type == hipMemoryTypeHost;
+}
+
+// One workgroup per segment, folded over x and y (x <= 2^20) so that any count fits a grid;
+// at most kHostCopyGroups workgroups when an end of the copy is host memory.
+dim3 grid_for(size_t total_segs, bool host_end = false)
+{
+    if (host_end && total_segs > kHostCopyGroups) total_segs = kHostCopyGroups;
     const size_t gx = total_segs < (1u << 20) ? (total_segs ? total_segs : 1) : (1u << 20);
     const size_t gy = (total_segs + gx - 1) / gx;
     return dim3((unsigned)gx, (unsigned)(gy ? gy : 1));
+}
+
+// Staging buffer with room for `want` bytes (at most kStageBytes are asked for); grows by
+// replacing the buffer once the stream has drained.
+int ensure_stage(ucm_trans_stream* s, size_t want)
+{
+    if (s->stage_cap >= want) return UCM_OK;
+    if (s->stage) {
+        UCM_HIP_TRY(hipStreamSynchronize(s->stream));
+        (void)hipFree(s->stage);
+        s->stage = nullptr;
+        s->stage_cap = 0;
+    }
+    size_t cap = (size_t)1 << 20;
+    while (cap < want) cap <<= 1;
+    UCM_HIP_TRY(hipMalloc(&s->stage, cap));
+    s->stage_cap = cap;
+    return UCM_OK;
 }
 
 int finish(ucm_trans_stream* s, int sync)
@@ -200,7 +250,39 @@ int table_copy(ucm_trans_stream* s, int mode, const void* const* src_tab,
                             : (mode == 2 ? (const uint64_t*)sl->dev + number : nullptr);
     }
     const size_t segs = (size + kSeg - 1) / kSeg;
-    const dim3 grid = grid_for(number * segs);
+    // host tables can be inspected; a device-resident table says nothing about what it points to
+    bool host_end = mode != 2 && is_host_memory(mode == 1 ? src_flat : dst_flat);
+    if (host_end && size <= kStageBytes) {
+        // two stages per piece of whole chunks: kernel <-> device staging, copy engine <-> host
+        const size_t per_piece = kStageBytes / size;
+        const size_t first_piece = number < per_piece ? number : per_piece;
+        int rc = ensure_stage(s, first_piece * size);
+        if (rc != UCM_OK) return rc;
+        for (size_t first = 0; first < number; first += per_piece) {
+            const size_t n = number - first < per_piece ? number - first : per_piece;
+            const dim3 pgrid = grid_for(n * segs);
+            if (mode == 0) {
+                hipLaunchKernelGGL(table_copy_kernel<0>, pgrid, dim3(kThreads), 0, s->stream, d_src + first, d_dst,
+                                   (const uint8_t*)nullptr, (uint8_t*)s->stage, size, n, segs);
+                UCM_HIP_TRY(hipMemcpyAsync((char*)dst_flat + first * size, s->stage, n * size,
+                                           hipMemcpyDeviceToHost, s->stream));
+            } else {
+                UCM_HIP_TRY(hipMemcpyAsync(s->stage, (const char*)src_flat + first * size, n * size,
+                                           hipMemcpyHostToDevice, s->stream));
+                hipLaunchKernelGGL(table_copy_kernel<1>, pgrid, dim3(kThreads), 0, s->stream, d_src, d_dst + first,
+                                   (const uint8_t*)s->stage, (uint8_t*)nullptr, size, n, segs);
+            }
+        }
+        rc = ucm::launch_status("table_copy_kernel");
+        if (rc != UCM_OK) return rc;
+        if (sl) {
+            rc = release_slot(s, sl);
+            if (rc != UCM_OK) return rc;
+        }
+        return finish(s, sync);
+    }
+    if (!host_end && mode == 2 && !table_on_device) host_end = is_host_memory(src_tab[0]) || is_host_memory(dst_tab[0]);
+    const dim3 grid = grid_for(number * segs, host_end);
     if (mode == 0)
         hipLaunchKernelGGL(table_copy_kernel<0>, grid, dim3(kThreads), 0, s->stream, d_src, d_dst,
                            (const uint8_t*)nullptr, (uint8_t*)dst_flat, size, number, segs);
@@ -276,6 +358,7 @@ extern "C" int ucm_trans_stream_destroy(ucm_trans_stream_t* s)
         if (sl.host) (void)hipHostFree(sl.host);
         if (sl.dev) (void)hipFree(sl.dev);
     }
+    if (s->stage) (void)hipFree(s->stage);
     (void)hipStreamDestroy(s->stream);
     delete s;
     return UCM_OK;
@@ -393,10 +476,28 @@ extern "C" int ucm_trans_paged_copy(ucm_trans_stream_t* s, const uint64_t* base,
     }
     std::memcpy(h + meta_words, block_ids, (size_t)n_blocks * 4);
     UCM_HIP_TRY(hipMemcpyAsync(sl->dev, sl->host, bytes, hipMemcpyHostToDevice, s->stream));
-    const dim3 grid = grid_for((size_t)n_blocks * segs_per_row);
-    hipLaunchKernelGGL(paged_copy_kernel, grid, dim3(kThreads), 0, s->stream,
-                       (const uint64_t*)sl->dev, (int)n_cols, segs_per_row, row_bytes,
-                       (size_t)n_blocks, (uint8_t*)flat, to_cache);
+    const bool host_end = is_host_memory(flat);
+    if (host_end && row_bytes <= kStageBytes) {
+        // two stages per piece of whole blocks, as in table_copy()
+        const size_t per_piece = kStageBytes / row_bytes;
+        const size_t first_piece = (size_t)n_blocks < per_piece ? (size_t)n_blocks : per_piece;
+        rc = ensure_stage(s, first_piece * row_bytes);
+        if (rc != UCM_OK) return rc;
+        for (size_t first = 0; first < (size_t)n_blocks; first += per_piece) {
+            const size_t n = (size_t)n_blocks - first < per_piece ? (size_t)n_blocks - first : per_piece;
+            const dim3 pgrid = grid_for(n * segs_per_row);
+            char* hp = (char*)flat + first * row_bytes;
+            if (to_cache) UCM_HIP_TRY(hipMemcpyAsync(s->stage, hp, n * row_bytes, hipMemcpyHostToDevice, s->stream));
+            hipLaunchKernelGGL(paged_copy_kernel, pgrid, dim3(kThreads), 0, s->stream, (const uint64_t*)sl->dev,
+                               (int)n_cols, segs_per_row, row_bytes, n, (uint8_t*)s->stage, to_cache, first);
+            if (!to_cache) UCM_HIP_TRY(hipMemcpyAsync(hp, s->stage, n * row_bytes, hipMemcpyDeviceToHost, s->stream));
+        }
+    } else {
+        const dim3 grid = grid_for((size_t)n_blocks * segs_per_row, host_end);
+        hipLaunchKernelGGL(paged_copy_kernel, grid, dim3(kThreads), 0, s->stream,
+                           (const uint64_t*)sl->dev, (int)n_cols, segs_per_row, row_bytes,
+                           (size_t)n_blocks, (uint8_t*)flat, to_cache, (size_t)0);
+    }
     rc = ucm::launch_status("paged_copy_kernel");
     if (rc != UCM_OK) return rc;
     rc = release_slot(s, sl);
