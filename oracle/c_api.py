@@ -154,8 +154,9 @@ def hamming_score(q, kc, table, lens, max_seq_len, sink=0, recent=0, reduce_head
 
 
 def hamming_topk(q, kc, table, lens, k, sink=0, recent=0, flags=0, head_major=False,
-                 max_blocks=None, nthreads=1):
-    """-> (idx, score) int32 [B, Hkv|1, k]."""
+                 max_blocks=None, nthreads=1, head_items=False):
+    """-> (idx, score) int32 [B, Hkv|1, k].  head_items: the threads take (request, KV head)
+    items from a shared counter, each pinned to a core (per-head output only)."""
     q = _c(q, np.uint32)
     lens = _c(lens, np.int32)
     NB, BS, Hkv, Wd, ks = _cache_args(kc, head_major)
@@ -170,7 +171,9 @@ def hamming_topk(q, kc, table, lens, k, sink=0, recent=0, flags=0, head_major=Fa
     Ho = 1 if (flags & F_REDUCE_HEADS) else Hkv
     idx = np.zeros((B, Ho, k), np.int32)
     sc = np.zeros((B, Ho, k), np.int32)
-    lib().oracle_hamming_topk(_p(q), C.c_int64(Hq * Wd), C.c_int64(Wd), _p(kc), C.c_int64(NB),
+    assert not (head_items and (flags & F_REDUCE_HEADS))
+    fn = lib().oracle_hamming_topk_items if head_items else lib().oracle_hamming_topk
+    fn(_p(q), C.c_int64(Hq * Wd), C.c_int64(Wd), _p(kc), C.c_int64(NB),
                               C.c_int32(BS), C.c_int32(Hkv), C.c_int32(Wd), C.c_int64(ks[0]),
                               C.c_int64(ks[1]), C.c_int64(ks[2]), _p(table), C.c_int32(ts),
                               C.c_int32(mb), _p(lens), C.c_int32(B), C.c_int32(Hq), C.c_int32(k),

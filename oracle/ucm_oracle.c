@@ -9,9 +9,11 @@
  * request, which is the reference CPU backend's execution model
  * (ucm/sparse/gsa_on_device/csrc/cuda/hash_retrieval/cpy/hash_retrieval_backend.cpp:180-199,338).
  */
+#define _GNU_SOURCE
 #include <limits.h>
 #include <math.h>
 #include <pthread.h>
+#include <sched.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -333,6 +335,75 @@ static void* topk_range(void* arg)
                  a->recent, a->flags, a->out_idx + (int64_t)b * Ho * a->k,
                  a->out_score ? a->out_score + (int64_t)b * Ho * a->k : NULL);
     return NULL;
+}
+
+/*
+ * The same top-k with the work cut into (request, KV head) items that `nthreads` threads take
+ * from a shared counter, each thread pinned to one of the cores this process may run on (the
+ * reference's CPU backend pins its workers the same way, hash_retrieval_backend.cpp:188-199).
+ * Timing variant for hosts with more cores than requests; per-head output only (no head reduce).
+ */
+typedef struct {
+    topk_job_t job;
+    volatile int32_t* next;
+    int32_t core;
+} topk_item_worker_t;
+
+static void* topk_items(void* arg)
+{
+    topk_item_worker_t* w = (topk_item_worker_t*)arg;
+    const topk_job_t* a = &w->job;
+    if (w->core >= 0) {
+        cpu_set_t set;
+        CPU_ZERO(&set);
+        CPU_SET(w->core, &set);
+        (void)pthread_setaffinity_np(pthread_self(), sizeof(set), &set);
+    }
+    const int32_t G = a->Hq / a->Hkv;
+    const int32_t total = a->B * a->Hkv;
+    for (;;) {
+        const int32_t i = __sync_fetch_and_add(w->next, 1);
+        if (i >= total) break;
+        const int32_t b = i / a->Hkv, h = i % a->Hkv;
+        topk_one(a->q + b * a->q_stride_b + (int64_t)h * G * a->q_stride_h, a->q_stride_h,
+                 a->kc + (int64_t)h * a->ks_head, a->NB, a->BS, 1, a->Wd, a->ks_block, a->ks_token,
+                 a->ks_head, a->table ? a->table + (int64_t)b * a->table_stride : NULL,
+                 (int64_t)b * a->max_blocks, a->lens[b], a->max_blocks, G, a->k, a->sink, a->recent,
+                 a->flags & ~F_REDUCE_HEADS, a->out_idx + ((int64_t)b * a->Hkv + h) * a->k,
+                 a->out_score ? a->out_score + ((int64_t)b * a->Hkv + h) * a->k : NULL);
+    }
+    return NULL;
+}
+
+void oracle_hamming_topk_items(const uint32_t* q, int64_t q_stride_b, int64_t q_stride_h,
+                               const uint32_t* kc, int64_t NB, int32_t BS, int32_t Hkv, int32_t Wd,
+                               int64_t ks_block, int64_t ks_token, int64_t ks_head,
+                               const int32_t* table, int32_t table_stride, int32_t max_blocks,
+                               const int32_t* lens, int32_t B, int32_t Hq, int32_t k, int32_t sink,
+                               int32_t recent, uint32_t flags, int32_t* out_idx, int32_t* out_score,
+                               int32_t nthreads)
+{
+    topk_job_t base = {q,  q_stride_b, q_stride_h, kc,     NB,        BS,    Hkv,
+                       Wd, ks_block,   ks_token,   ks_head, table,     table_stride,
+                       max_blocks, lens, B, Hq, k, sink, recent, flags, out_idx, out_score, 0, B};
+    if (nthreads < 1) nthreads = 1;
+    cpu_set_t allowed;
+    int32_t cores[1024], ncores = 0;
+    if (sched_getaffinity(0, sizeof(allowed), &allowed) == 0)
+        for (int32_t c = 0; c < 1024 && c < CPU_SETSIZE; ++c)
+            if (CPU_ISSET(c, &allowed)) cores[ncores++] = c;
+    volatile int32_t next = 0;
+    pthread_t* th = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)nthreads);
+    topk_item_worker_t* ws = (topk_item_worker_t*)malloc(sizeof(topk_item_worker_t) * (size_t)nthreads);
+    for (int32_t i = 0; i < nthreads; ++i) {
+        ws[i].job = base;
+        ws[i].next = &next;
+        ws[i].core = ncores ? cores[i % ncores] : -1;
+        pthread_create(&th[i], NULL, topk_items, &ws[i]);
+    }
+    for (int32_t i = 0; i < nthreads; ++i) pthread_join(th[i], NULL);
+    free(ws);
+    free(th);
 }
 
 /*

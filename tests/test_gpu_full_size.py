@@ -272,3 +272,49 @@ def test_config4_kv_block_transfer_round_trip_full_payload():
         for l in range(L):  # restore the canary for the next request
             dst[l][:, n] = 0x5A5A
     torch.cuda.synchronize()
+
+
+def test_config5_encode_from_bf16_latents_at_full_size():
+    """BASELINE.json config 5 from its floating-point inputs: 16 x 65,536 latent rows of 576 bf16
+    values of which the first 512 are hashed with a 512 x 256 projection into the paged code cache
+    (64-token blocks, permuted table), and the 16 x 128 query rows with the same projection.  The
+    codes are checked with the margin rule on sampled rows (|projection| < 1e-2 * ||x|| is the only
+    place a bit may differ from the float64 oracle), the top-128 on those codes bit-exactly."""
+    from oracle import brute
+    from ucm_amd.sparse import HashEncoder, hamming_topk
+
+    B, CTX, HQ, KIN, KROW, N, BS, K = 16, 65536, 128, 512, 576, 256, 64, 128
+    NBLK = CTX // BS
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1005)
+    W = torch.randn((KIN, N), generator=gen, device="cuda").to(torch.bfloat16)
+    enc = HashEncoder(KIN, N, torch.bfloat16, torch.device("cuda:0"))
+    enc.set_hash_weight(W)
+    cache = torch.zeros((B * NBLK, BS, 1, N // 32), dtype=torch.int32, device="cuda")
+    table = torch.randperm(B * NBLK, device="cuda", generator=gen).to(torch.int32).reshape(B, NBLK)
+    Wf = W.float().cpu().numpy()
+    rng = np.random.default_rng(55)
+    for b in range(B):
+        latent = torch.randn((CTX, 1, KROW), generator=gen, device="cuda").to(torch.bfloat16)
+        slots = (table[b].long().repeat_interleave(BS) * BS + torch.arange(BS, device="cuda").repeat(NBLK))
+        enc.compute_hash_and_cache(latent[:, :, :KIN], slots, cache, BS)  # rows of 576, 512 hashed
+        if b in (0, 9, 15):
+            rows = np.sort(rng.choice(CTX, size=300, replace=False))
+            x = latent[rows, 0, :KIN].float().cpu().numpy()
+            torch.cuda.synchronize()
+            got = np_u32(cache).reshape(-1, N // 32)[slots.cpu().numpy()[rows]]
+            ref = brute.hash_encode(x, Wf)
+            diff = np.unpackbits((got ^ ref).view(np.uint8), axis=-1, bitorder="little").astype(bool)
+            assert not np.any(diff & (brute.margins(x, Wf) >= 1e-2)), "code bit flipped outside the margin"
+    qx = torch.randn((B, HQ, KIN), generator=gen, device="cuda").to(torch.bfloat16)
+    q = enc.compute_hash(qx).view(torch.int32)
+    qref = brute.hash_encode(qx.float().cpu().numpy().reshape(-1, KIN), Wf)
+    qdiff = np.unpackbits((np_u32(q).reshape(-1, N // 32) ^ qref).view(np.uint8), axis=-1, bitorder="little").astype(bool)
+    assert not np.any(qdiff & (brute.margins(qx.float().cpu().numpy().reshape(-1, KIN), Wf) >= 1e-2))
+    lens = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
+    idx, sc = hamming_topk(q, cache, table, lens, K)
+    sel = [2, 7, 11]
+    oi, osc = c_api.hamming_topk(np_u32(q)[sel], np_u32(cache), table.cpu().numpy()[sel],
+                                 lens.cpu().numpy()[sel], K, nthreads=3)
+    assert np.array_equal(idx.cpu().numpy()[sel], oi)
+    assert np.array_equal(sc.cpu().numpy()[sel], osc)

@@ -361,3 +361,13 @@ def test_paged_copy_variable_columns():
     c_api.paged_copy([c.ctypes.data for c in cols2], col_bytes, ids2, flat, to_cache=True)
     for c, c2 in zip(cols, cols2):
         assert np.array_equal(c2[ids2], c[ids])
+
+
+def test_topk_request_head_items_mode_equals_the_request_mode():
+    """The timing variant that hands (request, KV head) items to pinned threads computes the
+    same lists as one thread per request."""
+    q, kc, table, lens = make_paged_case(4711, 3, 8, 4, 2, 8, [70, 33, 8], table_pad=1)
+    ref = c_api.hamming_topk(q, kc, table, lens, 3, 4, 8)
+    for nt in (1, 2, 5):
+        got = c_api.hamming_topk(q, kc, table, lens, 3, 4, 8, nthreads=nt, head_items=True)
+        assert np.array_equal(got[0], ref[0]) and np.array_equal(got[1], ref[1])
