@@ -57,13 +57,16 @@ def parse():
     ap.add_argument("--skip-extras", action="store_true",
                     help="only the headline workload (no encoder / gather side figures)")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--legs", default=",".join(ALL_LEGS),
+                    help="comma-separated side figures to run (default: all): " + ", ".join(ALL_LEGS))
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="only run a plain device-to-device copy of known size (1 GiB read + 1 GiB "
                          "written per launch) so that hardware byte counters can be scaled")
     ap.add_argument("--graph-steps", type=int, default=4,
                     help="decode steps captured per HIP graph (each on the next rotated cache)")
     ap.add_argument("--no-graph", action="store_true",
-                    help="time eager launches instead of HIP graph replays")
+                    help="time eager launches instead of HIP graph replays; no graph is captured "
+                         "anywhere and no hold kernel is queued (the mode for hardware-counter runs)")
     return ap.parse_args()
 
 
@@ -265,6 +268,17 @@ def graph_ms(torch, fn, reps=20, replays=5):
     """Milliseconds per call of fn(i) with `reps` calls captured in one HIP graph and the graph
     replayed: the launches run back to back on the GPU, so the figure is the kernels' time, not
     the host's time to issue them one by one from Python."""
+    if NO_GRAPH:  # counter runs: the same calls issued one by one (host-bound for small kernels)
+        for i in range(3):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         for i in range(3):
@@ -283,6 +297,12 @@ def graph_ms(torch, fn, reps=20, replays=5):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / (reps * replays)
+
+
+NO_GRAPH = False  # set by --no-graph: no HIP graph is captured anywhere and no hold kernel is queued
+
+ALL_LEGS = ("encoder", "prefix_rehash", "float_retrieval", "retrieval_shapes", "token_scores", "gather",
+            "plugin", "beside")
 
 
 def encoder_cache_build(torch, enc_k, gen, launches=9):
@@ -362,6 +382,8 @@ def plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots):
         gaps = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(n))
         res = {"eager_p50_us": gaps[n // 2], "eager_p90_us": gaps[int(n * 0.9)], "eager_wall_us_per_call": wall}
         try:
+            if NO_GRAPH:
+                raise RuntimeError("graphs switched off (--no-graph)")
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -475,301 +497,307 @@ def gather_beside_decode(torch, gen, run_step, steps_per_call):
     return out
 
 
-def extras(torch, enc_k, gen):
+def extras(torch, enc_k, gen, legs=ALL_LEGS):
     """Side figures: encoder at cache-build shape, device gather, pinned-host dump."""
     import numpy as np
     from ucm_amd.trans import Device
 
     out = {}
-    # --- encoder: one request's keys (32768 x 8 rows of 128) per call ---
-    keys = torch.randn((CTX, HKV, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
-    cache = torch.empty((NBLK, BS, HKV, WD), dtype=torch.int32, device="cuda")
-    slots = torch.arange(CTX, device="cuda", dtype=torch.int64)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    reps = 20
-    ms = graph_ms(torch, lambda i: enc_k.compute_hash_and_cache(keys, slots, cache, BS))
-    rows = CTX * HKV
-    enc_bytes = rows * D * 2 + rows * WD * 4 + HKV * D * D * 2
-    out["encoder_one_request_cache_warm"] = {
-        "rows": rows, "ms": ms, "GBps": enc_bytes / ms / 1e6, "TFLOPs": 2.0 * rows * D * D / ms / 1e9,
-        "input": "one 67 MB key tensor replayed: served by the 256 MB last-level cache, not an HBM figure"}
-    del keys, cache
+    if "encoder" in legs:
+        # --- encoder: one request's keys (32768 x 8 rows of 128) per call ---
+        keys = torch.randn((CTX, HKV, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+        cache = torch.empty((NBLK, BS, HKV, WD), dtype=torch.int32, device="cuda")
+        slots = torch.arange(CTX, device="cuda", dtype=torch.int64)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 20
+        ms = graph_ms(torch, lambda i: enc_k.compute_hash_and_cache(keys, slots, cache, BS))
+        rows = CTX * HKV
+        enc_bytes = rows * D * 2 + rows * WD * 4 + HKV * D * D * 2
+        out["encoder_one_request_cache_warm"] = {
+            "rows": rows, "ms": ms, "GBps": enc_bytes / ms / 1e6, "TFLOPs": 2.0 * rows * D * D / ms / 1e9,
+            "input": "one 67 MB key tensor replayed: served by the 256 MB last-level cache, not an HBM figure"}
+        del keys, cache
 
-    # --- encoder at cache-build size: the keys of all 32 requests (8,388,608 rows of 128 bf16 =
-    #     2.1 GB, far beyond the last-level cache: a cold-HBM figure) hashed into the paged code
-    #     cache through the permuted block table (compute_hash_and_cache, hash_encoder.py:548-662) ---
-    out["encoder_cache_build"] = encoder_cache_build(torch, enc_k, gen)
+        # --- encoder at cache-build size: the keys of all 32 requests (8,388,608 rows of 128 bf16 =
+        #     2.1 GB, far beyond the last-level cache: a cold-HBM figure) hashed into the paged code
+        #     cache through the permuted block table (compute_hash_and_cache, hash_encoder.py:548-662) ---
+        out["encoder_cache_build"] = encoder_cache_build(torch, enc_k, gen)
 
-    # --- prefix-cache rehash: keys of 256 blocks read in place from a paged key cache, against
-    #     the reference's recipe (gather the blocks into a copy, then encode with a slot map) ---
-    NBK = 1024
-    kcache = torch.empty((NBK, BS, HKV, D), dtype=torch.bfloat16, device="cuda").normal_(generator=gen)
-    codes = torch.empty((NBK, BS, HKV, WD), dtype=torch.int32, device="cuda")
-    perms = [torch.randperm(NBK, generator=gen, device="cuda")[:NBLK].to(torch.int32) for _ in range(4)]
-    tok = torch.arange(CTX, device="cuda")
+    if "prefix_rehash" in legs:
+        # --- prefix-cache rehash: keys of 256 blocks read in place from a paged key cache, against
+        #     the reference's recipe (gather the blocks into a copy, then encode with a slot map) ---
+        NBK = 1024
+        kcache = torch.empty((NBK, BS, HKV, D), dtype=torch.bfloat16, device="cuda").normal_(generator=gen)
+        codes = torch.empty((NBK, BS, HKV, WD), dtype=torch.int32, device="cuda")
+        perms = [torch.randperm(NBK, generator=gen, device="cuda")[:NBLK].to(torch.int32) for _ in range(4)]
+        tok = torch.arange(CTX, device="cuda")
 
-    def fused(i):
-        enc_k.compute_hash_from_paged_cache(kcache, perms[i % 4], CTX, codes, BS)
+        def fused(i):
+            enc_k.compute_hash_from_paged_cache(kcache, perms[i % 4], CTX, codes, BS)
 
-    def recipe(i):
-        ids = perms[i % 4]
-        gathered = kcache[ids.long()].reshape(-1, HKV, D)
-        slot_map = ids.long()[tok // BS] * BS + tok % BS
-        enc_k.compute_hash_and_cache(gathered, slot_map, codes, BS)
+        def recipe(i):
+            ids = perms[i % 4]
+            gathered = kcache[ids.long()].reshape(-1, HKV, D)
+            slot_map = ids.long()[tok // BS] * BS + tok % BS
+            enc_k.compute_hash_and_cache(gathered, slot_map, codes, BS)
 
-    for name, fn in (("fused", fused), ("reference_recipe", recipe)):
-        ms = graph_ms(torch, fn)
-        out.setdefault("prefix_rehash", {})[name] = {
-            "tokens": CTX, "ms": ms, "key_GBps": rows * D * 2 / ms / 1e6}
-    del kcache, codes
+        for name, fn in (("fused", fused), ("reference_recipe", recipe)):
+            ms = graph_ms(torch, fn)
+            out.setdefault("prefix_rehash", {})[name] = {
+                "tokens": CTX, "ms": ms, "key_GBps": rows * D * 2 / ms / 1e6}
+        del kcache, codes
 
-    # --- float retrieval (ESA): the shape of the reference's own driver
-    #     (esa/retrieval/retrieval_worker.py:45-60): 25600 block vectors of dim 1024, 2 requests,
-    #     8000 candidates each, top-3000 ---
-    from ucm_amd.sparse.esa_retrieval_worker import dot_topk
+    if "float_retrieval" in legs:
+        # --- float retrieval (ESA): the shape of the reference's own driver
+        #     (esa/retrieval/retrieval_worker.py:45-60): 25600 block vectors of dim 1024, 2 requests,
+        #     8000 candidates each, top-3000 ---
+        from ucm_amd.sparse.esa_retrieval_worker import dot_topk
 
-    vecs = torch.rand((25600, 1024), generator=gen, device="cuda", dtype=torch.float32)
-    qv = torch.rand((2, 1024), generator=gen, device="cuda", dtype=torch.float32)
-    cand = torch.stack([torch.randperm(25600, generator=gen, device="cuda")[:8000] for _ in range(2)]).to(torch.int32)
-    ws = torch.empty(_esa_ws(2, 8000), dtype=torch.uint8, device="cuda")
-    ms = graph_ms(torch, lambda i: dot_topk(vecs, qv, cand, 3000, ws))
-    out["esa_dot_topk"] = {"candidates": 2 * 8000, "dim": 1024, "topk": 3000, "ms": ms,
-                           "gather_GBps": 2 * 8000 * 4096 / ms / 1e6}
-    del vecs
+        vecs = torch.rand((25600, 1024), generator=gen, device="cuda", dtype=torch.float32)
+        qv = torch.rand((2, 1024), generator=gen, device="cuda", dtype=torch.float32)
+        cand = torch.stack([torch.randperm(25600, generator=gen, device="cuda")[:8000] for _ in range(2)]).to(torch.int32)
+        ws = torch.empty(_esa_ws(2, 8000), dtype=torch.uint8, device="cuda")
+        ms = graph_ms(torch, lambda i: dot_topk(vecs, qv, cand, 3000, ws))
+        out["esa_dot_topk"] = {"candidates": 2 * 8000, "dim": 1024, "topk": 3000, "ms": ms,
+                               "gather_GBps": 2 * 8000 * 4096 / ms / 1e6}
+        del vecs
 
-    # --- float retrieval (KVStar) ---
-    from ucm_amd.sparse.kvstar_retrieve import kvstar_topk
+        # --- float retrieval (KVStar) ---
+        from ucm_amd.sparse.kvstar_retrieve import kvstar_topk
 
-    kq, kk, kp = (torch.from_numpy(t).cuda() for t in _kvstar_case(np))
-    kws = torch.empty(_lib_mod().lib().ucm_kvstar_topk_workspace_bytes(8, 32, 253, 64), dtype=torch.uint8,
-                      device="cuda")
-    out["kvstar_topk"] = {"queries": 8, "q_heads": 32, "blocks": 253, "representatives": 253 * 64,
-                          "dim": 32, "topk": 64,
-                          "ms": graph_ms(torch, lambda i: kvstar_topk(kq, kk, kp, 64, kws))}
+        kq, kk, kp = (torch.from_numpy(t).cuda() for t in _kvstar_case(np))
+        kws = torch.empty(_lib_mod().lib().ucm_kvstar_topk_workspace_bytes(8, 32, 253, 64), dtype=torch.uint8,
+                          device="cuda")
+        out["kvstar_topk"] = {"queries": 8, "q_heads": 32, "blocks": 253, "representatives": 253 * 64,
+                              "dim": 32, "topk": 64,
+                              "ms": graph_ms(torch, lambda i: kvstar_topk(kq, kk, kp, 64, kws))}
 
-    # --- the other retrieval shapes of BASELINE.json (parity-tested in tests/test_gpu_full_size.py),
-    #     timed here on random codes: top-k = score + select; the per-token scorer alone ---
-    from ucm_amd.sparse import hamming_score, hamming_topk
+    if "retrieval_shapes" in legs:
+        # --- the other retrieval shapes of BASELINE.json (parity-tested in tests/test_gpu_full_size.py),
+        #     timed here on random codes: top-k = score + select; the per-token scorer alone ---
+        from ucm_amd.sparse import hamming_score, hamming_topk
 
-    def codes(shape):
-        return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device="cuda", generator=gen)
+        def codes(shape):
+            return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device="cuda", generator=gen)
 
-    # config 3: batch 8, lengths uniform in [16384, 131072], 128-bit codes, top-128
-    lens3 = torch.randint(16384, 131072 + 1, (8,), generator=gen, device="cuda").to(torch.int32)
-    nblk3 = (lens3.long() + BS - 1) // BS
-    nb3 = int(nblk3.sum())
-    cache3 = codes((nb3, BS, HKV, WD))
-    table3 = torch.zeros((8, int(nblk3.max())), dtype=torch.int32, device="cuda")
-    perm3 = torch.randperm(nb3, generator=gen, device="cuda").to(torch.int32)
-    o = 0
-    for b in range(8):
-        table3[b, : int(nblk3[b])] = perm3[o:o + int(nblk3[b])]
-        o += int(nblk3[b])
-    q3 = codes((8, HQ, WD))
-    ms = graph_ms(torch, lambda i: hamming_topk(q3, cache3, table3, lens3, 128))
-    tok3 = int(lens3.sum())
-    out["config3_ragged_topk128"] = {"tokens": tok3, "ms": ms, "tokens_per_s": tok3 / ms * 1e3,
-                                     "code_GBps": tok3 * HKV * WD * 4 / ms / 1e6}
-    del cache3, table3
-    # config 5: MLA, one latent head, 128 q heads, 256-bit codes, 16 x 65536 tokens, 64-token blocks, top-128
-    b5, ctx5, bs5, wd5 = 16, 65536, 64, 8
-    cache5 = codes((b5 * ctx5 // bs5, bs5, 1, wd5))
-    table5 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
-    lens5 = torch.full((b5,), ctx5, dtype=torch.int32, device="cuda")
-    q5 = codes((b5, 128, wd5))
-    ms = graph_ms(torch, lambda i: hamming_topk(q5, cache5, table5, lens5, 128))
-    out["config5_mla_topk128"] = {"tokens": b5 * ctx5, "ms": ms, "tokens_per_s": b5 * ctx5 / ms * 1e3,
-                                  "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6}
-    del cache5, table5
-    # the reference's own latent-attention setting: 18-word codes (512 nope + 64 rope bits), 64 query
-    # heads after its head reduction (128 heads, reduction 2), same 16 x 65536 tokens
-    wd6 = 18
-    cache6 = codes((b5 * ctx5 // bs5, bs5, 1, wd6))
-    table6 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
-    q6 = codes((b5, 64, wd6))
-    ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6, table6, lens5, 128))
-    ms_tok = graph_ms(torch, lambda i: hamming_score(cache6, q6, table6, lens5, ctx5, 0, 0, False), reps=5)
-    # the whole decode step of that layout in one native call: both parts of 16 new keys into the cache,
-    # both parts of the 16 x 64 query rows hashed, score, select
-    from ucm_amd.sparse import SparseDecodeStepMLA
-    bf = lambda *shape: torch.randn(*shape, device="cuda", dtype=torch.bfloat16, generator=gen)
-    stm = SparseDecodeStepMLA(bf(512, 512), bf(64, 64), 64, b5, ctx5 // bs5, 128, block_size=bs5,
-                              sink_token=bs5, recent_token=4 * bs5, return_physical=True)
-    kn6, kr6, qn6, qr6 = bf(b5, 512), bf(b5, 64), bf(b5, 64, 512), bf(b5, 64, 64)
-    slots6 = (table6[:, -1].to(torch.int64) * bs5 + bs5 - 1)
-    cache6v = cache6.view(cache6.shape[0], bs5, wd6)
-    ms_step = graph_ms(torch, lambda i: stm.step(kn6, kr6, slots6, qn6, qr6, cache6v, table6, lens5))
-    out["mla_576bit_64heads"] = {"tokens": b5 * ctx5, "topk128_ms": ms, "token_scores_ms": ms_tok,
-                                 "decode_step_ms": ms_step,
-                                 "tokens_per_s": b5 * ctx5 / ms * 1e3,
-                                 "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6}
-    del cache6, table6
-    # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
-    cache2 = codes((NB, BS, HKV, WD))
-    table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, NBLK)
-    lens2 = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
-    q2 = codes((B, HQ, WD))
-    ms = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, False), reps=10)
-    byt = B * CTX * HKV * (WD * 4 + 2)
-    # the reference's own GQA call reduces over the KV heads (hamming_topk.py:33): one fp16 row per request
-    ms_red = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, True), reps=10)
-    byt_red = B * CTX * (HKV * WD * 4 + 2)
-    out["token_scores_config2"] = {"tokens": B * CTX, "ms": ms, "tokens_per_s": B * CTX / ms * 1e3,
-                                   "hbm_GBps": byt / ms / 1e6, "hbm_frac": byt / ms / 1e6 / HBM_PEAK_GBPS,
-                                   "reduce_kvhead_ms": ms_red,
-                                   "reduce_kvhead_hbm_frac": byt_red / ms_red / 1e6 / HBM_PEAK_GBPS}
-    del cache2, table2
+        # config 3: batch 8, lengths uniform in [16384, 131072], 128-bit codes, top-128
+        lens3 = torch.randint(16384, 131072 + 1, (8,), generator=gen, device="cuda").to(torch.int32)
+        nblk3 = (lens3.long() + BS - 1) // BS
+        nb3 = int(nblk3.sum())
+        cache3 = codes((nb3, BS, HKV, WD))
+        table3 = torch.zeros((8, int(nblk3.max())), dtype=torch.int32, device="cuda")
+        perm3 = torch.randperm(nb3, generator=gen, device="cuda").to(torch.int32)
+        o = 0
+        for b in range(8):
+            table3[b, : int(nblk3[b])] = perm3[o:o + int(nblk3[b])]
+            o += int(nblk3[b])
+        q3 = codes((8, HQ, WD))
+        ms = graph_ms(torch, lambda i: hamming_topk(q3, cache3, table3, lens3, 128))
+        tok3 = int(lens3.sum())
+        out["config3_ragged_topk128"] = {"tokens": tok3, "ms": ms, "tokens_per_s": tok3 / ms * 1e3,
+                                         "code_GBps": tok3 * HKV * WD * 4 / ms / 1e6}
+        del cache3, table3
+        # config 5: MLA, one latent head, 128 q heads, 256-bit codes, 16 x 65536 tokens, 64-token blocks, top-128
+        b5, ctx5, bs5, wd5 = 16, 65536, 64, 8
+        cache5 = codes((b5 * ctx5 // bs5, bs5, 1, wd5))
+        table5 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
+        lens5 = torch.full((b5,), ctx5, dtype=torch.int32, device="cuda")
+        q5 = codes((b5, 128, wd5))
+        ms = graph_ms(torch, lambda i: hamming_topk(q5, cache5, table5, lens5, 128))
+        out["config5_mla_topk128"] = {"tokens": b5 * ctx5, "ms": ms, "tokens_per_s": b5 * ctx5 / ms * 1e3,
+                                      "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6}
+        del cache5, table5
+        # the reference's own latent-attention setting: 18-word codes (512 nope + 64 rope bits), 64 query
+        # heads after its head reduction (128 heads, reduction 2), same 16 x 65536 tokens
+        wd6 = 18
+        cache6 = codes((b5 * ctx5 // bs5, bs5, 1, wd6))
+        table6 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
+        q6 = codes((b5, 64, wd6))
+        ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6, table6, lens5, 128))
+        ms_tok = graph_ms(torch, lambda i: hamming_score(cache6, q6, table6, lens5, ctx5, 0, 0, False), reps=5)
+        # the whole decode step of that layout in one native call: both parts of 16 new keys into the cache,
+        # both parts of the 16 x 64 query rows hashed, score, select
+        from ucm_amd.sparse import SparseDecodeStepMLA
+        bf = lambda *shape: torch.randn(*shape, device="cuda", dtype=torch.bfloat16, generator=gen)
+        stm = SparseDecodeStepMLA(bf(512, 512), bf(64, 64), 64, b5, ctx5 // bs5, 128, block_size=bs5,
+                                  sink_token=bs5, recent_token=4 * bs5, return_physical=True)
+        kn6, kr6, qn6, qr6 = bf(b5, 512), bf(b5, 64), bf(b5, 64, 512), bf(b5, 64, 64)
+        slots6 = (table6[:, -1].to(torch.int64) * bs5 + bs5 - 1)
+        cache6v = cache6.view(cache6.shape[0], bs5, wd6)
+        ms_step = graph_ms(torch, lambda i: stm.step(kn6, kr6, slots6, qn6, qr6, cache6v, table6, lens5))
+        out["mla_576bit_64heads"] = {"tokens": b5 * ctx5, "topk128_ms": ms, "token_scores_ms": ms_tok,
+                                     "decode_step_ms": ms_step,
+                                     "tokens_per_s": b5 * ctx5 / ms * 1e3,
+                                     "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6}
+        del cache6, table6
+    if "token_scores" in legs:
+        # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
+        cache2 = codes((NB, BS, HKV, WD))
+        table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, NBLK)
+        lens2 = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
+        q2 = codes((B, HQ, WD))
+        ms = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, False), reps=10)
+        byt = B * CTX * HKV * (WD * 4 + 2)
+        # the reference's own GQA call reduces over the KV heads (hamming_topk.py:33): one fp16 row per request
+        ms_red = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, True), reps=10)
+        byt_red = B * CTX * (HKV * WD * 4 + 2)
+        out["token_scores_config2"] = {"tokens": B * CTX, "ms": ms, "tokens_per_s": B * CTX / ms * 1e3,
+                                       "hbm_GBps": byt / ms / 1e6, "hbm_frac": byt / ms / 1e6 / HBM_PEAK_GBPS,
+                                       "reduce_kvhead_ms": ms_red,
+                                       "reduce_kvhead_hbm_frac": byt_red / ms_red / 1e6 / HBM_PEAK_GBPS}
+        del cache2, table2
 
-    # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---
-    L, NBP, n_req, n_sel = 32, 256, 4, 64
-    chunk = BS * HKV * D * 2  # 256 KiB
-    kv = [torch.empty((2, NBP, BS, HKV, D), dtype=torch.bfloat16, device="cuda").normal_(generator=gen)
-          for _ in range(L)]
-    base = np.array([[t[0].data_ptr(), t[1].data_ptr()] for t in kv], np.uint64).reshape(-1)
-    sizes = np.full(base.shape, chunk, np.uint64)
-    ids = np.concatenate([np.random.Generator(np.random.PCG64(1004 + r)).choice(NBP, n_sel, replace=False)
-                          for r in range(n_req)]).astype(np.int32)
-    payload = len(ids) * L * 2 * chunk
-    dev_flat = torch.empty(payload, dtype=torch.uint8, device="cuda")
-    host = torch.empty(payload, dtype=torch.uint8).pin_memory()
-    d = Device()
-    d.Setup(0)
-    st = d.MakeSMStream()
-    addrs = (ids.astype(np.uint64)[:, None] * sizes[None, :] + base[None, :]).reshape(-1)
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
-    side = torch.cuda.ExternalStream(st.handle)
+    if "gather" in legs:
+        # --- KV block gather (config 4 shape, bounded: 4 requests x 64 blocks) ---
+        L, NBP, n_req, n_sel = 32, 256, 4, 64
+        chunk = BS * HKV * D * 2  # 256 KiB
+        kv = [torch.empty((2, NBP, BS, HKV, D), dtype=torch.bfloat16, device="cuda").normal_(generator=gen)
+              for _ in range(L)]
+        base = np.array([[t[0].data_ptr(), t[1].data_ptr()] for t in kv], np.uint64).reshape(-1)
+        sizes = np.full(base.shape, chunk, np.uint64)
+        ids = np.concatenate([np.random.Generator(np.random.PCG64(1004 + r)).choice(NBP, n_sel, replace=False)
+                              for r in range(n_req)]).astype(np.int32)
+        payload = len(ids) * L * 2 * chunk
+        dev_flat = torch.empty(payload, dtype=torch.uint8, device="cuda")
+        host = torch.empty(payload, dtype=torch.uint8).pin_memory()
+        d = Device()
+        d.Setup(0)
+        st = d.MakeSMStream()
+        addrs = (ids.astype(np.uint64)[:, None] * sizes[None, :] + base[None, :]).reshape(-1)
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        side = torch.cuda.ExternalStream(st.handle)
 
-    def timed(fn, reps):
-        fn()
-        st.Synchronized()
-        ev0.record(side)
-        for _ in range(reps):
+        def timed(fn, reps):
             fn()
-        ev1.record(side)
-        st.Synchronized()
-        return ev0.elapsed_time(ev1) / reps
+            st.Synchronized()
+            ev0.record(side)
+            for _ in range(reps):
+                fn()
+            ev1.record(side)
+            st.Synchronized()
+            return ev0.elapsed_time(ev1) / reps
 
-    ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids, dev_flat.data_ptr()), 5)
-    out["gather_device"] = {"payload_GiB": payload / 2**30, "ms": ms, "payload_GBps": payload / ms / 1e6,
-                            "hbm_GBps": 2 * payload / ms / 1e6,
-                            "hbm_frac": 2 * payload / ms / 1e6 / HBM_PEAK_GBPS, "form": "paged (table-free)"}
-    ms = timed(lambda: st.DeviceToHostGatherAsync(addrs, dev_flat.data_ptr(), chunk, len(addrs)), 5)
-    out["gather_device_ptr_table"] = {"ms": ms, "hbm_GBps": 2 * payload / ms / 1e6}
-    ms = timed(lambda: st.PagedScatterAsync(dev_flat.data_ptr(), base, sizes, ids), 5)
-    out["scatter_device"] = {"ms": ms, "hbm_GBps": 2 * payload / ms / 1e6}
-    ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids, host.data_ptr()), 2)
-    out["gather_to_pinned_host"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6,
-                                    "form": "per 64 MiB piece: compaction kernel into device staging, one copy-engine transfer"}
-    ms = timed(lambda: st.DeviceToHostAsync(dev_flat.data_ptr(), host.data_ptr(), payload), 2)
-    out["d2h_copy_engine_flat"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
-    ms = timed(lambda: st.PagedScatterAsync(host.data_ptr(), base, sizes, ids), 2)
-    out["scatter_from_pinned_host"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
-    del host, dev_flat
+        ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids, dev_flat.data_ptr()), 5)
+        out["gather_device"] = {"payload_GiB": payload / 2**30, "ms": ms, "payload_GBps": payload / ms / 1e6,
+                                "hbm_GBps": 2 * payload / ms / 1e6,
+                                "hbm_frac": 2 * payload / ms / 1e6 / HBM_PEAK_GBPS, "form": "paged (table-free)"}
+        ms = timed(lambda: st.DeviceToHostGatherAsync(addrs, dev_flat.data_ptr(), chunk, len(addrs)), 5)
+        out["gather_device_ptr_table"] = {"ms": ms, "hbm_GBps": 2 * payload / ms / 1e6}
+        ms = timed(lambda: st.PagedScatterAsync(dev_flat.data_ptr(), base, sizes, ids), 5)
+        out["scatter_device"] = {"ms": ms, "hbm_GBps": 2 * payload / ms / 1e6}
+        ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids, host.data_ptr()), 2)
+        out["gather_to_pinned_host"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6,
+                                        "form": "per 64 MiB piece: compaction kernel into device staging, one copy-engine transfer"}
+        ms = timed(lambda: st.DeviceToHostAsync(dev_flat.data_ptr(), host.data_ptr(), payload), 2)
+        out["d2h_copy_engine_flat"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
+        ms = timed(lambda: st.PagedScatterAsync(host.data_ptr(), base, sizes, ids), 2)
+        out["scatter_from_pinned_host"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
+        del host, dev_flat
 
-    # --- config 4 at its full size, device side: 32 requests x 64 blocks x 32 layers x {K,V} x 256 KiB
-    #     = 32 GiB gathered from the 4 GiB cache into one device buffer by one launch, and scattered back ---
-    ids_full = np.concatenate([np.random.Generator(np.random.PCG64(1004 + r)).choice(NBP, n_sel, replace=False)
-                               for r in range(32)]).astype(np.int32)
-    full_payload = len(ids_full) * L * 2 * chunk
-    try:
-        dev_full = torch.empty(full_payload, dtype=torch.uint8, device="cuda")
-        ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids_full, dev_full.data_ptr()), 3)
-        ms_s = timed(lambda: st.PagedScatterAsync(dev_full.data_ptr(), base, sizes, ids_full), 3)
-        out["gather_device_full_config4"] = {"payload_GiB": full_payload / 2**30, "gather_ms": ms, "scatter_ms": ms_s,
-                                             "gather_hbm_GBps": 2 * full_payload / ms / 1e6,
-                                             "gather_hbm_frac": 2 * full_payload / ms / 1e6 / HBM_PEAK_GBPS,
-                                             "scatter_hbm_GBps": 2 * full_payload / ms_s / 1e6}
-        del dev_full
-    except Exception as e:  # noqa: BLE001 - a side figure
-        out["gather_device_full_config4"] = {"error": str(e)[:200]}
-    # ... and host side: the same 32 GiB into one contiguous pinned buffer, request by request
-    # (1 GiB each), and back into the cache
-    try:
-        host_full = torch.empty(full_payload, dtype=torch.uint8).pin_memory()
-        per_req = n_sel * L * 2 * chunk
+        # --- config 4 at its full size, device side: 32 requests x 64 blocks x 32 layers x {K,V} x 256 KiB
+        #     = 32 GiB gathered from the 4 GiB cache into one device buffer by one launch, and scattered back ---
+        ids_full = np.concatenate([np.random.Generator(np.random.PCG64(1004 + r)).choice(NBP, n_sel, replace=False)
+                                   for r in range(32)]).astype(np.int32)
+        full_payload = len(ids_full) * L * 2 * chunk
+        try:
+            dev_full = torch.empty(full_payload, dtype=torch.uint8, device="cuda")
+            ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids_full, dev_full.data_ptr()), 3)
+            ms_s = timed(lambda: st.PagedScatterAsync(dev_full.data_ptr(), base, sizes, ids_full), 3)
+            out["gather_device_full_config4"] = {"payload_GiB": full_payload / 2**30, "gather_ms": ms, "scatter_ms": ms_s,
+                                                 "gather_hbm_GBps": 2 * full_payload / ms / 1e6,
+                                                 "gather_hbm_frac": 2 * full_payload / ms / 1e6 / HBM_PEAK_GBPS,
+                                                 "scatter_hbm_GBps": 2 * full_payload / ms_s / 1e6}
+            del dev_full
+        except Exception as e:  # noqa: BLE001 - a side figure
+            out["gather_device_full_config4"] = {"error": str(e)[:200]}
+        # ... and host side: the same 32 GiB into one contiguous pinned buffer, request by request
+        # (1 GiB each), and back into the cache
+        try:
+            host_full = torch.empty(full_payload, dtype=torch.uint8).pin_memory()
+            per_req = n_sel * L * 2 * chunk
 
-        def dump_all():
-            for r in range(32):
-                st.PagedGatherAsync(base, sizes, ids_full[r * n_sel:(r + 1) * n_sel], host_full.data_ptr() + r * per_req)
+            def dump_all():
+                for r in range(32):
+                    st.PagedGatherAsync(base, sizes, ids_full[r * n_sel:(r + 1) * n_sel], host_full.data_ptr() + r * per_req)
 
-        def restore_all():
-            for r in range(32):
-                st.PagedScatterAsync(host_full.data_ptr() + r * per_req, base, sizes, ids_full[r * n_sel:(r + 1) * n_sel])
+            def restore_all():
+                for r in range(32):
+                    st.PagedScatterAsync(host_full.data_ptr() + r * per_req, base, sizes, ids_full[r * n_sel:(r + 1) * n_sel])
 
-        ms_d = timed(dump_all, 1)
-        ms_r = timed(restore_all, 1)
-        out["config4_full_host_roundtrip"] = {"payload_GiB": full_payload / 2**30, "pinned_buffer_GiB": full_payload / 2**30,
-                                              "dump_ms": ms_d, "dump_pcie_GBps": full_payload / ms_d / 1e6,
-                                              "restore_ms": ms_r, "restore_pcie_GBps": full_payload / ms_r / 1e6}
-        del host_full
-    except Exception as e:  # noqa: BLE001 - 32 GiB of pinned memory may not be available
-        out["config4_full_host_roundtrip"] = {"error": str(e)[:200]}
+            ms_d = timed(dump_all, 1)
+            ms_r = timed(restore_all, 1)
+            out["config4_full_host_roundtrip"] = {"payload_GiB": full_payload / 2**30, "pinned_buffer_GiB": full_payload / 2**30,
+                                                  "dump_ms": ms_d, "dump_pcie_GBps": full_payload / ms_d / 1e6,
+                                                  "restore_ms": ms_r, "restore_pcie_GBps": full_payload / ms_r / 1e6}
+            del host_full
+        except Exception as e:  # noqa: BLE001 - 32 GiB of pinned memory may not be available
+            out["config4_full_host_roundtrip"] = {"error": str(e)[:200]}
 
-    # --- the same blocks through the native cache store (task queues + pinned staging nodes):
-    #     submit -> wait, one request (64 blocks = 1 GiB) per task, as the connector's
-    #     save_speed / load_speed are measured ---
-    from ucm_amd.store import CacheStore
+        # --- the same blocks through the native cache store (task queues + pinned staging nodes):
+        #     submit -> wait, one request (64 blocks = 1 GiB) per task, as the connector's
+        #     save_speed / load_speed are measured ---
+        from ucm_amd.store import CacheStore
 
-    n_tensors = 2 * L
-    store = CacheStore({"tensor_size_list": [chunk] * n_tensors,
-                        "buffer_capacity_bytes": len(ids) * n_tensors * chunk})
-    rows = (ids.astype(np.uint64)[:, None] * sizes[None, :] + base[None, :])  # [blocks, tensors]
-    bids = [int(i).to_bytes(8, "little") * 2 for i in range(len(ids))]
-    per_task = n_sel
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    tasks = [store.dump_data(bids[i:i + per_task], [0] * per_task, rows[i:i + per_task])
-             for i in range(0, len(ids), per_task)]
-    for t in tasks:
-        store.wait(t)
-    t1 = time.perf_counter()
-    tasks = [store.load_data(bids[i:i + per_task], [0] * per_task, rows[i:i + per_task])
-             for i in range(0, len(ids), per_task)]
-    for t in tasks:
-        store.wait(t)
-    t2 = time.perf_counter()
-    out["cache_store"] = {"payload_GiB": payload / 2**30, "tasks": len(tasks),
-                          "dump_GBps": payload / (t1 - t0) / 1e9, "load_GBps": payload / (t2 - t1) / 1e9}
-    store.close()
-
-    # --- "Cache|Posix" pipeline: the same shards on to block files in a temporary directory
-    #     (page cache included: a figure of the software path, not of a disk) ---
-    import shutil
-    import tempfile
-
-    from ucm_amd.store import UcmPipelineStore
-
-    root = tempfile.mkdtemp(prefix="ucm_bench_posix_")
-    try:
-        shard = n_tensors * chunk
-        n_blk, per_task = 32, 8
-        pipe = UcmPipelineStore({"store_pipeline": "Cache|Posix", "storage_backends": [root], "device_id": 0,
-                                 "tensor_size": chunk, "shard_size": shard, "block_size": shard,
-                                 "data_dir_shard_bytes": 2, "posix_data_trans_concurrency": 16,
-                                 "buffer_capacity_bytes": 2 * per_task * shard})
-        watcher = UcmPipelineStore({"store_pipeline": "Posix", "storage_backends": [root],
-                                    "data_dir_shard_bytes": 2})
-        pbids = [(1000 + i).to_bytes(8, "little") * 2 for i in range(n_blk)]
+        n_tensors = 2 * L
+        store = CacheStore({"tensor_size_list": [chunk] * n_tensors,
+                            "buffer_capacity_bytes": len(ids) * n_tensors * chunk})
+        rows = (ids.astype(np.uint64)[:, None] * sizes[None, :] + base[None, :])  # [blocks, tensors]
+        bids = [int(i).to_bytes(8, "little") * 2 for i in range(len(ids))]
+        per_task = n_sel
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(0, n_blk, per_task):
-            pipe.wait(pipe.dump_data(pbids[i:i + per_task], [0] * per_task, rows[i:i + per_task]))
-            while watcher.lookup_on_prefix(pbids[i:i + per_task]) + 1 < per_task:  # files committed
-                time.sleep(0.0005)
+        tasks = [store.dump_data(bids[i:i + per_task], [0] * per_task, rows[i:i + per_task])
+                 for i in range(0, len(ids), per_task)]
+        for t in tasks:
+            store.wait(t)
         t1 = time.perf_counter()
-        for i in range(0, n_blk, per_task):
-            pipe.wait(pipe.load_data(pbids[i:i + per_task], [0] * per_task, rows[i:i + per_task]))
+        tasks = [store.load_data(bids[i:i + per_task], [0] * per_task, rows[i:i + per_task])
+                 for i in range(0, len(ids), per_task)]
+        for t in tasks:
+            store.wait(t)
         t2 = time.perf_counter()
-        pbytes = n_blk * shard
-        out["cache_posix_pipeline"] = {"payload_GiB": pbytes / 2**30, "dir": os.path.dirname(root),
-                                       "dump_to_files_GBps": pbytes / (t1 - t0) / 1e9,
-                                       "load_from_files_GBps": pbytes / (t2 - t1) / 1e9}
-        pipe.close()
-        watcher.close()
-    except Exception as e:  # noqa: BLE001 - a side figure must not take the headline down
-        out["cache_posix_pipeline"] = {"error": str(e)[:200]}
-    finally:
-        shutil.rmtree(root, ignore_errors=True)
+        out["cache_store"] = {"payload_GiB": payload / 2**30, "tasks": len(tasks),
+                              "dump_GBps": payload / (t1 - t0) / 1e9, "load_GBps": payload / (t2 - t1) / 1e9}
+        store.close()
+
+        # --- "Cache|Posix" pipeline: the same shards on to block files in a temporary directory
+        #     (page cache included: a figure of the software path, not of a disk) ---
+        import shutil
+        import tempfile
+
+        from ucm_amd.store import UcmPipelineStore
+
+        root = tempfile.mkdtemp(prefix="ucm_bench_posix_")
+        try:
+            shard = n_tensors * chunk
+            n_blk, per_task = 32, 8
+            pipe = UcmPipelineStore({"store_pipeline": "Cache|Posix", "storage_backends": [root], "device_id": 0,
+                                     "tensor_size": chunk, "shard_size": shard, "block_size": shard,
+                                     "data_dir_shard_bytes": 2, "posix_data_trans_concurrency": 16,
+                                     "buffer_capacity_bytes": 2 * per_task * shard})
+            watcher = UcmPipelineStore({"store_pipeline": "Posix", "storage_backends": [root],
+                                        "data_dir_shard_bytes": 2})
+            pbids = [(1000 + i).to_bytes(8, "little") * 2 for i in range(n_blk)]
+            t0 = time.perf_counter()
+            for i in range(0, n_blk, per_task):
+                pipe.wait(pipe.dump_data(pbids[i:i + per_task], [0] * per_task, rows[i:i + per_task]))
+                while watcher.lookup_on_prefix(pbids[i:i + per_task]) + 1 < per_task:  # files committed
+                    time.sleep(0.0005)
+            t1 = time.perf_counter()
+            for i in range(0, n_blk, per_task):
+                pipe.wait(pipe.load_data(pbids[i:i + per_task], [0] * per_task, rows[i:i + per_task]))
+            t2 = time.perf_counter()
+            pbytes = n_blk * shard
+            out["cache_posix_pipeline"] = {"payload_GiB": pbytes / 2**30, "dir": os.path.dirname(root),
+                                           "dump_to_files_GBps": pbytes / (t1 - t0) / 1e9,
+                                           "load_from_files_GBps": pbytes / (t2 - t1) / 1e9}
+            pipe.close()
+            watcher.close()
+        except Exception as e:  # noqa: BLE001 - a side figure must not take the headline down
+            out["cache_posix_pipeline"] = {"error": str(e)[:200]}
+        finally:
+            shutil.rmtree(root, ignore_errors=True)
     return out
 
 
@@ -794,7 +822,9 @@ def pmc_calibration(torch):
 
 
 def main():
+    global NO_GRAPH
     args = parse()
+    NO_GRAPH = args.no_graph
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no cross-GPU exchange "
               "(requests and KV heads shard without communication); run with --gpus 1",
@@ -839,6 +869,8 @@ def main():
     graphs = None
     if not args.no_graph:
         try:
+            if NO_GRAPH:
+                raise RuntimeError("graphs switched off (--no-graph)")
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -900,9 +932,10 @@ def main():
     # busy queue, 23.4 us after a 24 us gap, and 6 % of those above 25 us).  The timed region has no
     # such gaps (graph replays), so the eager steps are queued behind a kernel that keeps the GPU
     # busy while the host enqueues them, and then run back to back like the replays.
-    hold_ms = args.steps * 0.06 + 3.0
+    hold_ms = 0.0 if args.no_graph else args.steps * 0.06 + 3.0
     try:
-        torch.cuda._sleep(int(hold_ms * 1e-3 * 2.0e9))
+        if hold_ms:
+            torch.cuda._sleep(int(hold_ms * 1e-3 * 2.0e9))
     except Exception:  # noqa: BLE001 - no spin kernel in this build: fills of 1 GiB (about 0.3 ms each)
         pad = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
         for _ in range(int(hold_ms / 0.3) + 1):
@@ -973,18 +1006,24 @@ def main():
         line["cpu_baseline"] = cpu_baseline(torch, caches[0], tables[0], qc, lens)
         line["gpu_over_cpu"] = line["value"] / line["cpu_baseline"]["value"]
     if not args.skip_extras:
-        plug = plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots)
-        line["plugin_attention_begin_p50_us"] = {
-            "single_call_graph": plug["single_call"].get("graph_p50_us"),
-            "single_call_eager": plug["single_call"]["eager_p50_us"],
-            "separate_operators_graph": plug["separate_operators"].get("graph_p50_us"),
-            "separate_operators_eager": plug["separate_operators"]["eager_p50_us"]}
-        beside = gather_beside_decode(torch, gen, run_launch, GS)
+        legs = tuple(x for x in args.legs.split(",") if x)
+        plug = beside = None
+        if "plugin" in legs:
+            plug = plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots)
+            line["plugin_attention_begin_p50_us"] = {
+                "single_call_graph": plug["single_call"].get("graph_p50_us"),
+                "single_call_eager": plug["single_call"]["eager_p50_us"],
+                "separate_operators_graph": plug["separate_operators"].get("graph_p50_us"),
+                "separate_operators_eager": plug["separate_operators"]["eager_p50_us"]}
+        if "beside" in legs:
+            beside = gather_beside_decode(torch, gen, run_launch, GS)
         del caches[1:], tables[1:]
         torch.cuda.empty_cache()
-        line["extras"] = extras(torch, enc_k, gen)
-        line["extras"]["plugin_surface"] = plug
-        line["extras"]["gather_beside_decode"] = beside
+        line["extras"] = extras(torch, enc_k, gen, legs)
+        if plug is not None:
+            line["extras"]["plugin_surface"] = plug
+        if beside is not None:
+            line["extras"]["gather_beside_decode"] = beside
         if not args.skip_cpu:
             line["extras"].update(cpu_side_baselines(torch))
     print(json.dumps(line))
