@@ -28,7 +28,7 @@ TOPK_SHAPES = {
     "config3_one_long_request": (1, 32, 8, 4, 128, [70001], 128, {},
                                  "block_score_one<1,8,1,4,1>+select_group_kernel<4>"),
     "config5_two_requests": (2, 128, 1, 8, 64, [65536, 700], 128, {},
-                             "plane_kernel+block_score_lanes64<4,0,8>+select_group_kernel<4>"),
+                             "block_score_lanes64<8>+select_group_kernel<4>"),
     "plugin_reduced_physical": (2, 8, 8, 4, 128, [4096, 3000], 8,
                                 {"reduce_heads": True, "return_physical": True},
                                 "block_score_one<1,8,1,1,1>+select_wave_kernel<4>"),
@@ -99,3 +99,32 @@ def test_per_token_scorer_takes_its_kernels_and_matches_the_checker(name):
     torch.cuda.synchronize()
     ref = c_api.hamming_score(q, kc, table, lens, msl)
     assert np.array_equal(out.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("G", [3, 5, 8, 15, 16, 31, 33, 64, 100, 127, 128, 200])
+def test_planes_built_inside_the_scorer_for_every_group_size(G):
+    """64-token blocks of 8-word codes, one KV head: the scorer builds the bit planes of the G query
+    heads itself (no plane kernel).  Ragged lengths (an empty request, a length that ends inside a
+    block, runs that end inside a workgroup), table entries out of range, forced blocks."""
+    from ucm_amd import _lib
+    from ucm_amd.sparse import hamming_topk
+
+    lens = [0, 1, 63, 64, 65, 700, 1024 + 17, 5000, 16 * 64 * 3 + 1]
+    B = len(lens)
+    q, kc, table, lens = make_paged_case(77 + G, B, G, 1, 8, 64, lens)
+    rng = np.random.default_rng(G)
+    if G % 2:  # low-entropy queries: many per-bit counts of 0 and of G
+        q[:, :, :4] = q[:, :1, :4]
+        q[:, :, 4] = 0
+        q[:, :, 5] = 0xFFFFFFFF
+    table[5, 3] = -1
+    table[7, 11] = kc.shape[0] + 5
+    k = 9
+    planes = max(4, int(G).bit_length())
+    for sink, recent in ((0, 0), (64, 256)):
+        idx, sc = hamming_topk(_dev(q), _dev(kc), _dev(table), _dev(lens), k, sink, recent)
+        assert _lib.last_dispatch().startswith("block_score_lanes64<%d>+" % planes)
+        torch.cuda.synchronize()
+        oi, os_ = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, 0)
+        assert np.array_equal(sc.cpu().numpy(), os_)
+        assert np.array_equal(idx.cpu().numpy(), oi)

@@ -71,6 +71,15 @@ __device__ __forceinline__ T code_load(const T* p)
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+// popcount(x) + acc as the one instruction it is; as plain C++ the sum of many popcounts is
+// re-associated into a tree with extra adds.
+__device__ __forceinline__ int popc_add(uint32_t x, int acc)
+{
+    int r;
+    asm("v_bcnt_u32_b32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(acc));
+    return r;
+}
+
 __device__ __forceinline__ int popc4(u32x4 v)
 {
     return __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
@@ -394,11 +403,20 @@ __global__ __launch_bounds__(kThreads) void block_score_one(ScoreArgs a)
             for (int u = 0; u < 4; ++u) {
                 int d;
                 if (DIRECT) {
-                    d = 0;
+                    // one accumulating popcount per word, chained: left to itself the compiler
+                    // splits the sum into several chains and joins them with three-input adds
+                    // (28 of 245 vector instructions per wave at four query heads)
+                    d = __popc(kv[u].x ^ qr[0][0]);
+                    d = popc_add(kv[u].y ^ qr[0][1], d);
+                    d = popc_add(kv[u].z ^ qr[0][2], d);
+                    d = popc_add(kv[u].w ^ qr[0][3], d);
 #pragma unroll
-                    for (int g = 0; g < GP; ++g)
-                        d += __popc(kv[u].x ^ qr[g][0]) + __popc(kv[u].y ^ qr[g][1]) +
-                             __popc(kv[u].z ^ qr[g][2]) + __popc(kv[u].w ^ qr[g][3]);
+                    for (int g = 1; g < GP; ++g) {
+                        d = popc_add(kv[u].x ^ qr[g][0], d);
+                        d = popc_add(kv[u].y ^ qr[g][1], d);
+                        d = popc_add(kv[u].z ^ qr[g][2], d);
+                        d = popc_add(kv[u].w ^ qr[g][3], d);
+                    }
                 } else {
                     int acc = 0;
 #pragma unroll
@@ -1054,107 +1072,220 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     }
 }
 
-// The same walk for 64-token blocks (one round per block), several blocks per wave: with one
-// block per wave a wave's whole life is three dependent round trips to memory (table entry,
-// codes, and the bit planes behind a barrier) around some 250 instructions, and the counters show
-// it (16 x 65,536 tokens of 256-bit codes, 128 query heads: vector ALU busy 11 % of a wave's
-// resident cycles, 82 % spent waiting).  Here a wave owns kLaneRun consecutive logical blocks:
-// their table entries arrive in one load, the codes of all of them are requested together (the
-// whole problem is a few tens of MB: everything should be in flight at once), the planes are
-// staged once per 4 * kLaneRun blocks, and the run's scores leave in one store.
+// 64-token blocks of 8-word codes against one KV head whose G query heads enter as bit planes
+// (16 requests x 65,536 tokens, 128 query heads: 33 MB of codes, 4096 waves).  With one block per
+// wave a wave's life is three dependent round trips to memory around some 250 instructions, and a
+// separate launch builds the planes first.  Here
+//  * a wave owns kLaneRun consecutive blocks: their table entries arrive in one load and all of
+//    their codes are requested at once, a whole code per lane (two 16-byte loads at a lane stride of
+//    32 bytes: no transpose through LDS);
+//  * while those loads are in flight, wave 0 of the workgroup builds the request's bit planes from
+//    the query codes: lane (w, g) counts bit-sliced over up to 16 heads with a carry-save adder
+//    tree (11 full + 4 half adders for 16 words), three bit-sliced additions across the lane
+//    groups finish the counts, and the planes of word w go to LDS.  No plane kernel runs;
+//  * after one barrier every wave keeps the planes in registers (GP * 8 of them) for its blocks;
+//  * the minima of the run's blocks are reduced together (the first two butterfly steps halve the
+//    number of values per lane) and leave in one store.
 constexpr int kLaneRun = 4;
 
-template <int LC, bool DIRECT, int GP>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void block_score_lanes64(ScoreArgs a)
+__device__ __forceinline__ void full_add(uint32_t x, uint32_t y, uint32_t z, uint32_t& sum, uint32_t& carry)
 {
-    using LCd = LaneCode<LC, DIRECT, GP>;
-    constexpr int WD = LCd::WD;
-    __shared__ __align__(16) uint32_t strip[kThreads / kWave][LCd::kRoundWords];
-    __shared__ __align__(16) uint32_t pl[DIRECT ? 8 : WD * 8];
-    __shared__ int ctot[LC];
+    const uint32_t t = x ^ y;
+    sum = t ^ z;
+    carry = (t & z) | (~t & x);  // majority(x, y, z)
+}
+__device__ __forceinline__ void half_add(uint32_t x, uint32_t y, uint32_t& sum, uint32_t& carry)
+{
+    sum = x ^ y;
+    carry = x & y;
+}
+
+// Bit-sliced count of 16 words: n[p] bit i = bit p of the number of words with bit i set.
+__device__ __forceinline__ void count16(const uint32_t (&x)[16], uint32_t (&n)[5])
+{
+    uint32_t s[6], c1[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) full_add(x[3 * i], x[3 * i + 1], x[3 * i + 2], s[i], c1[i]);
+    s[5] = x[15];
+    // weight 1: six sums
+    uint32_t a0, a1, k0, k1, k2;
+    full_add(s[0], s[1], s[2], a0, k0);
+    full_add(s[3], s[4], s[5], a1, k1);
+    half_add(a0, a1, n[0], k2);
+    // weight 2: c1[0..4], k0, k1, k2
+    uint32_t b0, b1, m0, m1, m2, m3;
+    full_add(c1[0], c1[1], c1[2], b0, m0);
+    full_add(c1[3], c1[4], k0, b1, m1);
+    uint32_t b2;
+    full_add(b0, b1, k1, b2, m2);
+    half_add(b2, k2, n[1], m3);
+    // weight 4: m0..m3
+    uint32_t d0, e0, e1;
+    full_add(m0, m1, m2, d0, e0);
+    half_add(d0, m3, n[2], e1);
+    // weight 8: e0, e1
+    half_add(e0, e1, n[3], n[4]);
+}
+
+template <int GP>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void block_score_lanes64(ScoreArgs a)
+{
+    constexpr int WD = 8;
+    __shared__ __align__(16) uint32_t pl[WD * 8];  // pl[w * 8 + p]
+    __shared__ int base_s;
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
     const int j0 = (blockIdx.x * (kThreads / kWave) + wid) * kLaneRun;
-    const int len = a.lens[b];
-    // the run's table entries: lane i holds block j0 + i
+    // the run's table entries: lane i holds block j0 + i (requested before the length is looked at)
     int my_entry = 0;
     {
         const int j = j0 + (lane < kLaneRun ? lane : 0);
         const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
-        if (a.table) my_entry = a.table[(int64_t)b * a.table_stride + (jc < 0 ? 0 : jc)];
+        if (a.table) my_entry = a.table[(int64_t)b * a.table_stride + jc];
         else my_entry = b * a.max_blocks + jc;
     }
-    LCd::stage_planes(a, b, pl, ctot);
-    if (!DIRECT) __syncthreads();
+    const int len = a.lens[b];
     int nblk = len > 0 ? (len + 63) >> 6 : 0;
     if (nblk > a.max_blocks) nblk = a.max_blocks;
-    if (j0 >= nblk) return;
-    const int run = (nblk - j0 < kLaneRun) ? nblk - j0 : kLaneRun;
-    u32x4* mine = reinterpret_cast<u32x4*>(strip[wid]);
-    const uint32_t* row = strip[wid] + lane * WD;
-    const uint32_t* qp = a.q + b * a.q_stride_b;
-    int base = 0;
-    if (!DIRECT) {
+    if ((int)blockIdx.x * (kThreads / kWave) * kLaneRun >= nblk) return;  // the whole workgroup
+    const int run = nblk - j0 < kLaneRun ? nblk - j0 : kLaneRun;  // <= 0: nothing to score
+    // a whole code per lane; blocks past the run re-read its first block (never used)
+    u32x4 v[kLaneRun][2];
+    auto request_codes = [&]() {
 #pragma unroll
-        for (int i = 0; i < LC; ++i) base += ctot[i];
-    }
-    auto block_src = [&](int i) -> const u32x4* {
-        int64_t pb = __shfl(my_entry, i);
-        if (pb < 0 || pb >= a.NB) pb = 0;  // scored as -1 below
-        return reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block);
+        for (int i = 0; i < kLaneRun; ++i) {
+            int64_t pb = __shfl(my_entry, (run > 0 && i < run) ? i : 0);
+            if (pb < 0 || pb >= a.NB) pb = 0;  // scored as -1 below
+            const u32x4* src = reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + 2 * lane;
+            v[i][0] = code_load(src);
+            v[i][1] = code_load(src + 1);
+        }
     };
-    // the codes of the whole run are requested at once (blocks past the run re-read its first)
-    u32x4 v[kLaneRun][LCd::kLoads];
+    if (wid != 0) {
+        request_codes();
+    } else {
+        // lane (w = lane & 7, g = lane >> 3) takes word w of heads g, g + 8, g + 16, ...; the query
+        // words are requested before the codes, so that waiting for them leaves the codes in flight
+        const int w = lane & 7, g = lane >> 3;
+        const uint32_t* qb = a.q + b * a.q_stride_b + w;
+        const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
+        uint32_t acc[8];
 #pragma unroll
-    for (int i = 0; i < kLaneRun; ++i) LCd::load_round(block_src(i < run ? i : 0), 0, lane, v[i]);
-    int result = 0;  // lane i: score of block j0 + i
-    const int full = a.G * 32 * a.Wd;
+        for (int p = 0; p < 8; ++p) acc[p] = 0;
+        // 128 heads at a time; the first round is straight-line code with the code loads in its
+        // middle, so that the waits for the query words are counted exactly and leave the codes
+        // in flight (a load under a condition makes every later wait cover it)
+        auto add_heads = [&](int h0, bool first) __attribute__((always_inline)) {
+            uint32_t x[16], n[5];
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int h = h0 + t * 8 + g;  // heads past the group re-read the last one, as zero
+                x[t] = qb[(h < a.G ? h : a.G - 1) * qs];
+            }
+            if (first) request_codes();
+#pragma unroll
+            for (int t = 0; t < 16; ++t) x[t] = (h0 + t * 8 + g < a.G) ? x[t] : 0u;
+            count16(x, n);
+            uint32_t cy = 0;
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                uint32_t sum, c2;
+                if (p < 5) full_add(acc[p], n[p], cy, sum, c2);
+                else half_add(acc[p], cy, sum, c2);
+                acc[p] = sum;
+                cy = c2;
+            }
+        };
+        add_heads(0, true);
+        for (int h0 = 128; h0 < a.G; h0 += 128) add_heads(h0, false);
+        // the eight lane groups add up (every lane ends with the full counts of its word)
+#pragma unroll
+        for (int st = 8; st < kWave; st <<= 1) {
+            uint32_t o[8], cy = 0;
+#pragma unroll
+            for (int p = 0; p < 8; ++p) o[p] = __shfl_xor(acc[p], st);
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                uint32_t sum, c2;
+                full_add(acc[p], o[p], cy, sum, c2);
+                acc[p] = sum;
+                cy = c2;
+            }
+        }
+        int c = 0;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) c += __popc(acc[p]) << p;
+        c += __shfl_xor(c, 1);
+        c += __shfl_xor(c, 2);
+        c += __shfl_xor(c, 4);
+        if (lane < 8) {
+            u32x4* dst = reinterpret_cast<u32x4*>(pl + lane * 8);
+            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
+            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
+        }
+        if (lane == 0) base_s = c;  // sum over all code bits of the per-bit counts
+    }
+    __syncthreads();
+    if (run <= 0) return;
+    const int base = base_s;
+    uint32_t P[WD][GP];
+#pragma unroll
+    for (int w = 0; w < WD; ++w) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(pl + w * 8);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(pl + w * 8 + 4);
+#pragma unroll
+        for (int p = 0; p < GP; ++p) P[w][p] = p < 4 ? lo[p] : hi[p - 4];
+    }
+    int d[kLaneRun];
 #pragma unroll
     for (int i = 0; i < kLaneRun; ++i) {
-        if (i >= run) break;
-        LCd::store_round(mine, lane, v[i]);
-        asm volatile("" ::: "memory");  // the planes are re-read from LDS for every block
-        int d = 0;
-        if (DIRECT) {
+        int acc[GP], pk = 0;
 #pragma unroll
-            for (int w = 0; w < LC; ++w) {
-                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * w);
+        for (int p = 0; p < GP; ++p) acc[p] = 0;
 #pragma unroll
-                for (int g = 0; g < GP; ++g)
-                    d += __popc(k.x ^ qp[g * a.q_stride_h + 2 * w]) + __popc(k.y ^ qp[g * a.q_stride_h + 2 * w + 1]);
-            }
-        } else {
-            int acc[GP], pk = 0;
+        for (int w = 0; w < WD; ++w) {
+            const uint32_t k = v[i][w >> 2][w & 3];
+            pk += __popc(k);
 #pragma unroll
-            for (int p = 0; p < GP; ++p) acc[p] = 0;
-#pragma unroll
-            for (int w = 0; w < LC; ++w) {
-                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * w);
-                pk += __popc(k.x) + __popc(k.y);
-#pragma unroll
-                for (int p = 0; p < GP; ++p)
-                    acc[p] += __popc(k.x & pl[(2 * w) * 8 + p]) + __popc(k.y & pl[(2 * w + 1) * 8 + p]);
-            }
-            int x = 0;
-#pragma unroll
-            for (int p = 0; p < GP; ++p) x += acc[p] << p;
-            d = base + a.G * pk - 2 * x;
+            for (int p = 0; p < GP; ++p) acc[p] += __popc(k & P[w][p]);
         }
-        asm volatile("" ::: "memory");  // the strip is rewritten by the next block
+        int x = 0;
+#pragma unroll
+        for (int p = 0; p < GP; ++p) x += acc[p] << p;
         const int pos0 = (j0 + i) << 6;
-        const int ntok = (64 < len - pos0) ? 64 : len - pos0;
-        int m = lane < ntok ? d : kInf;
-#pragma unroll
-        for (int st = 1; st < kWave; st <<= 1) {
-            const int o = __shfl_xor(m, st);
-            m = o < m ? o : m;
-        }
-        const int entry = __shfl(my_entry, i);
-        const bool forced = (pos0 < a.sink) || (pos0 + ntok > len - a.recent);
-        const int sc = (entry < 0 || entry >= a.NB) ? -1 : (forced ? full : full - m);
-        if (lane == i) result = sc;
+        d[i] = (i < run && pos0 + lane < len) ? base + a.G * pk - 2 * x : kInf;
     }
-    if (lane < run) a.scores[(int64_t)b * a.max_blocks + j0 + lane] = result;
+    // minima of the four blocks together: after the steps over lane bits 0 and 1 a lane holds one
+    // value, that of block 2 * (lane & 1) + ((lane >> 1) & 1)
+    static_assert(kLaneRun == 4, "the reduction below is written for runs of four blocks");
+    const bool odd = lane & 1, up = lane & 2;
+    int ka = odd ? d[2] : d[0], kb = odd ? d[3] : d[1];
+    {
+        const int oa = __shfl_xor(odd ? d[0] : d[2], 1), ob = __shfl_xor(odd ? d[1] : d[3], 1);
+        ka = oa < ka ? oa : ka;
+        kb = ob < kb ? ob : kb;
+    }
+    int m = up ? kb : ka;
+    {
+        const int o = __shfl_xor(up ? ka : kb, 2);
+        m = o < m ? o : m;
+    }
+#pragma unroll
+    for (int st = 4; st < kWave; st <<= 1) {
+        const int o = __shfl_xor(m, st);
+        m = o < m ? o : m;
+    }
+    const int i = 2 * (lane & 1) + ((lane >> 1) & 1);
+    const int entry = __shfl(my_entry, i);
+    if (lane < 4) {
+        if (i < run) {
+            const int pos0 = (j0 + i) << 6;
+            const int ntok = (64 < len - pos0) ? 64 : len - pos0;
+            const bool forced = (pos0 < a.sink) || (pos0 + ntok > len - a.recent);
+            const int full = a.G * 32 * a.Wd;
+            a.scores[(int64_t)b * a.max_blocks + j0 + i] = (entry < 0 || entry >= a.NB) ? -1 : (forced ? full : full - m);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -2041,21 +2172,6 @@ template <int LC>
 void dispatch_lanes(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
     const bool dir = LC == 9 && (a.G == 1 || a.G == 2 || a.G == 4);
-    // 64-token blocks of 8-word codes: runs of kLaneRun blocks per wave (wider codes hold too
-    // many registers for the run's loads: 18 words measured 21.9 against 18.4 us)
-    if (a.BS == 64 && LC == 4) {
-        note_score("block_score_lanes64", LC, dir, dir ? a.G : (pmax < 4 ? 4 : (pmax > 8 ? 8 : pmax)));
-        const dim3 g64((unsigned)ucm::ceil_div(a.max_blocks, (kThreads / kWave) * kLaneRun), grid.y);
-        if (LC == 9 && a.G == 1) launch_score(block_score_lanes64<9, true, 1>, g64, 0, st, a);
-        else if (LC == 9 && a.G == 2) launch_score(block_score_lanes64<9, true, 2>, g64, 0, st, a);
-        else if (LC == 9 && a.G == 4) launch_score(block_score_lanes64<9, true, 4>, g64, 0, st, a);
-        else if (pmax == 4) launch_score(block_score_lanes64<LC, false, 4>, g64, 0, st, a);
-        else if (pmax == 5) launch_score(block_score_lanes64<LC, false, 5>, g64, 0, st, a);
-        else if (pmax == 6) launch_score(block_score_lanes64<LC, false, 6>, g64, 0, st, a);
-        else if (pmax == 7) launch_score(block_score_lanes64<LC, false, 7>, g64, 0, st, a);
-        else launch_score(block_score_lanes64<LC, false, 8>, g64, 0, st, a);
-        return;
-    }
     note_score("block_score_lanes", LC, dir, dir ? a.G : (pmax < 4 ? 4 : (pmax > 8 ? 8 : pmax)));
     if (LC == 9 && a.G == 1) launch_score(block_score_lanes<9, true, 1>, grid, 0, st, a);
     else if (LC == 9 && a.G == 2) launch_score(block_score_lanes<9, true, 2>, grid, 0, st, a);
@@ -2258,7 +2374,9 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         while ((1 << pmax) <= a.G) ++pmax;  // bit planes that hold the counts 0..G
         if (pmax < 4) pmax = 4;
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
-        if (!direct) {
+        // 64-token blocks of 8-word codes: the scorer builds the planes itself
+        const bool planes_inside = !direct && Wd == 8 && BS == 64 && pmax <= 8 && lanes_layout(a, k_cache, direct);
+        if (!direct && !planes_inside) {
             g_note.planes = "plane_kernel";
             hipLaunchKernelGGL(plane_kernel, dim3(B * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
                                q_stride_b, q_stride_h, 1, a.G, Wd, pmax, ws.planes);
@@ -2268,7 +2386,17 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         const dim3 pgrid((unsigned)ucm::ceil_div(max_blocks, kThreads / kWave), (unsigned)B);
         // 18-word codes (and 8- or 16-word codes with bit planes) in blocks of 64, 128, ...
         // tokens: a whole code per lane
-        if (lanes_layout(a, k_cache, direct)) {
+        if (planes_inside) {
+            note_score("block_score_lanes64", pmax);
+            const dim3 g64((unsigned)ucm::ceil_div(max_blocks, (kThreads / kWave) * kLaneRun), (unsigned)B);
+            switch (pmax) {
+                case 4: launch_score(block_score_lanes64<4>, g64, 0, st, a); break;
+                case 5: launch_score(block_score_lanes64<5>, g64, 0, st, a); break;
+                case 6: launch_score(block_score_lanes64<6>, g64, 0, st, a); break;
+                case 7: launch_score(block_score_lanes64<7>, g64, 0, st, a); break;
+                default: launch_score(block_score_lanes64<8>, g64, 0, st, a); break;
+            }
+        } else if (lanes_layout(a, k_cache, direct)) {
             if (Wd == 18) dispatch_lanes<9>(a, pmax, pgrid, st);
             else if (Wd == 16) dispatch_lanes<8>(a, pmax, pgrid, st);
             else dispatch_lanes<4>(a, pmax, pgrid, st);
