@@ -47,7 +47,7 @@ TOPK_SHAPES = {
                                         "plane_kernel+block_score_pairs<0,5>+select_wave_kernel<4>"),
     "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], 8, {}, "block_score_lanes<9,1,1>+select_wave_kernel<4>"),
     "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], 8, {},
-                                       "plane_kernel+block_score_lanes<9,0,7>+select_wave_kernel<4>"),
+                                       "block_score_lanes_run<9,7>+select_wave_kernel<4>"),
     "config5_blocks_of_128": (2, 128, 1, 8, 128, [8192, 700], 8, {},
                               "plane_kernel+block_score_lanes<4,0,8>+select_wave_kernel<4>"),
     "odd_code_width": (2, 6, 2, 3, 16, [1024, 300], 8, {}, "block_score_generic+select_wave_kernel<4>"),
@@ -101,18 +101,19 @@ def test_per_token_scorer_takes_its_kernels_and_matches_the_checker(name):
     assert np.array_equal(out.cpu().numpy(), ref)
 
 
-@pytest.mark.parametrize("G", [3, 5, 8, 15, 16, 31, 33, 64, 100, 127, 128, 200])
-def test_planes_built_inside_the_scorer_for_every_group_size(G):
-    """64-token blocks of 8-word codes, one KV head: the scorer builds the bit planes of the G query
-    heads itself (no plane kernel).  Ragged lengths (an empty request, a length that ends inside a
-    block, runs that end inside a workgroup), table entries out of range, forced blocks."""
+@pytest.mark.parametrize("Wd,BS", [(8, 64), (18, 64), (16, 64), (8, 128), (18, 128)])
+@pytest.mark.parametrize("G", [3, 5, 8, 15, 16, 31, 33, 48, 49, 64, 100, 127, 128, 200])
+def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
+    """One KV head, a whole code per lane: the scorer builds the bit planes of the G query heads
+    itself (no plane kernel) when the blocks hold 64 tokens - for every G with 8-word codes, up to
+    128 heads with 16- and 18-word codes; larger blocks keep the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
+    that end inside a workgroup), table entries out of range, forced blocks."""
     from ucm_amd import _lib
     from ucm_amd.sparse import hamming_topk
 
     lens = [0, 1, 63, 64, 65, 700, 1024 + 17, 5000, 16 * 64 * 3 + 1]
     B = len(lens)
-    q, kc, table, lens = make_paged_case(77 + G, B, G, 1, 8, 64, lens)
-    rng = np.random.default_rng(G)
+    q, kc, table, lens = make_paged_case(77 + G + Wd, B, G, 1, Wd, BS, lens)
     if G % 2:  # low-entropy queries: many per-bit counts of 0 and of G
         q[:, :, :4] = q[:, :1, :4]
         q[:, :, 4] = 0
@@ -123,7 +124,13 @@ def test_planes_built_inside_the_scorer_for_every_group_size(G):
     planes = max(4, int(G).bit_length())
     for sink, recent in ((0, 0), (64, 256)):
         idx, sc = hamming_topk(_dev(q), _dev(kc), _dev(table), _dev(lens), k, sink, recent)
-        assert _lib.last_dispatch().startswith("block_score_lanes64<%d>+" % planes)
+        got = _lib.last_dispatch()
+        if (Wd, BS) == (8, 64):
+            assert got.startswith("block_score_lanes64<%d>+" % planes)
+        elif BS == 64 and G <= 128:
+            assert got.startswith("block_score_lanes_run<%d,%d>+" % (Wd // 2, planes))
+        else:
+            assert got.startswith("plane_kernel+block_score_lanes<%d,0,%d>+" % (Wd // 2, min(planes, 8)))
         torch.cuda.synchronize()
         oi, os_ = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, 0)
         assert np.array_equal(sc.cpu().numpy(), os_)

@@ -549,8 +549,7 @@ __global__ __launch_bounds__(kThreads) void block_score_small(ScoreArgs a)
                     d = 0;
 #pragma unroll
                     for (int g = 0; g < GP; ++g)
-                        d += __popc(k4.x ^ qr[g][0]) + __popc(k4.y ^ qr[g][1]) +
-                             __popc(k4.z ^ qr[g][2]) + __popc(k4.w ^ qr[g][3]);
+                        d = popc_add(k4.w ^ qr[g][3], popc_add(k4.z ^ qr[g][2], popc_add(k4.y ^ qr[g][1], popc_add(k4.x ^ qr[g][0], d))));
                 } else {
                     int acc = 0;
 #pragma unroll
@@ -660,8 +659,7 @@ __global__ __launch_bounds__(kThreads) void block_score_rows(ScoreArgs a)
             int d = 0;
 #pragma unroll
             for (int g = 0; g < GP; ++g)
-                d += __popc(k4.x ^ qr[g][0]) + __popc(k4.y ^ qr[g][1]) + __popc(k4.z ^ qr[g][2]) +
-                     __popc(k4.w ^ qr[g][3]);
+                d = popc_add(k4.w ^ qr[g][3], popc_add(k4.z ^ qr[g][2], popc_add(k4.y ^ qr[g][1], popc_add(k4.x ^ qr[g][0], d))));
             if (CPU >= 2) d += __shfl_xor(d, 1);
             if (CPU >= 4) d += __shfl_xor(d, 2);
             const int t = ((r << 6) + lane) / PERIOD;
@@ -751,8 +749,7 @@ __global__ __launch_bounds__(kThreads) void block_score_tiny(ScoreArgs a, int bp
         int d = 0;
 #pragma unroll
         for (int g = 0; g < GP; ++g)
-            d += __popc(kv[u].x ^ qr[g][0]) + __popc(kv[u].y ^ qr[g][1]) + __popc(kv[u].z ^ qr[g][2]) +
-                 __popc(kv[u].w ^ qr[g][3]);
+            d = popc_add(kv[u].w ^ qr[g][3], popc_add(kv[u].z ^ qr[g][2], popc_add(kv[u].y ^ qr[g][1], popc_add(kv[u].x ^ qr[g][0], d))));
         if (CPU >= 2) d += __shfl_xor(d, 1);
         if (CPU >= 4) d += __shfl_xor(d, 2);
         int m = (pos0 + (lb >> pshift) < len) ? d : kInf;
@@ -936,6 +933,46 @@ __global__ __launch_bounds__(kThreads) void block_score_pairs(ScoreArgs a, int L
 // piece-per-lane kernels; the bit planes are the same for all lanes and are read from LDS as
 // broadcasts (padded to 8 words per code word).
 // ---------------------------------------------------------------------------------------
+// Bit-sliced adders: every bit position of a word is a counter of its own.
+__device__ __forceinline__ void full_add(uint32_t x, uint32_t y, uint32_t z, uint32_t& sum, uint32_t& carry)
+{
+    const uint32_t t = x ^ y;
+    sum = t ^ z;
+    carry = (t & z) | (~t & x);  // majority(x, y, z)
+}
+__device__ __forceinline__ void half_add(uint32_t x, uint32_t y, uint32_t& sum, uint32_t& carry)
+{
+    sum = x ^ y;
+    carry = x & y;
+}
+
+// Bit-sliced count of 16 words: n[p] bit i = bit p of the number of words with bit i set.
+__device__ __forceinline__ void count16(const uint32_t (&x)[16], uint32_t (&n)[5])
+{
+    uint32_t s[6], c1[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) full_add(x[3 * i], x[3 * i + 1], x[3 * i + 2], s[i], c1[i]);
+    s[5] = x[15];
+    // weight 1: six sums
+    uint32_t a0, a1, k0, k1, k2;
+    full_add(s[0], s[1], s[2], a0, k0);
+    full_add(s[3], s[4], s[5], a1, k1);
+    half_add(a0, a1, n[0], k2);
+    // weight 2: c1[0..4], k0, k1, k2
+    uint32_t b0, b1, m0, m1, m2, m3;
+    full_add(c1[0], c1[1], c1[2], b0, m0);
+    full_add(c1[3], c1[4], k0, b1, m1);
+    uint32_t b2;
+    full_add(b0, b1, k1, b2, m2);
+    half_add(b2, k2, n[1], m3);
+    // weight 4: m0..m3
+    uint32_t d0, e0, e1;
+    full_add(m0, m1, m2, d0, e0);
+    half_add(d0, m3, n[2], e1);
+    // weight 8: e0, e1
+    half_add(e0, e1, n[3], n[4]);
+}
+
 template <int LC, bool DIRECT, int GP>
 struct LaneCode {
     static constexpr int WD = 2 * LC;
@@ -1035,8 +1072,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
                 const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
 #pragma unroll
                 for (int g = 0; g < GP; ++g)
-                    d += __popc(k.x ^ qp[g * a.q_stride_h + 2 * i]) +
-                         __popc(k.y ^ qp[g * a.q_stride_h + 2 * i + 1]);
+                    d = popc_add(k.y ^ qp[g * a.q_stride_h + 2 * i + 1], popc_add(k.x ^ qp[g * a.q_stride_h + 2 * i], d));
             }
         } else {
             int acc[GP], pk = 0;
@@ -1045,10 +1081,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
 #pragma unroll
             for (int i = 0; i < LC; ++i) {
                 const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
-                pk += __popc(k.x) + __popc(k.y);
+                pk = popc_add(k.y, popc_add(k.x, pk));
+                // the 8 plane slots of a code word as two 16-byte broadcast reads
+                const u32x4* pw = reinterpret_cast<const u32x4*>(pl + (2 * i) * 8);
+                const u32x4 x0 = pw[0], x1 = pw[1], y0 = pw[2], y1 = pw[3];
 #pragma unroll
                 for (int p = 0; p < GP; ++p)
-                    acc[p] += __popc(k.x & pl[(2 * i) * 8 + p]) + __popc(k.y & pl[(2 * i + 1) * 8 + p]);
+                    acc[p] = popc_add(k.y & (p < 4 ? y0[p & 3] : y1[p & 3]), popc_add(k.x & (p < 4 ? x0[p & 3] : x1[p & 3]), acc[p]));
             }
             int x = 0;
 #pragma unroll
@@ -1072,6 +1111,180 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     }
 }
 
+// 64-token blocks of 16- or 18-word codes with bit planes: block_score_lanes' walk (a round of 64
+// tokens through the wave's LDS strip, planes re-read from LDS) over a run of kLaneRun consecutive
+// blocks per wave - the next block's codes are requested before the current one is computed - with
+// the planes built by wave 0 of the workgroup while the first codes are in flight (up to 128 query
+// heads): lane (w = lane % WD, g = lane / WD) counts, bit-sliced, word w of heads g, g + NG, ...
+// 16 at a time, the NG lane groups meet in LDS.  No plane kernel runs.  (One block per wave with
+// the planes built per workgroup was slower than the separate plane kernel: 22.7 against 16.1 +
+// 4.4 us at 16 x 65,536 tokens; a run of four blocks shares one build between 16 blocks: 18.6 us;
+// runs of two or eight blocks: 19.7 / 20.0 us.)
+constexpr int kLaneRun = 4;         // block_score_lanes64
+constexpr int kLanesRunBlocks = 4;  // block_score_lanes_run
+
+template <int LC, int GP>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void block_score_lanes_run(ScoreArgs a)
+{
+    using LCd = LaneCode<LC, false, GP>;
+    constexpr int kRun = kLanesRunBlocks;
+    constexpr int WD = LCd::WD;
+    constexpr int NG = kWave / WD;                        // lane groups (3 for 18 words)
+    constexpr int NCH = (128 + 16 * NG - 1) / (16 * NG);  // rounds of 16 heads per lane
+    __shared__ __align__(16) uint32_t strip[kThreads / kWave][LCd::kRoundWords];
+    __shared__ __align__(16) uint32_t pl[WD * 8];
+    __shared__ __align__(16) uint32_t ptmp[(NG - 1) * WD * 8];
+    const int b = blockIdx.y;
+    const int lane = lane_id(), wid = wave_id();
+    const int j0 = (blockIdx.x * (kThreads / kWave) + wid) * kRun;
+    // the run's table entries: lane i holds block j0 + i
+    int my_entry = 0;
+    {
+        const int j = j0 + (lane < kRun ? lane : 0);
+        const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+        if (a.table) my_entry = a.table[(int64_t)b * a.table_stride + jc];
+        else my_entry = b * a.max_blocks + jc;
+    }
+    const bool builder = wid == 0;
+    const int pw = lane % WD, pg = lane / WD;
+    uint32_t qx[NCH][16];
+    if (builder) {
+        const uint32_t* qb = a.q + b * a.q_stride_b + pw;
+        const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (c * 16 * NG < a.G) {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) {
+                    const int h = (c * 16 + t) * NG + pg;  // heads past the group re-read the last one
+                    qx[c][t] = qb[(h < a.G ? h : a.G - 1) * qs];
+                }
+            }
+        }
+    }
+    const int len = a.lens[b];
+    int nblk = len > 0 ? (len + 63) >> 6 : 0;
+    if (nblk > a.max_blocks) nblk = a.max_blocks;
+    if ((int)blockIdx.x * (kThreads / kWave) * kRun >= nblk) return;  // the whole workgroup
+    const int run = nblk - j0 < kRun ? nblk - j0 : kRun;  // <= 0: nothing to score
+    auto block_src = [&](int i) -> const u32x4* {
+        int64_t pb = __shfl(my_entry, i);
+        if (pb < 0 || pb >= a.NB) pb = 0;  // scored as -1 below
+        return reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block);
+    };
+    u32x4* mine = reinterpret_cast<u32x4*>(strip[wid]);
+    const uint32_t* row = strip[wid] + lane * WD;
+    // the first block's codes go out before anything waits for the planes
+    u32x4 cur[LCd::kLoads], nxt[LCd::kLoads];
+    LCd::load_round(block_src(0), 0, lane, cur);
+#pragma unroll
+    for (int u = 0; u < LCd::kLoads; ++u) nxt[u] = cur[u];
+    if (builder) {
+        uint32_t acc[8];
+#pragma unroll
+        for (int p = 0; p < 8; ++p) acc[p] = 0;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (c * 16 * NG < a.G) {
+                uint32_t n[5], cy = 0;
+#pragma unroll
+                for (int t = 0; t < 16; ++t)
+                    qx[c][t] = ((c * 16 + t) * NG + pg < a.G && pg < NG) ? qx[c][t] : 0u;
+                count16(qx[c], n);
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    uint32_t sum, c2;
+                    if (p < 5) full_add(acc[p], n[p], cy, sum, c2);
+                    else half_add(acc[p], cy, sum, c2);
+                    acc[p] = sum;
+                    cy = c2;
+                }
+            }
+        }
+        if (pg > 0 && pg < NG) {
+            u32x4* dst = reinterpret_cast<u32x4*>(ptmp + ((pg - 1) * WD + pw) * 8);
+            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
+            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
+        }
+        // the same wave reads what it has just written: LDS operations of a wave complete in order
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (pg == 0) {
+#pragma unroll
+            for (int g = 1; g < NG; ++g) {
+                const u32x4* o4 = reinterpret_cast<const u32x4*>(ptmp + ((g - 1) * WD + pw) * 8);
+                const u32x4 lo = o4[0], hi = o4[1];
+                uint32_t cy = 0;
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    uint32_t sum, c2;
+                    full_add(acc[p], p < 4 ? lo[p & 3] : hi[p & 3], cy, sum, c2);
+                    acc[p] = sum;
+                    cy = c2;
+                }
+            }
+            u32x4* dst = reinterpret_cast<u32x4*>(pl + pw * 8);
+            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
+            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
+        }
+    }
+    __syncthreads();
+    if (run <= 0) return;
+    // sum over all code bits of the per-bit counts, from the planes in LDS
+    int base = 0;
+    {
+        int c = 0;
+        if (lane < WD) {
+            const u32x4* w4 = reinterpret_cast<const u32x4*>(pl + lane * 8);
+            const u32x4 lo = w4[0], hi = w4[1];
+#pragma unroll
+            for (int p = 0; p < 8; ++p) c += __popc(p < 4 ? lo[p & 3] : hi[p & 3]) << p;
+        }
+#pragma unroll
+        for (int st = 1; st < 32; st <<= 1) c += __shfl_xor(c, st);
+        base = __builtin_amdgcn_readfirstlane(c);
+    }
+    const int full = a.G * 32 * a.Wd;
+    int result = 0;  // lane i: score of block j0 + i
+    for (int r = 0; r < run; ++r) {
+        if (r + 1 < run) LCd::load_round(block_src(r + 1), 0, lane, nxt);
+        LCd::store_round(mine, lane, cur);
+        asm volatile("" ::: "memory");  // the planes are re-read from LDS for every block
+        int acc[GP], pk = 0;
+#pragma unroll
+        for (int p = 0; p < GP; ++p) acc[p] = 0;
+#pragma unroll
+        for (int i = 0; i < LC; ++i) {
+            const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
+            pk = popc_add(k.y, popc_add(k.x, pk));
+            const u32x4* pw4 = reinterpret_cast<const u32x4*>(pl + (2 * i) * 8);
+            const u32x4 x0 = pw4[0], x1 = pw4[1], y0 = pw4[2], y1 = pw4[3];
+#pragma unroll
+            for (int p = 0; p < GP; ++p)
+                acc[p] = popc_add(k.y & (p < 4 ? y0[p & 3] : y1[p & 3]), popc_add(k.x & (p < 4 ? x0[p & 3] : x1[p & 3]), acc[p]));
+        }
+        asm volatile("" ::: "memory");  // the strip is rewritten by the next block
+        int x = 0;
+#pragma unroll
+        for (int p = 0; p < GP; ++p) x += acc[p] << p;
+        const int d = base + a.G * pk - 2 * x;
+        const int pos0 = (j0 + r) << 6;
+        const int ntok = (64 < len - pos0) ? 64 : len - pos0;
+        int m = lane < ntok ? d : kInf;
+#pragma unroll
+        for (int st = 1; st < kWave; st <<= 1) {
+            const int o = __shfl_xor(m, st);
+            m = o < m ? o : m;
+        }
+        const int entry = __shfl(my_entry, r);
+        const bool forced = (pos0 < a.sink) || (pos0 + ntok > len - a.recent);
+        const int sc = (entry < 0 || entry >= a.NB) ? -1 : (forced ? full : full - m);
+        if (lane == r) result = sc;
+#pragma unroll
+        for (int u = 0; u < LCd::kLoads; ++u) cur[u] = nxt[u];
+    }
+    if (lane < run) a.scores[(int64_t)b * a.max_blocks + j0 + lane] = result;
+}
+
 // 64-token blocks of 8-word codes against one KV head whose G query heads enter as bit planes
 // (16 requests x 65,536 tokens, 128 query heads: 33 MB of codes, 4096 waves).  With one block per
 // wave a wave's life is three dependent round trips to memory around some 250 instructions, and a
@@ -1086,46 +1299,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
 //  * after one barrier every wave keeps the planes in registers (GP * 8 of them) for its blocks;
 //  * the minima of the run's blocks are reduced together (the first two butterfly steps halve the
 //    number of values per lane) and leave in one store.
-constexpr int kLaneRun = 4;
-
-__device__ __forceinline__ void full_add(uint32_t x, uint32_t y, uint32_t z, uint32_t& sum, uint32_t& carry)
-{
-    const uint32_t t = x ^ y;
-    sum = t ^ z;
-    carry = (t & z) | (~t & x);  // majority(x, y, z)
-}
-__device__ __forceinline__ void half_add(uint32_t x, uint32_t y, uint32_t& sum, uint32_t& carry)
-{
-    sum = x ^ y;
-    carry = x & y;
-}
-
-// Bit-sliced count of 16 words: n[p] bit i = bit p of the number of words with bit i set.
-__device__ __forceinline__ void count16(const uint32_t (&x)[16], uint32_t (&n)[5])
-{
-    uint32_t s[6], c1[5];
-#pragma unroll
-    for (int i = 0; i < 5; ++i) full_add(x[3 * i], x[3 * i + 1], x[3 * i + 2], s[i], c1[i]);
-    s[5] = x[15];
-    // weight 1: six sums
-    uint32_t a0, a1, k0, k1, k2;
-    full_add(s[0], s[1], s[2], a0, k0);
-    full_add(s[3], s[4], s[5], a1, k1);
-    half_add(a0, a1, n[0], k2);
-    // weight 2: c1[0..4], k0, k1, k2
-    uint32_t b0, b1, m0, m1, m2, m3;
-    full_add(c1[0], c1[1], c1[2], b0, m0);
-    full_add(c1[3], c1[4], k0, b1, m1);
-    uint32_t b2;
-    full_add(b0, b1, k1, b2, m2);
-    half_add(b2, k2, n[1], m3);
-    // weight 4: m0..m3
-    uint32_t d0, e0, e1;
-    full_add(m0, m1, m2, d0, e0);
-    half_add(d0, m3, n[2], e1);
-    // weight 8: e0, e1
-    half_add(e0, e1, n[3], n[4]);
-}
 
 template <int GP>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void block_score_lanes64(ScoreArgs a)
@@ -1245,9 +1418,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
 #pragma unroll
         for (int w = 0; w < WD; ++w) {
             const uint32_t k = v[i][w >> 2][w & 3];
-            pk += __popc(k);
+            pk = popc_add(k, pk);
 #pragma unroll
-            for (int p = 0; p < GP; ++p) acc[p] += __popc(k & P[w][p]);
+            for (int p = 0; p < GP; ++p) acc[p] = popc_add(k & P[w][p], acc[p]);
         }
         int x = 0;
 #pragma unroll
@@ -2169,6 +2342,18 @@ bool lanes_layout(const ScoreArgs& a, const uint32_t* k_cache, bool direct)
 }
 
 template <int LC>
+void launch_lanes_run(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
+{
+    switch (pmax) {
+        case 4: launch_score(block_score_lanes_run<LC, 4>, grid, 0, st, a); break;
+        case 5: launch_score(block_score_lanes_run<LC, 5>, grid, 0, st, a); break;
+        case 6: launch_score(block_score_lanes_run<LC, 6>, grid, 0, st, a); break;
+        case 7: launch_score(block_score_lanes_run<LC, 7>, grid, 0, st, a); break;
+        default: launch_score(block_score_lanes_run<LC, 8>, grid, 0, st, a); break;
+    }
+}
+
+template <int LC>
 void dispatch_lanes(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
     const bool dir = LC == 9 && (a.G == 1 || a.G == 2 || a.G == 4);
@@ -2376,7 +2561,10 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
         // 64-token blocks of 8-word codes: the scorer builds the planes itself
         const bool planes_inside = !direct && Wd == 8 && BS == 64 && pmax <= 8 && lanes_layout(a, k_cache, direct);
-        if (!direct && !planes_inside) {
+        // the other code-per-lane shapes build them in wave 0 of every workgroup (up to 128 query heads)
+        const bool planes_in_lanes = !direct && !planes_inside && a.G <= 128 && BS == 64 && (Wd == 16 || Wd == 18) &&
+                                     lanes_layout(a, k_cache, direct);
+        if (!direct && !planes_inside && !planes_in_lanes) {
             g_note.planes = "plane_kernel";
             hipLaunchKernelGGL(plane_kernel, dim3(B * ((Wd + 1) / 2)), dim3(kThreads), 0, st, q_codes,
                                q_stride_b, q_stride_h, 1, a.G, Wd, pmax, ws.planes);
@@ -2396,6 +2584,11 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
                 case 7: launch_score(block_score_lanes64<7>, g64, 0, st, a); break;
                 default: launch_score(block_score_lanes64<8>, g64, 0, st, a); break;
             }
+        } else if (planes_in_lanes) {
+            note_score("block_score_lanes_run", Wd / 2, pmax);
+            const dim3 g64((unsigned)ucm::ceil_div(max_blocks, (kThreads / kWave) * kLanesRunBlocks), (unsigned)B);
+            if (Wd == 18) launch_lanes_run<9>(a, pmax, g64, st);
+            else launch_lanes_run<8>(a, pmax, g64, st);
         } else if (lanes_layout(a, k_cache, direct)) {
             if (Wd == 18) dispatch_lanes<9>(a, pmax, pgrid, st);
             else if (Wd == 16) dispatch_lanes<8>(a, pmax, pgrid, st);
@@ -2732,8 +2925,7 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t, int tb
             int d = 0;
 #pragma unroll
             for (int g = 0; g < G; ++g)
-                d += __popc(kw[u].x ^ qw[g][0]) + __popc(kw[u].y ^ qw[g][1]) +
-                     __popc(kw[u].z ^ qw[g][2]) + __popc(kw[u].w ^ qw[g][3]);
+                d = popc_add(kw[u].w ^ qw[g][3], popc_add(kw[u].z ^ qw[g][2], popc_add(kw[u].y ^ qw[g][1], popc_add(kw[u].x ^ qw[g][0], d))));
             for (int o = 1; o < P; o <<= 1) d += __shfl_xor(d, o);
             if (part == 0 && tt < TT) dyn[h * TT + tt] = (uint32_t)d;
         }
