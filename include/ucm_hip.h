@@ -243,7 +243,7 @@ int ucm_hamming_topk_set_profile_events(void* before, void* after);
  * ucm_hamming_topk / ucm_hamming_topk_static / ucm_sparse_decode_step* / ucm_gsa_decode_step /
  * ucm_hamming_score call on the calling thread launched, e.g.
  * "block_score_one<1,8,1,4,1>+select_wave_kernel<4>" or
- * "plane_kernel+block_score_lanes<4,0,8>+select_group_kernel<4>" (family, then its template
+ * "plane_kernel+block_score_lanes<4,0,8>+select_wave_kernel<4>" (family, then its template
  * arguments), cut to cap - 1 characters.  Returns the full length.  Several kernel families give
  * the same results at very different speeds; this lets a test pin which one a shape takes.
  */
