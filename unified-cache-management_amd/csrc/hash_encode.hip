@@ -638,13 +638,14 @@ __device__ __forceinline__ void stream_wait_lds()
 // ACCS: accumulator tiles in flight (the MFMAs of ACCS column tiles are interleaved, so that a
 // wave's consecutive MFMAs do not depend on each other).
 //
-// Stores: one 16-byte store per row and head.  Handing the codes of neighbouring heads to one
-// wave through LDS, which then writes whole 128-byte runs, was built and measured: the writes
-// got cheaper and the arrival counters, the extra LDS traffic and the waves waiting for each
-// other cost more than that (2.1 GB of keys: 476-520 us against 446 us).  What the stores cost
-// is not their size: on this part a read stream slows down by a fifth as soon as ANY write
-// stream runs beside it (2 GiB of plain 16-byte loads: 304 us alone, 350 us with 1.6 % writes,
-// 400 us with 6.25 % writes in 1 KiB runs, whatever the store's cache policy).
+// Stores: one 16-byte store per row and head.  Their size is what they cost: beside a 2 GiB read
+// stream (304 us alone) the same 6.25 % of bytes written back take the stream to 392-405 us as
+// whole 128-byte lines, 408 us as 64-byte pieces, 425-436 us as 32-byte pieces and 450-472 us as
+// 16-byte pieces of lines that other workgroups complete (no arithmetic in any of these; the
+// stores' cache policy and their clustering in time change nothing).  This kernel sits at the
+// last figure.  Handing the codes of neighbouring heads to one wave through LDS, which then
+// writes whole 128-byte runs, was built in its simplest form (arrival counters, the storing wave
+// in step with the slowest of the eight) and measured slower: 476-520 us against 446 us.
 template <typename V, int KS, int NT, int SLOT, int ACCS>
 __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void encode_stream_kernel(
     EncArgs a, int64_t ntiles, int nstreams)
