@@ -334,8 +334,9 @@ def encoder_cache_build(torch, enc_k, gen, launches=9):
             "note": "a plain 16-byte-load stream of 2 GiB with 6.25 % of its bytes written back (this "
                     "operator's traffic shape, no arithmetic) takes 392-405 us on this part when the writes "
                     "are whole 128-byte lines (0.71-0.73 of the published peak) and 450-472 us when they are "
-                    "16-byte pieces of lines that other workgroups complete, as this kernel's are; the same "
-                    "reads alone take 304 us"}
+                    "16-byte pieces of lines that other workgroups complete; the kernel stores whole lines "
+                    "(the eight head waves of a token stream take turns, codes exchanged through LDS); "
+                    "the same reads alone take 304 us"}
 
 
 def plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots):

@@ -65,6 +65,11 @@ CASES = [
     (6, 2048 + 1, 1, 64, 64, torch.float16, torch.int64, True),
     (7, 1500, 12, 128, 128, torch.bfloat16, torch.int64, False),       # head count that is no power of two
     (8, 70000, 8, 128, 128, torch.bfloat16, torch.int64, False),       # several tiles per wave
+    # eight heads of 128-bit codes: whole cache rows stored by one wave (ring of tiles in LDS)
+    (9, 70000 + 13, 8, 128, 128, torch.float16, torch.int32, False),   # ragged end after many tiles
+    (10, 200000, 8, 64, 128, torch.bfloat16, torch.int64, True),       # 24 tiles per wave, ring reused 4x
+    (11, 32 * 256 * 5 + 1, 8, 128, 128, torch.bfloat16, torch.int32, False),  # one tile more than the ring
+    (12, 32 * 256 * 2, 8, 128, 128, torch.bfloat16, torch.int64, True),       # exactly the store delay
 ]
 
 
@@ -84,6 +89,10 @@ def test_streaming_kernel_matches_oracle_and_tiled_kernel(stream_everything, see
     slots_in[drop[0]] = -1
     if len(drop) > 1:
         slots_in[drop[1]] = NB * BS + 4
+    if T > 50000:  # whole tiles and runs of rows without a slot
+        more = np.concatenate([np.arange(32 * 300, 32 * 302), np.arange(40001, 40040)])
+        slots_in[more] = -1
+        drop = np.concatenate([drop[:2], more, drop[2:]])
     slots = torch.from_numpy(slots_in).to(sdt).cuda()
     canary = 0x5A5A5A5A
     got = torch.full((NB, BS, H, N // 32), canary, dtype=torch.int32, device="cuda")
@@ -101,7 +110,7 @@ def test_streaming_kernel_matches_oracle_and_tiled_kernel(stream_everything, see
     flat = g.reshape(-1, H, N // 32)
     used = np.zeros(NB * BS, bool)
     keep = np.ones(T, bool)
-    keep[drop[:2]] = False
+    keep[drop[:-3] if T > 50000 else drop[:2]] = False
     used[slots_np[keep]] = True
     assert np.all(flat[~used] == canary)
     rows = np.flatnonzero(keep)
@@ -126,6 +135,30 @@ def test_streaming_kernel_dense_output(stream_everything):
     o = out.cpu().numpy().view(np.uint32)
     rows = np.sort(rng.choice(T, size=500, replace=False))
     _check_against_oracle(o[:, None].reshape(T, 1, H, N // 32), x, W, np.arange(T), 1, 1, rows)
+
+
+def test_streaming_kernel_dense_output_many_tiles(stream_everything):
+    """Dense [T, 8, 4] output over many tiles per wave (whole 128-byte rows stored by one wave):
+    identical to the tiled kernel, rows past the end untouched."""
+    from ucm_amd import _lib
+
+    L = stream_everything
+    rng = rng_for(22)
+    T, H, K, N = 32 * 256 * 7 + 19, 8, 128, 128
+    x = torch.from_numpy(rng.standard_normal((T, H, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    W = torch.from_numpy(rng.standard_normal((H, K, N)).astype(np.float32)).to(torch.bfloat16).cuda()
+    outs = []
+    for thr in (1, 1 << 62):
+        L.ucm_hash_encode_set_stream_threshold(thr)
+        out = torch.full((T + 64, H, N // 32), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+        _lib.check(L.ucm_hash_encode(x.data_ptr(), 0, T, H, K, x.stride(0), x.stride(1), W.data_ptr(), 0, H, 1, N,
+                                     out.data_ptr(), out.stride(0), out.stride(1),
+                                     torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        outs.append(out)
+    L.ucm_hash_encode_set_stream_threshold(1)
+    assert torch.equal(outs[0], outs[1])
+    assert bool((outs[0][T:] == 0x5A5A5A5A).all())
 
 
 def test_cache_build_size_takes_the_streaming_kernel_by_default():

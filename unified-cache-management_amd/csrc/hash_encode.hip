@@ -638,15 +638,60 @@ __device__ __forceinline__ void stream_wait_lds()
 // ACCS: accumulator tiles in flight (the MFMAs of ACCS column tiles are interleaved, so that a
 // wave's consecutive MFMAs do not depend on each other).
 //
-// Stores: one 16-byte store per row and head.  Their size is what they cost: beside a 2 GiB read
+// Stores: one 16-byte code per row and head.  Their size is what they cost: beside a 2 GiB read
 // stream (304 us alone) the same 6.25 % of bytes written back take the stream to 392-405 us as
 // whole 128-byte lines, 408 us as 64-byte pieces, 425-436 us as 32-byte pieces and 450-472 us as
 // 16-byte pieces of lines that other workgroups complete (no arithmetic in any of these; the
-// stores' cache policy and their clustering in time change nothing).  This kernel sits at the
-// last figure.  Handing the codes of neighbouring heads to one wave through LDS, which then
-// writes whole 128-byte runs, was built in its simplest form (arrival counters, the storing wave
-// in step with the slowest of the eight) and measured slower: 476-520 us against 446 us.
-template <typename V, int KS, int NT, int SLOT, int ACCS>
+// stores' cache policy and their clustering in time change nothing).  With one store per row and
+// head this kernel sits at the last figure (2.1 GB of keys: 455-470 us into the paged cache).
+//
+// COMB (eight heads of four-word codes side by side in a token's cache row, one stream per
+// workgroup): the waves hand their codes to one another through a ring of kRing tiles in LDS and
+// take turns storing whole 128-byte rows, kCombDelay tiles after the codes were produced, so that
+// the storing wave normally finds all eight heads there and nobody runs in step with anybody.
+// Two counters per ring slot: pub (codes handed in) and done (tiles stored); plain LDS
+// operations of one wave complete in order, so a counter update that follows the data in program
+// order is seen after the data.  Every wait is bounded: a wave that does not see its counter
+// move gives up waiting and goes on (the results are then wrong, the kernel still ends).
+// 2.1 GB of keys: 403-411 us against 455-470 us = 5.6 TB/s of algorithmic bytes.  What made earlier
+// forms of this slower than the plain stores (476-545 us): counters as volatile / atomic C++
+// accesses (each waits for the row loads in flight), spilled registers reloaded inside the loop
+// (scratch reloads count as vector loads and wait behind the row loads: hence two accumulator
+// tiles here, not four), and the storing wave in step with the slowest of the eight.
+constexpr int kRing = 5;
+constexpr int kCombDelay = 2;
+constexpr int kRingSlotBytes = 4096 + 128;  // 32 rows x 8 heads x 16 bytes, then the rows' 32 slots
+constexpr int kSpinLimit = 1 << 22;  // some tenths of a second
+
+// Counter reads and updates as single LDS instructions with a wait of their own: a volatile or
+// atomic access in C++ makes the compiler wait for every outstanding memory operation, the row
+// loads in flight included.  The read waits inside the same statement: a register that an LDS read
+// fills later, behind the compiler's back, may have been given to another value by then.
+__device__ __forceinline__ int lds_peek(const int* counter)
+{
+    int v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                 : "=v"(v)
+                 : "v"((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) int*)counter)
+                 : "memory");
+    return v;
+}
+__device__ __forceinline__ void lds_bump(int* counter)
+{
+    const uint32_t one = 1;
+    asm volatile("ds_add_u32 %0, %1" ::"v"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) int*)counter), "v"(one)
+                 : "memory");
+}
+__device__ __forceinline__ void lds_wait_at_least(const int* counter, int want)
+{
+    int spins = 0;
+    while (lds_peek(counter) < want) {
+        if (++spins > kSpinLimit) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+template <typename V, int KS, int NT, int SLOT, int ACCS, bool COMB>
 __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void encode_stream_kernel(
     EncArgs a, int64_t ntiles, int nstreams)
 {
@@ -759,13 +804,65 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
     // one shift, two 32-bit multiplications, one store.
     uint32_t words_prev[NT];
     uint32_t* dst_prev = nullptr;
+    int32_t slot_prev = -1;  // COMB: the previous tile's slot of this lane's row, -1 = no store
+    int prev_idx = -1;       // COMB: the previous tile's number in this stream (0, 1, 2, ...)
+    int done_seen = 0;       // COMB: `done` of the ring slot the previous tile goes to, read in step()
 #pragma unroll
     for (int q = 0; q < NT; ++q) words_prev[q] = 0;
     const int64_t n_slots = a.NB << a.bs_shift;
     uint32_t* const cache_h = a.cache + (int64_t)h * a.cs_head;
     const uint32_t csb = (uint32_t)a.cs_block, cst = (uint32_t)a.cs_token;
 
+    uint8_t* const ring = stream_lds + (size_t)kStreamWaves * 2 * kBufBytes;
+    int* const pub = reinterpret_cast<int*>(ring + kRing * kRingSlotBytes);
+    int* const done = pub + kRing;
+    if constexpr (COMB) {
+        if (threadIdx.x < 2 * kRing) pub[threadIdx.x] = 0;
+        __syncthreads();
+    }
+    // the wave whose turn it is stores tile j of this stream as 32 whole cache rows
+    auto store_tile = [&](int j) {
+        const int s = j % kRing;
+        lds_wait_at_least(pub + s, kStreamWaves * (j / kRing + 1));
+        asm volatile("" ::: "memory");
+        const uint8_t* slot_base = ring + s * kRingSlotBytes;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int piece = u * 64 + lane;  // row piece / 8 of the tile, head piece % 8
+            const int ph = piece & 7, pr = piece >> 3;
+            const u32x4 code = *reinterpret_cast<const u32x4*>(slot_base + ph * 512 + ((pr ^ (2 * ph)) << 4));
+            const int32_t sv = *reinterpret_cast<const int32_t*>(slot_base + 4096 + (piece >> 3) * 4);
+            if (sv >= 0) {
+                const uint32_t svl = (uint32_t)sv;
+                uint32_t* dst = a.cache + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) + (piece & 7) * 4;
+                *reinterpret_cast<u32x4*>(dst) = code;
+            }
+        }
+        asm volatile("" ::: "memory");
+        if (lane == 0) lds_bump(done + s);
+    };
+
     auto store_prev = [&]() {
+        if constexpr (COMB) {
+            if (prev_idx < 0) return;
+            const int s = prev_idx % kRing, gen = prev_idx / kRing;
+            // the slot's previous tile has been stored: normally known from the read in step()
+            if (gen > 0 && done_seen < gen) lds_wait_at_least(done + s, gen);
+            asm volatile("" ::: "memory");
+            uint8_t* slot_base = ring + s * kRingSlotBytes;
+            if (lane < 32) {
+                const u32x4 v = {words_prev[0], words_prev[1 % NT], words_prev[2 % NT], words_prev[3 % NT]};
+                // head-major in the ring, rows swizzled with the head: the 32 lanes of this write and
+                // the 64 lanes of the storing wave's reads (8 heads x 8 rows) each cover all banks
+                *reinterpret_cast<u32x4*>(slot_base + h * 512 + ((r ^ (2 * h)) << 4)) = v;
+                if ((prev_idx & 7) == h) *reinterpret_cast<int32_t*>(slot_base + 4096 + r * 4) = slot_prev;
+            }
+            asm volatile("" ::: "memory");
+            if (lane == 0) lds_bump(pub + s);
+            const int j = prev_idx - kCombDelay;
+            if (j >= 0 && (j & 7) == h) store_tile(j);
+            return;
+        }
         if (dst_prev) {
             if constexpr (NT == 4) {
                 u32x4 v = {words_prev[0], words_prev[1 % NT], words_prev[2 % NT], words_prev[3 % NT]};
@@ -778,7 +875,7 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
     };
 
     // newer: the next tile's loads are in flight behind this tile's; more: a tile two ahead exists
-    auto step = [&](int64_t tile, int b, bool newer, bool more) {
+    auto step = [&](int64_t tile, int local, int b, bool newer, bool more) {
         const uint8_t* buf = mybuf + b * kBufBytes;
         if (newer) stream_wait_loads<kLoads>();  // everything but the newest tile's loads has landed
         else stream_wait_loads<0>();
@@ -790,13 +887,20 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
         int64_t sv = t;
         if constexpr (SLOT == 2) sv = *reinterpret_cast<const int64_t*>(buf + kTileBytes + r * 8);
         if constexpr (SLOT == 1) sv = *reinterpret_cast<const int32_t*>(buf + kTileBytes + r * 4);
-        stream_wait_lds();  // the buffer may be overwritten from here on
+        // the buffer may be overwritten from here on (COMB: the counter read shares the wait)
+        if constexpr (COMB) done_seen = lds_peek(done + (prev_idx < 0 ? 0 : prev_idx % kRing));
+        else stream_wait_lds();
         store_prev();
         if (more) issue(tile + 2 * (int64_t)nstreams, b);
 
         const bool ok = t < a.T && lane < 32 && sv >= 0 && sv < n_slots;
         const uint32_t svl = (uint32_t)sv;  // below 2^31 when ok
-        dst_prev = ok ? cache_h + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) : nullptr;
+        if constexpr (COMB) {
+            slot_prev = ok ? (int32_t)svl : -1;
+            prev_idx = local;
+        } else {
+            dst_prev = ok ? cache_h + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) : nullptr;
+        }
 
 #pragma unroll
         for (int n0 = 0; n0 < NT; n0 += ACCS) {
@@ -821,13 +925,19 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
     if (n > 0) issue(tile, 0);
     if (n > 1) issue(tile + nstreams, 1);
     for (int64_t i = 0; i < n; i += 2) {
-        step(tile, 0, i + 1 < n, i + 2 < n);
+        step(tile, (int)i, 0, i + 1 < n, i + 2 < n);
         tile += nstreams;
         if (i + 1 >= n) break;
-        step(tile, 1, i + 2 < n, i + 3 < n);
+        step(tile, (int)i + 1, 1, i + 2 < n, i + 3 < n);
         tile += nstreams;
     }
+    if constexpr (COMB) done_seen = lds_peek(done + (prev_idx < 0 ? 0 : prev_idx % kRing));
     store_prev();
+    if constexpr (COMB) {
+        // the last kCombDelay tiles have been handed in but not stored yet
+        for (int j = (int)n - kCombDelay < 0 ? 0 : (int)n - kCombDelay; j < (int)n; ++j)
+            if ((j & 7) == h) store_tile(j);
+    }
     // no load may still be writing into this workgroup's LDS when the wave ends
     stream_wait_loads<0>();
 }
@@ -1112,13 +1222,15 @@ bool stream_eligible(const EncArgs& a, int x_dtype, int w_dtype)
     return a.H <= waves;
 }
 
-template <typename V, int KS, int NT, int SLOT, int ACCS>
+template <typename V, int KS, int NT, int SLOT, int ACCS, bool COMB>
 int launch_stream_a(const EncArgs& a, hipStream_t st)
 {
-    constexpr size_t lds = (size_t)kStreamWaves * 2 * (kRowsPerWave * KS * 32 + 256);
+    constexpr size_t lds = (size_t)kStreamWaves * 2 * (kRowsPerWave * KS * 32 + 256) +
+                           (COMB ? kRing * kRingSlotBytes + 2 * kRing * sizeof(int) : 0);
+    static_assert(lds <= 160 * 1024, "row buffers and ring exceed the LDS");
     static int opted = 0;  // 0 = not tried, 1 = allowed, -1 = refused by the runtime
     if (opted == 0) {
-        const hipError_t e = hipFuncSetAttribute((const void*)encode_stream_kernel<V, KS, NT, SLOT, ACCS>,
+        const hipError_t e = hipFuncSetAttribute((const void*)encode_stream_kernel<V, KS, NT, SLOT, ACCS, COMB>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) (void)hipGetLastError();
         opted = (e == hipSuccess) ? 1 : -1;
@@ -1130,15 +1242,26 @@ int launch_stream_a(const EncArgs& a, hipStream_t st)
     if ((wgs * kStreamWaves) % a.H) return UCM_EUNSUPPORTED;
     const int nstreams = wgs * kStreamWaves / a.H;
     const int64_t ntiles = ucm::ceil_div(a.T, kRowsPerWave);
-    hipLaunchKernelGGL((encode_stream_kernel<V, KS, NT, SLOT, ACCS>), dim3((unsigned)wgs), dim3(kStreamThreads),
+    hipLaunchKernelGGL((encode_stream_kernel<V, KS, NT, SLOT, ACCS, COMB>), dim3((unsigned)wgs), dim3(kStreamThreads),
                        lds, st, a, ntiles, nstreams);
     return ucm::launch_status("encode_stream_kernel");
+}
+
+// Whole cache rows from one wave: eight heads of four-word codes that lie side by side in a
+// 128-byte aligned token row, and fewer than 2^31 tiles per stream.
+bool stream_combine(const EncArgs& a)
+{
+    return a.H == 8 && a.N == 128 && a.cs_head == 4 && a.cs_token == 32 && a.cs_block % 32 == 0 &&
+           (((uintptr_t)a.cache) & 127) == 0;
 }
 
 template <typename V, int KS, int NT, int SLOT>
 int launch_stream_i(const EncArgs& a, hipStream_t st)
 {
-    return launch_stream_a<V, KS, NT, SLOT, (NT == 4 ? 4 : 2)>(a, st);
+    if constexpr (NT == 4) {
+        if (stream_combine(a)) return launch_stream_a<V, KS, NT, SLOT, 2, true>(a, st);
+    }
+    return launch_stream_a<V, KS, NT, SLOT, (NT == 4 ? 4 : 2), false>(a, st);
 }
 
 template <typename V, int KS, int NT>
