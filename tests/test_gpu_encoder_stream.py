@@ -70,6 +70,10 @@ CASES = [
     (10, 200000, 8, 64, 128, torch.bfloat16, torch.int64, True),       # 24 tiles per wave, ring reused 4x
     (11, 32 * 256 * 5 + 1, 8, 128, 128, torch.bfloat16, torch.int32, False),  # one tile more than the ring
     (12, 32 * 256 * 2, 8, 128, 128, torch.bfloat16, torch.int64, True),       # exactly the store delay
+    # four and two heads: 64- and 32-byte rows, two and four streams per workgroup
+    (13, 150000, 4, 128, 128, torch.bfloat16, torch.int64, False),
+    (14, 150000 + 7, 2, 128, 128, torch.float16, torch.int32, True),
+    (15, 300000, 2, 64, 128, torch.bfloat16, torch.int64, False),
 ]
 
 

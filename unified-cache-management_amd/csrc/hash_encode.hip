@@ -645,10 +645,11 @@ __device__ __forceinline__ void stream_wait_lds()
 // stores' cache policy and their clustering in time change nothing).  With one store per row and
 // head this kernel sits at the last figure (2.1 GB of keys: 455-470 us into the paged cache).
 //
-// COMB (eight heads of four-word codes side by side in a token's cache row, one stream per
-// workgroup): the waves hand their codes to one another through a ring of kRing tiles in LDS and
-// take turns storing whole 128-byte rows, kCombDelay tiles after the codes were produced, so that
-// the storing wave normally finds all eight heads there and nobody runs in step with anybody.
+// HC > 0 (HC = 2, 4 or 8 heads of four-word codes side by side in a token's cache row; the HC
+// waves of a stream sit in one workgroup): the waves hand their codes to one another through a
+// ring of kRing tiles in LDS and take turns storing whole rows (128 bytes at eight heads),
+// kCombDelay tiles after the codes were produced, so that the storing wave normally finds all
+// heads there and nobody runs in step with anybody.
 // Two counters per ring slot: pub (codes handed in) and done (tiles stored); plain LDS
 // operations of one wave complete in order, so a counter update that follows the data in program
 // order is seen after the data.  Every wait is bounded: a wave that does not see its counter
@@ -660,7 +661,11 @@ __device__ __forceinline__ void stream_wait_lds()
 // tiles here, not four), and the storing wave in step with the slowest of the eight.
 constexpr int kRing = 5;
 constexpr int kCombDelay = 2;
-constexpr int kRingSlotBytes = 4096 + 128;  // 32 rows x 8 heads x 16 bytes, then the rows' 32 slots
+constexpr int ring_slot_bytes(int hc) { return 512 * hc + 128; }  // 32 rows x hc heads x 16 bytes, then the rows' 32 slots
+constexpr int ring_lds_bytes(int hc)  // rings and counters of the 8 / hc streams of a workgroup
+{
+    return hc ? (8 / hc) * (kRing * ring_slot_bytes(hc) + 2 * kRing * (int)sizeof(int)) : 0;
+}
 constexpr int kSpinLimit = 1 << 22;  // some tenths of a second
 
 // Counter reads and updates as single LDS instructions with a wait of their own: a volatile or
@@ -682,19 +687,27 @@ __device__ __forceinline__ void lds_bump(int* counter)
     asm volatile("ds_add_u32 %0, %1" ::"v"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) int*)counter), "v"(one)
                  : "memory");
 }
-__device__ __forceinline__ void lds_wait_at_least(const int* counter, int want)
+// gave_up: set once a wait of this wave has run into the limit; the wave then never waits again,
+// so a kernel that has gone wrong ends after one limit per wave, not one per tile.
+__device__ __forceinline__ void lds_wait_at_least(const int* counter, int want, bool& gave_up)
 {
+    if (gave_up) return;
     int spins = 0;
     while (lds_peek(counter) < want) {
-        if (++spins > kSpinLimit) break;
+        if (++spins > kSpinLimit) {
+            gave_up = true;
+            break;
+        }
         __builtin_amdgcn_s_sleep(1);
     }
 }
 
-template <typename V, int KS, int NT, int SLOT, int ACCS, bool COMB>
+template <typename V, int KS, int NT, int SLOT, int ACCS, int HC>
 __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void encode_stream_kernel(
     EncArgs a, int64_t ntiles, int nstreams)
 {
+    constexpr bool COMB = HC > 0;
+    constexpr int HCn = HC > 0 ? HC : 8;  // keeps the index arithmetic of the unused branch well-formed
     extern __shared__ __attribute__((aligned(1024))) uint8_t stream_lds[];
     constexpr int K = KS * 16;
     constexpr int LN = KS / 4;                      // 128-byte lines per row
@@ -807,34 +820,38 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
     int32_t slot_prev = -1;  // COMB: the previous tile's slot of this lane's row, -1 = no store
     int prev_idx = -1;       // COMB: the previous tile's number in this stream (0, 1, 2, ...)
     int done_seen = 0;       // COMB: `done` of the ring slot the previous tile goes to, read in step()
+    bool gave_up = false;    // COMB: a wait of this wave has hit its limit
 #pragma unroll
     for (int q = 0; q < NT; ++q) words_prev[q] = 0;
     const int64_t n_slots = a.NB << a.bs_shift;
     uint32_t* const cache_h = a.cache + (int64_t)h * a.cs_head;
     const uint32_t csb = (uint32_t)a.cs_block, cst = (uint32_t)a.cs_token;
 
-    uint8_t* const ring = stream_lds + (size_t)kStreamWaves * 2 * kBufBytes;
-    int* const pub = reinterpret_cast<int*>(ring + kRing * kRingSlotBytes);
+    // this stream's ring and its counters (a workgroup holds 8 / HC streams)
+    constexpr int kSlotBytes = ring_slot_bytes(HCn);
+    constexpr int kStreamRing = kRing * kSlotBytes + 2 * kRing * (int)sizeof(int);
+    uint8_t* const ring = stream_lds + (size_t)kStreamWaves * 2 * kBufBytes + (COMB ? (wave / HCn) * kStreamRing : 0);
+    int* const pub = reinterpret_cast<int*>(ring + kRing * kSlotBytes);
     int* const done = pub + kRing;
     if constexpr (COMB) {
-        if (threadIdx.x < 2 * kRing) pub[threadIdx.x] = 0;
+        if ((wave % HCn) == 0 && lane < 2 * kRing) pub[lane] = 0;
         __syncthreads();
     }
     // the wave whose turn it is stores tile j of this stream as 32 whole cache rows
     auto store_tile = [&](int j) {
         const int s = j % kRing;
-        lds_wait_at_least(pub + s, kStreamWaves * (j / kRing + 1));
+        lds_wait_at_least(pub + s, HCn * (j / kRing + 1), gave_up);
         asm volatile("" ::: "memory");
-        const uint8_t* slot_base = ring + s * kRingSlotBytes;
+        const uint8_t* slot_base = ring + s * kSlotBytes;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int piece = u * 64 + lane;  // row piece / 8 of the tile, head piece % 8
-            const int ph = piece & 7, pr = piece >> 3;
+        for (int u = 0; u < HCn / 2; ++u) {
+            const int piece = u * 64 + lane;  // row piece / HC of the tile, head piece % HC
+            const int ph = piece % HCn, pr = piece / HCn;
             const u32x4 code = *reinterpret_cast<const u32x4*>(slot_base + ph * 512 + ((pr ^ (2 * ph)) << 4));
-            const int32_t sv = *reinterpret_cast<const int32_t*>(slot_base + 4096 + (piece >> 3) * 4);
+            const int32_t sv = *reinterpret_cast<const int32_t*>(slot_base + 512 * HCn + pr * 4);
             if (sv >= 0) {
                 const uint32_t svl = (uint32_t)sv;
-                uint32_t* dst = a.cache + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) + (piece & 7) * 4;
+                uint32_t* dst = a.cache + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) + ph * 4;
                 *reinterpret_cast<u32x4*>(dst) = code;
             }
         }
@@ -847,20 +864,20 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
             if (prev_idx < 0) return;
             const int s = prev_idx % kRing, gen = prev_idx / kRing;
             // the slot's previous tile has been stored: normally known from the read in step()
-            if (gen > 0 && done_seen < gen) lds_wait_at_least(done + s, gen);
+            if (gen > 0 && done_seen < gen) lds_wait_at_least(done + s, gen, gave_up);
             asm volatile("" ::: "memory");
-            uint8_t* slot_base = ring + s * kRingSlotBytes;
+            uint8_t* slot_base = ring + s * kSlotBytes;
             if (lane < 32) {
                 const u32x4 v = {words_prev[0], words_prev[1 % NT], words_prev[2 % NT], words_prev[3 % NT]};
                 // head-major in the ring, rows swizzled with the head: the 32 lanes of this write and
-                // the 64 lanes of the storing wave's reads (8 heads x 8 rows) each cover all banks
+                // (at eight heads) the 64 lanes of the storing wave's reads each cover all banks
                 *reinterpret_cast<u32x4*>(slot_base + h * 512 + ((r ^ (2 * h)) << 4)) = v;
-                if ((prev_idx & 7) == h) *reinterpret_cast<int32_t*>(slot_base + 4096 + r * 4) = slot_prev;
+                if ((prev_idx % HCn) == h) *reinterpret_cast<int32_t*>(slot_base + 512 * HCn + r * 4) = slot_prev;
             }
             asm volatile("" ::: "memory");
             if (lane == 0) lds_bump(pub + s);
             const int j = prev_idx - kCombDelay;
-            if (j >= 0 && (j & 7) == h) store_tile(j);
+            if (j >= 0 && (j % HCn) == h) store_tile(j);
             return;
         }
         if (dst_prev) {
@@ -936,7 +953,7 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
     if constexpr (COMB) {
         // the last kCombDelay tiles have been handed in but not stored yet
         for (int j = (int)n - kCombDelay < 0 ? 0 : (int)n - kCombDelay; j < (int)n; ++j)
-            if ((j & 7) == h) store_tile(j);
+            if ((j % HCn) == h) store_tile(j);
     }
     // no load may still be writing into this workgroup's LDS when the wave ends
     stream_wait_loads<0>();
@@ -1222,15 +1239,14 @@ bool stream_eligible(const EncArgs& a, int x_dtype, int w_dtype)
     return a.H <= waves;
 }
 
-template <typename V, int KS, int NT, int SLOT, int ACCS, bool COMB>
+template <typename V, int KS, int NT, int SLOT, int ACCS, int HC>
 int launch_stream_a(const EncArgs& a, hipStream_t st)
 {
-    constexpr size_t lds = (size_t)kStreamWaves * 2 * (kRowsPerWave * KS * 32 + 256) +
-                           (COMB ? kRing * kRingSlotBytes + 2 * kRing * sizeof(int) : 0);
+    constexpr size_t lds = (size_t)kStreamWaves * 2 * (kRowsPerWave * KS * 32 + 256) + ring_lds_bytes(HC);
     static_assert(lds <= 160 * 1024, "row buffers and ring exceed the LDS");
     static int opted = 0;  // 0 = not tried, 1 = allowed, -1 = refused by the runtime
     if (opted == 0) {
-        const hipError_t e = hipFuncSetAttribute((const void*)encode_stream_kernel<V, KS, NT, SLOT, ACCS, COMB>,
+        const hipError_t e = hipFuncSetAttribute((const void*)encode_stream_kernel<V, KS, NT, SLOT, ACCS, HC>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) (void)hipGetLastError();
         opted = (e == hipSuccess) ? 1 : -1;
@@ -1242,26 +1258,32 @@ int launch_stream_a(const EncArgs& a, hipStream_t st)
     if ((wgs * kStreamWaves) % a.H) return UCM_EUNSUPPORTED;
     const int nstreams = wgs * kStreamWaves / a.H;
     const int64_t ntiles = ucm::ceil_div(a.T, kRowsPerWave);
-    hipLaunchKernelGGL((encode_stream_kernel<V, KS, NT, SLOT, ACCS, COMB>), dim3((unsigned)wgs), dim3(kStreamThreads),
+    hipLaunchKernelGGL((encode_stream_kernel<V, KS, NT, SLOT, ACCS, HC>), dim3((unsigned)wgs), dim3(kStreamThreads),
                        lds, st, a, ntiles, nstreams);
     return ucm::launch_status("encode_stream_kernel");
 }
 
-// Whole cache rows from one wave: eight heads of four-word codes that lie side by side in a
-// 128-byte aligned token row, and fewer than 2^31 tiles per stream.
-bool stream_combine(const EncArgs& a)
+// Whole cache rows from one wave: 2, 4 or 8 heads of four-word codes that lie side by side in a
+// token row aligned to its own size.  Returns the head count, 0 when the shape does not qualify.
+int stream_combine(const EncArgs& a)
 {
-    return a.H == 8 && a.N == 128 && a.cs_head == 4 && a.cs_token == 32 && a.cs_block % 32 == 0 &&
-           (((uintptr_t)a.cache) & 127) == 0;
+    if (!(a.H == 2 || a.H == 4 || a.H == 8) || a.N != 128 || a.cs_head != 4) return 0;
+    if (a.cs_token != 4 * a.H || a.cs_block % (4 * a.H) || (((uintptr_t)a.cache) & (16 * a.H - 1))) return 0;
+    return a.H;
 }
 
 template <typename V, int KS, int NT, int SLOT>
 int launch_stream_i(const EncArgs& a, hipStream_t st)
 {
     if constexpr (NT == 4) {
-        if (stream_combine(a)) return launch_stream_a<V, KS, NT, SLOT, 2, true>(a, st);
+        switch (stream_combine(a)) {
+            case 8: return launch_stream_a<V, KS, NT, SLOT, 2, 8>(a, st);
+            case 4: return launch_stream_a<V, KS, NT, SLOT, 2, 4>(a, st);
+            case 2: return launch_stream_a<V, KS, NT, SLOT, 2, 2>(a, st);
+            default: break;
+        }
     }
-    return launch_stream_a<V, KS, NT, SLOT, (NT == 4 ? 4 : 2), false>(a, st);
+    return launch_stream_a<V, KS, NT, SLOT, (NT == 4 ? 4 : 2), 0>(a, st);
 }
 
 template <typename V, int KS, int NT>
