@@ -35,6 +35,10 @@ TOPK_SHAPES = {
     "blocks_of_32_KiB": (2, 32, 8, 4, 256, [4096, 3000], 4, {}, "block_score_one<1,8,1,4,0>+select_wave_kernel<4>"),
     "eight_query_heads_per_kv_head": (2, 64, 8, 4, 128, [4096, 3000], 8, {},
                                       "plane_kernel+block_score_one<1,8,0,4,1>+select_wave_kernel<4>"),
+    "sixteen_query_heads_per_kv_head": (2, 128, 8, 4, 128, [4096, 3000], 8, {},
+                                        "plane_kernel+block_score_one<1,8,0,5,1>+select_wave_kernel<4>"),
+    "thirty_one_query_heads_one_kv_head": (2, 31, 1, 4, 1024, [8192, 3000], 4, {},
+                                           "plane_kernel+block_score_one<1,1,0,5,1>+select_wave_kernel<4>"),
     "blocks_of_64_tokens": (2, 32, 8, 4, 64, [4096, 3000], 8, {}, "block_score_rows<1,8,4,8>+select_wave_kernel<4>"),
     "blocks_of_16_tokens": (2, 32, 8, 4, 16, [1024, 700], 8, {}, "block_score_rows<1,8,4,2>+select_wave_kernel<4>"),
     "small_blocks_bit_planes": (2, 16, 2, 4, 32, [2048, 700], 8, {},
