@@ -2215,8 +2215,9 @@ bool dispatch_fast(const ScoreArgs& a, int pmax, int split, int u, dim3 grid, hi
 template <int CPU, int HKV, bool EXACT>
 void dispatch_one_e(const ScoreArgs& a, int pmax, dim3 grid, hipStream_t st)
 {
-    // (eight query heads compared directly, without the plane kernel, were measured: 42.3 against
-    // 31.2 us for planes at the config 2 shape)
+    // (measured at the config 2 shape with eight query heads per KV head, 31.2 us with the plane
+    // kernel in front: the eight heads compared directly 42.3 us; the planes built by wave 0 of every
+    // workgroup behind a barrier 31.3 us - what the plane kernel costs, the scorer then loses)
     const bool dir = a.G == 1 || a.G == 2 || a.G == 4;
     note_score("block_score_one", CPU, HKV, dir, dir ? a.G : (pmax <= 5 ? pmax : 8), EXACT);
     if (a.G == 1) launch_score(block_score_one<CPU, HKV, true, 1, EXACT>, grid, 0, st, a);
