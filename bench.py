@@ -299,6 +299,35 @@ def graph_ms(torch, fn, reps=20, replays=5):
     return e0.elapsed_time(e1) / (reps * replays)
 
 
+def scorer_kernel_us(torch, fn, n=30):
+    """Mean duration in microseconds of the block-score dispatch inside fn(): the library attaches
+    the two events to that dispatch as its start / stop events (eager launches)."""
+    L = _lib_mod().lib()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in ev:  # creates the underlying hipEvent_t
+        a.record()
+        b.record()
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    for a, b in ev:
+        L.ucm_hamming_topk_set_profile_events(a.cuda_event, b.cuda_event)
+        fn()
+    torch.cuda.synchronize()
+    L.ucm_hamming_topk_set_profile_events(None, None)
+    ts = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+    return sum(ts[: max(1, n * 3 // 4)]) / max(1, n * 3 // 4)  # without the slowest quarter: eager launches after idle gaps
+
+
+def topk_split(torch, fn, ms, code_bytes):
+    """Operator-level and scorer-level HBM fractions of a top-k call that takes `ms` per call in a graph."""
+    sc = scorer_kernel_us(torch, fn)
+    return {"hbm_frac_operator": code_bytes / ms / 1e6 / HBM_PEAK_GBPS, "scorer_us": sc,
+            "scorer_hbm_frac": code_bytes / sc / 1e3 / HBM_PEAK_GBPS, "selection_and_rest_us": ms * 1e3 - sc,
+            "scorer_timing": "eager launches, dispatch start/stop events (a launch after an idle gap runs "
+                             "1-2 us longer than inside a graph; the committed kernel traces hold both)"}
+
+
 NO_GRAPH = False  # set by --no-graph: no HIP graph is captured anywhere and no hold kernel is queued
 
 ALL_LEGS = ("encoder", "prefix_rehash", "float_retrieval", "retrieval_shapes", "token_scores", "gather",
@@ -598,7 +627,9 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         ms = graph_ms(torch, lambda i: hamming_topk(q3, cache3, table3, lens3, 128))
         tok3 = int(lens3.sum())
         out["config3_ragged_topk128"] = {"tokens": tok3, "ms": ms, "tokens_per_s": tok3 / ms * 1e3,
-                                         "code_GBps": tok3 * HKV * WD * 4 / ms / 1e6}
+                                         "code_GBps": tok3 * HKV * WD * 4 / ms / 1e6,
+                                         **topk_split(torch, lambda: hamming_topk(q3, cache3, table3, lens3, 128), ms,
+                                                      tok3 * HKV * WD * 4)}
         del cache3, table3
         # config 5: MLA, one latent head, 128 q heads, 256-bit codes, 16 x 65536 tokens, 64-token blocks, top-128
         b5, ctx5, bs5, wd5 = 16, 65536, 64, 8
@@ -608,7 +639,9 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         q5 = codes((b5, 128, wd5))
         ms = graph_ms(torch, lambda i: hamming_topk(q5, cache5, table5, lens5, 128))
         out["config5_mla_topk128"] = {"tokens": b5 * ctx5, "ms": ms, "tokens_per_s": b5 * ctx5 / ms * 1e3,
-                                      "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6}
+                                      "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6,
+                                      **topk_split(torch, lambda: hamming_topk(q5, cache5, table5, lens5, 128), ms,
+                                                   b5 * ctx5 * wd5 * 4)}
         del cache5, table5
         # the reference's own latent-attention setting: 18-word codes (512 nope + 64 rope bits), 64 query
         # heads after its head reduction (128 heads, reduction 2), same 16 x 65536 tokens
@@ -617,6 +650,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         table6 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
         q6 = codes((b5, 64, wd6))
         ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6, table6, lens5, 128))
+        split6 = topk_split(torch, lambda: hamming_topk(q6, cache6, table6, lens5, 128), ms, b5 * ctx5 * wd6 * 4)
         ms_tok = graph_ms(torch, lambda i: hamming_score(cache6, q6, table6, lens5, ctx5, 0, 0, False), reps=5)
         # the whole decode step of that layout in one native call: both parts of 16 new keys into the cache,
         # both parts of the 16 x 64 query rows hashed, score, select
@@ -631,7 +665,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         out["mla_576bit_64heads"] = {"tokens": b5 * ctx5, "topk128_ms": ms, "token_scores_ms": ms_tok,
                                      "decode_step_ms": ms_step,
                                      "tokens_per_s": b5 * ctx5 / ms * 1e3,
-                                     "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6}
+                                     "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6, **split6}
         del cache6, table6
     if "token_scores" in legs:
         # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
