@@ -1015,18 +1015,55 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
     }
+    // The wave's 32 columns of W in operand layout (8 consecutive k of one column per lane and
+    // k-step).  16-byte aligned weights: lanes fetch 8 x 8 patches (eight 16-byte rows each),
+    // transpose them in registers and pass them through LDS - K / 16 loads per lane; fetching the
+    // operands directly takes eight 2-byte loads per k-step (K / 2 per lane: 256 at K = 512).
+    constexpr int KP = K + kPad;
+    __shared__ __align__(16) uint16_t wt[32 * KP];
+    V bv[KS];
+    if ((reinterpret_cast<uintptr_t>(a.w) & 15) == 0) {
+        constexpr int kPatches = (K / 8) * 4;
+        constexpr int kIters = (kPatches + 63) / 64;
+        const uint16_t* wslice = (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N + nt * 32;
+        u32x4 row[kIters][8];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
+        for (int it = 0; it < kIters; ++it) {
+            const int idx = (it * 64 + lane) % kPatches;  // lanes past the last patch repeat one
+            const uint16_t* src = wslice + (int64_t)((idx >> 2) * 8) * a.N + 8 * (idx & 3);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) bw[ks][i] = wsrc[(int64_t)(ks * 16 + kb * 8 + i) * a.N];
+            for (int i = 0; i < 8; ++i) row[it][i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * a.N);
+        }
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+            const int idx = (it * 64 + lane) % kPatches;
+            const int kq = idx >> 2, j = idx & 3;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                u32x4 o;
+                o.x = __builtin_amdgcn_perm(row[it][1][c >> 1], row[it][0][c >> 1], sel);
+                o.y = __builtin_amdgcn_perm(row[it][3][c >> 1], row[it][2][c >> 1], sel);
+                o.z = __builtin_amdgcn_perm(row[it][5][c >> 1], row[it][4][c >> 1], sel);
+                o.w = __builtin_amdgcn_perm(row[it][7][c >> 1], row[it][6][c >> 1], sel);
+                *reinterpret_cast<u32x4*>(wt + (8 * j + c) * KP + kq * 8) = o;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) bv[ks] = *reinterpret_cast<const V*>(wt + r * KP + ks * 16 + kb * 8);
+    } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) bw[ks][i] = wsrc[(int64_t)(ks * 16 + kb * 8 + i) * a.N];
+            __builtin_memcpy(&bv[ks], bw[ks], 16);
+        }
+    }
 
     f32x16 acc = acc_start();
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        V bv;
-        __builtin_memcpy(&bv, bw[ks], 16);
-        acc = Mfma<V>::run(bv, av[ks], acc);
-    }
+    for (int ks = 0; ks < KS; ++ks) acc = Mfma<V>::run(bv[ks], av[ks], acc);
     const uint32_t half = pack_half(acc);
     const uint32_t word = join_halves(kb ? half << 4 : half);
     if (row_ok && lane < 32) {
