@@ -93,6 +93,16 @@ int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int3
 int ucm_hash_encode_set_stream_threshold(int64_t rows);
 
 /*
+ * Diagnostic, no counterpart in the reference.  With 2, 4 or 8 heads of 128-bit codes side by side
+ * in a cache row the streaming kernel's waves exchange their codes through LDS and wait for one
+ * another with a bounded number of polls; a wave that reaches the bound goes on without waiting, so
+ * that a launch always ends, and the codes of that launch may then be wrong.  This returns how many
+ * waits have reached the bound on the current device since the library was loaded (0 in a healthy
+ * process; synchronises with the device), or a negative status.
+ */
+int64_t ucm_hash_encode_stream_timeouts(void);
+
+/*
  * Re-encodes keys that already sit in the paged KV cache (prefix-cache hit): replaces the
  * gather `kv_cache[0][0][prefix_block_ids]` followed by compute_hash_and_cache with the
  * prefix slot mapping (ucm/sparse/gsa_on_device/gsa_on_device.py:574-588; the slot rule is

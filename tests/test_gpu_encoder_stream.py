@@ -165,10 +165,20 @@ def test_streaming_kernel_dense_output_many_tiles(stream_everything):
     assert bool((outs[0][T:] == 0x5A5A5A5A).all())
 
 
+def test_no_exchange_wait_reached_its_bound():
+    """The waves of the streaming kernel wait for one another with bounded polls (a launch always
+    ends); after the encoder tests of this process no wait may have reached the bound."""
+    from ucm_amd import _lib
+
+    assert _lib.lib().ucm_hash_encode_stream_timeouts() == 0
+
+
 def test_cache_build_size_takes_the_streaming_kernel_by_default():
     """2^20 rows (131,072 tokens x 8 KV heads of 128 -> 128 bits): the default threshold; sampled
     rows against the oracle, everything against the tiled kernel."""
     from ucm_amd import _lib
+
+    timeouts_before = _lib.lib().ucm_hash_encode_stream_timeouts()
 
     L = _lib.lib()
     L.ucm_hash_encode_set_stream_threshold(0)
@@ -190,3 +200,4 @@ def test_cache_build_size_takes_the_streaming_kernel_by_default():
     assert torch.equal(got, ref)
     rows = np.sort(rng.choice(T, size=400, replace=False))
     _check_against_oracle(got.cpu().numpy().view(np.uint32), x, W, slots_np, BS, 1, rows)
+    assert L.ucm_hash_encode_stream_timeouts() == timeouts_before

@@ -687,6 +687,9 @@ __device__ __forceinline__ void lds_bump(int* counter)
     asm volatile("ds_add_u32 %0, %1" ::"v"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) int*)counter), "v"(one)
                  : "memory");
 }
+// Waits that ran into their limit, since the library was loaded (ucm_hash_encode_stream_timeouts).
+__device__ unsigned int g_stream_wait_timeouts = 0;
+
 // gave_up: set once a wait of this wave has run into the limit; the wave then never waits again,
 // so a kernel that has gone wrong ends after one limit per wave, not one per tile.
 __device__ __forceinline__ void lds_wait_at_least(const int* counter, int want, bool& gave_up)
@@ -696,6 +699,7 @@ __device__ __forceinline__ void lds_wait_at_least(const int* counter, int want, 
     while (lds_peek(counter) < want) {
         if (++spins > kSpinLimit) {
             gave_up = true;
+            if ((threadIdx.x & 63) == 0) atomicAdd(&g_stream_wait_timeouts, 1u);
             break;
         }
         __builtin_amdgcn_s_sleep(1);
@@ -1563,6 +1567,18 @@ extern "C" int ucm_hash_encode(const void* x, int x_dtype, int64_t T, int32_t H,
     a.w = w; a.n_w = n_w; a.heads_per_w = heads_per_w; a.N = N_bits;
     a.out = out; a.out_stride_t = out_stride_t; a.out_stride_h = out_stride_h;
     return encode_common(a, x_dtype, w_dtype, (hipStream_t)stream);
+}
+
+extern "C" int64_t ucm_hash_encode_stream_timeouts(void)
+{
+    ucm::clear_error();
+    unsigned int n = 0;
+    const hipError_t e = hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_stream_wait_timeouts), sizeof(n));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return ucm::fail(UCM_ERROR, "reading the timeout counter: %s", hipGetErrorString(e));
+    }
+    return (int64_t)n;
 }
 
 extern "C" int ucm_hash_encode_set_stream_threshold(int64_t rows)

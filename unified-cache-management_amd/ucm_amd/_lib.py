@@ -29,6 +29,7 @@ _SIGNATURES = {
     "ucm_hash_encode_cache": (ci, [vp, ci, i64, i32, i32, i64, i64, vp, ci, i32, i32, i32, vp, ci,
                                    vp, i64, i32, i64, i64, i64, vp]),
     "ucm_hash_encode_set_stream_threshold": (ci, [i64]),
+    "ucm_hash_encode_stream_timeouts": (i64, []),
     "ucm_hash_encode_paged": (ci, [vp, ci, i64, i32, i32, i32, i64, i64, i64, vp, i64, i64, vp, ci,
                                    i32, i32, i32, vp, i64, i64, i64, i64, vp]),
     "ucm_code_scatter": (ci, [vp, i64, i32, i32, i64, i64, vp, ci, vp, i64, i32, i64, i64, i64, vp]),
