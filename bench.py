@@ -631,6 +631,20 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
                                          **topk_split(torch, lambda: hamming_topk(q3, cache3, table3, lens3, 128), ms,
                                                       tok3 * HKV * WD * 4)}
         del cache3, table3
+        # config 2's cache with more query heads per KV head (64 / 8- and 128 / 8-head models): bit planes,
+        # four of them up to 15 query heads per KV head, five up to 31
+        cache2 = [codes((NB, BS, HKV, WD)) for _ in range(3)]  # rotated: 3 x 128 MiB exceed the last-level cache
+        table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, -1)
+        lens2 = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
+        more = {}
+        for hq in (64, 128):
+            q2 = codes((B, hq, WD))
+            ms2 = graph_ms(torch, lambda i: hamming_topk(q2, cache2[i % 3], table2, lens2, 64), reps=18)
+            more["%d_query_heads" % hq] = {"ms": ms2, "tokens_per_s": B * CTX / ms2 * 1e3,
+                                           "hbm_frac_operator": B * CTX * HKV * WD * 4 / ms2 / 1e6 / HBM_PEAK_GBPS,
+                                           "kernels": _lib_mod().last_dispatch()}
+        out["config2_shape_more_query_heads_top64"] = more
+        del cache2, table2
         # config 5: MLA, one latent head, 128 q heads, 256-bit codes, 16 x 65536 tokens, 64-token blocks, top-128
         b5, ctx5, bs5, wd5 = 16, 65536, 64, 8
         cache5 = codes((b5 * ctx5 // bs5, bs5, 1, wd5))
