@@ -28,7 +28,7 @@ TOPK_SHAPES = {
     "config3_one_long_request": (1, 32, 8, 4, 128, [70001], 128, {},
                                  "block_score_one<1,8,1,4,1>+select_group_kernel<4>"),
     "config5_two_requests": (2, 128, 1, 8, 64, [65536, 700], 128, {},
-                             "block_score_lanes64<8>+select_group_kernel<4>"),
+                             "block_score_dot64<2>+select_group_kernel<4>"),
     "plugin_reduced_physical": (2, 8, 8, 4, 128, [4096, 3000], 8,
                                 {"reduce_heads": True, "return_physical": True},
                                 "block_score_one<1,8,1,1,1>+select_wave_kernel<4>"),
@@ -108,9 +108,10 @@ def test_per_token_scorer_takes_its_kernels_and_matches_the_checker(name):
 @pytest.mark.parametrize("Wd,BS", [(8, 64), (18, 64), (16, 64), (8, 128), (18, 128)])
 @pytest.mark.parametrize("G", [3, 5, 8, 15, 16, 31, 33, 48, 49, 64, 100, 127, 128, 200])
 def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
-    """One KV head, a whole code per lane: the scorer builds the bit planes of the G query heads
-    itself (no plane kernel) when the blocks hold 64 tokens - for every G with 8-word codes, up to
-    128 heads with 16- and 18-word codes; larger blocks keep the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
+    """One KV head: the scorer reduces the G query heads to per-bit counts itself (no plane kernel)
+    when the blocks hold 64 tokens - for every G with 8-word codes (counts as nibble digits for the
+    4-bit dot product), up to 128 heads with 16- and 18-word codes (bit planes); larger blocks keep
+    the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
     that end inside a workgroup), table entries out of range, forced blocks."""
     from ucm_amd import _lib
     from ucm_amd.sparse import hamming_topk
@@ -130,7 +131,7 @@ def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
         idx, sc = hamming_topk(_dev(q), _dev(kc), _dev(table), _dev(lens), k, sink, recent)
         got = _lib.last_dispatch()
         if (Wd, BS) == (8, 64):
-            assert got.startswith("block_score_lanes64<%d>+" % planes)
+            assert got.startswith("block_score_dot64<%d>+" % (1 if G <= 15 else 2))
         elif BS == 64 and G <= 128:
             assert got.startswith("block_score_lanes_run<%d,%d>+" % (Wd // 2, planes))
         else:

@@ -1120,7 +1120,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
 // the planes built per workgroup was slower than the separate plane kernel: 22.7 against 16.1 +
 // 4.4 us at 16 x 65,536 tokens; a run of four blocks shares one build between 16 blocks: 18.6 us;
 // runs of two or eight blocks: 19.7 / 20.0 us.)
-constexpr int kLaneRun = 4;         // block_score_lanes64
 constexpr int kLanesRunBlocks = 4;  // block_score_lanes_run
 
 template <int LC, int GP>
@@ -1285,79 +1284,131 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     if (lane < run) a.scores[(int64_t)b * a.max_blocks + j0 + lane] = result;
 }
 
-// 64-token blocks of 8-word codes against one KV head whose G query heads enter as bit planes
-// (16 requests x 65,536 tokens, 128 query heads: 33 MB of codes, 4096 waves).  With one block per
-// wave a wave's life is three dependent round trips to memory around some 250 instructions, and a
-// separate launch builds the planes first.  Here
-//  * a wave owns kLaneRun consecutive blocks: their table entries arrive in one load and all of
-//    their codes are requested at once, a whole code per lane (two 16-byte loads at a lane stride of
-//    32 bytes: no transpose through LDS);
-//  * while those loads are in flight, wave 0 of the workgroup builds the request's bit planes from
-//    the query codes: lane (w, g) counts bit-sliced over up to 16 heads with a carry-save adder
-//    tree (11 full + 4 half adders for 16 words), three bit-sliced additions across the lane
-//    groups finish the counts, and the planes of word w go to LDS.  No plane kernel runs;
-//  * after one barrier every wave keeps the planes in registers (GP * 8 of them) for its blocks;
-//  * the minima of the run's blocks are reduced together (the first two butterfly steps halve the
-//    number of values per lane) and leave in one store.
+// 64-token blocks of 8-word codes against one KV head whose G query heads enter as per-bit counts
+// (16 requests x 65,536 tokens, 128 query heads: 33 MB of codes in 16,384 blocks of 2 KiB).
+//
+// Arithmetic.  With c_b the number of query heads whose bit b is set, the group-summed distance
+// of a cached code k is  sum_b c_b + G * popc(k) - 2 * sum_b k_b * c_b.  The last sum is a dot
+// product of the code's bits with small integers, and v_dot8_u32_u4 multiplies eight 4-bit pairs
+// per lane and instruction: k & (0x11111111 << j) holds bits j, j + 4, ... of a word as nibbles
+// of value 2^j, the counts of those eight bits enter as two nibble digits (c = lo + 16 * hi), and
+// an accumulator per (j, digit) carries the factor 2^j until the end of the code.  4 ands, 8 dot
+// products and one popcount per code word (13 operations) against 17 with eight bit planes; up
+// to 15 query heads need one digit (9 operations).  Exact: every intermediate is an integer far
+// below 2^32.
+//
+// Loads.  Lane l of a wave takes 16-byte pieces l and 64 + l of a block (two instructions of 1 KiB
+// contiguous each): half (l & 1) of the codes of tokens l >> 1 and 32 + (l >> 1); the two halves
+// of a code meet with one lane swap.  A lane's weight words (its four code words x four bit
+// residues x two digits) stay in 32 registers.  Whatever a wave asks of memory once the code
+// loads of the whole grid are under way is answered microseconds later, the smallest scalar read
+// included (measured: a table entry or a length requested behind the codes took 3 to 7 us).  So
+// every read that needs the kernel arguments only goes out first and together - the run's table
+// entries, the length, the builder's query words - and nothing at all is requested after the codes:
+// no kernel argument, no dispatch-packet field (a private array indexed at run time is kept in
+// LDS behind the flat thread id, which the compiler fetches from the dispatch packet right there).
+//
+// Weights.  Wave 0 of the workgroup builds them while the others wait: lane (w, g) counts word w
+// of heads g, g + 8, ... bit-sliced with a carry-save adder tree, three bit-sliced additions join
+// the lane groups, lane (w, (j, digit)) assembles one weight word and drops it into LDS.  No wave
+// requests codes before the builder holds its query words (first barrier): queued behind the
+// codes of the 31 other waves of its compute unit they took 5 us (median), and every wave of the
+// workgroup then stood at the barrier that long.  The second barrier hands the weights over; both
+// are bare s_barrier instructions - __syncthreads() makes a wave wait for its own loads in flight,
+// i.e. for all of its codes.
+constexpr int kDotRun = 4;    // blocks per wave
+constexpr int kDotWaves = 8;  // waves per workgroup
 
-template <int GP>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void block_score_lanes64(ScoreArgs a)
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ int dpp_min_step(int x)
 {
-    constexpr int WD = 8;
-    __shared__ __align__(16) uint32_t pl[WD * 8];  // pl[w * 8 + p]
+    const int t = __builtin_amdgcn_update_dpp(x, x, CTRL, ROWMASK, 0xf, false);
+    return t < x ? t : x;
+}
+// Minimum over the 64 lanes, valid in lane 63: butterflies inside a row of 16 lanes, then the
+// last lane of a row broadcast into the next row(s).
+__device__ __forceinline__ int wave_min_lane63(int x)
+{
+    x = dpp_min_step<0xB1, 0xf>(x);   // quad_perm [1,0,3,2]
+    x = dpp_min_step<0x4E, 0xf>(x);   // quad_perm [2,3,0,1]
+    x = dpp_min_step<0x141, 0xf>(x);  // row_half_mirror
+    x = dpp_min_step<0x140, 0xf>(x);  // row_mirror
+    x = dpp_min_step<0x142, 0xa>(x);  // row_bcast15 into rows 1 and 3
+    x = dpp_min_step<0x143, 0xc>(x);  // row_bcast31 into rows 2 and 3
+    return x;
+}
+
+template <int ND>
+__global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs a)
+{
+    constexpr int RUN = kDotRun;
+    __shared__ __align__(16) uint32_t wl[64];  // weight word [w][j][digit]
     __shared__ int base_s;
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
-    const int j0 = (blockIdx.x * (kThreads / kWave) + wid) * kLaneRun;
-    // the run's table entries: lane i holds block j0 + i (requested before the length is looked at)
-    int my_entry = 0;
+    const int j0 = (blockIdx.x * kDotWaves + wid) * RUN;
+    // round 1: the reads that need the kernel arguments only
+    const int len = a.lens[b];
+    int my_entry;  // lane i: table entry of block j0 + i
     {
-        const int j = j0 + (lane < kLaneRun ? lane : 0);
+        const int j = j0 + (lane & 7);
         const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
         if (a.table) my_entry = a.table[(int64_t)b * a.table_stride + jc];
         else my_entry = b * a.max_blocks + jc;
     }
-    const int len = a.lens[b];
-    int nblk = len > 0 ? (len + 63) >> 6 : 0;
-    if (nblk > a.max_blocks) nblk = a.max_blocks;
-    if ((int)blockIdx.x * (kThreads / kWave) * kLaneRun >= nblk) return;  // the whole workgroup
-    const int run = nblk - j0 < kLaneRun ? nblk - j0 : kLaneRun;  // <= 0: nothing to score
-    // a whole code per lane; blocks past the run re-read its first block (never used)
-    u32x4 v[kLaneRun][2];
-    auto request_codes = [&]() {
+    uint32_t x[16];
+    const int qw = lane & 7, qg = lane >> 3;
+    const uint32_t* qb = a.q + b * a.q_stride_b + qw;
+    const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
+    const int G = a.G;
+    if (wid == 0) {
 #pragma unroll
-        for (int i = 0; i < kLaneRun; ++i) {
-            int64_t pb = __shfl(my_entry, (run > 0 && i < run) ? i : 0);
-            if (pb < 0 || pb >= a.NB) pb = 0;  // scored as -1 below
-            const u32x4* src = reinterpret_cast<const u32x4*>(a.kc + pb * a.ks_block) + 2 * lane;
-            v[i][0] = code_load(src);
-            v[i][1] = code_load(src + 1);
+        for (int t = 0; t < 16; ++t) {
+            const int h = t * 8 + qg;  // heads past the group re-read the last one, as zero
+            x[t] = qb[(h < G ? h : G - 1) * qs];
         }
-    };
-    if (wid != 0) {
-        request_codes();
-    } else {
-        // lane (w = lane & 7, g = lane >> 3) takes word w of heads g, g + 8, g + 16, ...; the query
-        // words are requested before the codes, so that waiting for them leaves the codes in flight
-        const int w = lane & 7, g = lane >> 3;
-        const uint32_t* qb = a.q + b * a.q_stride_b + w;
-        const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
+    }
+    // everything the rest of the kernel takes from its arguments, now
+    const int64_t NB = a.NB, ks_block = a.ks_block;
+    const uint32_t* kc = a.kc;
+    const int sink = a.sink, recent = a.recent, max_blocks = a.max_blocks;
+    int32_t* scores = a.scores;
+    asm volatile("" ::"s"(sink), "s"(recent), "s"(scores), "s"(NB), "s"(G), "s"(max_blocks));
+    int nblk = len > 0 ? (len + 63) >> 6 : 0;
+    if (nblk > max_blocks) nblk = max_blocks;
+    if ((int)blockIdx.x * kDotWaves * RUN >= nblk) return;  // the whole workgroup
+    const int run = nblk - j0 < RUN ? nblk - j0 : RUN;  // <= 0: nothing to score
+    int entry[RUN];
+#pragma unroll
+    for (int i = 0; i < RUN; ++i) entry[i] = __builtin_amdgcn_readlane(my_entry, i);
+    if (wid == 0) {
+        uint32_t o = 0;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) o |= x[t];
+        asm volatile("" ::"v"(o));  // the query words are here
+    }
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    // round 2: the codes
+    u32x4 v[RUN][2];
+#pragma unroll
+    for (int i = 0; i < RUN; ++i) {
+        int64_t pb = entry[i];
+        if (pb < 0 || pb >= NB) pb = 0;  // scored as -1 below
+        const u32x4* src = reinterpret_cast<const u32x4*>(kc + pb * ks_block);
+        v[i][0] = code_load(src + lane);
+        v[i][1] = code_load(src + 64 + lane);
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (wid == 0) {
         uint32_t acc[8];
 #pragma unroll
         for (int p = 0; p < 8; ++p) acc[p] = 0;
-        // 128 heads at a time; the first round is straight-line code with the code loads in its
-        // middle, so that the waits for the query words are counted exactly and leave the codes
-        // in flight (a load under a condition makes every later wait cover it)
-        auto add_heads = [&](int h0, bool first) __attribute__((always_inline)) {
-            uint32_t x[16], n[5];
+        auto add16 = [&](int h0) __attribute__((always_inline)) {
+            uint32_t n[5];
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                const int h = h0 + t * 8 + g;  // heads past the group re-read the last one, as zero
-                x[t] = qb[(h < a.G ? h : a.G - 1) * qs];
-            }
-            if (first) request_codes();
-#pragma unroll
-            for (int t = 0; t < 16; ++t) x[t] = (h0 + t * 8 + g < a.G) ? x[t] : 0u;
+            for (int t = 0; t < 16; ++t) x[t] = (h0 + t * 8 + qg < G) ? x[t] : 0u;
             count16(x, n);
             uint32_t cy = 0;
 #pragma unroll
@@ -1369,14 +1420,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
                 cy = c2;
             }
         };
-        add_heads(0, true);
-        for (int h0 = 128; h0 < a.G; h0 += 128) add_heads(h0, false);
+        // straight-line code for the first 128 heads: a load inside the loop below makes the
+        // compiler wait for the codes at the loop's head
+        add16(0);
+        for (int h0 = 128; h0 < G; h0 += 128) {
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int h = h0 + t * 8 + qg;
+                x[t] = qb[(h < G ? h : G - 1) * qs];
+            }
+            add16(h0);
+        }
         // the eight lane groups add up (every lane ends with the full counts of its word)
 #pragma unroll
         for (int st = 8; st < kWave; st <<= 1) {
             uint32_t o[8], cy = 0;
 #pragma unroll
-            for (int p = 0; p < 8; ++p) o[p] = __shfl_xor(acc[p], st);
+            for (int p = 0; p < 8; ++p) o[p] = __builtin_amdgcn_ds_bpermute((lane ^ st) << 2, acc[p]);
 #pragma unroll
             for (int p = 0; p < 8; ++p) {
                 uint32_t sum, c2;
@@ -1388,77 +1448,69 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4))
         int c = 0;
 #pragma unroll
         for (int p = 0; p < 8; ++p) c += __popc(acc[p]) << p;
-        c += __shfl_xor(c, 1);
-        c += __shfl_xor(c, 2);
-        c += __shfl_xor(c, 4);
-        if (lane < 8) {
-            u32x4* dst = reinterpret_cast<u32x4*>(pl + lane * 8);
-            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
-            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
+        c += __builtin_amdgcn_ds_bpermute((lane ^ 1) << 2, c);
+        c += __builtin_amdgcn_ds_bpermute((lane ^ 2) << 2, c);
+        c += __builtin_amdgcn_ds_bpermute((lane ^ 4) << 2, c);
+        // lane (w, g = 2 * j + digit) assembles weight word [w][j][digit]: nibble n = that digit of
+        // the count of bit 4 * n + j (both digits are computed, one is kept: no run-time index)
+        const int jj = qg >> 1;
+        uint32_t r0 = 0, r1 = 0;
+#pragma unroll
+        for (int pp = 0; pp < 4; ++pp) {
+            r0 |= ((acc[pp] >> jj) & 0x11111111u) << pp;
+            r1 |= ((acc[4 + pp] >> jj) & 0x11111111u) << pp;
         }
+        wl[qw * 8 + qg] = (qg & 1) ? r1 : r0;
         if (lane == 0) base_s = c;  // sum over all code bits of the per-bit counts
     }
-    __syncthreads();
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (run <= 0) return;
+    u32x4 M[8];  // [w][j / 2] -> {lo, hi of j even; lo, hi of j odd} for the lane's four code words
+    {
+        const u32x4* src = reinterpret_cast<const u32x4*>(wl + (lane & 1) * 32);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) M[i] = src[i];
+    }
     const int base = base_s;
-    uint32_t P[WD][GP];
+    const int full = G * 256;
+    int result = 0;  // lane i: score of block j0 + i
 #pragma unroll
-    for (int w = 0; w < WD; ++w) {
-        const u32x4 lo = *reinterpret_cast<const u32x4*>(pl + w * 8);
-        const u32x4 hi = *reinterpret_cast<const u32x4*>(pl + w * 8 + 4);
+    for (int i = 0; i < RUN; ++i) {
+        int dd[2];
 #pragma unroll
-        for (int p = 0; p < GP; ++p) P[w][p] = p < 4 ? lo[p] : hi[p - 4];
-    }
-    int d[kLaneRun];
+        for (int h = 0; h < 2; ++h) {
+            int pk = 0;
+            uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < kLaneRun; ++i) {
-        int acc[GP], pk = 0;
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t k = v[i][h][w];
+                pk = popc_add(k, pk);
 #pragma unroll
-        for (int p = 0; p < GP; ++p) acc[p] = 0;
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t e = k & (0x11111111u << j);
+                    lo[j] = __builtin_amdgcn_udot8(e, M[w * 2 + (j >> 1)][(j & 1) * 2], lo[j], false);
+                    if (ND > 1) hi[j] = __builtin_amdgcn_udot8(e, M[w * 2 + (j >> 1)][(j & 1) * 2 + 1], hi[j], false);
+                }
+            }
+            uint32_t t[4];
 #pragma unroll
-        for (int w = 0; w < WD; ++w) {
-            const uint32_t k = v[i][w >> 2][w & 3];
-            pk = popc_add(k, pk);
-#pragma unroll
-            for (int p = 0; p < GP; ++p) acc[p] = popc_add(k & P[w][p], acc[p]);
+            for (int j = 0; j < 4; ++j) t[j] = ND > 1 ? lo[j] + (hi[j] << 4) : lo[j];
+            const uint32_t x8 = (((((t[0] << 1) + t[1]) << 1) + t[2]) << 1) + t[3];  // 8 * sum_b k_b * c_b
+            dd[h] = G * pk - (int)(x8 >> 2);
+            dd[h] += __builtin_amdgcn_update_dpp(0, dd[h], 0xB1, 0xf, 0xf, true);  // the code's other half
         }
-        int x = 0;
-#pragma unroll
-        for (int p = 0; p < GP; ++p) x += acc[p] << p;
         const int pos0 = (j0 + i) << 6;
-        d[i] = (i < run && pos0 + lane < len) ? base + a.G * pk - 2 * x : kInf;
+        const int t0 = pos0 + (lane >> 1);
+        int d = (i < run && t0 < len) ? dd[0] : kInf;
+        const int d1 = (i < run && t0 + 32 < len) ? dd[1] : kInf;
+        d = d1 < d ? d1 : d;
+        const int m = __builtin_amdgcn_readlane(wave_min_lane63(d), 63) + base;
+        const int ntok = (64 < len - pos0) ? 64 : len - pos0;
+        const bool forced = (pos0 < sink) || (pos0 + ntok > len - recent);
+        const int sc = (entry[i] < 0 || entry[i] >= NB) ? -1 : (forced ? full : full - m);
+        if (lane == i) result = sc;
     }
-    // minima of the four blocks together: after the steps over lane bits 0 and 1 a lane holds one
-    // value, that of block 2 * (lane & 1) + ((lane >> 1) & 1)
-    static_assert(kLaneRun == 4, "the reduction below is written for runs of four blocks");
-    const bool odd = lane & 1, up = lane & 2;
-    int ka = odd ? d[2] : d[0], kb = odd ? d[3] : d[1];
-    {
-        const int oa = __shfl_xor(odd ? d[0] : d[2], 1), ob = __shfl_xor(odd ? d[1] : d[3], 1);
-        ka = oa < ka ? oa : ka;
-        kb = ob < kb ? ob : kb;
-    }
-    int m = up ? kb : ka;
-    {
-        const int o = __shfl_xor(up ? ka : kb, 2);
-        m = o < m ? o : m;
-    }
-#pragma unroll
-    for (int st = 4; st < kWave; st <<= 1) {
-        const int o = __shfl_xor(m, st);
-        m = o < m ? o : m;
-    }
-    const int i = 2 * (lane & 1) + ((lane >> 1) & 1);
-    const int entry = __shfl(my_entry, i);
-    if (lane < 4) {
-        if (i < run) {
-            const int pos0 = (j0 + i) << 6;
-            const int ntok = (64 < len - pos0) ? 64 : len - pos0;
-            const bool forced = (pos0 < a.sink) || (pos0 + ntok > len - a.recent);
-            const int full = a.G * 32 * a.Wd;
-            a.scores[(int64_t)b * a.max_blocks + j0 + i] = (entry < 0 || entry >= a.NB) ? -1 : (forced ? full : full - m);
-        }
-    }
+    if (lane < run) scores[(int64_t)b * max_blocks + j0 + lane] = result;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -2571,7 +2623,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         while ((1 << pmax) <= a.G) ++pmax;  // bit planes that hold the counts 0..G
         if (pmax < 4) pmax = 4;
         const bool direct = a.G == 1 || a.G == 2 || a.G == 4;
-        // 64-token blocks of 8-word codes: the scorer builds the planes itself
+        // 64-token blocks of 8-word codes: the scorer builds its weights (per-bit counts) itself
         const bool planes_inside = !direct && Wd == 8 && BS == 64 && pmax <= 8 && lanes_layout(a, k_cache, direct);
         // the other code-per-lane shapes build them in wave 0 of every workgroup (up to 128 query heads)
         const bool planes_in_lanes = !direct && !planes_inside && a.G <= 128 && BS == 64 && (Wd == 16 || Wd == 18) &&
@@ -2587,14 +2639,18 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         // 18-word codes (and 8- or 16-word codes with bit planes) in blocks of 64, 128, ...
         // tokens: a whole code per lane
         if (planes_inside) {
-            note_score("block_score_lanes64", pmax);
-            const dim3 g64((unsigned)ucm::ceil_div(max_blocks, (kThreads / kWave) * kLaneRun), (unsigned)B);
-            switch (pmax) {
-                case 4: launch_score(block_score_lanes64<4>, g64, 0, st, a); break;
-                case 5: launch_score(block_score_lanes64<5>, g64, 0, st, a); break;
-                case 6: launch_score(block_score_lanes64<6>, g64, 0, st, a); break;
-                case 7: launch_score(block_score_lanes64<7>, g64, 0, st, a); break;
-                default: launch_score(block_score_lanes64<8>, g64, 0, st, a); break;
+            // one nibble digit of the per-bit counts up to 15 query heads, two up to 255
+            const int nd = a.G <= 15 ? 1 : 2;
+            note_score("block_score_dot64", nd);
+            const dim3 g64((unsigned)ucm::ceil_div(max_blocks, kDotWaves * kDotRun), (unsigned)B);
+            ++g_note.score_launches;
+            const dim3 threads(kDotWaves * kWave);
+            if (g_prof_before && g_prof_after) {
+                if (nd == 1) hipExtLaunchKernelGGL(block_score_dot64<1>, g64, threads, 0, st, g_prof_before, g_prof_after, 0, a);
+                else hipExtLaunchKernelGGL(block_score_dot64<2>, g64, threads, 0, st, g_prof_before, g_prof_after, 0, a);
+            } else {
+                if (nd == 1) hipLaunchKernelGGL(block_score_dot64<1>, g64, threads, 0, st, a);
+                else hipLaunchKernelGGL(block_score_dot64<2>, g64, threads, 0, st, a);
             }
         } else if (planes_in_lanes) {
             note_score("block_score_lanes_run", Wd / 2, pmax);
