@@ -1226,7 +1226,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
             dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
         }
     }
-    __syncthreads();
+    // a bare barrier: __syncthreads() would make every wave wait for its codes in flight
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (run <= 0) return;
     // sum over all code bits of the per-bit counts, from the planes in LDS
     int base = 0;
