@@ -26,6 +26,7 @@ extern "C" {
 #define UCM_EPARAM       (-50000)
 #define UCM_EOOM         (-50001)
 #define UCM_EOSERROR     (-50002)
+#define UCM_ERETRY       (-50004)
 #define UCM_ENOOBJ       (-50005)
 #define UCM_EUNSUPPORTED (-50008)
 #define UCM_ETIMEOUT     (-50010)
@@ -88,19 +89,33 @@ int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int3
  * Tuning and test hook, no counterpart in the reference.  Inputs of at least `rows` rows (tokens x
  * heads) with 64 or 128 input dimensions and 64 or 128 hash bits take the streaming kernel
  * (persistent waves, projection matrix in registers, rows loaded straight into LDS); smaller ones
- * take the tiled kernel.  Both give identical codes.  rows <= 0 restores the default (2^20).
+ * take the tiled kernel.  Both give identical codes.  rows <= 0 restores the default (2^20).  The
+ * setting belongs to the calling thread: encodes issued by other threads are not affected.
  */
 int ucm_hash_encode_set_stream_threshold(int64_t rows);
 
 /*
- * Diagnostic, no counterpart in the reference.  With 2, 4 or 8 heads of 128-bit codes side by side
- * in a cache row the streaming kernel's waves exchange their codes through LDS and wait for one
- * another with a bounded number of polls; a wave that reaches the bound goes on without waiting, so
- * that a launch always ends, and the codes of that launch may then be wrong.  This returns how many
- * waits have reached the bound on the current device since the library was loaded (0 in a healthy
- * process; synchronises with the device), or a negative status.
+ * The streaming kernel's time-out contract, no counterpart in the reference.  With 2, 4 or 8 heads
+ * of 128-bit codes side by side in a cache row the streaming kernel's waves exchange their codes
+ * through LDS and wait for one another with a bounded number of polls; a wave that reaches the bound
+ * goes on without waiting, so that a launch always ends.  The codes that launch wrote are then
+ * undefined.  The wave reports it in a word of pinned host memory, and from then on EVERY encode entry
+ * point (ucm_hash_encode, ucm_hash_encode_cache, ucm_hash_encode_paged and the decode-step calls that
+ * encode) returns UCM_ERROR on that device, with a ucm_last_error() text that says so, before it
+ * launches anything - a host-side read, no device synchronisation.  The failed launch itself has
+ * returned UCM_OK (it ran later, asynchronously): a caller that must know before it uses the codes
+ * synchronises the stream and calls ucm_hash_encode_stream_timeouts().  After rebuilding the codes
+ * the caller acknowledges with ucm_hash_encode_clear_stream_timeouts().
+ *
+ * ucm_hash_encode_stream_timeouts: how many waits have reached the bound on the current device since
+ * the library was loaded (0 in a healthy process; synchronises with the device), or a negative status.
+ * ucm_hash_encode_clear_stream_timeouts: clears the current device's latch (not the count).
+ * ucm_hash_encode_debug_trip_stream_latch: sets the current device's latch from the host, as a timed-out
+ * wave would - for tests of the error path; no kernel is involved.
  */
 int64_t ucm_hash_encode_stream_timeouts(void);
+int ucm_hash_encode_clear_stream_timeouts(void);
+int ucm_hash_encode_debug_trip_stream_latch(void);
 
 /*
  * Re-encodes keys that already sit in the paged KV cache (prefix-cache hit): replaces the
@@ -621,7 +636,12 @@ int ucm_posix_store_dump(ucm_posix_store_t* store, const uint8_t* block_ids,
 int ucm_posix_store_load(ucm_posix_store_t* store, const uint8_t* block_ids,
                          const uint64_t* shard_idx, void* const* host_addrs, size_t n,
                          int64_t* task);
-/* PosixStore::Check / Wait (posix_store.cc:94-103): as ucm_cache_store_check / _wait. */
+/* PosixStore::Check / Wait (posix_store.cc:94-103): as ucm_cache_store_check / _wait.  A wait that
+ * times out does not return while a file worker may still read or write the task's buffers: it waits
+ * up to four more time-outs for them to come back (queued units are skipped).  Normally it then
+ * returns UCM_ETIMEOUT and forgets the task; if the workers are still stuck (a dead mount) it
+ * returns UCM_ERETRY, keeps the task, and the buffers must not be reused or freed until a later wait
+ * on the same task has returned something else. */
 int ucm_posix_store_check(ucm_posix_store_t* store, int64_t task, int32_t* finished);
 int ucm_posix_store_wait(ucm_posix_store_t* store, int64_t task);
 /* One turn of the collector's loop now (ShardGarbageCollector::GCCheckLoop, shard_gc.cc:85-108):

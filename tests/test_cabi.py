@@ -95,3 +95,44 @@ def test_no_product_code_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower() or f == "README.md", f
+
+
+def test_encoder_timeout_latch_refuses_further_encodes_until_cleared():
+    """A streaming encode whose bounded LDS wait gave up leaves undefined codes behind; from then on
+    every encode entry point on that device must fail with UCM_ERROR and say why, before it touches
+    the device, until the caller acknowledges.  The latch is tripped from the host here (what a
+    timed-out wave does from the device), so the whole error path runs without a GPU."""
+    import numpy as np
+
+    from ucm_amd import _lib
+
+    lib = _lib.lib()
+    x = np.zeros((4, 1, 128), np.uint16)
+    w = np.zeros((128, 128), np.uint16)
+    out = np.zeros((4, 1, 4), np.uint32)
+    cache = np.zeros((1, 4, 1, 4), np.uint32)
+    slots = np.arange(4, dtype=np.int32)
+
+    def encode():
+        return lib.ucm_hash_encode(x.ctypes.data, _lib.DT_BF16, 4, 1, 128, 128, 128, w.ctypes.data, _lib.DT_BF16,
+                                   1, 1, 128, out.ctypes.data, 4, 4, None)
+
+    def encode_cache():
+        return lib.ucm_hash_encode_cache(x.ctypes.data, _lib.DT_BF16, 4, 1, 128, 128, 128, w.ctypes.data,
+                                         _lib.DT_BF16, 1, 1, 128, slots.ctypes.data, 0, cache.ctypes.data,
+                                         1, 4, 16, 4, 4, None)
+
+    assert lib.ucm_hash_encode_clear_stream_timeouts() == _lib.UCM_OK
+    try:
+        assert lib.ucm_hash_encode_debug_trip_stream_latch() == _lib.UCM_OK
+        for call in (encode, encode_cache):
+            assert call() == _lib.UCM_ERROR
+            msg = _lib.last_error()
+            assert "gave up waiting" in msg and "ucm_hash_encode_clear_stream_timeouts" in msg
+        # sticky: a second call fails the same way
+        assert encode() == _lib.UCM_ERROR
+    finally:
+        assert lib.ucm_hash_encode_clear_stream_timeouts() == _lib.UCM_OK
+    # acknowledged: the call gets past the latch (whatever it returns without a GPU, it is not the latch)
+    encode()
+    assert "gave up waiting" not in _lib.last_error()

@@ -201,3 +201,22 @@ def test_cache_build_size_takes_the_streaming_kernel_by_default():
     rows = np.sort(rng.choice(T, size=400, replace=False))
     _check_against_oracle(got.cpu().numpy().view(np.uint32), x, W, slots_np, BS, 1, rows)
     assert L.ucm_hash_encode_stream_timeouts() == timeouts_before
+
+
+def test_tripped_timeout_latch_surfaces_in_the_host_mirror():
+    """The latch a timed-out wave sets (tripped from the host here) makes the encoder object raise
+    instead of returning codes, and clearing it restores the operator."""
+    from ucm_amd import _lib
+    from ucm_amd.sparse import HashEncoder
+
+    L = _lib.lib()
+    enc = HashEncoder(128, 128, torch.bfloat16, torch.device("cuda"))
+    x = torch.randn(64, 128, device="cuda", dtype=torch.bfloat16)
+    good = enc.compute_hash(x).clone()
+    assert L.ucm_hash_encode_debug_trip_stream_latch() == _lib.UCM_OK
+    try:
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            enc.compute_hash(x)
+    finally:
+        assert L.ucm_hash_encode_clear_stream_timeouts() == _lib.UCM_OK
+    assert torch.equal(enc.compute_hash(x), good)

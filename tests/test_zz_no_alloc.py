@@ -92,3 +92,52 @@ def test_static_entry_point_rejects_shapes_beyond_its_scratch():
                                    out.data_ptr(), None, _lib.stream_ptr(dq.device))
     assert rc == _lib.UCM_EPARAM
     assert b"scratch" in L.ucm_last_error()
+
+
+def test_static_entry_point_allocates_nothing_and_replays_in_a_graph():
+    """What the entry point exists for: after a first call on the device (which looks up the scratch
+    array's address) a call takes no device memory - free memory is the same before and after -
+    and can be captured into a HIP graph whose replays, with eager work and synchronisations in
+    between, all give the workspace entry point's result."""
+    from ucm_amd import _lib
+
+    L = _lib.lib()
+    seed, B, Hq, Hkv, Wd, BS, lens, k, flags = MLA_CALLS[0]
+    q, kc, table, lens = make_paged_case(seed, B, Hq, Hkv, Wd, BS, lens)
+    ref_i, ref_s = _call(False, q, kc, table, lens, k, flags)
+    _call(True, q, kc, table, lens, k, flags)  # warm-up: address look-up, code object load
+
+    NB, mb = kc.shape[0], table.shape[1]
+    dq, dk, dt, dl = _dev(q.view(np.int32)), _dev(kc.view(np.int32)), _dev(table), _dev(lens)
+    idx = torch.full((B, 1, k), -7, dtype=torch.int32, device="cuda")
+    sc = torch.full((B, 1, k), -7, dtype=torch.int32, device="cuda")
+
+    def launch(stream_ptr):
+        _lib.check(L.ucm_hamming_topk_static(
+            dq.data_ptr(), Hq * Wd, Wd, dk.data_ptr(), NB, BS, Hkv, Wd, BS * Hkv * Wd, Hkv * Wd, Wd,
+            dt.data_ptr(), mb, mb, dl.data_ptr(), B, Hq, k, 0, 0, flags, idx.data_ptr(), sc.data_ptr(),
+            stream_ptr))
+
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    launch(_lib.stream_ptr(dq.device))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert np.array_equal(idx.cpu().numpy(), ref_i) and np.array_equal(sc.cpu().numpy(), ref_s)
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            launch(side.cuda_stream)
+    for rep in range(3):
+        idx.fill_(-7)
+        sc.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(idx.cpu().numpy(), ref_i), rep
+        assert np.array_equal(sc.cpu().numpy(), ref_s), rep
+        # eager work of the program's own between the replays
+        got_i, _ = _call(True, q, kc, table, lens, k, flags)
+        assert np.array_equal(got_i, ref_i)

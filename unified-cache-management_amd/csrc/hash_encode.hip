@@ -21,6 +21,7 @@
 #include <hip/hip_fp16.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "common.h"
 
@@ -69,6 +70,9 @@ struct EncArgs {
     int gmean;
     int64_t x_stride_g;
     int bs_shift;  // log2(BS) when BS is a power of two, else -1
+    // streaming kernel: a word in pinned host memory that a wave sets when one of its bounded waits
+    // gives up; the host reads it without touching the device (see stream_latch_tripped())
+    unsigned int* timeout_flag;
 };
 
 __device__ __forceinline__ int weight_index(const EncArgs& a, int h)
@@ -653,7 +657,8 @@ __device__ __forceinline__ void stream_wait_lds()
 // Two counters per ring slot: pub (codes handed in) and done (tiles stored); plain LDS
 // operations of one wave complete in order, so a counter update that follows the data in program
 // order is seen after the data.  Every wait is bounded: a wave that does not see its counter
-// move gives up waiting and goes on (the results are then wrong, the kernel still ends).
+// move gives up waiting and goes on: the kernel still ends, the codes of that launch are undefined,
+// and the host refuses further encodes on the device until the caller has acknowledged it.
 // 2.1 GB of keys: 403-411 us against 455-470 us = 5.6 TB/s of algorithmic bytes.  What made earlier
 // forms of this slower than the plain stores (476-545 us): counters as volatile / atomic C++
 // accesses (each waits for the row loads in flight), spilled registers reloaded inside the loop
@@ -662,9 +667,14 @@ __device__ __forceinline__ void stream_wait_lds()
 constexpr int kRing = 5;
 constexpr int kCombDelay = 2;
 constexpr int ring_slot_bytes(int hc) { return 512 * hc + 128; }  // 32 rows x hc heads x 16 bytes, then the rows' 32 slots
+// the two counters per ring slot, padded so that the next stream's ring starts 16-byte aligned
+// (the ring is read and written with 16-byte LDS operations)
+constexpr int kRingCounterBytes = 48;
+static_assert(2 * kRing * (int)sizeof(int) <= kRingCounterBytes && kRingCounterBytes % 16 == 0, "counter area");
+constexpr int ring_stream_bytes(int hc) { return kRing * ring_slot_bytes(hc) + kRingCounterBytes; }
 constexpr int ring_lds_bytes(int hc)  // rings and counters of the 8 / hc streams of a workgroup
 {
-    return hc ? (8 / hc) * (kRing * ring_slot_bytes(hc) + 2 * kRing * (int)sizeof(int)) : 0;
+    return hc ? (8 / hc) * ring_stream_bytes(hc) : 0;
 }
 constexpr int kSpinLimit = 1 << 22;  // some tenths of a second
 
@@ -691,15 +701,20 @@ __device__ __forceinline__ void lds_bump(int* counter)
 __device__ unsigned int g_stream_wait_timeouts = 0;
 
 // gave_up: set once a wait of this wave has run into the limit; the wave then never waits again,
-// so a kernel that has gone wrong ends after one limit per wave, not one per tile.
-__device__ __forceinline__ void lds_wait_at_least(const int* counter, int want, bool& gave_up)
+// so a kernel that has gone wrong ends after one limit per wave, not one per tile.  The codes of
+// such a launch are undefined; `flag` (pinned host memory) tells the host, which refuses every
+// later encode on the device until the caller has acknowledged it.
+__device__ __forceinline__ void lds_wait_at_least(const int* counter, int want, bool& gave_up, unsigned int* flag)
 {
     if (gave_up) return;
     int spins = 0;
     while (lds_peek(counter) < want) {
         if (++spins > kSpinLimit) {
             gave_up = true;
-            if ((threadIdx.x & 63) == 0) atomicAdd(&g_stream_wait_timeouts, 1u);
+            if ((threadIdx.x & 63) == 0) {
+                atomicAdd(&g_stream_wait_timeouts, 1u);
+                if (flag) __hip_atomic_store(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
             break;
         }
         __builtin_amdgcn_s_sleep(1);
@@ -833,7 +848,8 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
 
     // this stream's ring and its counters (a workgroup holds 8 / HC streams)
     constexpr int kSlotBytes = ring_slot_bytes(HCn);
-    constexpr int kStreamRing = kRing * kSlotBytes + 2 * kRing * (int)sizeof(int);
+    constexpr int kStreamRing = ring_stream_bytes(HCn);
+    static_assert(kStreamRing % 16 == 0, "every stream's ring starts 16-byte aligned");
     uint8_t* const ring = stream_lds + (size_t)kStreamWaves * 2 * kBufBytes + (COMB ? (wave / HCn) * kStreamRing : 0);
     int* const pub = reinterpret_cast<int*>(ring + kRing * kSlotBytes);
     int* const done = pub + kRing;
@@ -844,7 +860,7 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
     // the wave whose turn it is stores tile j of this stream as 32 whole cache rows
     auto store_tile = [&](int j) {
         const int s = j % kRing;
-        lds_wait_at_least(pub + s, HCn * (j / kRing + 1), gave_up);
+        lds_wait_at_least(pub + s, HCn * (j / kRing + 1), gave_up, a.timeout_flag);
         asm volatile("" ::: "memory");
         const uint8_t* slot_base = ring + s * kSlotBytes;
 #pragma unroll
@@ -868,7 +884,7 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
             if (prev_idx < 0) return;
             const int s = prev_idx % kRing, gen = prev_idx / kRing;
             // the slot's previous tile has been stored: normally known from the read in step()
-            if (gen > 0 && done_seen < gen) lds_wait_at_least(done + s, gen, gave_up);
+            if (gen > 0 && done_seen < gen) lds_wait_at_least(done + s, gen, gave_up, a.timeout_flag);
             asm volatile("" ::: "memory");
             uint8_t* slot_base = ring + s * kSlotBytes;
             if (lane < 32) {
@@ -1245,7 +1261,7 @@ bool mfma_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 // the tiled kernel (65,536 rows: 14.8 against 12.4 us; 1M rows: 67.6 against 71.8 us; 4M rows: 225
 // against 262 us)
 constexpr int64_t kStreamMinRows = (int64_t)1 << 20;
-std::atomic<int64_t> g_stream_min_rows{kStreamMinRows};
+thread_local int64_t t_stream_min_rows = kStreamMinRows;  // per calling thread: a test hook must not move other threads' encodes
 
 int stream_workgroups()
 {
@@ -1266,7 +1282,7 @@ bool stream_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 {
     if (!mfma_eligible(a, x_dtype, w_dtype) || a.src_blocks) return false;
     if (!((a.K == 128 && (a.N == 128 || a.N == 64)) || (a.K == 64 && (a.N == 128 || a.N == 64)))) return false;
-    if (a.T * a.H < g_stream_min_rows.load(std::memory_order_relaxed)) return false;
+    if (a.T * a.H < t_stream_min_rows) return false;
     if (a.slot && ((uintptr_t)a.slot & 3)) return false;
     // one shift per slot, one 16-byte store per four-word code (set_block_shift() has run)
     if (a.bs_shift < 0) return false;
@@ -1510,8 +1526,73 @@ bool small_eligible(const EncArgs& a, int x_dtype, int w_dtype)
     return small_us < lds_floor_us;
 }
 
+// ---- the streaming kernel's time-out latch ----
+// A wave of the streaming kernel whose bounded wait gave up sets a word in pinned host memory (one
+// per device, allocated with the first streaming launch on it).  Every encode entry point reads that
+// word first - a plain host read, no device call - and fails with UCM_ERROR while it is set: the
+// codes of the launch that tripped it are undefined, so the caller must rebuild them and acknowledge
+// with ucm_hash_encode_clear_stream_timeouts().
+constexpr int kLatchDevices = 64;
+std::mutex g_latch_mu;
+unsigned int* g_latch_host[kLatchDevices] = {nullptr};  // pinned, mapped
+unsigned int* g_latch_dev[kLatchDevices] = {nullptr};   // the same words as the device sees them
+std::atomic<unsigned int> g_latch_forced[kLatchDevices];  // ucm_hash_encode_debug_trip_stream_latch()
+
+int latch_device()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        dev = 0;  // no device at all: the latch still works for its host-side users
+    }
+    return dev >= 0 && dev < kLatchDevices ? dev : 0;
+}
+
+// Device address of the current device's flag word; null when pinned memory cannot be had (the
+// kernel then only counts in g_stream_wait_timeouts).
+unsigned int* stream_latch_flag()
+{
+    const int dev = latch_device();
+    std::lock_guard<std::mutex> g(g_latch_mu);
+    if (!g_latch_dev[dev]) {
+        void* h = nullptr;
+        void* d = nullptr;
+        if (hipHostMalloc(&h, 64, hipHostMallocMapped) != hipSuccess || !h ||
+            hipHostGetDevicePointer(&d, h, 0) != hipSuccess || !d) {
+            (void)hipGetLastError();
+            if (h) (void)hipHostFree(h);
+            return nullptr;
+        }
+        *static_cast<volatile unsigned int*>(h) = 0;
+        g_latch_host[dev] = static_cast<unsigned int*>(h);
+        g_latch_dev[dev] = static_cast<unsigned int*>(d);
+    }
+    return g_latch_dev[dev];
+}
+
+bool stream_latch_tripped(int dev)
+{
+    if (g_latch_forced[dev].load(std::memory_order_relaxed)) return true;
+    const volatile unsigned int* h = g_latch_host[dev];  // written once under the mutex, then constant
+    return h && *h != 0;
+}
+
+int stream_latch_check()
+{
+    const int dev = latch_device();
+    if (!stream_latch_tripped(dev)) return UCM_OK;
+    return ucm::fail(UCM_ERROR,
+                     "an earlier streaming encode on device %d gave up waiting for its workgroup's code exchange: "
+                     "the codes that launch wrote are undefined; rebuild them, then call "
+                     "ucm_hash_encode_clear_stream_timeouts()", dev);
+}
+
 int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
 {
+    {
+        const int lrc = stream_latch_check();
+        if (lrc != UCM_OK) return lrc;
+    }
     set_block_shift(a);
     int rc = check_shape(a, x_dtype, w_dtype);
     if (rc != UCM_OK) return rc;
@@ -1526,6 +1607,7 @@ int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
                                       : launch_small<f16x8>(js, js.waves0, a.K, st);
     }
     if (stream_eligible(a, x_dtype, w_dtype)) {
+        a.timeout_flag = stream_latch_flag();
         rc = x_dtype == UCM_DT_BF16 ? launch_stream<bf16x8>(a, st) : launch_stream<f16x8>(a, st);
         if (rc != UCM_EUNSUPPORTED) return rc;  // no large-LDS opt-in: the tiled kernel below
         ucm::clear_error();
@@ -1581,10 +1663,27 @@ extern "C" int64_t ucm_hash_encode_stream_timeouts(void)
     return (int64_t)n;
 }
 
+extern "C" int ucm_hash_encode_clear_stream_timeouts(void)
+{
+    ucm::clear_error();
+    const int dev = latch_device();
+    g_latch_forced[dev].store(0, std::memory_order_relaxed);
+    std::lock_guard<std::mutex> g(g_latch_mu);
+    if (g_latch_host[dev]) *static_cast<volatile unsigned int*>(g_latch_host[dev]) = 0;
+    return UCM_OK;
+}
+
+extern "C" int ucm_hash_encode_debug_trip_stream_latch(void)
+{
+    ucm::clear_error();
+    g_latch_forced[latch_device()].store(1, std::memory_order_relaxed);
+    return UCM_OK;
+}
+
 extern "C" int ucm_hash_encode_set_stream_threshold(int64_t rows)
 {
     ucm::clear_error();
-    g_stream_min_rows.store(rows > 0 ? rows : kStreamMinRows, std::memory_order_relaxed);
+    t_stream_min_rows = rows > 0 ? rows : kStreamMinRows;
     return UCM_OK;
 }
 
@@ -1743,6 +1842,8 @@ int encode_pair(const PairSpec& p, hipStream_t st)
 {
     EncArgs kk, kq;
     bool has_keys;
+    const int lrc = stream_latch_check();
+    if (lrc != UCM_OK) return lrc;
     const int rc = build_pair(p, kk, kq, has_keys);
     if (rc != UCM_OK) return rc;
     return launch_pair(p, kk, kq, has_keys, st);
@@ -1752,7 +1853,9 @@ int encode_two_pairs(const PairSpec& pa, const PairSpec& pb, hipStream_t st)
 {
     EncArgs ka, qa, kb, qb;
     bool ha, hb;
-    int rc = build_pair(pa, ka, qa, ha);
+    int rc = stream_latch_check();
+    if (rc != UCM_OK) return rc;
+    rc = build_pair(pa, ka, qa, ha);
     if (rc != UCM_OK) return rc;
     rc = build_pair(pb, kb, qb, hb);
     if (rc != UCM_OK) return rc;

@@ -517,7 +517,15 @@ int64_t be_load(void* ctx, const uint8_t* ids, const uint64_t* idx, void* const*
 {
     return be_move((ucm_posix_store*)ctx, true, ids, idx, host, n, shard_size);
 }
-int be_wait(void* ctx, int64_t handle) { return ucm_posix_store_wait((ucm_posix_store_t*)ctx, handle); }
+// The cache store hands the waited-for staging nodes to other keys as soon as this returns, so
+// here "the workers still hold the buffers" is not an answer: keep waiting.
+int be_wait(void* ctx, int64_t handle)
+{
+    int rc;
+    while ((rc = ucm_posix_store_wait((ucm_posix_store_t*)ctx, handle)) == UCM_ERETRY) {
+    }
+    return rc;
+}
 
 }  // namespace
 
@@ -714,9 +722,17 @@ extern "C" int ucm_posix_store_wait(ucm_posix_store_t* st, int64_t task)
             st->failures.insert(task);  // shards still queued are skipped
         }
         // the caller's buffers are free to reuse once this returns, so the units that are queued
-        // (now skipped) or in the middle of their read / write must have drained first
-        while (!w->wait_for(1000)) {
-        }
+        // (now skipped) or in the middle of their read / write must have drained first.  That drain
+        // is bounded too (a worker stuck in a read or write on a dead mount never returns): after
+        // four more time-outs the task stays registered and the caller is told that its buffers are
+        // still in use.
+        bool drained = false;
+        for (int i = 0; i < 4 && !drained; ++i) drained = w->wait_for(st->timeout_ms ? st->timeout_ms : 1000);
+        if (!drained)
+            return ucm::fail(UCM_ERETRY,
+                             "task %lld timed out and its file workers have not returned after %zu ms more: the "
+                             "buffers of this task must not be reused or freed; wait on the task again",
+                             (long long)task, 4 * st->timeout_ms);
     }
     bool failed;
     {

@@ -9,6 +9,7 @@ UCM_OK = 0
 UCM_ERROR = -1
 UCM_EPARAM = -50000
 UCM_EOOM = -50001
+UCM_ERETRY = -50004
 UCM_ENOOBJ = -50005
 UCM_EUNSUPPORTED = -50008
 UCM_ETIMEOUT = -50010
@@ -30,6 +31,8 @@ _SIGNATURES = {
                                    vp, i64, i32, i64, i64, i64, vp]),
     "ucm_hash_encode_set_stream_threshold": (ci, [i64]),
     "ucm_hash_encode_stream_timeouts": (i64, []),
+    "ucm_hash_encode_clear_stream_timeouts": (ci, []),
+    "ucm_hash_encode_debug_trip_stream_latch": (ci, []),
     "ucm_hash_encode_paged": (ci, [vp, ci, i64, i32, i32, i32, i64, i64, i64, vp, i64, i64, vp, ci,
                                    i32, i32, i32, vp, i64, i64, i64, i64, vp]),
     "ucm_code_scatter": (ci, [vp, i64, i32, i32, i64, i64, vp, ci, vp, i64, i32, i64, i64, i64, vp]),

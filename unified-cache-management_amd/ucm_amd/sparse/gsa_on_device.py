@@ -76,7 +76,8 @@ class GSAOnDevice(UcmSparseBase):
         else:
             self.hash_encoder = HashEncoder(self.head_dim, self.hash_bits, self.dtype, self.device)
         self._saved = {}
-        self._fused_steps = {}  # (requests, table width) -> GSADecodeStep
+        self._fused_steps = {}  # (requests, table width, projection) -> GSADecodeStep, least recently used first
+        self._max_fused_steps = 8
         # one native call per layer at decode; False keeps the separate operators (same results)
         self.fused_decode = bool(cfg.get("fused_decode", True))
         self.has_pc_hit = False
@@ -246,7 +247,7 @@ class GSAOnDevice(UcmSparseBase):
             k_cache = attn.kv_cache[forward_context.virtual_engine][0]
         is_rollback_layer, _ = self.get_layer_state(layer_name)
         decode = phase == "decode" and not is_rollback_layer
-        if decode and self._fused_decode_ok(attn_metadata):
+        if decode and self._fused_decode_ok(attn_metadata, k_hash):
             self._fused_decode_step(query, key, attn_metadata, k_hash, k_cache, layer_name)
             return query, key, value, output
         self.cache_k_hash_gqa(key, attn_metadata, k_hash, k_cache)
@@ -271,11 +272,14 @@ class GSAOnDevice(UcmSparseBase):
             attn_metadata.seq_lens = new_lens
         return query, key, value, output
 
-    def _fused_decode_ok(self, attn_metadata):
-        """The single-call decode step takes 16-bit inputs with one projection, int32 metadata
-        and tables of at most 4096 blocks per request; anything else runs the separate operators."""
+    def _fused_decode_ok(self, attn_metadata, k_hash):
+        """The single-call decode step takes 16-bit inputs with one projection, int32 metadata,
+        tables of at most 4096 blocks per request and a code cache it can write in place (unit
+        stride over a whole number of 32-bit words: anything else would be written into a copy);
+        every other case runs the separate operators."""
         bt, sl = attn_metadata.block_table, attn_metadata.seq_lens
         return (self.fused_decode and self.dtype in (torch.bfloat16, torch.float16)
+                and k_hash.stride(-1) == 1 and (k_hash.shape[-1] * k_hash.element_size()) % 4 == 0
                 and self.head_dim in (64, 128, 256, 512) and self.hash_bits % 32 == 0
                 and self.num_q_heads >= self.num_key_heads
                 and bt.dtype == torch.int32 and sl.dtype == torch.int32 and bt.shape[1] <= 4096
@@ -290,13 +294,15 @@ class GSAOnDevice(UcmSparseBase):
         num_reqs = sl.shape[0]
         w = self.hash_encoder.hash_weights
         key_ = (num_reqs, bt.shape[1], w.data_ptr())
-        step = self._fused_steps.get(key_)
+        step = self._fused_steps.pop(key_, None)  # re-inserted below: most recently used last
         if step is None:
+            while len(self._fused_steps) >= self._max_fused_steps:  # each entry holds device buffers
+                self._fused_steps.pop(next(iter(self._fused_steps)))
             step = GSADecodeStep(w, self.num_q_heads, self.num_key_heads, num_reqs,
                                  bt.shape[1], self.hash_topk_tokens, block_size=self.block_size,
                                  sink_token=self.sink_tokens, recent_token=self.recent_tokens,
                                  seq_len_threshold=self.seq_len_threshold)
-            self._fused_steps[key_] = step
+        self._fused_steps[key_] = step
         slots = attn_metadata.slot_mapping.flatten()
         n = slots.numel()
         keys = key[:n].view(n, self.num_key_heads, self.head_dim)
