@@ -399,49 +399,99 @@ def plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots):
                     "sink 128 + recent 512 tokens kept", "cache_rotation": R}
     for mode in ("single_call", "separate_operators"):
         plugin.fused_decode = mode == "single_call"
-        for i in range(2 * R):
-            call(i)
+        out[mode] = _time_plugin_calls(torch, call, R)
+    return out
+
+
+def _time_plugin_calls(torch, call, R):
+    """call(i) = one attention_begin + attention_finished pair on rotation slot i % R: eager (events
+    between calls, wall clock around the loop) and as HIP-graph replays of R calls."""
+    for i in range(2 * R):
+        call(i)
+    torch.cuda.synchronize()
+    n = 100
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+    t0 = time.perf_counter()
+    for i in range(n):
+        ev[i].record()
+        call(i)
+    ev[n].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / n * 1e6
+    gaps = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(n))
+    res = {"eager_p50_us": gaps[n // 2], "eager_p90_us": gaps[int(n * 0.9)], "eager_wall_us_per_call": wall}
+    try:
+        if NO_GRAPH:
+            raise RuntimeError("graphs switched off (--no-graph)")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(R):
+                call(i)
+        torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        n = 100
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
-        t0 = time.perf_counter()
-        for i in range(n):
-            ev[i].record()
-            call(i)
-        ev[n].record()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(R):
+                call(i)
+        g.replay()
         torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) / n * 1e6
-        gaps = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(n))
-        res = {"eager_p50_us": gaps[n // 2], "eager_p90_us": gaps[int(n * 0.9)], "eager_wall_us_per_call": wall}
-        try:
-            if NO_GRAPH:
-                raise RuntimeError("graphs switched off (--no-graph)")
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                for i in range(R):
-                    call(i)
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for i in range(R):
-                    call(i)
+        m = 50
+        ge = [torch.cuda.Event(enable_timing=True) for _ in range(m + 1)]
+        for i in range(m):
+            ge[i].record()
             g.replay()
-            torch.cuda.synchronize()
-            m = 50
-            ge = [torch.cuda.Event(enable_timing=True) for _ in range(m + 1)]
-            for i in range(m):
-                ge[i].record()
-                g.replay()
-            ge[m].record()
-            torch.cuda.synchronize()
-            gg = sorted(ge[i].elapsed_time(ge[i + 1]) * 1e3 / R for i in range(m))
-            res["graph_p50_us"] = gg[m // 2]
-            res["graph_p90_us"] = gg[int(m * 0.9)]
-        except Exception as e:  # noqa: BLE001
-            res["graph_error"] = str(e)[:200]
-        out[mode] = res
+        ge[m].record()
+        torch.cuda.synchronize()
+        gg = sorted(ge[i].elapsed_time(ge[i + 1]) * 1e3 / R for i in range(m))
+        res["graph_p50_us"] = gg[m // 2]
+        res["graph_p90_us"] = gg[int(m * 0.9)]
+    except Exception as e:  # noqa: BLE001
+        res["graph_error"] = str(e)[:200]
+    return res
+
+
+def plugin_surface_mla(torch, gen):
+    """The latent-attention decode step at the plugin surface (GSAOnDevice with is_mla, the
+    reference's DeepSeek setting: 512 + 64 hash bits, 128 query heads reduced by 2, 64-token
+    blocks): 16 requests x 65,536 tokens, top-128 blocks, once as the single native call and once
+    as the separate operators."""
+    import types
+
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa_on_device import GSAOnDevice
+
+    b5, ctx5, bs5, hq, red, topk = 16, 65536, 64, 128, 2, 128
+    name = "model.layers.1.self_attn.attn"
+    cfg = {"ucm_sparse_config": {"GSAOnDevice": {
+        "num_q_heads": hq, "num_kv_heads": 1, "head_dim": 576, "block_size": bs5, "is_mla": True,
+        "kv_lora_rank": 512, "qk_rope_head_dim": 64, "vllm_hash_attention_reduction_head_num": red,
+        "vllm_hash_attention_topk": topk * bs5, "seed": 4}}}
+    plugin = GSAOnDevice(cfg, UcmSparseRole.WORKER)
+    nb = b5 * ctx5 // bs5
+    R = 4  # 4 x 75 MB of codes: beyond the last-level cache
+    caches = [torch.randint(-2**31, 2**31 - 1, (nb, bs5, 18), dtype=torch.int32, device="cuda", generator=gen)
+              for _ in range(R)]
+    tables = [torch.randperm(nb, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1) for _ in range(R)]
+    lens = torch.full((b5,), ctx5, dtype=torch.int32, device="cuda")
+    bf = lambda *shape: torch.randn(*shape, device="cuda", dtype=torch.bfloat16, generator=gen)
+    kn, kr, ql, qp = bf(b5, 512), bf(b5, 64), bf(b5, hq, 512), bf(b5, hq, 64)
+    slots = [(t[:, -1].to(torch.int64) * bs5 + bs5 - 1) for t in tables]
+    decs = [types.SimpleNamespace(block_table=tables[r], seq_lens=lens) for r in range(R)]
+    metas = [types.SimpleNamespace(slot_mapping=slots[r], decode=decs[r]) for r in range(R)]
+    ctxs = [types.SimpleNamespace(attn_metadata={name: m}) for m in metas]
+
+    def call(i):
+        r = i % R
+        plugin.attention_begin(None, kn, kr, name, ctxs[r], phase="decode", k_hash=caches[r],
+                               decode_ql_nope=ql, decode_q_pe=qp)
+        plugin.attention_finished(None, None, None, None, name, ctxs[r], phase="decode")
+
+    out = {"shape": "16 x 65536 tokens, 18-word codes, 128 query heads reduced by 2, top-128 blocks of 64 tokens, "
+                    "sink 64 + recent 256 tokens kept", "cache_rotation": R}
+    for mode in ("single_call", "separate_operators"):
+        plugin.fused_decode = mode == "single_call"
+        out[mode] = _time_plugin_calls(torch, call, R)
     return out
 
 
@@ -1073,6 +1123,7 @@ def main():
         line["extras"] = extras(torch, enc_k, gen, legs)
         if plug is not None:
             line["extras"]["plugin_surface"] = plug
+            line["extras"]["plugin_surface_latent_attention"] = plugin_surface_mla(torch, gen)
         if beside is not None:
             line["extras"]["gather_beside_decode"] = beside
         if not args.skip_cpu:

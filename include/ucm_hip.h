@@ -371,6 +371,43 @@ int ucm_gsa_decode_step(const void* new_keys, int64_t T, int64_t k_stride_t, int
                         int32_t* new_seq_lens, void* workspace, size_t workspace_bytes,
                         ucm_stream_t stream);
 
+/*
+ * The same for the latent-attention (MLA) plugin: replaces GSAOnDevice.attention_begin at decode with
+ * is_mla (ucm/sparse/gsa_on_device/gsa_on_device.py:426-455 cache_k_hash_mla_cuda, :376-393 the head
+ * reduction of hash_code, :667-709 update_decode_topk_mla_cuda) - two compute_hash + concat_and_cache_mla
+ * launches for the keys, two means, two compute_hash and a cat for the queries, the scorer, min, topk,
+ * sort, gather, zeros_like and a slice assignment there; three kernel launches here.
+ *
+ *   1. both parts of the step's new latent keys are hashed and written side by side into the paged
+ *      code cache (nope words first);
+ *   2. the Hq query heads are reduced to Hq / reduction_head_num rows - row i is the mean of heads
+ *      i, i + Hq / R, i + 2 Hq / R, ... (`view(T, R, Hq / R, D).mean(1)`: fp32 sum, times 1 / R,
+ *      rounded to the input type) - and both parts hashed: q_codes uint32 [B, Hq / R, Wd];
+ *   3. every block is scored with the sum over those rows, blocks holding a position < sink_tok or
+ *      >= len - recent_tok are always kept, the topk_tok / BS best are selected;
+ *   4. new_block_table / new_seq_lens / seq_len_threshold as in ucm_gsa_decode_step.
+ *
+ * Arguments as in ucm_sparse_decode_step_mla and ucm_gsa_decode_step; reduction_head_num >= 1 divides
+ * Hq.  Allocates nothing.
+ */
+int ucm_gsa_decode_step_mla(const void* new_nope, int64_t nope_stride_t,
+                            const void* new_rope, int64_t rope_stride_t, int64_t T,
+                            const void* slot_mapping, int slot_is_i64,
+                            const void* q_nope, int64_t qn_stride_b, int64_t qn_stride_h,
+                            const void* q_rope, int64_t qr_stride_b, int64_t qr_stride_h,
+                            int x_dtype, int32_t K_nope, int32_t K_rope,
+                            const void* w_nope, const void* w_rope, int w_dtype,
+                            int32_t N_nope_bits, int32_t N_rope_bits,
+                            uint32_t* k_cache, int64_t NB, int32_t BS,
+                            int64_t ks_block, int64_t ks_token,
+                            const int32_t* block_table, int32_t table_stride, int32_t max_blocks,
+                            const int32_t* seq_lens, int32_t B, int32_t Hq,
+                            int32_t reduction_head_num, int32_t topk_tok,
+                            int32_t sink_tok, int32_t recent_tok, int32_t seq_len_threshold,
+                            uint32_t* q_codes, int32_t* new_block_table, int32_t new_table_stride,
+                            int32_t* new_seq_lens, void* workspace, size_t workspace_bytes,
+                            ucm_stream_t stream);
+
 /* Replaces update_seq_lens (hamming_topk.py:7-12):
  * out[b] = len[b] - ceil(max(len[b] - topk_tok, 0) / BS) * BS. */
 int ucm_update_seq_lens(const int32_t* seq_lens, int32_t B, int32_t topk_tok, int32_t BS,

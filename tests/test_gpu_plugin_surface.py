@@ -326,6 +326,119 @@ def test_plugin_latent_attention_mode():
     assert torch.equal(dec.block_table, table) and torch.equal(dec.seq_lens, lens)
 
 
+@pytest.mark.parametrize("threshold,red", [(0, 2), (1000, 2), (0, 1), (0, 8)])
+def test_plugin_single_call_latent_decode_equals_separate_operators_and_oracle(threshold, red):
+    """attention_begin at decode with is_mla as ONE native call (ucm_gsa_decode_step_mla) against the
+    same hook running the separate operators (two encode-and-cache calls, two head reductions, two
+    hashes, cat, top-k, torch table swap) and against the CPU checker: identical code cache, query
+    codes, replacement table and lengths.  Lengths include a request shorter than the top-k budget,
+    one shorter than the threshold and a ragged last block."""
+    from ucm_amd.sparse.base import UcmSparseFactory, UcmSparseRole
+
+    B, Hq, BS, nblk, topk_tok = 5, 16, 64, 40, 1024
+    name = "model.layers.3.self_attn.attn"
+    rng = rng_for(93 + red)
+    NB = B * nblk + 3
+    base_codes = torch.from_numpy(rng.integers(0, 256, size=(NB, BS, 72), dtype=np.uint8)).cuda()
+    table = torch.from_numpy(rng.permutation(NB)[: B * nblk].astype(np.int32).reshape(B, nblk)).cuda()
+    lens = torch.tensor([nblk * BS, nblk * BS - 100, 9 * BS + 1, 700, 17 * BS], dtype=torch.int32, device="cuda")
+    ql = torch.from_numpy(rng.standard_normal((B, Hq, 512)).astype(np.float32)).to(torch.bfloat16).cuda()
+    qp = torch.from_numpy(rng.standard_normal((B, Hq, 64)).astype(np.float32)).to(torch.bfloat16).cuda()
+    lat = torch.from_numpy(rng.standard_normal((B, 576)).astype(np.float32)).to(torch.bfloat16).cuda()
+    pos = lens.long() - 1
+    slots = table[torch.arange(B), pos // BS].long() * BS + pos % BS
+    results = []
+    for fused in (True, False):
+        cfg = {"ucm_sparse_config": {"GSAOnDevice": {
+            "num_q_heads": Hq, "num_kv_heads": 1, "head_dim": 576, "block_size": BS, "is_mla": True,
+            "kv_lora_rank": 512, "qk_rope_head_dim": 64, "vllm_hash_attention_reduction_head_num": red,
+            "vllm_hash_attention_topk": topk_tok, "gpu_seq_len_threshold": threshold,
+            "fused_decode": fused, "seed": 13}}}
+        plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+        k_hash = base_codes.clone().view(torch.bfloat16)  # [NB, BS, 36] as the engine allocates it
+        dec = types.SimpleNamespace(block_table=table.clone(), seq_lens=lens.clone())
+        meta = types.SimpleNamespace(slot_mapping=slots, decode=dec)
+        ctx = types.SimpleNamespace(attn_metadata={name: meta})
+        for _ in range(2):  # twice: the step's buffers are reused
+            plugin.attention_begin(None, lat[:, :512].contiguous(), lat[:, 512:].contiguous(), name, ctx,
+                                   phase="decode", k_hash=k_hash, decode_ql_nope=ql, decode_q_pe=qp)
+            torch.cuda.synchronize()
+            out = (k_hash.clone(), dec.block_table.clone(), dec.seq_lens.clone())
+            plugin.attention_finished(None, None, None, None, name, ctx, phase="decode")
+            assert torch.equal(dec.block_table, table) and torch.equal(dec.seq_lens, lens)
+        results.append((plugin, out))
+    (pf, (kh_f, bt_f, sl_f)), (ps, (kh_s, bt_s, sl_s)) = results
+    assert len(pf._fused_steps) == 1 and not ps._fused_steps
+    assert torch.equal(pf.hash_encoder_nope.hash_weights, ps.hash_encoder_nope.hash_weights)
+    # (compared as bytes: as bfloat16 some codes are NaN patterns)
+    assert torch.equal(kh_f.view(torch.uint8), kh_s.view(torch.uint8)), \
+        "code cache differs between the single call and the separate operators"
+    assert not torch.equal(kh_f.view(torch.uint8), base_codes)
+    assert torch.equal(bt_f, bt_s) and torch.equal(sl_f, sl_s)
+    # the query codes of the single call are the codes of torch's strided head mean
+    step = next(iter(pf._fused_steps.values()))
+    qn, qr = ps.hash_code(nope=ql, rope=qp, reduction_head_num=red)
+    qc_sep = torch.cat([qn, qr], dim=-1).view(torch.int32)
+    assert tuple(step.q_codes.shape) == (B, Hq // red, 18)
+    assert torch.equal(step.q_codes, qc_sep)
+    # and the CPU checker on the codes now in the cache
+    kblk = topk_tok // BS
+    oi, _ = c_api.hamming_topk(step.q_codes.cpu().numpy().view(np.uint32),
+                               kh_f.view(torch.uint8).cpu().numpy().view(np.uint32).reshape(NB, BS, 1, 18),
+                               table.cpu().numpy(), lens.cpu().numpy(), kblk, BS, 4 * BS,
+                               flags=c_api.F_REDUCE_HEADS | c_api.F_PHYSICAL)
+    exp_t = np.zeros((B, nblk), np.int32)
+    exp_t[:, :kblk] = np.maximum(oi[:, 0], 0)
+    exp_l = c_api.update_seq_lens(lens.cpu().numpy(), topk_tok, BS)
+    if threshold:
+        short = lens.cpu().numpy() < threshold
+        exp_t[short] = table.cpu().numpy()[short]
+        exp_l[short] = lens.cpu().numpy()[short]
+        assert short.any() and not short.all()
+    assert np.array_equal(bt_f.cpu().numpy(), exp_t)
+    assert np.array_equal(sl_f.cpu().numpy(), exp_l)
+
+
+def test_single_call_latent_decode_step_in_a_hip_graph():
+    """GSADecodeStepMLA allocates nothing: captured once, replayed with changing inputs and the
+    program's own eager work in between, every replay checked against an eager call."""
+    from ucm_amd.sparse import GSADecodeStepMLA
+
+    B, Hq, red, BS, nblk, topk_tok = 4, 16, 2, 64, 48, 1024
+    rng = rng_for(94)
+    NB = B * nblk
+    bf = lambda *shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(torch.bfloat16).cuda()
+    wn, wr = bf(512, 512), bf(64, 64)
+    cache0 = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=(NB, BS, 18), dtype=np.int64).astype(np.int32)).cuda()
+    table = torch.from_numpy(rng.permutation(NB).astype(np.int32).reshape(B, nblk)).cuda()
+    lens = torch.full((B,), nblk * BS, dtype=torch.int32, device="cuda")
+    slots = (table[:, -1].long() * BS + BS - 1)
+    ql, qp = torch.empty((B, Hq, 512), dtype=torch.bfloat16, device="cuda"), torch.empty((B, Hq, 64), dtype=torch.bfloat16, device="cuda")
+    kn, kr = torch.empty((B, 512), dtype=torch.bfloat16, device="cuda"), torch.empty((B, 64), dtype=torch.bfloat16, device="cuda")
+    cache_g, cache_e = cache0.clone(), cache0.clone()
+    step = GSADecodeStepMLA(wn, wr, Hq, red, B, nblk, topk_tok, block_size=BS)
+    eager = GSADecodeStepMLA(wn, wr, Hq, red, B, nblk, topk_tok, block_size=BS)
+    for t in (ql, qp, kn, kr):
+        t.copy_(bf(*t.shape))
+    step.step(kn, kr, slots, ql, qp, cache_g, table, lens)  # warm-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step.step(kn, kr, slots, ql, qp, cache_g, table, lens)
+    for rep in range(4):
+        for t in (ql, qp, kn, kr):
+            t.copy_(bf(*t.shape))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        et, el = eager.step(kn, kr, slots, ql, qp, cache_e, table, lens)
+        torch.cuda.synchronize()
+        assert torch.equal(step.new_table, et) and torch.equal(step.new_lens, el), rep
+        assert torch.equal(step.q_codes, eager.q_codes) and torch.equal(cache_g, cache_e), rep
+
+
 def test_host_memory_store_dump_lookup_load_roundtrip():
     """The store contract of the reference's e2e test (ucm/store/test/e2e/cache_on_empty_test.py:
     46-79): dump -> lookup -> load -> bit-exact."""

@@ -55,6 +55,9 @@ struct PairSpec {
     uint32_t* q_codes; int64_t qc_stride_b, qc_stride_h;
     int x_dtype; int K; const void* w; int w_dtype; int n_w; int N_bits;
     int q_group_mean = 0;  // hash the mean of every KV head's query group: q_codes is [B, Hkv, Wd]
+    // latent attention's head reduction: query row i of the Hq / q_reduce that are hashed is the mean
+    // of heads i, i + Hq / q_reduce, i + 2 * Hq / q_reduce, ... (q_codes is [B, Hq / q_reduce, Wd])
+    int q_reduce = 0;
 };
 // one launch when both jobs are small
 int encode_pair(const PairSpec& p, hipStream_t st);

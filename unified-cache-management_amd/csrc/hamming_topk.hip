@@ -2901,6 +2901,48 @@ extern "C" int ucm_sparse_decode_step_mla(
                             workspace_bytes, stream);
 }
 
+/* One latent-attention decode step as the reference's plugin performs it, see ucm_hip.h. */
+extern "C" int ucm_gsa_decode_step_mla(
+    const void* new_nope, int64_t nope_stride_t, const void* new_rope, int64_t rope_stride_t, int64_t T,
+    const void* slot_mapping, int slot_is_i64, const void* q_nope, int64_t qn_stride_b,
+    int64_t qn_stride_h, const void* q_rope, int64_t qr_stride_b, int64_t qr_stride_h, int x_dtype,
+    int32_t K_nope, int32_t K_rope, const void* w_nope, const void* w_rope, int w_dtype,
+    int32_t N_nope_bits, int32_t N_rope_bits, uint32_t* k_cache, int64_t NB, int32_t BS,
+    int64_t ks_block, int64_t ks_token, const int32_t* block_table, int32_t table_stride,
+    int32_t max_blocks, const int32_t* seq_lens, int32_t B, int32_t Hq, int32_t reduction_head_num,
+    int32_t topk_tok, int32_t sink_tok, int32_t recent_tok, int32_t seq_len_threshold, uint32_t* q_codes,
+    int32_t* new_block_table, int32_t new_table_stride, int32_t* new_seq_lens, void* workspace,
+    size_t workspace_bytes, ucm_stream_t stream)
+{
+    ucm::clear_error();
+    UCM_REQUIRE(Hq > 0 && reduction_head_num >= 1 && Hq % reduction_head_num == 0,
+                "%d query heads do not reduce by %d", Hq, reduction_head_num);
+    UCM_REQUIRE(N_nope_bits > 0 && N_nope_bits % 32 == 0 && N_rope_bits > 0 && N_rope_bits % 32 == 0,
+                "hash_bits of both parts must be multiples of 32");
+    UCM_REQUIRE(q_codes && k_cache, "q_codes or k_cache is null");
+    // the reference's own checks (hamming_topk.py:30-31)
+    UCM_REQUIRE(BS > 0 && topk_tok > 0 && topk_tok % BS == 0, "topk_token %d is no multiple of the block size %d",
+                topk_tok, BS);
+    UCM_REQUIRE(recent_tok > 0 && topk_tok > sink_tok + recent_tok, "topk_token must exceed sink + recent > 0");
+    const int32_t Wn = N_nope_bits / 32, Wd = Wn + N_rope_bits / 32;
+    UCM_REQUIRE(ks_token >= Wd, "cache rows of %lld words do not hold %d-word codes", (long long)ks_token, Wd);
+    const int32_t Hr = Hq / reduction_head_num;  // rows that are hashed and scored
+    ucm::PairSpec nope{new_nope, T, 1, nope_stride_t, 0, slot_mapping, slot_is_i64, k_cache, NB, BS,
+                       ks_block, ks_token, ks_token, q_nope, B, Hq, qn_stride_b, qn_stride_h,
+                       q_codes, (int64_t)Hr * Wd, Wd, x_dtype, K_nope, w_nope, w_dtype, 1, N_nope_bits};
+    ucm::PairSpec rope{new_rope, T, 1, rope_stride_t, 0, slot_mapping, slot_is_i64, k_cache + Wn, NB,
+                       BS, ks_block, ks_token, ks_token, q_rope, B, Hq, qr_stride_b, qr_stride_h,
+                       q_codes + Wn, (int64_t)Hr * Wd, Wd, x_dtype, K_rope, w_rope, w_dtype, 1, N_rope_bits};
+    nope.q_reduce = rope.q_reduce = reduction_head_num;
+    const int rc = ucm::encode_two_pairs(nope, rope, (hipStream_t)stream);
+    if (rc != UCM_OK) return rc;
+    const StepOut so{new_block_table, new_table_stride, new_seq_lens, seq_len_threshold, topk_tok};
+    return hamming_topk_run(q_codes, (int64_t)Hr * Wd, Wd, k_cache, NB, BS, 1, Wd, ks_block, ks_token, ks_token,
+                            block_table, table_stride, max_blocks, seq_lens, B, Hr, topk_tok / BS, sink_tok,
+                            recent_tok, UCM_TOPK_RETURN_PHYSICAL, nullptr, nullptr, workspace, workspace_bytes,
+                            stream, &so);
+}
+
 extern "C" int64_t ucm_hamming_last_dispatch(char* buf, size_t cap)
 {
     char tmp[256];

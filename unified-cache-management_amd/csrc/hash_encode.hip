@@ -1772,6 +1772,13 @@ int build_pair(const PairSpec& p, EncArgs& kk, EncArgs& kq, bool& has_keys)
         kq.x_stride_g = p.q_stride_h;
         kq.x_stride_h = p.q_stride_h * kq.gmean;
         kq.heads_per_w = p.n_w > 1 ? 1 : 0;
+    } else if (p.q_reduce > 1) {
+        // the reference's view(T, R, H / R, D).mean(1) (gsa_on_device.py:378-391): members of a group
+        // lie H / R heads apart
+        if (p.Hq % p.q_reduce) return ucm::fail(UCM_EPARAM, "%d query heads do not reduce by %d", p.Hq, p.q_reduce);
+        kq.H = p.Hq / p.q_reduce;
+        kq.gmean = p.q_reduce;
+        kq.x_stride_g = p.q_stride_h * kq.H;
     }
     kq.out = p.q_codes; kq.out_stride_t = p.qc_stride_b; kq.out_stride_h = p.qc_stride_h;
     int rc = check_shape(kq, p.x_dtype, p.w_dtype);

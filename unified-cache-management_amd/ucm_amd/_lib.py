@@ -52,6 +52,9 @@ _SIGNATURES = {
     "ucm_sparse_decode_step_mla": (ci, [vp, i64, vp, i64, i64, vp, ci, vp, i64, i64, vp, i64, i64, ci, i32, i32,
                                         vp, vp, ci, i32, i32, vp, i64, i32, i64, i64, vp, i32, i32, vp, i32,
                                         i32, i32, i32, i32, u32, vp, vp, vp, vp, sz, vp]),
+    "ucm_gsa_decode_step_mla": (ci, [vp, i64, vp, i64, i64, vp, ci, vp, i64, i64, vp, i64, i64, ci, i32, i32,
+                                     vp, vp, ci, i32, i32, vp, i64, i32, i64, i64, vp, i32, i32, vp, i32,
+                                     i32, i32, i32, i32, i32, i32, vp, vp, i32, vp, vp, sz, vp]),
     "ucm_hamming_score": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
                                vp, i32, i32, i32, i32, i32, ci, vp, ci, vp, sz, vp]),
     "ucm_hamming_score_workspace_bytes": (sz, [i32, i32, i32]),

@@ -256,3 +256,82 @@ class GSADecodeStep:
             return result
 
         return run
+
+
+class GSADecodeStepMLA:
+    """The latent-attention plugin's per-layer decode work in one native call
+    (ucm_gsa_decode_step_mla): both parts of the step's new latent keys into the paged code cache
+    (cache_k_hash_mla_cuda, gsa_on_device.py:426-455), the head reduction and both hashes of the
+    queries (hash_code, :376-393), block scores with sink / recent blocks kept and the selection
+    (update_decode_topk_mla_cuda, :667-709), and the replacement block table and sequence lengths
+    the attention backend reads.  Buffers are allocated once here; `step` allocates nothing and
+    can be captured in a HIP graph."""
+
+    def __init__(self, w_nope, w_rope, num_q_heads, reduction_head_num, batch, table_width, topk_tokens,
+                 block_size=64, sink_token=None, recent_token=None, seq_len_threshold=0):
+        if w_nope.dtype != w_rope.dtype or w_nope.dtype not in _DT or w_nope.dtype == torch.float32:
+            raise ValueError("the fused step needs two bfloat16 or float16 projections of one dtype")
+        if w_nope.dim() != 2 or w_rope.dim() != 2:
+            raise ValueError("projections must be [K, N]")
+        self.wn, self.wr = w_nope.contiguous(), w_rope.contiguous()
+        self.Kn, self.Nn = (int(v) for v in w_nope.shape)
+        self.Kr, self.Nr = (int(v) for v in w_rope.shape)
+        if self.Nn % 32 or self.Nr % 32:
+            raise ValueError("hash_bits of both parts must be multiples of 32")
+        self.Wd = (self.Nn + self.Nr) // 32
+        self.Hq, self.R, self.B = int(num_q_heads), max(1, int(reduction_head_num)), int(batch)
+        if self.Hq % self.R:
+            raise ValueError(f"{self.Hq} query heads do not reduce by {self.R}")
+        self.width, self.BS, self.topk = int(table_width), int(block_size), int(topk_tokens)
+        self.sink = self.BS if sink_token is None else int(sink_token)
+        self.recent = 4 * self.BS if recent_token is None else int(recent_token)
+        self.threshold = int(seq_len_threshold)
+        assert self.topk % self.BS == 0
+        assert self.recent > 0 and self.topk > self.sink + self.recent
+        dev = w_nope.device
+        self.q_codes = torch.empty((self.B, self.Hq // self.R, self.Wd), dtype=torch.int32, device=dev)
+        self.new_table = torch.empty((self.B, self.width), dtype=torch.int32, device=dev)
+        self.new_lens = torch.empty((self.B,), dtype=torch.int32, device=dev)
+        nbytes = _lib.lib().ucm_hamming_topk_workspace_bytes(self.B, 1, self.width)
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+    def step(self, new_nope, new_rope, slot_mapping, q_nope, q_rope, k_hash_cache, block_table, seq_lens):
+        """new_nope [T,K_nope], new_rope [T,K_rope] + slot_mapping [T] (T may be 0); q_nope
+        [B,Hq,K_nope], q_rope [B,Hq,K_rope] (all Hq heads: the reduction happens inside);
+        k_hash_cache int32 [NB,BS,Wd]; block_table int32 [B,width]; seq_lens int32 [B].
+        Returns (new_block_table [B, width], new_seq_lens [B]): buffers reused by every call."""
+        dt = self.wn.dtype
+        T = 0 if new_nope is None else int(new_nope.shape[0])
+        for t in (q_nope, q_rope) + ((new_nope, new_rope) if T else ()):
+            if t.dtype != dt or t.stride(-1) != 1:
+                raise ValueError("keys, queries and weights must share one dtype and have contiguous rows")
+        if tuple(q_nope.shape) != (self.B, self.Hq, self.Kn) or tuple(q_rope.shape) != (self.B, self.Hq, self.Kr):
+            raise ValueError("queries must be [B,Hq,K_nope] and [B,Hq,K_rope]")
+        if k_hash_cache.dtype != torch.int32 or k_hash_cache.dim() != 3 or k_hash_cache.shape[1] != self.BS \
+                or k_hash_cache.shape[2] != self.Wd or k_hash_cache.stride(-1) != 1:
+            raise ValueError(f"k_hash_cache must be int32 [NB,{self.BS},{self.Wd}]")
+        if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
+            raise ValueError("block_table and seq_lens must be int32")
+        if tuple(block_table.shape) != (self.B, self.width) or block_table.stride(-1) != 1:
+            raise ValueError(f"block_table must be {(self.B, self.width)}")
+        if seq_lens.numel() != self.B or not seq_lens.is_contiguous():
+            raise ValueError("seq_lens must be a contiguous [B] tensor")
+        if T:
+            if tuple(new_nope.shape) != (T, self.Kn) or tuple(new_rope.shape) != (T, self.Kr):
+                raise ValueError("new keys must be [T,K_nope] and [T,K_rope]")
+            if slot_mapping.dtype not in (torch.int32, torch.int64) or slot_mapping.numel() != T \
+                    or not slot_mapping.is_contiguous():
+                raise ValueError("slot_mapping must be a contiguous int32/int64 [T] tensor")
+        s = _lib.stride
+        _lib.check(_lib.lib().ucm_gsa_decode_step_mla(
+            new_nope.data_ptr() if T else None, s(new_nope, 0) if T else 0,
+            new_rope.data_ptr() if T else None, s(new_rope, 0) if T else 0, T,
+            slot_mapping.data_ptr() if T else None, int(T > 0 and slot_mapping.dtype == torch.int64),
+            q_nope.data_ptr(), s(q_nope, 0), s(q_nope, 1), q_rope.data_ptr(), s(q_rope, 0), s(q_rope, 1),
+            _DT[dt], self.Kn, self.Kr, self.wn.data_ptr(), self.wr.data_ptr(), _DT[dt], self.Nn, self.Nr,
+            k_hash_cache.data_ptr(), k_hash_cache.shape[0], self.BS, s(k_hash_cache, 0), s(k_hash_cache, 1),
+            block_table.data_ptr(), max(s(block_table, 0), self.width), self.width,
+            seq_lens.data_ptr(), self.B, self.Hq, self.R, self.topk, self.sink, self.recent, self.threshold,
+            self.q_codes.data_ptr(), self.new_table.data_ptr(), self.width, self.new_lens.data_ptr(),
+            self.workspace.data_ptr(), self.workspace.numel(), _lib.stream_ptr(q_nope.device)))
+        return self.new_table, self.new_lens

@@ -29,7 +29,7 @@ from typing import List, Optional, Union
 import torch
 
 from .base import UcmSparseBase, UcmSparseMetadata, UcmSparseRole
-from .decode_step import GSADecodeStep
+from .decode_step import GSADecodeStep, GSADecodeStepMLA
 from .hamming_topk import _as_words, cuda_hamming_topk, update_seq_lens
 from .hash_encoder import HashEncoder
 
@@ -191,17 +191,22 @@ class GSAOnDevice(UcmSparseBase):
         self.hash_encoder_rope.compute_hash_and_cache(
             rope[:n].reshape(n, 1, self.qk_rope_head_dim), slots, c_rope, block_size=self.block_size)
         if self.has_pc_hit:
-            # kv_cache [NB, BS, kv_lora_rank + qk_rope_head_dim]: both parts are read in place
-            if kv_cache is None:
-                raise ValueError("a prefix-cache hit needs the layer's latent cache")
-            kc = kv_cache if kv_cache.ndim == 4 else kv_cache.unsqueeze(2)
-            k_nope, k_rope = kc[..., :self.kv_lora_rank], kc[..., self.kv_lora_rank:]
-            for first, n_blk, n_tok in self._prefix_segments:
-                ids = self.prefix_block_ids[first:first + n_blk]
-                self.hash_encoder_nope.compute_hash_from_paged_cache(k_nope, ids, n_tok, c_nope,
-                                                                     block_size=self.block_size)
-                self.hash_encoder_rope.compute_hash_from_paged_cache(k_rope, ids, n_tok, c_rope,
-                                                                     block_size=self.block_size)
+            self._rehash_prefix_mla(k_hash, kv_cache)
+
+    def _rehash_prefix_mla(self, k_hash, kv_cache):
+        """Codes of the prefix tokens that came from the store, read where their latents lie:
+        kv_cache [NB, BS, kv_lora_rank + qk_rope_head_dim] (gsa_on_device.py:438-455)."""
+        if kv_cache is None:
+            raise ValueError("a prefix-cache hit needs the layer's latent cache")
+        c_nope, c_rope = self._mla_code_views(k_hash)
+        kc = kv_cache if kv_cache.ndim == 4 else kv_cache.unsqueeze(2)
+        k_nope, k_rope = kc[..., :self.kv_lora_rank], kc[..., self.kv_lora_rank:]
+        for first, n_blk, n_tok in self._prefix_segments:
+            ids = self.prefix_block_ids[first:first + n_blk]
+            self.hash_encoder_nope.compute_hash_from_paged_cache(k_nope, ids, n_tok, c_nope,
+                                                                 block_size=self.block_size)
+            self.hash_encoder_rope.compute_hash_from_paged_cache(k_rope, ids, n_tok, c_rope,
+                                                                 block_size=self.block_size)
 
     def update_decode_topk_mla(self, layer_name, attn_metadata, decode_ql_nope, decode_q_pe, k_hash):
         """Top-k block table of a latent-attention decode step
@@ -218,8 +223,64 @@ class GSAOnDevice(UcmSparseBase):
         self._saved[layer_name] = (meta.block_table, meta.seq_lens)
         new_table = torch.zeros_like(meta.block_table)
         new_table[:, :topk_table.shape[1]] = topk_table
+        new_lens = update_seq_lens(meta.seq_lens, self.hash_topk_tokens, self.block_size)
+        if self.seq_len_threshold > 0:  # short requests keep their full table
+            short = meta.seq_lens < self.seq_len_threshold
+            new_table = torch.where(short[:, None], meta.block_table, new_table)
+            new_lens = torch.where(short, meta.seq_lens, new_lens)
         meta.block_table = new_table
-        meta.seq_lens = update_seq_lens(meta.seq_lens, self.hash_topk_tokens, self.block_size)
+        meta.seq_lens = new_lens
+
+    def _fused_decode_ok_mla(self, meta, k_hash, decode_ql_nope, decode_q_pe):
+        """The single-call latent-attention step takes 16-bit inputs, int32 metadata, tables of at
+        most 4096 blocks per request and a code cache [NB, BS, code] it can write in place as
+        32-bit words; every other case runs the separate operators."""
+        bt, sl = meta.block_table, meta.seq_lens
+        code_bytes = (self.kv_lora_rank + self.qk_rope_head_dim) // 8
+        return (self.fused_decode and self.dtype in (torch.bfloat16, torch.float16)
+                and self.kv_lora_rank in (64, 128, 256, 512) and self.qk_rope_head_dim in (64, 128, 256, 512)
+                and k_hash.dim() in (3, 4) and k_hash.is_contiguous()
+                and k_hash.shape[-1] * k_hash.element_size() == code_bytes and code_bytes % 4 == 0
+                and (k_hash.dim() == 3 or k_hash.shape[2] == 1)
+                and decode_ql_nope is not None and decode_q_pe is not None
+                and decode_ql_nope.dim() == 3 and decode_q_pe.dim() == 3
+                and decode_ql_nope.stride(-1) == 1 and decode_q_pe.stride(-1) == 1
+                and decode_ql_nope.shape[1] % self.hash_reduction_head_num == 0
+                and bt.dtype == torch.int32 and sl.dtype == torch.int32 and bt.shape[1] <= 4096
+                and bt.stride(-1) == 1 and sl.is_contiguous()
+                and self.hash_topk_tokens % self.block_size == 0
+                and self.hash_topk_tokens > 5 * self.block_size)
+
+    def _fused_decode_step_mla(self, nope, rope, k_hash, attn_metadata, meta, decode_ql_nope, decode_q_pe,
+                               kv_cache, layer_name):
+        """cache_k_hash_mla + hash_code + cuda_hamming_topk + the table / length swap
+        (gsa_on_device.py:426-455, 376-393, 667-709) as one native call."""
+        bt, sl = meta.block_table, meta.seq_lens
+        num_reqs = sl.shape[0]
+        wn, wr = self.hash_encoder_nope.hash_weights, self.hash_encoder_rope.hash_weights
+        hq = decode_ql_nope.shape[1]
+        key_ = (num_reqs, bt.shape[1], hq, wn.data_ptr())
+        step = self._fused_steps.pop(key_, None)  # re-inserted below: most recently used last
+        if step is None:
+            while len(self._fused_steps) >= self._max_fused_steps:  # each entry holds device buffers
+                self._fused_steps.pop(next(iter(self._fused_steps)))
+            step = GSADecodeStepMLA(wn, wr, hq, self.hash_reduction_head_num, num_reqs, bt.shape[1],
+                                    self.hash_topk_tokens, block_size=self.block_size,
+                                    sink_token=self.block_size, recent_token=4 * self.block_size,
+                                    seq_len_threshold=self.seq_len_threshold)
+        self._fused_steps[key_] = step
+        slots = attn_metadata.slot_mapping.flatten()
+        n = slots.numel()
+        if self.has_pc_hit:  # prefix latents are re-encoded where they lie (gsa_on_device.py:438-455)
+            self._rehash_prefix_mla(k_hash, kv_cache)
+        words = k_hash.view(torch.int32)
+        words = words.view(words.shape[0], words.shape[1], words.shape[-1])
+        new_table, new_lens = step.step(nope[:n].reshape(n, self.kv_lora_rank),
+                                        rope[:n].reshape(n, self.qk_rope_head_dim), slots,
+                                        decode_ql_nope[:num_reqs], decode_q_pe[:num_reqs], words, bt, sl)
+        self._saved[layer_name] = (bt, sl)
+        meta.block_table = new_table
+        meta.seq_lens = new_lens
 
     # ---- hooks ----
     def attention_begin(self, query, key, value, layer_name: str, forward_context, output=None,
@@ -234,9 +295,15 @@ class GSAOnDevice(UcmSparseBase):
             if self.has_pc_hit:
                 attn = forward_context.no_compile_layers[layer_name]
                 kv_cache = attn.kv_cache[forward_context.virtual_engine]
-            self.cache_k_hash_mla(key, value, k_hash, attn_metadata, kv_cache)
             is_rollback_layer, _ = self.get_layer_state(layer_name)
-            if phase == "decode" and not is_rollback_layer:
+            decode = phase == "decode" and not is_rollback_layer
+            meta = getattr(attn_metadata, "decode", attn_metadata)
+            if decode and self._fused_decode_ok_mla(meta, k_hash, decode_ql_nope, decode_q_pe):
+                self._fused_decode_step_mla(key, value, k_hash, attn_metadata, meta, decode_ql_nope,
+                                            decode_q_pe, kv_cache, layer_name)
+                return query, key, value, output
+            self.cache_k_hash_mla(key, value, k_hash, attn_metadata, kv_cache)
+            if decode:
                 self.update_decode_topk_mla(layer_name, attn_metadata, decode_ql_nope, decode_q_pe,
                                             k_hash)
             return query, key, value, output
