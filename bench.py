@@ -368,6 +368,60 @@ def encoder_cache_build(torch, enc_k, gen, launches=9):
                     "the same reads alone take 304 us"}
 
 
+def encoder_latent_cache_build(torch, gen, launches=7):
+    """The K = 512 encoders at cache-build size: 1,048,576 latent rows of 576 bf16 (512 hashed),
+    cold (two 1.2 GB inputs in turn), written through a permuted slot mapping into the paged code
+    cache - 512 -> 256 bits (config 5's projection, 8-word code rows) and 512 -> 512 bits (the nope
+    part of the reference's 18-word latent codes, hash_encoder.py:548-662 via
+    gsa_on_device.py:426-455).  At 512 bits the matrix cores bind (about 480 flop per byte), at 256
+    bits memory and matrix cores bind about equally: both fractions are reported, and the tiled
+    kernel (the projection sliced over workgroups, rows re-read per slice) beside them."""
+    from ucm_amd import _lib
+    from ucm_amd.sparse import HashEncoder
+
+    T, K, BS5 = 1 << 20, 512, 64
+    NB5 = T // BS5
+    lat = [torch.randn((T, 576), generator=gen, device="cuda", dtype=torch.bfloat16) for _ in range(2)]
+    perm = torch.randperm(NB5, generator=gen, device="cuda")
+    slots = (perm.repeat_interleave(BS5) * BS5 + torch.arange(BS5, device="cuda").repeat(NB5)).to(torch.int64)
+    out = {}
+    for n_bits, cwords in ((256, 8), (512, 18)):
+        enc = HashEncoder(K, n_bits, torch.bfloat16, torch.device("cuda"))
+        cache = torch.empty((NB5, BS5, 1, cwords), dtype=torch.int32, device="cuda")
+        view = cache[..., : n_bits // 32]
+        res = {}
+        for kernel, thr in (("encode_wide_kernel", 0), ("encode_mfma_kernel (tiled)", 1 << 62)):
+            _lib.lib().ucm_hash_encode_set_stream_threshold(thr)
+            for i in range(2):
+                enc.compute_hash_and_cache(lat[i][:, :K].unsqueeze(1), slots, view, BS5)
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+            for i in range(launches):
+                ev[i].record()
+                enc.compute_hash_and_cache(lat[i % 2][:, :K].unsqueeze(1), slots, view, BS5)
+            ev[launches].record()
+            torch.cuda.synchronize()
+            ts = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(launches))
+            ms = ts[len(ts) // 2]
+            alg = T * K * 2 + T * n_bits // 8 + K * n_bits * 2 + T * 8  # rows, codes, projection, slot mapping
+            flops = 2.0 * T * K * n_bits
+            res[kernel] = {"ms_median": ms, "ms_min": ts[0], "GBps": alg / ms / 1e6,
+                           "hbm_frac": alg / ms / 1e6 / HBM_PEAK_GBPS, "TFLOPs": flops / ms / 1e9,
+                           "mfma_frac_of_2500_TFLOPs": flops / ms / 1e9 / 2500.0}
+        _lib.lib().ucm_hash_encode_set_stream_threshold(0)
+        alg = T * K * 2 + T * n_bits // 8 + K * n_bits * 2 + T * 8
+        flops = 2.0 * T * K * n_bits
+        floor_ms = max(alg / (HBM_PEAK_GBPS * 1e6), flops / 2500e9)
+        res["rows"] = T
+        res["algorithmic_bytes"] = alg
+        res["flops"] = flops
+        res["binding_roofline"] = "mfma" if flops / 2500e9 > alg / (HBM_PEAK_GBPS * 1e6) else "hbm"
+        res["roofline_floor_ms"] = floor_ms
+        res["frac_of_binding_roofline"] = floor_ms / res["encode_wide_kernel"]["ms_median"]
+        out["512_to_%d_bits" % n_bits] = res
+        del cache
+    return out
+
+
 def plugin_surface(torch, caches, tables, lens, new_keys, queries, new_slots):
     """The same decode step at the reference's plugin surface: GSAOnDevice.attention_begin +
     attention_finished per layer (group-mean query, best KV head per block, sink = one block,
@@ -604,6 +658,8 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         #     2.1 GB, far beyond the last-level cache: a cold-HBM figure) hashed into the paged code
         #     cache through the permuted block table (compute_hash_and_cache, hash_encoder.py:548-662) ---
         out["encoder_cache_build"] = encoder_cache_build(torch, enc_k, gen)
+        # --- the same for latent vectors (K = 512): config 5's 512 -> 256 and the reference's 512 -> 512 ---
+        out["encoder_latent_cache_build"] = encoder_latent_cache_build(torch, gen)
 
     if "prefix_rehash" in legs:
         # --- prefix-cache rehash: keys of 256 blocks read in place from a paged key cache, against

@@ -165,6 +165,92 @@ def test_streaming_kernel_dense_output_many_tiles(stream_everything):
     assert bool((outs[0][T:] == 0x5A5A5A5A).all())
 
 
+# (seed, T, N, dtype, slot dtype, input row stride, code row words, first code word)
+WIDE_CASES = [
+    (31, 70000, 256, torch.bfloat16, torch.int64, 512, 8, 0),
+    (32, 70000 + 13, 512, torch.bfloat16, torch.int32, 576, 18, 0),   # latent rows of 576, 18-word code rows
+    (33, 40000, 512, torch.float16, torch.int64, 512, 16, 0),
+    (34, 300000, 256, torch.bfloat16, torch.int32, 576, 8, 0),        # 37 tiles per workgroup, ring reused 9x
+    (35, 32 * 256 * 4 + 1, 256, torch.bfloat16, torch.int64, 512, 12, 4),  # one tile more than the ring; codes at word 4
+    (36, 32 * 256 * 2, 512, torch.bfloat16, torch.int64, 512, 16, 0),  # exactly two tiles per workgroup pair
+]
+
+
+@pytest.mark.parametrize("seed,T,N,dtype,sdt,xstride,cwords,cfirst", WIDE_CASES)
+def test_wide_streaming_kernel_matches_oracle_and_tiled_kernel(stream_everything, seed, T, N, dtype, sdt, xstride,
+                                                               cwords, cfirst):
+    """K = 512 (latent vectors): the persistent kernel that shares each row tile between the eight
+    waves of a workgroup, against the fp64 closed form under the margin rule and against the tiled
+    kernel (same products, the k-steps added in two chains instead of one: codes may differ only where
+    the projection is within rounding of zero).  Dropped slots, words of a code row that belong to
+    somebody else (the rope part of a latent code) and rows past the end keep their canary."""
+    from ucm_amd import _lib
+
+    L = stream_everything
+    rng = rng_for(seed)
+    K, BS = 512, 64
+    NB = -(-T // BS) + 3
+    xfull = torch.from_numpy(rng.standard_normal((T, xstride)).astype(np.float32)).to(dtype).cuda()
+    x = xfull[:, :K].unsqueeze(1)  # [T, 1, 512] with rows xstride apart
+    W = torch.from_numpy(rng.standard_normal((1, K, N)).astype(np.float32)).to(dtype).cuda()
+    perm = rng.permutation(NB)
+    slots_np = (np.repeat(perm, BS)[:T] * BS + np.tile(np.arange(BS), NB)[:T]).astype(np.int64)
+    canary = 0x5A5A5A5A
+    drop = np.concatenate([rng.choice(T, size=5, replace=False), np.arange(32 * 300, 32 * 302),
+                           np.arange(12001, 12040)])
+    slots_in = slots_np.copy()
+    slots_in[drop] = -1
+    slots_in[drop[1]] = NB * BS + 4
+    slots = torch.from_numpy(slots_in).to(sdt).cuda()
+    outs = []
+    for thr in (1, 1 << 62):
+        L.ucm_hash_encode_set_stream_threshold(thr)
+        cache = torch.full((NB, BS, 1, cwords), canary, dtype=torch.int32, device="cuda")
+        view = cache[..., cfirst:cfirst + N // 32]
+        _encode_cache(L, x, W, slots, view, BS, 1, 0)
+        torch.cuda.synchronize()
+        outs.append(cache)
+    L.ucm_hash_encode_set_stream_threshold(1)
+    got, ref = (o.cpu().numpy().view(np.uint32) for o in outs)
+    codes = got[..., cfirst:cfirst + N // 32]
+    # only this call's words were written
+    other = np.ones(cwords, bool)
+    other[cfirst:cfirst + N // 32] = False
+    assert np.all(got[..., other] == canary)
+    flat = codes.reshape(-1, 1, N // 32)
+    keep = np.ones(T, bool)
+    keep[drop] = False
+    used = np.zeros(NB * BS, bool)
+    used[slots_np[keep]] = True
+    assert np.all(flat[~used] == canary)
+    # against the tiled kernel: the same bits except within rounding of a zero projection
+    diff_bits = np.unpackbits((got ^ ref).view(np.uint8)).sum()
+    assert diff_bits <= max(4, T * N // 200000), f"{diff_bits} bits differ from the tiled kernel"
+    rows = np.flatnonzero(keep)
+    if len(rows) > 400:
+        rows = np.sort(rng.choice(rows, size=400, replace=False))
+    _check_against_oracle(codes, x, W, slots_np, BS, 0, rows)
+
+
+def test_wide_streaming_kernel_dense_output(stream_everything):
+    from ucm_amd import _lib
+
+    L = stream_everything
+    rng = rng_for(41)
+    T, K, N = 50000 + 5, 512, 256
+    x = torch.from_numpy(rng.standard_normal((T, 1, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    W = torch.from_numpy(rng.standard_normal((1, K, N)).astype(np.float32)).to(torch.bfloat16).cuda()
+    out = torch.full((T + 40, 1, N // 32), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    _lib.check(L.ucm_hash_encode(x.data_ptr(), 0, T, 1, K, x.stride(0), x.stride(1), W.data_ptr(), 0, 1, 0, N,
+                                 out.data_ptr(), out.stride(0), out.stride(1),
+                                 torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    o = out.cpu().numpy().view(np.uint32)
+    assert np.all(o[T:] == 0x5A5A5A5A)
+    rows = np.sort(rng.choice(T, size=400, replace=False))
+    _check_against_oracle(o[:T].reshape(T, 1, 1, N // 32), x, W, np.arange(T), 1, 0, rows)
+
+
 def test_no_exchange_wait_reached_its_bound():
     """The waves of the streaming kernel wait for one another with bounded polls (a launch always
     ends); after the encoder tests of this process no wait may have reached the bound."""

@@ -979,6 +979,249 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
     stream_wait_loads<0>();
 }
 
+// ---------------------------------------------------------------------------------------
+// Wide streaming encoder: K = 512 input dimensions (the latent vector of latent attention), one
+// head, 256 or 512 hash bits, from some hundred thousand rows (building the code cache of a long
+// prompt or after a store hit).
+//
+// 512 x 256 bf16 are 256 KiB - half of a compute unit's register file - so the projection cannot
+// belong to one wave as in the 128-wide kernel above.  A persistent workgroup of eight waves owns a
+// slice of 256 hash columns for the kernel's lifetime, each wave 32 of them: 32 k-steps x 4
+// registers = 128 registers of MFMA A operands per lane.  (512 hash bits are two such slices, i.e. two
+// launches over the same rows.)  What the
+// eight waves share are the rows: a tile of 32 rows (32 KiB) is brought in once per workgroup,
+// straight from memory into LDS - every wave issues the loads of four rows, lane l of a load fetching
+// 16-byte piece l ^ (row & 7) so that the operand reads below hit all banks - and every wave
+// reads all of it as its B operands (one 16-byte LDS read per lane and MFMA).  Four tiles are
+// in the ring: at the barrier of tile i every wave has waited for its own loads of tile i, so the
+// tile is complete, and everybody is done with tile i - 1, so the loads of tile i + 3 go into its
+// slot: three tiles (96 KiB per compute unit) are in flight behind the one being multiplied.  One bare
+// barrier per tile.  Between two barriers the two waves of a SIMD
+// work in opposite order - one multiplies first and packs its signs afterwards, the other packs the
+// previous tile's signs first and multiplies then - so that the matrix cores are not left idle while
+// everybody packs (all waves in step: 0.25 ms per million rows at 256 bits; out of step: see below).
+// A wave's 32 x 32 products leave it as one word per row; the eight words of a row meet in a small
+// LDS buffer (three in turn), and two barriers later one wave - they take turns - stores the tile's
+// 32 code rows, 16 bytes per lane.  Roofline: 1 KiB read and 32 bytes written per row and slice
+// against 262,144 multiply-adds: at 256 bits memory and matrix cores bind about equally (0.14 ms
+// against 0.11 ms per million rows), at 512 bits the matrix cores do (0.22 ms).  The LDS read rate
+// (eight waves x 32 KiB per tile) equals the matrix cores' appetite exactly: both pipes would be
+// busy all the time in a perfect schedule.
+// ---------------------------------------------------------------------------------------
+constexpr int kWideWaves = 8;
+constexpr int kWideThreads = kWideWaves * 64;
+constexpr int kWideRing = 4;
+constexpr int kWideK = 512;
+constexpr int kWideTileBytes = kRowsPerWave * kWideK * 2;  // 32 KiB
+// a ring slot holds a tile; before the first tile it holds one wave's staged slice of W (32 rows of
+// K + kPad values)
+constexpr int kWideSlotBytes = kRowsPerWave * (kWideK + kPad) * 2;
+constexpr int kWideCodeBytes = kRowsPerWave * 32;  // 32 rows x 8 words
+constexpr int kWideMapRing = 8;                    // slot-mapping entries (256 bytes) of eight tiles
+constexpr size_t kWideLds = (size_t)kWideRing * kWideSlotBytes + 3 * kWideCodeBytes + kWideMapRing * 256;
+static_assert(kWideSlotBytes % 16 == 0 && kWideTileBytes <= kWideSlotBytes, "ring slot layout");
+static_assert(kWideLds <= 160 * 1024, "ring exceeds the LDS");
+
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+
+template <typename V, int SLOT>
+__global__ __launch_bounds__(kWideThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void encode_wide_kernel(
+    EncArgs a, int64_t ntiles, int nstreams, int col)
+{
+    extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[];
+    constexpr int K = kWideK, KS = K / 16;
+    constexpr int kLoads = 4 + (SLOT ? 1 : 0);  // load instructions per wave and tile
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 31, kb = lane >> 5;
+    const int stream = blockIdx.x;  // rows stream, stream + nstreams, ...; hash columns 256 col .. 256 col + 255
+    uint8_t* const codes = wide_lds + (size_t)kWideRing * kWideSlotBytes;
+    constexpr uint32_t kMapOff = (uint32_t)(kWideRing * kWideSlotBytes + 3 * kWideCodeBytes);
+
+    // ---- this wave's 32 columns of W as MFMA A operands, for the kernel's lifetime ----
+    // 8 x 8 patches (eight 16-byte rows each) are transposed in registers and written as 32 LDS
+    // rows of K values, then every lane reads its K / 16 operands.  A staged tile fills a ring
+    // slot, so the waves go in two shifts of four.
+    V wreg[KS];
+    {
+        constexpr int KP = K + kPad;
+        const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)weight_index(a, 0) * K * a.N + col * 256 + wave * 32;
+        uint16_t* wt = reinterpret_cast<uint16_t*>(wide_lds + (size_t)(wave & 3) * kWideSlotBytes);
+#pragma unroll
+        for (int shift = 0; shift < 2; ++shift) {
+            if ((wave >> 2) == shift) {
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {  // 256 patches, four per lane, two at a time
+                    u32x4 row[2][8];
+#pragma unroll
+                    for (int it = 0; it < 2; ++it) {
+                        const int idx = (half * 2 + it) * 64 + lane;
+                        const uint16_t* src = wsrc + (int64_t)((idx >> 2) * 8) * a.N + 8 * (idx & 3);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) row[it][i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * a.N);
+                    }
+#pragma unroll
+                    for (int it = 0; it < 2; ++it) {
+                        const int idx = (half * 2 + it) * 64 + lane;
+                        const int kq = idx >> 2, j = idx & 3;
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) {
+                            const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                            u32x4 o;
+                            o.x = __builtin_amdgcn_perm(row[it][1][c >> 1], row[it][0][c >> 1], sel);
+                            o.y = __builtin_amdgcn_perm(row[it][3][c >> 1], row[it][2][c >> 1], sel);
+                            o.z = __builtin_amdgcn_perm(row[it][5][c >> 1], row[it][4][c >> 1], sel);
+                            o.w = __builtin_amdgcn_perm(row[it][7][c >> 1], row[it][6][c >> 1], sel);
+                            *reinterpret_cast<u32x4*>(wt + (8 * j + c) * KP + kq * 8) = o;
+                        }
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    wreg[ks] = *reinterpret_cast<const V*>(wt + r * KP + ks * 16 + kb * 8);
+            }
+            __syncthreads();  // the staging area becomes the next shift's, then the row ring
+        }
+    }
+
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)wide_lds);
+    const uint32_t row_bytes = (uint32_t)(a.x_stride_t * 2);
+    constexpr int slot_sz = SLOT == 2 ? 8 : 4;
+    const uint32_t slot_e = SLOT == 2 ? (uint32_t)lane >> 1 : (uint32_t)lane & 31;
+    // A wave's share of a tile's loads: rows 4 * wave + j (j = 0..3), lane l fetching piece
+    // l ^ (row & 7); rows past the end of the input re-read its last row.  Every wave also fetches
+    // the tile's 32 slot-mapping entries into a ring of their own (all eight write the same values):
+    // one more instruction, so that every wave counts the same loads per tile.
+    uint32_t off_full[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t q = 4 * (uint32_t)wave + j;
+        off_full[j] = q * row_bytes + (((uint32_t)lane ^ (q & 7)) << 4);
+    }
+    const uint32_t slot_full = slot_e * slot_sz + (SLOT == 2 ? ((uint32_t)lane & 1) * 4 : 0);
+    auto issue = [&](int64_t tile, int local) {
+        const int64_t t0 = tile * kRowsPerWave;
+        const int64_t left64 = a.T - 1 - t0;
+        const uint64_t base = (uint64_t)(uintptr_t)((const uint16_t*)a.x + t0 * a.x_stride_t);
+        const uint32_t lds = lds0 + (local % kWideRing) * kWideSlotBytes;
+        uint32_t so = slot_full;
+        if (left64 >= 31) {
+            stream_issue_rows<1>(lds + wave * 4096, base, off_full);
+        } else {
+            const uint32_t left = (uint32_t)left64;
+            uint32_t off[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t q = 4 * (uint32_t)wave + j;
+                const uint32_t qq = q > left ? left : q;
+                off[j] = qq * row_bytes + (((uint32_t)lane ^ (q & 7)) << 4);
+            }
+            stream_issue_rows<1>(lds + wave * 4096, base, off);
+            const uint32_t ee = slot_e > left ? left : slot_e;
+            so = ee * slot_sz + (SLOT == 2 ? ((uint32_t)lane & 1) * 4 : 0);
+        }
+        if constexpr (SLOT != 0)
+            stream_issue_slots(lds0 + kMapOff + (local % kWideMapRing) * 256,
+                               (uint64_t)(uintptr_t)((const char*)a.slot + t0 * slot_sz), so);
+    };
+
+    // operand read offset of k-step ks: row r, piece (2 ks + kb) ^ (r & 7)
+    const uint32_t r_base = (uint32_t)r * 1024;
+    const uint32_t r_swz = (uint32_t)r & 7;
+    const int64_t n_slots = a.NB << a.bs_shift;
+    const uint32_t csb = (uint32_t)a.cs_block, cst = (uint32_t)a.cs_token;
+    uint32_t* const cache_c = a.cache + col * 8;
+
+    // Storing a tile's 32 code rows (lane l: half l & 1 of row l >> 1) takes two steps one tile apart:
+    // the slot-mapping entries are picked up first, the store follows when the last words have arrived.
+    int64_t held = -1;
+    auto pick_slots = [&](int64_t tile, int local) {
+        const uint8_t* slot_base = wide_lds + kMapOff + (local % kWideMapRing) * 256;
+        const int row = lane >> 1;
+        const int64_t t = tile * kRowsPerWave + row;
+        int64_t sv = t;
+        if constexpr (SLOT == 2) sv = *reinterpret_cast<const int64_t*>(slot_base + row * 8);
+        if constexpr (SLOT == 1) sv = *reinterpret_cast<const int32_t*>(slot_base + row * 4);
+        held = (t < a.T && sv >= 0 && sv < n_slots) ? sv : -1;
+    };
+    auto store_tile = [&](int local) {
+        const int row = lane >> 1, half = lane & 1;
+        const u32x4 code = *reinterpret_cast<const u32x4*>(codes + (local % 3) * kWideCodeBytes + row * 32 + half * 16);
+        if (held >= 0) {
+            const uint32_t svl = (uint32_t)held;
+            uint32_t* dst = cache_c + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) + half * 4;
+            *reinterpret_cast<u32x4_a4*>(dst) = code;
+        }
+    };
+    // a wave's 32 x 32 signs of a tile -> its word of each of the tile's 32 code rows
+    auto hand_in = [&](f32x16& acc0, const f32x16& acc1, int local) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc0[q] += acc1[q];
+        const uint32_t half = pack_half(acc0);
+        const uint32_t word = join_halves(kb ? half << 4 : half);
+        if (lane < 32) *reinterpret_cast<uint32_t*>(codes + (local % 3) * kWideCodeBytes + r * 32 + wave * 4) = word;
+    };
+
+    // The two waves of a SIMD (w and w + 4) take the work between two barriers in opposite order, so
+    // that one of them always has products for the matrix cores: waves 0..3 multiply tile i and hand
+    // its words in before the next barrier; waves 4..7 first hand in tile i - 1, then multiply tile i.
+    // A tile's words are therefore complete one barrier later, and its rows are stored after that.
+    const bool late = wave >= 4;
+    f32x16 acc0 = acc_start(), acc1;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc1[q] = 0.0f;
+
+    // tiles stream, stream + nstreams, ... : n of them
+    const int64_t n = stream < ntiles ? (ntiles - 1 - stream) / nstreams + 1 : 0;
+    int64_t tile = stream;
+    if (n > 0) issue(tile, 0);
+    if (n > 1) issue(tile + nstreams, 1);
+    if (n > 2) issue(tile + 2 * (int64_t)nstreams, 2);
+    for (int64_t i = 0; i < n + 2; ++i) {
+        const int local = (int)i;
+        if (i < n) {
+            // this wave's loads of tile i have landed (those of tiles i + 1 and i + 2 may be in flight)
+            if (i + 2 < n) stream_wait_loads<2 * kLoads>();
+            else if (i + 1 < n) stream_wait_loads<kLoads>();
+            else stream_wait_loads<0>();
+        }
+        // every wave's part of tile i is in LDS, and every wave is done reading tile i - 1: its ring
+        // slot takes tile i + 3
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (i + 3 < n) issue(tile + 3 * (int64_t)nstreams, local + 3);
+        if (late && i >= 1 && i <= n) {
+            hand_in(acc0, acc1, local - 1);
+            acc0 = acc_start();
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc1[q] = 0.0f;
+        }
+        if (i >= 2 && ((local - 2) % kWideWaves) == wave) store_tile(local - 2);
+        if (i >= 1 && i <= n && ((local - 1) % kWideWaves) == wave) pick_slots(tile - nstreams, local - 1);
+        if (i < n) {
+            const uint8_t* buf = wide_lds + (size_t)(local % kWideRing) * kWideSlotBytes;
+            // two accumulator chains in flight: the even and the odd k-steps, added at the end
+#pragma unroll
+            for (int ks = 0; ks < KS; ks += 2) {
+                const V b0 = *reinterpret_cast<const V*>(buf + r_base + ((((uint32_t)(2 * ks) + kb) ^ r_swz) << 4));
+                const V b1 = *reinterpret_cast<const V*>(buf + r_base + ((((uint32_t)(2 * ks + 2) + kb) ^ r_swz) << 4));
+                acc0 = Mfma<V>::run(wreg[ks], b0, acc0);
+                acc1 = Mfma<V>::run(wreg[ks + 1], b1, acc1);
+            }
+            if (!late) {
+                hand_in(acc0, acc1, local);
+                acc0 = acc_start();
+#pragma unroll
+                for (int q = 0; q < 16; ++q) acc1[q] = 0.0f;
+            }
+        }
+        tile += nstreams;
+    }
+    // no load may still be writing into this workgroup's LDS when the wave ends
+    stream_wait_loads<0>();
+}
+
 // Latency path for a handful of rows (decode): one wave per (job, head, 32 hash columns,
 // 32 rows).  No LDS and no persistent loop: the B operand is assembled straight from the
 // row-major projection matrix with eight 2-byte loads per k-step, all issued up front, so the
@@ -1261,7 +1504,14 @@ bool mfma_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 // the tiled kernel (65,536 rows: 14.8 against 12.4 us; 1M rows: 67.6 against 71.8 us; 4M rows: 225
 // against 262 us)
 constexpr int64_t kStreamMinRows = (int64_t)1 << 20;
-thread_local int64_t t_stream_min_rows = kStreamMinRows;  // per calling thread: a test hook must not move other threads' encodes
+// the wide (K = 512) kernel pays for itself earlier: it replaces a tiled kernel that re-reads the
+// rows once per slice of the projection (256 bits: 16,384 rows 19 against 26 us, 262,144 rows 74
+// against 164 us; 512 bits: 32,768 rows 36 against 34 us, 65,536 rows 52 against 65 us, 262,144 rows
+// 155 against 301 us)
+constexpr int64_t kWideMinRows256 = (int64_t)1 << 14;
+constexpr int64_t kWideMinRows512 = (int64_t)1 << 16;
+// 0 = the defaults above; set per calling thread (a test hook must not move other threads' encodes)
+thread_local int64_t t_stream_min_rows = 0;
 
 int stream_workgroups()
 {
@@ -1282,7 +1532,7 @@ bool stream_eligible(const EncArgs& a, int x_dtype, int w_dtype)
 {
     if (!mfma_eligible(a, x_dtype, w_dtype) || a.src_blocks) return false;
     if (!((a.K == 128 && (a.N == 128 || a.N == 64)) || (a.K == 64 && (a.N == 128 || a.N == 64)))) return false;
-    if (a.T * a.H < t_stream_min_rows) return false;
+    if (a.T * a.H < (t_stream_min_rows > 0 ? t_stream_min_rows : kStreamMinRows)) return false;
     if (a.slot && ((uintptr_t)a.slot & 3)) return false;
     // one shift per slot, one 16-byte store per four-word code (set_block_shift() has run)
     if (a.bs_shift < 0) return false;
@@ -1355,6 +1605,52 @@ int launch_stream(const EncArgs& a, hipStream_t st)
 {
     if (a.K == 128) return a.N == 128 ? launch_stream_s<V, 8, 4>(a, st) : launch_stream_s<V, 8, 2>(a, st);
     return a.N == 128 ? launch_stream_s<V, 4, 4>(a, st) : launch_stream_s<V, 4, 2>(a, st);
+}
+
+// The wide kernel takes one head of 512 input dimensions, 256 or 512 hash bits, dense rows.
+bool wide_eligible(const EncArgs& a, int x_dtype, int w_dtype)
+{
+    if (!mfma_eligible(a, x_dtype, w_dtype) || a.src_blocks || a.gmean > 1) return false;
+    if (a.K != kWideK || !(a.N == 256 || a.N == 512) || a.H != 1) return false;
+    if (a.T < (t_stream_min_rows > 0 ? t_stream_min_rows : (a.N == 256 ? kWideMinRows256 : kWideMinRows512))) return false;
+    if (a.slot && ((uintptr_t)a.slot & 3)) return false;
+    if (a.bs_shift < 0 || (((uintptr_t)a.cache) & 3)) return false;
+    // 32-bit offsets into the cache: non-negative strides, the last slot below 2^31 words
+    if (a.cs_block < 0 || a.cs_token < 0) return false;
+    if ((double)a.NB * (double)a.cs_block + (double)a.BS * (double)a.cs_token >= 2147483648.0) return false;
+    if ((double)a.NB * (double)a.BS >= 2147483648.0) return false;
+    return true;
+}
+
+template <typename V, int SLOT>
+int launch_wide_s(const EncArgs& a, hipStream_t st)
+{
+    static int opted = 0;  // 0 = not tried, 1 = allowed, -1 = refused by the runtime
+    if (opted == 0) {
+        const hipError_t e = hipFuncSetAttribute((const void*)encode_wide_kernel<V, SLOT>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLds);
+        if (e != hipSuccess) (void)hipGetLastError();
+        opted = (e == hipSuccess) ? 1 : -1;
+    }
+    if (opted < 0) return UCM_EUNSUPPORTED;
+    const int ncol = a.N / 256;
+    int wgs = stream_workgroups();
+    wgs -= wgs % 8;
+    if (wgs <= 0) return UCM_EUNSUPPORTED;
+    const int64_t ntiles = ucm::ceil_div(a.T, kRowsPerWave);
+    // one workgroup per compute unit and slice of 256 hash columns; a second slice is a second pass
+    // over the rows (two slices side by side, meeting in L2, measured the same)
+    for (int c = 0; c < ncol; ++c)
+        hipLaunchKernelGGL((encode_wide_kernel<V, SLOT>), dim3((unsigned)wgs), dim3(kWideThreads), kWideLds, st, a,
+                           ntiles, wgs, c);
+    return ucm::launch_status("encode_wide_kernel");
+}
+
+template <typename V>
+int launch_wide(const EncArgs& a, hipStream_t st)
+{
+    if (!a.slot) return launch_wide_s<V, 0>(a, st);
+    return a.slot_is_i64 ? launch_wide_s<V, 2>(a, st) : launch_wide_s<V, 1>(a, st);
 }
 
 int64_t small_waves(const EncArgs& a)
@@ -1606,6 +1902,11 @@ int encode_common(EncArgs a, int x_dtype, int w_dtype, hipStream_t st)
         return x_dtype == UCM_DT_BF16 ? launch_small<bf16x8>(js, js.waves0, a.K, st)
                                       : launch_small<f16x8>(js, js.waves0, a.K, st);
     }
+    if (wide_eligible(a, x_dtype, w_dtype)) {
+        rc = x_dtype == UCM_DT_BF16 ? launch_wide<bf16x8>(a, st) : launch_wide<f16x8>(a, st);
+        if (rc != UCM_EUNSUPPORTED) return rc;  // no large-LDS opt-in: the tiled kernel below
+        ucm::clear_error();
+    }
     if (stream_eligible(a, x_dtype, w_dtype)) {
         a.timeout_flag = stream_latch_flag();
         rc = x_dtype == UCM_DT_BF16 ? launch_stream<bf16x8>(a, st) : launch_stream<f16x8>(a, st);
@@ -1683,7 +1984,7 @@ extern "C" int ucm_hash_encode_debug_trip_stream_latch(void)
 extern "C" int ucm_hash_encode_set_stream_threshold(int64_t rows)
 {
     ucm::clear_error();
-    t_stream_min_rows = rows > 0 ? rows : kStreamMinRows;
+    t_stream_min_rows = rows > 0 ? rows : 0;
     return UCM_OK;
 }
 
