@@ -136,3 +136,18 @@ def test_encoder_timeout_latch_refuses_further_encodes_until_cleared():
     # acknowledged: the call gets past the latch (whatever it returns without a GPU, it is not the latch)
     encode()
     assert "gave up waiting" not in _lib.last_error()
+
+
+def test_torch_operator_library_registers_its_operators():
+    """torch.ops.ucm_amd.* (the TORCH_LIBRARY registration over the C ABI) loads without a GPU and
+    carries the three operators; a CPU tensor has no kernel behind it and is refused by the dispatcher."""
+    import torch
+
+    from ucm_amd import torch_ops
+
+    ops = torch_ops.load()
+    for name in ("hash_encode_cache", "hamming_topk", "gsa_decode_step"):
+        assert hasattr(ops, name)
+    z = torch.zeros((1, 1, 4), dtype=torch.int32)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        ops.hamming_topk(z, z.view(1, 1, 1, 4), z.view(1, 4)[:, :1], z.view(-1)[:1], 1, 0, 0, 0)

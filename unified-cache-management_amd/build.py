@@ -19,6 +19,8 @@ SRC = ["common.hip", "hamming_topk.hip", "hash_encode.hip", "trans.hip", "cache_
 LIB_DIR = os.path.join(HERE, "lib")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIB_DIR, "libucm_hip.so")
+TORCH_OPS_SRC = os.path.join(HERE, "csrc", "torch_ops.cpp")
+TORCH_OPS_LIB = os.path.join(LIB_DIR, "libucm_torch_ops.so")
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -66,7 +68,26 @@ def build(verbose=True, only_changed=False):
     with ThreadPoolExecutor(workers) as ex:
         list(ex.map(lambda c: _run(c, verbose), jobs))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB], verbose)
+    if not only_changed or _stale(TORCH_OPS_SRC, TORCH_OPS_LIB):
+        build_torch_ops(verbose)
     return LIB
+
+
+def build_torch_ops(verbose=True):
+    """libucm_torch_ops.so: the TORCH_LIBRARY registration (torch.ops.ucm_amd.*) over the C ABI.  Host
+    code only (g++), linked against libucm_hip.so and the installed PyTorch."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "csrc")]
+    cmd += ["-I" + p for p in ce.include_paths()] + ["-I/opt/rocm/include", "-w"]
+    cmd += [TORCH_OPS_SRC, "-o", TORCH_OPS_LIB, "-L" + LIB_DIR, "-lucm_hip", "-L" + tlib, "-ltorch", "-ltorch_cpu",
+            "-lc10", "-lc10_hip", "-ltorch_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + tlib]
+    _run(cmd, verbose)
+    return TORCH_OPS_LIB
 
 
 if __name__ == "__main__":
