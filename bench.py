@@ -845,7 +845,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         out["scatter_device"] = {"ms": ms, "hbm_GBps": 2 * payload / ms / 1e6}
         ms = timed(lambda: st.PagedGatherAsync(base, sizes, ids, host.data_ptr()), 2)
         out["gather_to_pinned_host"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6,
-                                        "form": "per 64 MiB piece: compaction kernel into device staging, one copy-engine transfer"}
+                                        "form": "per 256 MiB piece: compaction kernel into device staging, one copy-engine transfer"}
         ms = timed(lambda: st.DeviceToHostAsync(dev_flat.data_ptr(), host.data_ptr(), payload), 2)
         out["d2h_copy_engine_flat"] = {"ms": ms, "pcie_GBps": payload / ms / 1e6}
         ms = timed(lambda: st.PagedScatterAsync(host.data_ptr(), base, sizes, ids), 2)

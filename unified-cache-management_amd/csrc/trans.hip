@@ -17,7 +17,7 @@
 //       So gather / scatter / paged copies whose flat side is host memory go in two stages per
 //       piece of up to kStageBytes: the kernel compacts between the paged cache and a device
 //       staging buffer at HBM speed, and one copy-engine transfer moves the piece over PCIe
-//       (41-55 GB/s with the decode step running beside it at 33-37 us, no stalls).  Batch copies
+//       (54-56 GB/s with the decode step running beside it at 35-37 us, no stalls).  Batch copies
 //       (two pointer tables) with a host end keep the direct kernel on kHostCopyGroups
 //       workgroups.
 #include "common.h"
@@ -33,7 +33,12 @@ constexpr int kThreads = 256;
 constexpr size_t kSeg = (size_t)kThreads * 16;  // 4 KiB per workgroup
 constexpr int kSlots = 4;
 constexpr size_t kHostCopyGroups = 16;          // workgroups of a batch copy with a host end
-constexpr size_t kStageBytes = (size_t)64 << 20;  // device staging of host-ended copies, per stream
+// Device staging of host-ended copies, per stream.  A piece costs its kernel (40 us at this size) and
+// two dependent launches before the link is busy again: 64 MiB pieces reach 54.5 GB/s to the host,
+// 256 MiB pieces 55.8 GB/s (a flat copy-engine transfer: 57.0 GB/s).  Two staging buffers with the
+// transfers (or the kernels) on a second stream, joined by events, were slower than either: 37 and
+// 44 GB/s - every cross-stream dependency costs more than the kernel it would hide.
+constexpr size_t kStageBytes = (size_t)256 << 20;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
