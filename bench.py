@@ -302,7 +302,8 @@ def graph_ms(torch, fn, reps=20, replays=5):
 def scorer_kernel_us(torch, fn, n=30, with_call=False):
     """Mean duration in microseconds of the block-score dispatch inside fn(): the library attaches
     the two events to that dispatch as its start / stop events (eager launches).  with_call: also the
-    mean of (whole call - that dispatch) over the same launches, from events around each call."""
+    mean of (whole call - that dispatch) over the same launches, from events around each call, with
+    the launches queued behind a sleeping kernel (device time, no host launch gaps)."""
     L = _lib_mod().lib()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
     around = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
@@ -312,6 +313,10 @@ def scorer_kernel_us(torch, fn, n=30, with_call=False):
     for _ in range(3):
         fn()
     torch.cuda.synchronize()
+    if with_call and not NO_GRAPH:
+        # the launches below queue up behind a sleeping kernel, so the events around a call see the
+        # device's time for it and not the host's launch gaps
+        torch.cuda._sleep(int(n * 60e-6 * 2.0e9))
     for (a, b), (c0, c1) in zip(ev, around):
         L.ucm_hamming_topk_set_profile_events(a.cuda_event, b.cuda_event)
         c0.record()

@@ -51,7 +51,7 @@ TOPK_SHAPES = {
                                         "plane_kernel+block_score_pairs<0,5>+select_wave_kernel<4>"),
     "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], 8, {}, "block_score_lanes<9,1,1>+select_wave_kernel<4>"),
     "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], 8, {},
-                                       "block_score_lanes_run<9,7>+select_wave_kernel<4>"),
+                                       "block_score_strip18<2>+select_wave_kernel<4>"),
     "config5_blocks_of_128": (2, 128, 1, 8, 128, [8192, 700], 8, {},
                               "plane_kernel+block_score_lanes<4,0,8>+select_wave_kernel<4>"),
     "odd_code_width": (2, 6, 2, 3, 16, [1024, 300], 8, {}, "block_score_generic+select_wave_kernel<4>"),
@@ -110,8 +110,8 @@ def test_per_token_scorer_takes_its_kernels_and_matches_the_checker(name):
 def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
     """One KV head: the scorer reduces the G query heads to per-bit counts itself (no plane kernel)
     when the blocks hold 64 tokens - for every G with 8-word codes (counts as nibble digits for the
-    4-bit dot product), up to 128 heads with 16- and 18-word codes (bit planes); larger blocks keep
-    the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
+    4-bit dot product) and, up to 128 heads, with 18-word codes; up to 128 heads with 16-word codes
+    (bit planes); larger blocks keep the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
     that end inside a workgroup), table entries out of range, forced blocks."""
     from ucm_amd import _lib
     from ucm_amd.sparse import hamming_topk
@@ -132,6 +132,8 @@ def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
         got = _lib.last_dispatch()
         if (Wd, BS) == (8, 64):
             assert got.startswith("block_score_dot64<%d>+" % (1 if G <= 15 else 2))
+        elif (Wd, BS) == (18, 64) and G <= 128:
+            assert got.startswith("block_score_strip18<%d>+" % (1 if G <= 15 else 2))
         elif BS == 64 and G <= 128:
             assert got.startswith("block_score_lanes_run<%d,%d>+" % (Wd // 2, planes))
         else:

@@ -1111,7 +1111,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     }
 }
 
-// 64-token blocks of 16- or 18-word codes with bit planes: block_score_lanes' walk (a round of 64
+// 64-token blocks of 16-word codes with bit planes (18-word codes have block_score_strip18; the
+// figures below were taken with them): block_score_lanes' walk (a round of 64
 // tokens through the wave's LDS strip, planes re-read from LDS) over a run of kLaneRun consecutive
 // blocks per wave - the next block's codes are requested before the current one is computed - with
 // the planes built by wave 0 of the workgroup while the first codes are in flight (up to 128 query
@@ -1320,22 +1321,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
 constexpr int kDotRun = 4;    // blocks per wave
 constexpr int kDotWaves = 8;  // waves per workgroup
 
-template <int CTRL, int ROWMASK>
-__device__ __forceinline__ int dpp_min_step(int x)
-{
-    const int t = __builtin_amdgcn_update_dpp(x, x, CTRL, ROWMASK, 0xf, false);
-    return t < x ? t : x;
-}
 // Minimum over the 64 lanes, valid in lane 63: butterflies inside a row of 16 lanes, then the
-// last lane of a row broadcast into the next row(s).
+// last lane of a row broadcast into the next row(s).  Written out as v_min_i32 with a DPP operand
+// (the compiler turns the builtin into a copy, a DPP move and a minimum per step); a DPP operand
+// needs two idle cycles after the instruction that wrote it.
 __device__ __forceinline__ int wave_min_lane63(int x)
 {
-    x = dpp_min_step<0xB1, 0xf>(x);   // quad_perm [1,0,3,2]
-    x = dpp_min_step<0x4E, 0xf>(x);   // quad_perm [2,3,0,1]
-    x = dpp_min_step<0x141, 0xf>(x);  // row_half_mirror
-    x = dpp_min_step<0x140, 0xf>(x);  // row_mirror
-    x = dpp_min_step<0x142, 0xa>(x);  // row_bcast15 into rows 1 and 3
-    x = dpp_min_step<0x143, 0xc>(x);  // row_bcast31 into rows 2 and 3
+    asm volatile("s_nop 1\n\t"
+                 "v_min_i32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_min_i32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_min_i32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_min_i32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_min_i32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_min_i32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf"
+                 : "+v"(x));
     return x;
 }
 
@@ -1505,6 +1504,275 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
         int d = (i < run && t0 < len) ? dd[0] : kInf;
         const int d1 = (i < run && t0 + 32 < len) ? dd[1] : kInf;
         d = d1 < d ? d1 : d;
+        const int m = __builtin_amdgcn_readlane(wave_min_lane63(d), 63) + base;
+        const int ntok = (64 < len - pos0) ? 64 : len - pos0;
+        const bool forced = (pos0 < sink) || (pos0 + ntok > len - recent);
+        const int sc = (entry[i] < 0 || entry[i] >= NB) ? -1 : (forced ? full : full - m);
+        if (lane == i) result = sc;
+    }
+    if (lane < run) scores[(int64_t)b * max_blocks + j0 + lane] = result;
+}
+
+// 64-token blocks of 18-word codes against one KV head whose G query heads enter as per-bit
+// counts (the latent cache with position part: 16 requests x 65,536 tokens, 75 MB of codes in
+// 16,384 blocks of 4.5 KiB).  block_score_dot64's arithmetic with a whole code per lane:
+//
+// Codes.  A block goes from memory straight into the wave's LDS strip (load-to-LDS, five
+// instructions of 1 KiB, the last one half masked): no register holds a code on its way, no LDS
+// store instruction is issued.  The strip holds four blocks; a wave scores a run of eight and
+// requests block i + 4 the moment block i's reads are back.  Lane l reads token l's row (72 bytes
+// apart: 16 consecutive lanes cover all banks) as nine 8-byte reads.
+//
+// Weights.  The eight weight words of each of the 18 code words ([bit residue j][digit]) are
+// wave-uniform and stay in 144 registers for the whole run (two waves per SIMD: 256 registers a
+// lane), so a block costs 9 LDS reads and about 270 vector operations - against 50 and 370 with
+// bit planes re-read from LDS for every block.  Measured at 16 x 65,536 tokens, 64 query heads:
+// the loads alone (no arithmetic) 12.6 us, the arithmetic alone (no loads) 9.7 us, together
+// 16.7 us; the arithmetic (16 blocks a SIMD x 270 operations x 4 cycles) is what the waves wait
+// for once the codes flow, bit planes with popcounts (15 a word) and 8-bit dot products (16 a
+// word) need more of it than the 13 a word of the 4-bit dot product.
+//
+// Build.  All four waves build the weights in three steps with LDS in between (one wave doing
+// all of it held the workgroup for 2.4 to 5 us): lane (w, g) of wave v counts word w of heads
+// 3 v + g, 3 v + g + 12, ... bit-sliced; lane (w, p) counts the groups whose partial count has
+// bit p set; lane (w, j) adds those four numbers, shifted, and assembles the two weight words of
+// residue j.  Up to 128 query heads.  Only two of the four first blocks are requested before the
+// build: a compute unit takes one 1 KiB load instruction per 16 cycles, and the eight resident
+// waves' first four blocks each would keep every wave at its load instructions for a microsecond.
+constexpr int kStripWaves = 4;  // waves per workgroup
+constexpr int kStripRun = 8;    // blocks per wave
+constexpr int kStripSlots = 4;  // blocks of a wave in LDS
+constexpr int kStripFirst = 2;  // of those, requested before the weight build
+
+// One block of NL KiB (+ half a KiB when TAIL) from `base` into LDS at byte address `lds`.
+template <int NL, bool TAIL>
+__device__ __forceinline__ void strip_issue_block(uint32_t lds, uint64_t base, uint32_t off, bool low_half)
+{
+    static_assert(NL == 4, "a block of 64 codes of 16 or 18 words");
+    uint32_t keep;
+    asm volatile("s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[lds]\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %[o], %[base] nt\n\t"
+                 "global_load_lds_dwordx4 %[o], %[base] offset:1024 nt\n\t"
+                 "global_load_lds_dwordx4 %[o], %[base] offset:2048 nt\n\t"
+                 "global_load_lds_dwordx4 %[o], %[base] offset:3072 nt\n\t"
+                 "s_mov_b32 m0, %[keep]\n\t"
+                 : [keep] "=&s"(keep)
+                 : [lds] "s"(lds), [base] "s"(base), [o] "v"(off)
+                 : "memory");
+    if (TAIL) {
+        if (low_half) {
+            asm volatile("s_mov_b32 %[keep], m0\n\ts_add_u32 m0, %[lds], 4096\n\ts_nop 0\n\t"
+                         "global_load_lds_dwordx4 %[o], %[base] nt\n\t"
+                         "s_mov_b32 m0, %[keep]\n\t"
+                         : [keep] "=&s"(keep)
+                         : [lds] "s"(lds), [base] "s"(base), [o] "v"(off + 4096u)
+                         : "memory", "scc");
+        }
+    }
+}
+
+template <int ND>
+__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void block_score_strip18(ScoreArgs a)
+{
+
+    constexpr int WD = 18, RUN = kStripRun, kSlots = kStripSlots, kFirst = kStripFirst;
+    constexpr int NG = 3 * kStripWaves;  // head groups of the weight build: 3 per wave
+    constexpr int kBlockWords = 64 * WD;
+    constexpr int kLoadsPerBlock = 5;
+    __shared__ __align__(16) uint32_t strip[kStripWaves][kSlots * kBlockWords];
+    __shared__ __align__(16) uint32_t wl[WD * 8];        // weight word [w][j][digit]
+    __shared__ __align__(16) uint32_t part[NG * WD * 4];  // [group][w][plane]: counts of a group's heads
+    __shared__ __align__(16) uint32_t cnt[WD * 4 * 4];    // [w][plane p][plane]: groups with bit p set
+    __shared__ int base_s;
+    const int b = blockIdx.y;
+    const int lane = lane_id(), wid = wave_id();
+    const int j0 = (blockIdx.x * kStripWaves + wid) * RUN;
+    // round 1: the reads that need the kernel arguments only
+    const int len = a.lens[b];
+    int my_entry;  // lane i: table entry of block j0 + i
+    {
+        const int j = j0 + (lane & 7);
+        const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+        if (a.table) my_entry = a.table[(int64_t)b * a.table_stride + jc];
+        else my_entry = b * a.max_blocks + jc;
+    }
+    // lane (w, g) of wave v: word w of heads gi, gi + 12, ... with gi = 3 v + g (up to 11 heads)
+    const int pw = lane % WD, pg = lane / WD;
+    const int gi = wid * 3 + pg;
+    const int G = a.G;
+    uint32_t qx[16];
+    {
+        const uint32_t* qb = a.q + b * a.q_stride_b + pw;
+        const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
+#pragma unroll
+        for (int t = 0; t < 11; ++t) {
+            const int h = gi + NG * t;  // heads past the group re-read the last one, as zero
+            qx[t] = qb[(h < G ? h : G - 1) * qs];
+        }
+#pragma unroll
+        for (int t = 11; t < 16; ++t) qx[t] = 0;
+    }
+    // everything the rest of the kernel takes from its arguments, now
+    const int64_t NB = a.NB, ks_block = a.ks_block;
+    const uint32_t* kc = a.kc;
+    const int sink = a.sink, recent = a.recent, max_blocks = a.max_blocks;
+    int32_t* scores = a.scores;
+    asm volatile("" ::"s"(sink), "s"(recent), "s"(scores), "s"(NB), "s"(G), "s"(max_blocks));
+    int nblk = len > 0 ? (len + 63) >> 6 : 0;
+    if (nblk > max_blocks) nblk = max_blocks;
+    if ((int)blockIdx.x * kStripWaves * RUN >= nblk) return;  // the whole workgroup
+    const int run = nblk - j0 < RUN ? nblk - j0 : RUN;  // <= 0: nothing to score
+    int entry[RUN];
+#pragma unroll
+    for (int i = 0; i < RUN; ++i) entry[i] = __builtin_amdgcn_readlane(my_entry, i);
+    {
+        uint32_t o = 0;
+#pragma unroll
+        for (int t = 0; t < 11; ++t) o |= qx[t];
+        asm volatile("" ::"v"(o));  // the query words are here: no code is requested before
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // round 2: the first blocks of the run
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)strip[wid]);
+    const uint32_t off = (uint32_t)lane * 16u;
+    auto issue = [&](int i) __attribute__((always_inline)) {
+        int64_t pb = entry[i];
+        if (pb < 0 || pb >= NB) pb = 0;  // scored as -1 below
+        strip_issue_block<4, true>(lds0 + (uint32_t)(i % kSlots) * (kBlockWords * 4),
+                                   reinterpret_cast<uint64_t>(kc + pb * ks_block), off, lane < 32);
+    };
+#pragma unroll
+    for (int i = 0; i < kFirst; ++i)
+        if (i < run) issue(i);
+    __builtin_amdgcn_sched_barrier(0);
+    // The weights, by all four waves in three steps with LDS between them.  (A compute unit
+    // takes a 1 KiB load instruction every 16 cycles: the eight resident waves' first four
+    // blocks each would hold every wave at its load instructions for a microsecond before the
+    // build starts, so only the first kFirst go out here.)
+    // 1: every lane counts its group's heads bit-sliced (four planes, at most 11 heads).
+    {
+        uint32_t n[5];
+#pragma unroll
+        for (int t = 0; t < 11; ++t) qx[t] = (gi + NG * t < G && pg < 3) ? qx[t] : 0u;
+        count16(qx, n);
+        if (pg < 3) *reinterpret_cast<u32x4*>(part + (gi * WD + pw) * 4) = u32x4{n[0], n[1], n[2], n[3]};
+        if (threadIdx.x == 0) base_s = 0;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // 2: lane (w, p) of waves 0 and 1 counts the groups whose plane p has a bit set: the count of
+    //    a bit is  sum_p 2^p * (that number).
+    const int p2 = wid * 2 + pg;  // waves 0 and 1, lanes below 2 * WD
+    if (wid < 2 && lane < 2 * WD) {
+        uint32_t y[16], m[5];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) y[g] = part[(g * WD + pw) * 4 + p2];
+#pragma unroll
+        for (int g = NG; g < 16; ++g) y[g] = 0;
+        count16(y, m);
+        *reinterpret_cast<u32x4*>(cnt + (pw * 4 + p2) * 4) = u32x4{m[0], m[1], m[2], m[3]};
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // 3: the same lanes, now (w, j): add the four numbers, shifted, and assemble the two weight
+    //    words of bit residue j (nibble n = a digit of the count of bit 4 * n + j)
+    if (wid < 2 && lane < 2 * WD) {
+        uint32_t acc[8];
+        {
+            const u32x4 n0 = *reinterpret_cast<const u32x4*>(cnt + (pw * 4) * 4);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = i < 4 ? n0[i] : 0u;
+        }
+#pragma unroll
+        for (int p = 1; p < 4; ++p) {
+            const u32x4 np = *reinterpret_cast<const u32x4*>(cnt + (pw * 4 + p) * 4);
+            uint32_t cy = 0;
+#pragma unroll
+            for (int i = p; i < 8; ++i) {
+                uint32_t sum, c2;
+                if (i - p < 4) full_add(acc[i], np[i - p], cy, sum, c2);
+                else half_add(acc[i], cy, sum, c2);
+                acc[i] = sum;
+                cy = c2;
+            }
+        }
+        uint32_t r0 = 0, r1 = 0;
+#pragma unroll
+        for (int pp = 0; pp < 4; ++pp) {
+            r0 |= ((acc[pp] >> p2) & 0x11111111u) << pp;
+            r1 |= ((acc[4 + pp] >> p2) & 0x11111111u) << pp;
+        }
+        *reinterpret_cast<u32x2*>(wl + pw * 8 + 2 * p2) = u32x2{r0, r1};
+        if (p2 == 0) {
+            int c = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) c += __popc(acc[i]) << i;
+            atomicAdd(&base_s, c);  // sum over all code bits of the per-bit counts
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int i = kFirst; i < kSlots; ++i)
+        if (i < run) issue(i);
+    if (run <= 0) return;
+    const int base = base_s;
+    const int full = G * 32 * WD;
+    u32x4 W[WD][2];  // [w] -> {j = 0: lo, hi; j = 1: lo, hi}, {j = 2, j = 3}
+    {
+        const u32x4* src = reinterpret_cast<const u32x4*>(wl);
+#pragma unroll
+        for (int i = 0; i < WD; ++i) {
+            W[i][0] = src[2 * i];
+            W[i][1] = src[2 * i + 1];
+        }
+    }
+    int result = 0;  // lane i: score of block j0 + i
+#pragma unroll
+    for (int i = 0; i < RUN; ++i) {
+        if (i >= run) break;
+        // block i's codes have landed: loads complete in order, and at most the kSlots - 1 blocks
+        // requested behind it may still be under way
+        {
+            const int behind = run - 1 - i < kSlots - 1 ? run - 1 - i : kSlots - 1;
+            if (behind >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kLoadsPerBlock) : "memory");
+            else if (behind == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerBlock) : "memory");
+            else if (behind == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerBlock) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        const uint32_t* row = strip[wid] + (i % kSlots) * kBlockWords + lane * WD;
+        uint32_t k[WD];
+#pragma unroll
+        for (int w = 0; w < WD / 2; ++w) {
+            const u32x2 kk = *reinterpret_cast<const u32x2*>(row + 2 * w);
+            k[2 * w] = kk.x;
+            k[2 * w + 1] = kk.y;
+        }
+        int pk = 0;
+        uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int w = 0; w < WD; ++w) {
+            pk = popc_add(k[w], pk);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t e = k[w] & (0x11111111u << j);
+                lo[j] = __builtin_amdgcn_udot8(e, W[w][j >> 1][(j & 1) * 2], lo[j], false);
+                if (ND > 1) hi[j] = __builtin_amdgcn_udot8(e, W[w][j >> 1][(j & 1) * 2 + 1], hi[j], false);
+            }
+        }
+        // the sums exist here: left to the compiler they sink towards their last use, behind
+        // the branches below
+        asm volatile("" : "+v"(pk), "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]));
+        if (ND > 1) asm volatile("" : "+v"(hi[0]), "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3]));
+        if (i + kSlots < run) {
+            // this strip slot is free once its last reads are back
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            issue(i + kSlots);
+        }
+        uint32_t t[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[j] = ND > 1 ? lo[j] + (hi[j] << 4) : lo[j];
+        const uint32_t x8 = (((((t[0] << 1) + t[1]) << 1) + t[2]) << 1) + t[3];  // 8 * sum_b k_b * c_b
+        const int pos0 = (j0 + i) << 6;
+        const int d = pos0 + lane < len ? G * pk - (int)(x8 >> 2) : kInf;
         const int m = __builtin_amdgcn_readlane(wave_min_lane63(d), 63) + base;
         const int ntok = (64 < len - pos0) ? 64 : len - pos0;
         const bool forced = (pos0 < sink) || (pos0 + ntok > len - recent);
@@ -2653,11 +2921,23 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
                 if (nd == 1) hipLaunchKernelGGL(block_score_dot64<1>, g64, threads, 0, st, a);
                 else hipLaunchKernelGGL(block_score_dot64<2>, g64, threads, 0, st, a);
             }
+        } else if (planes_in_lanes && Wd == 18) {
+            const int nd = a.G <= 15 ? 1 : 2;
+            note_score("block_score_strip18", nd);
+            const dim3 g64((unsigned)ucm::ceil_div(max_blocks, kStripWaves * kStripRun), (unsigned)B);
+            ++g_note.score_launches;
+            const dim3 threads(kStripWaves * kWave);
+            if (g_prof_before && g_prof_after) {
+                if (nd == 1) hipExtLaunchKernelGGL(block_score_strip18<1>, g64, threads, 0, st, g_prof_before, g_prof_after, 0, a);
+                else hipExtLaunchKernelGGL(block_score_strip18<2>, g64, threads, 0, st, g_prof_before, g_prof_after, 0, a);
+            } else {
+                if (nd == 1) hipLaunchKernelGGL(block_score_strip18<1>, g64, threads, 0, st, a);
+                else hipLaunchKernelGGL(block_score_strip18<2>, g64, threads, 0, st, a);
+            }
         } else if (planes_in_lanes) {
             note_score("block_score_lanes_run", Wd / 2, pmax);
             const dim3 g64((unsigned)ucm::ceil_div(max_blocks, (kThreads / kWave) * kLanesRunBlocks), (unsigned)B);
-            if (Wd == 18) launch_lanes_run<9>(a, pmax, g64, st);
-            else launch_lanes_run<8>(a, pmax, g64, st);
+            launch_lanes_run<8>(a, pmax, g64, st);  // 16-word codes
         } else if (lanes_layout(a, k_cache, direct)) {
             if (Wd == 18) dispatch_lanes<9>(a, pmax, pgrid, st);
             else if (Wd == 16) dispatch_lanes<8>(a, pmax, pgrid, st);
