@@ -301,27 +301,20 @@ def graph_ms(torch, fn, reps=20, replays=5):
 
 def scorer_kernel_us(torch, fn, n=30, with_call=False):
     """Mean duration in microseconds of the block-score dispatch inside fn(): the library attaches
-    the two events to that dispatch as its start / stop events (eager launches).  with_call: also the
-    mean of (whole call - that dispatch) over the same launches, from events around each call, with
-    the launches queued behind a sleeping kernel (device time, no host launch gaps)."""
+    the two events to that dispatch as its start / stop events (eager launches).  with_call: also
+    (whole call - that dispatch), the call timed in the same mode: n eager calls queued behind a
+    sleeping kernel, so that the device runs them back to back, between one pair of events."""
     L = _lib_mod().lib()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-    around = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
     for a, b in ev:  # creates the underlying hipEvent_t
         a.record()
         b.record()
     for _ in range(3):
         fn()
     torch.cuda.synchronize()
-    if with_call and not NO_GRAPH:
-        # the launches below queue up behind a sleeping kernel, so the events around a call see the
-        # device's time for it and not the host's launch gaps
-        torch.cuda._sleep(int(n * 60e-6 * 2.0e9))
-    for (a, b), (c0, c1) in zip(ev, around):
+    for a, b in ev:
         L.ucm_hamming_topk_set_profile_events(a.cuda_event, b.cuda_event)
-        c0.record()
         fn()
-        c1.record()
     torch.cuda.synchronize()
     L.ucm_hamming_topk_set_profile_events(None, None)
     keep = max(1, n * 3 // 4)  # without the slowest quarter: eager launches after idle gaps
@@ -329,8 +322,16 @@ def scorer_kernel_us(torch, fn, n=30, with_call=False):
     sc = sum(ev[i][0].elapsed_time(ev[i][1]) for i in order) / keep * 1e3
     if not with_call:
         return sc
-    rest = sum(around[i][0].elapsed_time(around[i][1]) - ev[i][0].elapsed_time(ev[i][1]) for i in order) / keep * 1e3
-    return sc, rest
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    if not NO_GRAPH:
+        torch.cuda._sleep(int(n * 60e-6 * 2.0e9))
+    c0.record()
+    for _ in range(n):
+        fn()
+    c1.record()
+    torch.cuda.synchronize()
+    call = c0.elapsed_time(c1) / n * 1e3
+    return sc, max(call - sc, 0.0)
 
 
 def topk_split(torch, fn, ms, code_bytes):
@@ -340,9 +341,10 @@ def topk_split(torch, fn, ms, code_bytes):
     sc, rest = scorer_kernel_us(torch, fn, with_call=True)
     return {"hbm_frac_operator": code_bytes / ms / 1e6 / HBM_PEAK_GBPS, "scorer_us": sc,
             "scorer_hbm_frac": code_bytes / sc / 1e3 / HBM_PEAK_GBPS, "selection_and_rest_us": rest,
-            "scorer_timing": "eager launches: dispatch start/stop events of the scorer, events around the "
-                             "call for the rest (a launch after an idle gap runs 1-2 us longer than inside a "
-                             "graph; the committed kernel traces hold both)"}
+            "scorer_timing": "eager launches: dispatch start/stop events of the scorer; the rest is the mean "
+                             "device time of a call in a queue of eager calls minus that (a launch after an "
+                             "idle gap runs 1-2 us longer than inside a graph; the committed kernel traces "
+                             "hold both)"}
 
 
 OP_FLOOR_US = 25.3  # measured with stand-alone probes of the same traffic shape (see the design notes)

@@ -1880,16 +1880,39 @@ __device__ __forceinline__ bool plugin_row_prologue(const SelectArgs& a, int b, 
     return kk == 0;
 }
 
+// Inclusive prefix sum over the 64 lanes with DPP operands (row shifts inside a row of 16 lanes -
+// a lane without a source adds 0 - then the last lane of a row broadcast into the next row(s)):
+// six additions a few cycles apart, where six lane exchanges through the LDS pipe cost some
+// hundred cycles each, one after the other.
+__device__ __forceinline__ int wave_incl_scan(int v)
+{
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+// Maximum over the 64 lanes, valid in lane 63 (see wave_min_lane63).
+__device__ __forceinline__ int wave_max_lane63(int x)
+{
+    asm volatile("s_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\ts_nop 1\n\t"
+                 "v_max_i32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf"
+                 : "+v"(x));
+    return x;
+}
+
 // Exclusive prefix sum of one int per thread over the 256-thread workgroup; *total gets the
 // sum.  `wsum` is a 4-entry LDS array.
 __device__ __forceinline__ int block_exclusive_scan(int v, int* wsum, int* total)
 {
-    int inc = v;
-#pragma unroll
-    for (int s = 1; s < kWave; s <<= 1) {
-        const int o = __shfl_up(inc, s);
-        if (lane_id() >= s) inc += o;
-    }
+    const int inc = wave_incl_scan(v);
     __syncthreads();  // protects wsum from the previous use
     if (lane_id() == kWave - 1) wsum[threadIdx.x >> 6] = inc;
     __syncthreads();
@@ -1975,12 +1998,7 @@ __global__ __launch_bounds__(kThreads) void select_kernel(SelectArgs a)
             const int d0 = 255 - 4 * tid;
             const int c0 = hist[d0], c1 = hist[d0 - 1], c2 = hist[d0 - 2], c3 = hist[d0 - 3];
             const int mine = c0 + c1 + c2 + c3;
-            int inc = mine;
-#pragma unroll
-            for (int st = 1; st < kWave; st <<= 1) {
-                const int o = __shfl_up(inc, st);
-                if (tid >= st) inc += o;
-            }
+            const int inc = wave_incl_scan(mine);
             const int above = inc - mine;  // keys with a larger digit than any of mine
             if (above < need && need <= inc) {
                 int acc = above, digit = d0, cnt = c0;
@@ -2064,13 +2082,8 @@ __global__ __launch_bounds__(kThreads) void select_kernel(SelectArgs a)
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ int wave_excl_scan(int v, int* total)
 {
-    int inc = v;
-#pragma unroll
-    for (int s = 1; s < kWave; s <<= 1) {
-        const int o = __shfl_up(inc, s);
-        if (lane_id() >= s) inc += o;
-    }
-    *total = __shfl(inc, kWave - 1);
+    const int inc = wave_incl_scan(v);
+    *total = __builtin_amdgcn_readlane(inc, kWave - 1);
     return inc - v;
 }
 
@@ -2168,14 +2181,8 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
         if (lane * EL + e < n) lo = v[e] < lo ? v[e] : lo;
         hi = v[e] > hi ? v[e] : hi;
     }
-#pragma unroll
-    for (int st = 1; st < kWave; st <<= 1) {
-        const int l2 = __shfl_xor(lo, st), h2 = __shfl_xor(hi, st);
-        lo = l2 < lo ? l2 : lo;
-        hi = h2 > hi ? h2 : hi;
-    }
-    lo = __builtin_amdgcn_readfirstlane(lo);
-    hi = __builtin_amdgcn_readfirstlane(hi);
+    lo = __builtin_amdgcn_readlane(wave_min_lane63(lo), 63);
+    hi = __builtin_amdgcn_readlane(wave_max_lane63(hi), 63);
     while (lo < hi) {
         const int mid = lo + ((hi - lo + 1) >> 1);
         if (count_ge(mid) >= kk) lo = mid;
@@ -2286,13 +2293,9 @@ __global__ __launch_bounds__(kThreads) void select_group_kernel(SelectArgs a)
         else lo = v[e] < lo ? v[e] : lo;
         hi = v[e] > hi ? v[e] : hi;
     }
-#pragma unroll
-    for (int st = 1; st < kWave; st <<= 1) {
-        const int l2 = __shfl_xor(lo, st), h2 = __shfl_xor(hi, st);
-        lo = l2 < lo ? l2 : lo;
-        hi = h2 > hi ? h2 : hi;
-    }
-    if (lane == 0) {
+    lo = wave_min_lane63(lo);
+    hi = wave_max_lane63(hi);
+    if (lane == kWave - 1) {
         ext[0][wid] = lo;
         ext[1][wid] = hi;
     }
