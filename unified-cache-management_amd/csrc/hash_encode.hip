@@ -1251,6 +1251,9 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
     const bool row_ok = t < a.T;
     if (!row_ok) t = a.T - 1;
     const uint16_t* xr = (const uint16_t*)a.x + src_offset(a, t, h) + kb * 8;
+    // where the row's word goes (a read of the slot mapping): asked for with the operands and
+    // looked at after the matrix product - behind it, it is a round trip to memory of its own
+    const RawSlot raw = fetch_slot_flat(a, t);
 
     // K = 512 holds 128 + 256 operand registers: one wave per SIMD, which is all a launch of
     // this kernel has anyway
@@ -1330,14 +1333,31 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
     const uint32_t half = pack_half(acc);
     const uint32_t word = join_halves(kb ? half << 4 : half);
     if (row_ok && lane < 32) {
-        uint32_t* dst = row_dst(a, t, h);
+        uint32_t* dst = slot_dst(a, slot_value(a, raw, t), h);
         if (dst) dst[nt] = word;
     }
+}
+
+// Touches every 64-byte line of a kernel-argument struct at once.  The compiler fetches a field
+// where the code first needs it, behind the branches of the row addressing - a dozen scalar reads
+// one after the other in a kernel that lives for a few microseconds; with the lines already in the
+// scalar cache those reads are short.  (Copying the struct through pinned registers instead makes
+// its pointers lose their address space: every access becomes a flat one.)
+template <class T>
+__device__ __forceinline__ void warm_args(const T& args)
+{
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(&args);
+    uint32_t t = 0;
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(T) / 4; i += 16) t |= src[i];
+    t |= src[sizeof(T) / 4 - 1];
+    asm volatile("" ::"s"(t));
 }
 
 template <typename V, int KS>
 __global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
 {
+    warm_args(js);
     const bool second = (int)blockIdx.x >= js.waves0;
     encode_small_body<V, KS>(second ? js.job[1] : js.job[0],
                              second ? blockIdx.x - js.waves0 : blockIdx.x);
@@ -1353,6 +1373,7 @@ struct EncJobs4 {
 template <typename V, int KSA, int KSB>
 __global__ __launch_bounds__(64) void encode_small_mixed_kernel(EncJobs4 js)
 {
+    warm_args(js);
     const int w = blockIdx.x;
     if (w < js.end[1]) {
         const int j = w >= js.end[0] ? 1 : 0;
