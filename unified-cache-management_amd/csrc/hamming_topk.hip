@@ -2090,10 +2090,13 @@ __device__ __forceinline__ int wave_excl_scan(int v, int* total)
 template <int EL>
 __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int rows_total)
 {
-    const int rowid = blockIdx.x * (kThreads / kWave) + wave_id();
-    if (rowid >= rows_total) return;
+    // (a wave past the last row reads the last row and leaves below: with the exit up here the
+    // kernel's arguments would be fetched in two rounds, the row count first)
+    const int rowid_raw = blockIdx.x * (kThreads / kWave) + wave_id();
+    const int rowid = rowid_raw < rows_total ? rowid_raw : rows_total - 1;
     const int b = rowid / a.Ho, ho = rowid % a.Ho;
     const int lane = lane_id();
+    const int len = a.lens[b];
     // the row's scores go out before the length is known (in-range positions only, masked
     // below): one round trip to memory instead of two
     int raw[EL];
@@ -2121,7 +2124,7 @@ __global__ __launch_bounds__(kThreads) void select_wave_kernel(SelectArgs a, int
 #pragma unroll
         for (int e = 0; e < EL; ++e) tab[e] = physical ? b * a.max_blocks + lane * EL + e : lane * EL + e;
     }
-    const int len = a.lens[b];
+    if (rowid_raw >= rows_total) return;
     int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
     if (n > a.max_blocks) n = a.max_blocks;
     int32_t* oi = a.out_idx + ((int64_t)b * a.Ho + ho) * a.k;
@@ -2233,6 +2236,7 @@ __global__ __launch_bounds__(kThreads) void select_group_kernel(SelectArgs a)
     const int tid = threadIdx.x, lane = lane_id(), wid = wave_id();
     const bool reduce = (a.flags & UCM_TOPK_REDUCE_HEADS) && a.Hkv > 1;
     const int32_t* row = a.scores + ((int64_t)b * a.Hkv + (reduce ? 0 : ho)) * a.max_blocks;
+    const int len = a.lens[b];  // asked for with the scores: one round trip to memory
     int v[EL], tab[EL];
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
@@ -2251,7 +2255,6 @@ __global__ __launch_bounds__(kThreads) void select_group_kernel(SelectArgs a)
 #pragma unroll
         for (int e = 0; e < EL; ++e) tab[e] = physical ? b * a.max_blocks + tid * EL + e : tid * EL + e;
     }
-    const int len = a.lens[b];
     int n = len > 0 ? (len + a.BS - 1) / a.BS : 0;
     if (n > a.max_blocks) n = a.max_blocks;
     int32_t* oi = a.out_idx + ((int64_t)b * a.Ho + ho) * a.k;
