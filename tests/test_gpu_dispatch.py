@@ -51,7 +51,7 @@ TOPK_SHAPES = {
                                         "plane_kernel+block_score_pairs<0,5>+select_wave_kernel<4>"),
     "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], 8, {}, "block_score_lanes<9,1,1>+select_wave_kernel<4>"),
     "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], 8, {},
-                                       "block_score_strip18<2>+select_wave_kernel<4>"),
+                                       "block_score_strip18+select_wave_kernel<4>"),
     "config5_blocks_of_128": (2, 128, 1, 8, 128, [8192, 700], 8, {},
                               "plane_kernel+block_score_lanes<4,0,8>+select_wave_kernel<4>"),
     "odd_code_width": (2, 6, 2, 3, 16, [1024, 300], 8, {}, "block_score_generic+select_wave_kernel<4>"),
@@ -110,8 +110,9 @@ def test_per_token_scorer_takes_its_kernels_and_matches_the_checker(name):
 def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
     """One KV head: the scorer reduces the G query heads to per-bit counts itself (no plane kernel)
     when the blocks hold 64 tokens - for every G with 8-word codes (counts as nibble digits for the
-    4-bit dot product) and, up to 128 heads, with 18-word codes; up to 128 heads with 16-word codes
-    (bit planes); larger blocks keep the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
+    4-bit dot product), up to 128 heads with 18-word codes (signed base-4 digits of G - 2 * count as
+    FP4 operands of the matrix instruction) and with 16-word codes (bit planes); larger blocks keep
+    the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
     that end inside a workgroup), table entries out of range, forced blocks."""
     from ucm_amd import _lib
     from ucm_amd.sparse import hamming_topk
@@ -133,12 +134,43 @@ def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
         if (Wd, BS) == (8, 64):
             assert got.startswith("block_score_dot64<%d>+" % (1 if G <= 15 else 2))
         elif (Wd, BS) == (18, 64) and G <= 128:
-            assert got.startswith("block_score_strip18<%d>+" % (1 if G <= 15 else 2))
+            assert got.startswith("block_score_strip18+")
         elif BS == 64 and G <= 128:
             assert got.startswith("block_score_lanes_run<%d,%d>+" % (Wd // 2, planes))
         else:
             assert got.startswith("plane_kernel+block_score_lanes<%d,0,%d>+" % (Wd // 2, min(planes, 8)))
         torch.cuda.synchronize()
         oi, os_ = c_api.hamming_topk(q, kc, table, lens, k, sink, recent, 0)
+        assert np.array_equal(sc.cpu().numpy(), os_)
+        assert np.array_equal(idx.cpu().numpy(), oi)
+
+
+@pytest.mark.parametrize("G", [3, 63, 64, 112, 127, 128])
+def test_latent_18_word_scorer_extreme_weights(G):
+    """The 18-word scorer multiplies code bits with signed weights G - 2 * count on the matrix unit
+    (FP4 operands, float accumulation) and must stay exact at the ends of its range: every query
+    head equal (all counts 0 or G, weights of magnitude G, up to 128), all-ones and all-zero cached
+    codes (the largest sums), one bit set per word, and a run of blocks that ends inside a
+    workgroup's run with a last block of a single token."""
+    from ucm_amd import _lib
+    from ucm_amd.sparse import hamming_topk
+
+    lens = [64 * 9 + 1, 64 * 40, 17]
+    q, kc, table, lens = make_paged_case(900 + G, len(lens), G, 1, 18, 64, lens)
+    q[0, :, :] = q[0, :1, :]              # request 0: all heads equal
+    q[1, : G // 2, :] = 0xFFFFFFFF        # request 1: counts of G // 2 or G everywhere
+    q[1, G // 2:, :9] = 0
+    q[1, G // 2:, 9:] = 0xFFFFFFFF
+    nb = kc.shape[0]
+    kc[0::5] = 0xFFFFFFFF                 # whole blocks of all-ones / all-zero codes
+    kc[1::5] = 0
+    kc[2::5, ::2] = 0x80000001            # bits 0 and 31 of every word
+    kc[2::5, 1::2] = 0x00011000
+    assert nb >= 5
+    for sink, recent in ((0, 0), (64, 64)):
+        idx, sc = hamming_topk(_dev(q), _dev(kc), _dev(table), _dev(lens), 12, sink, recent)
+        assert _lib.last_dispatch().startswith("block_score_strip18+")
+        torch.cuda.synchronize()
+        oi, os_ = c_api.hamming_topk(q, kc, table, lens, 12, sink, recent, 0)
         assert np.array_equal(sc.cpu().numpy(), os_)
         assert np.array_equal(idx.cpu().numpy(), oi)

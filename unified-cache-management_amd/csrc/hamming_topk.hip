@@ -1524,30 +1524,44 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 
 // 64-token blocks of 18-word codes against one KV head whose G query heads enter as per-bit
 // counts (the latent cache with position part: 16 requests x 65,536 tokens, 75 MB of codes in
-// 16,384 blocks of 4.5 KiB).  block_score_dot64's arithmetic with a whole code per lane:
+// 16,384 blocks of 4.5 KiB).
+//
+// Arithmetic.  With c_b the number of query heads whose bit b is set, the group-summed distance of
+// a code k is  sum_b c_b + sum_b k_b * t_b  with the signed weight t_b = G - 2 c_b: per request a
+// matrix-vector product of the tokens' 576 code bits with one small-integer vector.  As vector
+// work it costs 13 operations a code word and token at best (4-bit dot products, as in
+// block_score_dot64): 270 a block and wave, 7.7 us a SIMD for the 16 blocks it gets - more than
+// the 9.6 us the codes take to arrive allow for in a kernel that also has to start and end
+// (measured: loads alone 12.6 us, arithmetic alone 9.7 us, together 16.1 to 16.7 us).  So the
+// product runs on the matrix unit, exactly: v_mfma_f32_16x16x128 with FP4 (E2M1) operands, one
+// instruction per code word.  A lane's word becomes 32 FP4 values with five operations -
+// k & 0x1111.., k & 0x2222.., k & 0x4444.. and (k >> 1) & 0x4444.. hold bit 4 i + j in nibble i as
+// 0.5, 1, 2, 2 - and |t_b| <= 128 is four base-4 digits whose products with those, digit x
+// {2, 1, 1/2, 1/2} = 0 ... 6 in steps FP4 has, carry t_b's sign.  Lane l supplies row l % 16 for the
+// K quarter l / 16, so token l is row l % 16 of quarter l / 16, and column 4 q + d of the other
+// operand carries digit d in quarter q and zeros elsewhere: all 16 columns are used, the result
+// register r of lane l is digit l % 4 of token 16 * ((l % 16) / 4) + 4 * (l / 16) + r.  Scaling by
+// 4^digit, a sum over the four lanes of a quad and a minimum finish the block.  Every term is a
+// small integer: the float accumulation is exact, and the scores equal the integer kernels' bit
+// for bit.  (v_mfma_f32_32x32x64 with the same operands fills 8 of its 32 columns and measured
+// 17.7 to 18.5 us, two accumulator chains 18.7 to 19.5: the instruction's own time is the limit
+// there.  16x16x128: 15.0 to 15.4 us.)
 //
 // Codes.  A block goes from memory straight into the wave's LDS strip (load-to-LDS, five
 // instructions of 1 KiB, the last one half masked): no register holds a code on its way, no LDS
 // store instruction is issued.  The strip holds four blocks; a wave scores a run of eight and
 // requests block i + 4 the moment block i's reads are back.  Lane l reads token l's row (72 bytes
-// apart: 16 consecutive lanes cover all banks) as nine 8-byte reads.
-//
-// Weights.  The eight weight words of each of the 18 code words ([bit residue j][digit]) are
-// wave-uniform and stay in 144 registers for the whole run (two waves per SIMD: 256 registers a
-// lane), so a block costs 9 LDS reads and about 270 vector operations - against 50 and 370 with
-// bit planes re-read from LDS for every block.  Measured at 16 x 65,536 tokens, 64 query heads:
-// the loads alone (no arithmetic) 12.6 us, the arithmetic alone (no loads) 9.7 us, together
-// 16.7 us; the arithmetic (16 blocks a SIMD x 270 operations x 4 cycles) is what the waves wait
-// for once the codes flow, bit planes with popcounts (15 a word) and 8-bit dot products (16 a
-// word) need more of it than the 13 a word of the 4-bit dot product.
+// apart: 16 consecutive lanes cover all banks) as nine 8-byte reads.  The 18 x 4 operand words of
+// the weights stay in registers for the whole run.
 //
 // Build.  All four waves build the weights in three steps with LDS in between (one wave doing
 // all of it held the workgroup for 2.4 to 5 us): lane (w, g) of wave v counts word w of heads
 // 3 v + g, 3 v + g + 12, ... bit-sliced; lane (w, p) counts the groups whose partial count has
-// bit p set; lane (w, j) adds those four numbers, shifted, and assembles the two weight words of
-// residue j.  Up to 128 query heads.  Only two of the four first blocks are requested before the
-// build: a compute unit takes one 1 KiB load instruction per 16 cycles, and the eight resident
-// waves' first four blocks each would keep every wave at its load instructions for a microsecond.
+// bit p set; lane (w, d) adds those four numbers, shifted, subtracts twice the sum from G (ten
+// bit-sliced bits), takes the magnitude and assembles the four operand words of digit d.  Up to
+// 128 query heads.  Only two of the four first blocks are requested before the build: a compute
+// unit takes one 1 KiB load instruction per 16 cycles, and the eight resident waves' first four
+// blocks each would keep every wave at its load instructions for a microsecond.
 constexpr int kStripWaves = 4;  // waves per workgroup
 constexpr int kStripRun = 8;    // blocks per wave
 constexpr int kStripSlots = 4;  // blocks of a wave in LDS
@@ -1580,7 +1594,9 @@ __device__ __forceinline__ void strip_issue_block(uint32_t lds, uint64_t base, u
     }
 }
 
-template <int ND>
+typedef int i32x8s __attribute__((ext_vector_type(8)));
+typedef float f32x4s __attribute__((ext_vector_type(4)));
+
 __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void block_score_strip18(ScoreArgs a)
 {
 
@@ -1589,7 +1605,8 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     constexpr int kBlockWords = 64 * WD;
     constexpr int kLoadsPerBlock = 5;
     __shared__ __align__(16) uint32_t strip[kStripWaves][kSlots * kBlockWords];
-    __shared__ __align__(16) uint32_t wl[WD * 8];        // weight word [w][j][digit]
+    __shared__ __align__(16) uint32_t wB[WD * 4 * 4];    // operand words [w][digit][j]
+    __shared__ __align__(16) uint32_t wzero[4];
     __shared__ __align__(16) uint32_t part[NG * WD * 4];  // [group][w][plane]: counts of a group's heads
     __shared__ __align__(16) uint32_t cnt[WD * 4 * 4];    // [w][plane p][plane]: groups with bit p set
     __shared__ int base_s;
@@ -1682,8 +1699,8 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
         *reinterpret_cast<u32x4*>(cnt + (pw * 4 + p2) * 4) = u32x4{m[0], m[1], m[2], m[3]};
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    // 3: the same lanes, now (w, j): add the four numbers, shifted, and assemble the two weight
-    //    words of bit residue j (nibble n = a digit of the count of bit 4 * n + j)
+    // 3: the same lanes, now (w, d): add the four numbers, shifted, turn the counts into signed
+    //    weights and assemble the four operand words of base-4 digit d
     if (wid < 2 && lane < 2 * WD) {
         uint32_t acc[8];
         {
@@ -1704,13 +1721,44 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
                 cy = c2;
             }
         }
-        uint32_t r0 = 0, r1 = 0;
+        // signed weight of every bit, t = G - 2 c (|t| <= G <= 128), bit-sliced: ten-bit
+        // subtraction, then the magnitude
+        uint32_t mag[8], sgn;
+        {
+            uint32_t diff[10], br = 0;
 #pragma unroll
-        for (int pp = 0; pp < 4; ++pp) {
-            r0 |= ((acc[pp] >> p2) & 0x11111111u) << pp;
-            r1 |= ((acc[4 + pp] >> p2) & 0x11111111u) << pp;
+            for (int i = 0; i < 10; ++i) {
+                const uint32_t g = ((G >> i) & 1) ? ~0u : 0u;
+                const uint32_t u = (i >= 1 && i <= 8) ? acc[i - 1] : 0u;
+                diff[i] = g ^ u ^ br;
+                br = (~g & (u | br)) | (u & br);
+            }
+            sgn = diff[9];
+            uint32_t cy = sgn;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t m = diff[i] ^ sgn;
+                mag[i] = m ^ cy;
+                cy = m & cy;
+            }
         }
-        *reinterpret_cast<u32x2*>(wl + pw * 8 + 2 * p2) = u32x2{r0, r1};
+        // this lane's base-4 digit of the magnitude (selected, not indexed: an array indexed at run
+        // time would be kept in LDS)
+        const uint32_t a0 = p2 == 0 ? mag[0] : p2 == 1 ? mag[2] : p2 == 2 ? mag[4] : mag[6];
+        const uint32_t a1 = p2 == 0 ? mag[1] : p2 == 1 ? mag[3] : p2 == 2 ? mag[5] : mag[7];
+        const uint32_t both = a0 & a1;
+        // FP4 (E2M1) code of digit * {2, 1, 1/2, 1/2} for bit residue j = 0, 1, 2, 3 - the code
+        // operand holds such a bit as 0.5, 1, 2, 2 - nibble i of word j for code bit 4 i + j
+        auto pack = [&](uint32_t b0, uint32_t b1, uint32_t b2, int j) {
+            constexpr uint32_t M = 0x11111111u;
+            return ((b0 >> j) & M) | (((b1 >> j) & M) << 1) | (((b2 >> j) & M) << 2) | (((sgn >> j) & M) << 3);
+        };
+        u32x4 bw;
+        bw.x = pack(both, a1, a0 | a1, 0);   // 0, 2, 4, 6 -> codes 0, 4, 6, 7
+        bw.y = pack(both, a0 & ~a1, a1, 1);  // 0, 1, 2, 3 -> codes 0, 2, 4, 5
+        bw.z = pack(a0, a1, 0u, 2);          // 0, 1/2, 1, 3/2 -> codes 0, 1, 2, 3
+        bw.w = pack(a0, a1, 0u, 3);
+        *reinterpret_cast<u32x4*>(wB + (pw * 4 + p2) * 4) = bw;
         if (p2 == 0) {
             int c = 0;
 #pragma unroll
@@ -1718,6 +1766,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
             atomicAdd(&base_s, c);  // sum over all code bits of the per-bit counts
         }
     }
+    if (threadIdx.x < 4) wzero[threadIdx.x] = 0;
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
     for (int i = kFirst; i < kSlots; ++i)
@@ -1725,15 +1774,22 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     if (run <= 0) return;
     const int base = base_s;
     const int full = G * 32 * WD;
-    u32x4 W[WD][2];  // [w] -> {j = 0: lo, hi; j = 1: lo, hi}, {j = 2, j = 3}
+    // v_mfma_f32_16x16x128 with FP4 operands, one per code word: 16 rows x 128 values of A times
+    // 128 x 16 of B.  Lane l supplies row l % 16 of A / column l % 16 of B for the K quarter l / 16,
+    // so token l (its word as four masked copies = 32 FP4 values) is row l % 16, quarter l / 16, and
+    // column 4 q + d carries digit d for the tokens of quarter q: zeros outside quarter q.  Result
+    // register r of lane l is row 4 * (l / 16) + r of column l % 16.
+    const int col = lane & 15, quarter = lane >> 4;
+    u32x4 Bw[WD];
     {
-        const u32x4* src = reinterpret_cast<const u32x4*>(wl);
+        const bool live = (col >> 2) == quarter;
+        const uint32_t* src = live ? wB + (col & 3) * 4 : wzero;
+        const int stride = live ? 16 : 0;
 #pragma unroll
-        for (int i = 0; i < WD; ++i) {
-            W[i][0] = src[2 * i];
-            W[i][1] = src[2 * i + 1];
-        }
+        for (int w = 0; w < WD; ++w) Bw[w] = *reinterpret_cast<const u32x4*>(src + w * stride);
     }
+    const float dscale = (col & 3) == 0 ? 1.0f : (col & 3) == 1 ? 4.0f : (col & 3) == 2 ? 16.0f : 64.0f;
+    const int tok0 = 16 * (col >> 2) + 4 * quarter;  // + r: the token of result register r
     int result = 0;  // lane i: score of block j0 + i
 #pragma unroll
     for (int i = 0; i < RUN; ++i) {
@@ -1755,35 +1811,34 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
             k[2 * w] = kk.x;
             k[2 * w + 1] = kk.y;
         }
-        int pk = 0;
-        uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
+        f32x4s c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int w = 0; w < WD; ++w) {
-            pk = popc_add(k[w], pk);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t e = k[w] & (0x11111111u << j);
-                lo[j] = __builtin_amdgcn_udot8(e, W[w][j >> 1][(j & 1) * 2], lo[j], false);
-                if (ND > 1) hi[j] = __builtin_amdgcn_udot8(e, W[w][j >> 1][(j & 1) * 2 + 1], hi[j], false);
-            }
+            const i32x8s A = {(int)(k[w] & 0x11111111u), (int)(k[w] & 0x22222222u), (int)(k[w] & 0x44444444u),
+                              (int)((k[w] >> 1) & 0x44444444u), 0, 0, 0, 0};
+            const i32x8s B = {(int)Bw[w].x, (int)Bw[w].y, (int)Bw[w].z, (int)Bw[w].w, 0, 0, 0, 0};
+            c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, c, 4, 4, 0, 0, 0, 0);  // FP4 x FP4, scales off
         }
-        // the sums exist here: left to the compiler they sink towards their last use, behind
-        // the branches below
-        asm volatile("" : "+v"(pk), "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]));
-        if (ND > 1) asm volatile("" : "+v"(hi[0]), "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3]));
         if (i + kSlots < run) {
             // this strip slot is free once its last reads are back
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             issue(i + kSlots);
         }
-        uint32_t t[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) t[j] = ND > 1 ? lo[j] + (hi[j] << 4) : lo[j];
-        const uint32_t x8 = (((((t[0] << 1) + t[1]) << 1) + t[2]) << 1) + t[3];  // 8 * sum_b k_b * c_b
+        // sum_b k_b t_b of a token = sum over its four digit columns of 4^digit * column: scale, add
+        // across the four lanes of a quad, then the minimum over this lane's four tokens
         const int pos0 = (j0 + i) << 6;
-        const int d = pos0 + lane < len ? G * pk - (int)(x8 >> 2) : kInf;
-        const int m = __builtin_amdgcn_readlane(wave_min_lane63(d), 63) + base;
         const int ntok = (64 < len - pos0) ? 64 : len - pos0;
+        float mn = 3.0e38f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = c[r] * dscale;
+            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+            if (tok0 + r >= ntok) v = 3.0e38f;  // the last block of a request
+            mn = v < mn ? v : mn;
+        }
+        const int d = (int)mn;  // exact: every term is an integer below 2^24 (all masked: saturates)
+        const int m = __builtin_amdgcn_readlane(wave_min_lane63(d), 63) + base;
         const bool forced = (pos0 < sink) || (pos0 + ntok > len - recent);
         const int sc = (entry[i] < 0 || entry[i] >= NB) ? -1 : (forced ? full : full - m);
         if (lane == i) result = sc;
@@ -2515,14 +2570,20 @@ void note_select(const char* family, int el = -1)
 }
 
 template <typename K, typename... Args>
-void launch_score(K kernel, dim3 grid, size_t lds, hipStream_t st, Args... args)
+void launch_score_threads(K kernel, dim3 grid, int threads, size_t lds, hipStream_t st, Args... args)
 {
     ++g_note.score_launches;
     if (g_prof_before && g_prof_after)
-        hipExtLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, st, g_prof_before, g_prof_after, 0,
+        hipExtLaunchKernelGGL(kernel, grid, dim3(threads), lds, st, g_prof_before, g_prof_after, 0,
                               args...);
     else
-        hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, st, args...);
+        hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, st, args...);
+}
+
+template <typename K, typename... Args>
+void launch_score(K kernel, dim3 grid, size_t lds, hipStream_t st, Args... args)
+{
+    launch_score_threads(kernel, grid, kThreads, lds, st, args...);
 }
 
 template <int CPU, bool DIRECT, int GP>
@@ -2937,18 +2998,9 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
                 else hipLaunchKernelGGL(block_score_dot64<2>, g64, threads, 0, st, a);
             }
         } else if (planes_in_lanes && Wd == 18) {
-            const int nd = a.G <= 15 ? 1 : 2;
-            note_score("block_score_strip18", nd);
+            note_score("block_score_strip18");
             const dim3 g64((unsigned)ucm::ceil_div(max_blocks, kStripWaves * kStripRun), (unsigned)B);
-            ++g_note.score_launches;
-            const dim3 threads(kStripWaves * kWave);
-            if (g_prof_before && g_prof_after) {
-                if (nd == 1) hipExtLaunchKernelGGL(block_score_strip18<1>, g64, threads, 0, st, g_prof_before, g_prof_after, 0, a);
-                else hipExtLaunchKernelGGL(block_score_strip18<2>, g64, threads, 0, st, g_prof_before, g_prof_after, 0, a);
-            } else {
-                if (nd == 1) hipLaunchKernelGGL(block_score_strip18<1>, g64, threads, 0, st, a);
-                else hipLaunchKernelGGL(block_score_strip18<2>, g64, threads, 0, st, a);
-            }
+            launch_score_threads(block_score_strip18, g64, kStripWaves * kWave, 0, st, a);
         } else if (planes_in_lanes) {
             note_score("block_score_lanes_run", Wd / 2, pmax);
             const dim3 g64((unsigned)ucm::ceil_div(max_blocks, (kThreads / kWave) * kLanesRunBlocks), (unsigned)B);
