@@ -1347,12 +1347,25 @@ __device__ __forceinline__ int wave_min_lane63(int x)
     return x;
 }
 
+// One LDS word, read and waited for in one statement (a register that an LDS read fills later,
+// behind the compiler's back, may have been given to another value by then).
+__device__ __forceinline__ int lds_flag_peek(const int* p)
+{
+    int v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                 : "=v"(v)
+                 : "v"((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) int*)p)
+                 : "memory");
+    return v;
+}
+
 template <int ND>
 __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs a)
 {
     constexpr int RUN = kDotRun;
     __shared__ __align__(16) uint32_t wl[64];  // weight word [w][j][digit]
     __shared__ int base_s;
+    __shared__ int ready_s;  // set by the building wave once the weights are in LDS
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
     const int j0 = (blockIdx.x * kDotWaves + wid) * RUN;
@@ -1395,19 +1408,28 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 #pragma unroll
         for (int t = 0; t < 16; ++t) o |= x[t];
         asm volatile("" ::"v"(o));  // the query words are here
+        if (lane == 0) ready_s = 0;
     }
-    asm volatile("s_barrier" ::: "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    // round 2: the codes
+    // round 2: the codes.  A wave stands at its load instructions until the unit's queue has room
+    // (a unit takes one 1 KiB instruction per 16 cycles and answers at its share of the memory
+    // rate), for microseconds when 16 waves ask for 8 KiB each.  Nobody may wait for that: the
+    // building wave builds first and requests its codes afterwards, and the weights are handed over
+    // with a flag in LDS that the others poll once their own requests are out - a barrier would make
+    // every wave wait for the slowest wave's requests (measured: weights ready after 1.8 ... 5.9 us).
     u32x4 v[RUN][2];
+    auto request = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < RUN; ++i) {
-        int64_t pb = entry[i];
-        if (pb < 0 || pb >= NB) pb = 0;  // scored as -1 below
-        const u32x4* src = reinterpret_cast<const u32x4*>(kc + pb * ks_block);
-        v[i][0] = code_load(src + lane);
-        v[i][1] = code_load(src + 64 + lane);
-    }
+        for (int i = 0; i < RUN; ++i) {
+            int64_t pb = entry[i];
+            if (pb < 0 || pb >= NB) pb = 0;  // scored as -1 below
+            const u32x4* src = reinterpret_cast<const u32x4*>(kc + pb * ks_block);
+            v[i][0] = code_load(src + lane);
+            v[i][1] = code_load(src + 64 + lane);
+        }
+    };
+    if (wid != 0) request();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     if (wid == 0) {
@@ -1440,12 +1462,25 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
             }
             add16(h0);
         }
-        // the eight lane groups add up (every lane ends with the full counts of its word)
+        // the eight lane groups add up (every lane ends with the full counts of its word): the
+        // partner lanes l ^ 8, l ^ 16, l ^ 32 through a row rotation and the two lane-swap
+        // instructions - a lane exchange through the LDS pipe (ds_bpermute) costs some hundred
+        // cycles, and 27 of them in a row kept seven waves waiting for this one
 #pragma unroll
         for (int st = 8; st < kWave; st <<= 1) {
             uint32_t o[8], cy = 0;
 #pragma unroll
-            for (int p = 0; p < 8; ++p) o[p] = __builtin_amdgcn_ds_bpermute((lane ^ st) << 2, acc[p]);
+            for (int p = 0; p < 8; ++p) {
+                if (st == 8) {
+                    o[p] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)acc[p], 0x128, 0xf, 0xf, false);  // row_ror:8
+                } else if (st == 16) {
+                    const auto sw = __builtin_amdgcn_permlane16_swap(acc[p], acc[p], false, false);
+                    o[p] = (lane & 16) ? sw[0] : sw[1];
+                } else {
+                    const auto sw = __builtin_amdgcn_permlane32_swap(acc[p], acc[p], false, false);
+                    o[p] = (lane & 32) ? sw[0] : sw[1];
+                }
+            }
 #pragma unroll
             for (int p = 0; p < 8; ++p) {
                 uint32_t sum, c2;
@@ -1457,9 +1492,9 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
         int c = 0;
 #pragma unroll
         for (int p = 0; p < 8; ++p) c += __popc(acc[p]) << p;
-        c += __builtin_amdgcn_ds_bpermute((lane ^ 1) << 2, c);
-        c += __builtin_amdgcn_ds_bpermute((lane ^ 2) << 2, c);
-        c += __builtin_amdgcn_ds_bpermute((lane ^ 4) << 2, c);
+        c += __builtin_amdgcn_update_dpp(0, c, 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+        c += __builtin_amdgcn_update_dpp(0, c, 0x4E, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
+        c += __builtin_amdgcn_update_dpp(0, c, 0x141, 0xf, 0xf, false);  // row_half_mirror: the other quad
         // lane (w, g = 2 * j + digit) assembles weight word [w][j][digit]: nibble n = that digit of
         // the count of bit 4 * n + j (both digits are computed, one is kept: no run-time index)
         const int jj = qg >> 1;
@@ -1471,8 +1506,16 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
         }
         wl[qw * 8 + qg] = (qg & 1) ? r1 : r0;
         if (lane == 0) base_s = c;  // sum over all code bits of the per-bit counts
+        // LDS operations of a wave complete in order: the flag lands behind the weights
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) ready_s = 1;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        request();
+    } else {
+        // the builder depends on nobody, so this ends; LDS reads do not wait for the codes in flight
+        while (lds_flag_peek(&ready_s) == 0) __builtin_amdgcn_s_sleep(1);
     }
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (run <= 0) return;
     u32x4 M[8];  // [w][j / 2] -> {lo, hi of j even; lo, hi of j odd} for the lane's four code words
     {
