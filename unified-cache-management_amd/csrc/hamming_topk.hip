@@ -1597,18 +1597,22 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 // apart: 16 consecutive lanes cover all banks) as nine 8-byte reads.  The 18 x 4 operand words of
 // the weights stay in registers for the whole run.
 //
-// Build.  All four waves build the weights in three steps with LDS in between (one wave doing
-// all of it held the workgroup for 2.4 to 5 us): lane (w, g) of wave v counts word w of heads
-// 3 v + g, 3 v + g + 12, ... bit-sliced; lane (w, p) counts the groups whose partial count has
-// bit p set; lane (w, d) adds those four numbers, shifted, subtracts twice the sum from G (ten
-// bit-sliced bits), takes the magnitude and assembles the four operand words of digit d.  Up to
-// 128 query heads.  Only two of the four first blocks are requested before the build: a compute
-// unit takes one 1 KiB load instruction per 16 cycles, and the eight resident waves' first four
-// blocks each would keep every wave at its load instructions for a microsecond.
+// Build.  Lane (s, g) of wave v counts code word 8 v + s over heads g, g + 8, ... bit-sliced (up to
+// 128 query heads), the eight lanes of a word add their counts with three DPP exchanges, subtract
+// twice the sum from G (ten bit-sliced bits), take the magnitude, and lanes g < 4 assemble the
+// four operand words of base-4 digit g: a wave takes its words from the query to the operands
+// without LDS and without meeting another wave; waves 0 and 1 build eight words each, wave 2
+// two, wave 3 none.  (Before: three steps by all four waves with LDS and a barrier between
+// them, 14.8 to 15.4 us; one wave doing all of it held the workgroup for 2.4 to 5 us.)  The
+// building waves request three of their first four blocks before the build and the fourth after
+// it, wave 3 all four at once: 14.3 to 14.6 us.  None before the build: 15.3 to 15.6 us; all
+// four: 15.0 to 15.5 us - a compute unit takes one 1 KiB load instruction per 16 cycles, and the
+// eight resident waves' first four blocks each keep every wave at its load instructions for a
+// microsecond before the build starts.
 constexpr int kStripWaves = 4;  // waves per workgroup
 constexpr int kStripRun = 8;    // blocks per wave
 constexpr int kStripSlots = 4;  // blocks of a wave in LDS
-constexpr int kStripFirst = 2;  // of those, requested before the weight build
+constexpr int kStripFirst = 3;  // of those, a building wave requests before the weight build
 
 // One block of NL KiB (+ half a KiB when TAIL) from `base` into LDS at byte address `lds`.
 template <int NL, bool TAIL>
@@ -1644,14 +1648,11 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
 {
 
     constexpr int WD = 18, RUN = kStripRun, kSlots = kStripSlots, kFirst = kStripFirst;
-    constexpr int NG = 3 * kStripWaves;  // head groups of the weight build: 3 per wave
     constexpr int kBlockWords = 64 * WD;
     constexpr int kLoadsPerBlock = 5;
     __shared__ __align__(16) uint32_t strip[kStripWaves][kSlots * kBlockWords];
     __shared__ __align__(16) uint32_t wB[WD * 4 * 4];    // operand words [w][digit][j]
     __shared__ __align__(16) uint32_t wzero[4];
-    __shared__ __align__(16) uint32_t part[NG * WD * 4];  // [group][w][plane]: counts of a group's heads
-    __shared__ __align__(16) uint32_t cnt[WD * 4 * 4];    // [w][plane p][plane]: groups with bit p set
     __shared__ int base_s;
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
@@ -1665,22 +1666,27 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
         if (a.table) my_entry = a.table[(int64_t)b * a.table_stride + jc];
         else my_entry = b * a.max_blocks + jc;
     }
-    // lane (w, g) of wave v: word w of heads gi, gi + 12, ... with gi = 3 v + g (up to 11 heads)
-    const int pw = lane % WD, pg = lane / WD;
-    const int gi = wid * 3 + pg;
+    // The build: lane (s, g) of wave v counts code word 8 v + s of heads g, g + 8, ... (16 of them,
+    // 128 query heads), bit-sliced.  The eight head groups of a word are eight neighbouring lanes,
+    // so they add up with three DPP exchanges and no LDS, and the same lanes turn the counts of
+    // their word into its operand words: a wave builds its words from the query words to the end
+    // without meeting another wave (waves 0 and 1 eight words each, wave 2 the last two).
+    const int bs = lane >> 3, bg = lane & 7;
+    const int word = wid * 8 + bs;
+    const bool has_word = word < WD;
     const int G = a.G;
     uint32_t qx[16];
-    {
-        const uint32_t* qb = a.q + b * a.q_stride_b + pw;
+    if (wid < 3) {
+        const uint32_t* qb = a.q + b * a.q_stride_b + (has_word ? word : 0);
         const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
 #pragma unroll
-        for (int t = 0; t < 11; ++t) {
-            const int h = gi + NG * t;  // heads past the group re-read the last one, as zero
+        for (int t = 0; t < 16; ++t) {
+            const int h = bg + 8 * t;  // heads past the group re-read the last one, as zero
             qx[t] = qb[(h < G ? h : G - 1) * qs];
         }
-#pragma unroll
-        for (int t = 11; t < 16; ++t) qx[t] = 0;
     }
+    if (threadIdx.x == 0) base_s = 0;
+    if (threadIdx.x < 4) wzero[threadIdx.x] = 0;
     // everything the rest of the kernel takes from its arguments, now
     const int64_t NB = a.NB, ks_block = a.ks_block;
     const uint32_t* kc = a.kc;
@@ -1694,14 +1700,9 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     int entry[RUN];
 #pragma unroll
     for (int i = 0; i < RUN; ++i) entry[i] = __builtin_amdgcn_readlane(my_entry, i);
-    {
-        uint32_t o = 0;
-#pragma unroll
-        for (int t = 0; t < 11; ++t) o |= qx[t];
-        asm volatile("" ::"v"(o));  // the query words are here: no code is requested before
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // round 2: the first blocks of the run
+    // base_s is zero for everybody (the waves get here within a few hundred nanoseconds of one
+    // another, long before the query words)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)strip[wid]);
     const uint32_t off = (uint32_t)lane * 16u;
@@ -1711,56 +1712,42 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
         strip_issue_block<4, true>(lds0 + (uint32_t)(i % kSlots) * (kBlockWords * 4),
                                    reinterpret_cast<uint64_t>(kc + pb * ks_block), off, lane < 32);
     };
+    if (wid < 3) {
+        {
+            uint32_t o = 0;
 #pragma unroll
-    for (int i = 0; i < kFirst; ++i)
-        if (i < run) issue(i);
-    __builtin_amdgcn_sched_barrier(0);
-    // The weights, by all four waves in three steps with LDS between them.  (A compute unit
-    // takes a 1 KiB load instruction every 16 cycles: the eight resident waves' first four
-    // blocks each would hold every wave at its load instructions for a microsecond before the
-    // build starts, so only the first kFirst go out here.)
-    // 1: every lane counts its group's heads bit-sliced (four planes, at most 11 heads).
-    {
-        uint32_t n[5];
+            for (int t = 0; t < 16; ++t) o |= qx[t];
+            asm volatile("" ::"v"(o));  // the query words are here: no code is requested before
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < 11; ++t) qx[t] = (gi + NG * t < G && pg < 3) ? qx[t] : 0u;
-        count16(qx, n);
-        if (pg < 3) *reinterpret_cast<u32x4*>(part + (gi * WD + pw) * 4) = u32x4{n[0], n[1], n[2], n[3]};
-        if (threadIdx.x == 0) base_s = 0;
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    // 2: lane (w, p) of waves 0 and 1 counts the groups whose plane p has a bit set: the count of
-    //    a bit is  sum_p 2^p * (that number).
-    const int p2 = wid * 2 + pg;  // waves 0 and 1, lanes below 2 * WD
-    if (wid < 2 && lane < 2 * WD) {
-        uint32_t y[16], m[5];
-#pragma unroll
-        for (int g = 0; g < NG; ++g) y[g] = part[(g * WD + pw) * 4 + p2];
-#pragma unroll
-        for (int g = NG; g < 16; ++g) y[g] = 0;
-        count16(y, m);
-        *reinterpret_cast<u32x4*>(cnt + (pw * 4 + p2) * 4) = u32x4{m[0], m[1], m[2], m[3]};
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    // 3: the same lanes, now (w, d): add the four numbers, shifted, turn the counts into signed
-    //    weights and assemble the four operand words of base-4 digit d
-    if (wid < 2 && lane < 2 * WD) {
+        for (int i = 0; i < kFirst; ++i)
+            if (i < run) issue(i);
+        __builtin_amdgcn_sched_barrier(0);
         uint32_t acc[8];
         {
-            const u32x4 n0 = *reinterpret_cast<const u32x4*>(cnt + (pw * 4) * 4);
+            uint32_t n[5];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[i] = i < 4 ? n0[i] : 0u;
+            for (int t = 0; t < 16; ++t) qx[t] = (bg + 8 * t < G && has_word) ? qx[t] : 0u;
+            count16(qx, n);
+#pragma unroll
+            for (int p = 0; p < 8; ++p) acc[p] = p < 5 ? n[p] : 0u;
         }
+        // the eight head groups of a word: lanes l ^ 1, l ^ 2 and the mirror lane of the other quad
 #pragma unroll
-        for (int p = 1; p < 4; ++p) {
-            const u32x4 np = *reinterpret_cast<const u32x4*>(cnt + (pw * 4 + p) * 4);
-            uint32_t cy = 0;
+        for (int st = 0; st < 3; ++st) {
+            uint32_t o[8], cy = 0;
 #pragma unroll
-            for (int i = p; i < 8; ++i) {
+            for (int p = 0; p < 8; ++p) {
+                if (st == 0) o[p] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)acc[p], 0xB1, 0xf, 0xf, false);
+                else if (st == 1) o[p] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)acc[p], 0x4E, 0xf, 0xf, false);
+                else o[p] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)acc[p], 0x141, 0xf, 0xf, false);
+            }
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
                 uint32_t sum, c2;
-                if (i - p < 4) full_add(acc[i], np[i - p], cy, sum, c2);
-                else half_add(acc[i], cy, sum, c2);
-                acc[i] = sum;
+                full_add(acc[p], o[p], cy, sum, c2);
+                acc[p] = sum;
                 cy = c2;
             }
         }
@@ -1785,8 +1772,9 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
                 cy = m & cy;
             }
         }
-        // this lane's base-4 digit of the magnitude (selected, not indexed: an array indexed at run
-        // time would be kept in LDS)
+        // lane g < 4 assembles base-4 digit g of the magnitude (selected, not indexed: an array
+        // indexed at run time would be kept in LDS)
+        const int p2 = bg & 3;
         const uint32_t a0 = p2 == 0 ? mag[0] : p2 == 1 ? mag[2] : p2 == 2 ? mag[4] : mag[6];
         const uint32_t a1 = p2 == 0 ? mag[1] : p2 == 1 ? mag[3] : p2 == 2 ? mag[5] : mag[7];
         const uint32_t both = a0 & a1;
@@ -1801,19 +1789,23 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
         bw.y = pack(both, a0 & ~a1, a1, 1);  // 0, 1, 2, 3 -> codes 0, 2, 4, 5
         bw.z = pack(a0, a1, 0u, 2);          // 0, 1/2, 1, 3/2 -> codes 0, 1, 2, 3
         bw.w = pack(a0, a1, 0u, 3);
-        *reinterpret_cast<u32x4*>(wB + (pw * 4 + p2) * 4) = bw;
-        if (p2 == 0) {
+        if (has_word && bg < 4) *reinterpret_cast<u32x4*>(wB + (word * 4 + p2) * 4) = bw;
+        if (has_word && bg == 0) {
             int c = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) c += __popc(acc[i]) << i;
             atomicAdd(&base_s, c);  // sum over all code bits of the per-bit counts
         }
-    }
-    if (threadIdx.x < 4) wzero[threadIdx.x] = 0;
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    } else {
 #pragma unroll
-    for (int i = kFirst; i < kSlots; ++i)
-        if (i < run) issue(i);
+        for (int i = 0; i < kSlots; ++i)
+            if (i < run) issue(i);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    const int first = wid < 3 ? kFirst : kSlots;
+#pragma unroll
+    for (int i = 0; i < kSlots; ++i)
+        if (i >= first && i < run) issue(i);
     if (run <= 0) return;
     const int base = base_s;
     const int full = G * 32 * WD;
