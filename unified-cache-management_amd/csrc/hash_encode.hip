@@ -985,104 +985,146 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
 // prompt or after a store hit).
 //
 // 512 x 256 bf16 are 256 KiB - half of a compute unit's register file - so the projection cannot
-// belong to one wave as in the 128-wide kernel above.  A persistent workgroup of eight waves owns a
-// slice of 256 hash columns for the kernel's lifetime, each wave 32 of them: 32 k-steps x 4
-// registers = 128 registers of MFMA A operands per lane.  (512 hash bits are two such slices, i.e. two
-// launches over the same rows.)  What the
-// eight waves share are the rows: a tile of 32 rows (32 KiB) is brought in once per workgroup,
-// straight from memory into LDS - every wave issues the loads of four rows, lane l of a load fetching
-// 16-byte piece l ^ (row & 7) so that the operand reads below hit all banks - and every wave
-// reads all of it as its B operands (one 16-byte LDS read per lane and MFMA).  Four tiles are
-// in the ring: at the barrier of tile i every wave has waited for its own loads of tile i, so the
-// tile is complete, and everybody is done with tile i - 1, so the loads of tile i + 3 go into its
-// slot: three tiles (96 KiB per compute unit) are in flight behind the one being multiplied.  One bare
-// barrier per tile.  Between two barriers the two waves of a SIMD
-// work in opposite order - one multiplies first and packs its signs afterwards, the other packs the
-// previous tile's signs first and multiplies then - so that the matrix cores are not left idle while
-// everybody packs (all waves in step: 0.25 ms per million rows at 256 bits; out of step: see below).
-// A wave's 32 x 32 products leave it as one word per row; the eight words of a row meet in a small
-// LDS buffer (three in turn), and two barriers later one wave - they take turns - stores the tile's
-// 32 code rows, 16 bytes per lane.  Roofline: 1 KiB read and 32 bytes written per row and slice
-// against 262,144 multiply-adds: at 256 bits memory and matrix cores bind about equally (0.14 ms
-// against 0.11 ms per million rows), at 512 bits the matrix cores do (0.22 ms).  The LDS read rate
-// (eight waves x 32 KiB per tile) equals the matrix cores' appetite exactly: both pipes would be
-// busy all the time in a perfect schedule.
+// belong to one wave as in the 128-wide kernel above.  A persistent workgroup of four waves, one
+// per SIMD, owns a slice of 256 hash columns for the kernel's lifetime, each wave 64 of them: 2 x
+// 32 k-steps x 4 registers = 256 registers of MFMA A operands per lane, the whole accumulation
+// half of the wave's register file.  The matrix instructions are written out (inline assembly)
+// because the compiler will not keep operands there on its own: given the builtin it holds them
+// in the other half, spills and copies.  (512 hash bits are two such slices, i.e. two launches
+// over the same rows.)  What the four waves share are the rows: a tile of 32 rows (32 KiB) is
+// brought in once per workgroup, straight from memory into LDS - every wave issues the loads of
+// eight rows, lane l of a load fetching 16-byte piece l ^ (row & 7) so that the operand reads hit
+// all banks - and every wave reads all of it as its B operands, each 16-byte read feeding two
+// matrix instructions (128 KiB of LDS reads per tile; eight waves of 32 columns read 256 KiB).
+//
+// A wave has its SIMD to itself, so nothing hides what it waits for: the stream of matrix
+// instructions must never stop.  Operand reads run eight k-steps ahead in a ring of registers -
+// never more than 15 LDS operations in flight: the counter the waits are written against has
+// four bits, and with 16 reads ahead the first of a pair of matrix instructions now and then
+// read its operand before it had arrived.  Four tiles are in the ring.  One bare barrier per
+// tile, in its middle: behind it the next tile is complete in LDS (its reads start with the
+// second half of this tile's matrix instructions, so the stream runs on from tile to tile),
+// everybody is done with the previous tile (its slot takes the tile three ahead, one load
+// instruction per k-step), and the words of the tile before that are complete.  The signs of
+// tile i - 1 are packed while tile i is multiplied, from a second set of accumulators, four
+// instructions per k-step (a wave issues about seven vector instructions between two pairs of
+// matrix instructions for free; 25 in one place cost 70 cycles of matrix time).  A sum starts
+// from a constant register set given to the tile's first matrix instruction as its C operand:
+// no accumulator is ever re-initialised.  A wave's 2 x 32 x 32 products leave it as two words per
+// row; the eight words of a row meet in a small LDS buffer (three in turn), and one wave - they
+// take turns - stores the tile's 32 code rows, 16 bytes per lane.
+//
+// Measured on the part (shader clock counter against the 100 MHz counter, inside the kernel):
+// a launch over 2^20 rows takes 440,000 cycles, and the clock under this load settles at 1.27
+// to 1.55 GHz (1.9 GHz in the first launches): 0.31 ms.  262,144 of the cycles are matrix
+// instructions (8,192 per wave x 32).  Without the row loads the same kernel takes 375,000
+// cycles, with loads that hit in L2 about the same: what the loads cost is their issue - an
+// instruction that finds the load path busy holds its wave, 80 cycles per instruction on
+// average - not the wait for their data (leaving the waits out changes nothing).  Spreading the
+// loads over the whole tile instead (each wave alone in its k-step) shortens their lead and was
+// slower (590,000 to 655,000 cycles).  Eight waves of 32 columns, two per SIMD, one reading while
+// the other multiplies: 465,000 to 508,000 cycles, 0.33 ms.
 // ---------------------------------------------------------------------------------------
-constexpr int kWideWaves = 8;
+constexpr int kWideWaves = 4;
 constexpr int kWideThreads = kWideWaves * 64;
 constexpr int kWideRing = 4;
 constexpr int kWideK = 512;
 constexpr int kWideTileBytes = kRowsPerWave * kWideK * 2;  // 32 KiB
-// a ring slot holds a tile; before the first tile it holds one wave's staged slice of W (32 rows of
-// K + kPad values)
+// a ring slot holds a tile; before the first tile it holds one wave's staged 32 columns of W (32
+// rows of K + kPad values)
 constexpr int kWideSlotBytes = kRowsPerWave * (kWideK + kPad) * 2;
 constexpr int kWideCodeBytes = kRowsPerWave * 32;  // 32 rows x 8 words
 constexpr int kWideMapRing = 8;                    // slot-mapping entries (256 bytes) of eight tiles
+constexpr int kWideAhead = 8;                      // operand reads ahead of the matrix instructions, in k-steps
 constexpr size_t kWideLds = (size_t)kWideRing * kWideSlotBytes + 3 * kWideCodeBytes + kWideMapRing * 256;
 static_assert(kWideSlotBytes % 16 == 0 && kWideTileBytes <= kWideSlotBytes, "ring slot layout");
 static_assert(kWideLds <= 160 * 1024, "ring exceeds the LDS");
+static_assert(kWideAhead + 4 <= 15 && (kWideK / 16) % kWideAhead == 0, "LDS operations in flight; ring index");
 
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 
+// v_mfma_f32_32x32x16 with the A operand in the accumulation registers
+template <typename V>
+__device__ __forceinline__ void wide_mfma(f32x16& acc, const u32x4& w, const u32x4& b)
+{
+    if constexpr (std::is_same<V, bf16x8>::value)
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "a"(w), "v"(b));
+    else
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "a"(w), "v"(b));
+}
+
+// first matrix instruction of a tile: the sum starts from `start` (which stays as it is)
+template <typename V>
+__device__ __forceinline__ void wide_mfma_first(f32x16& acc, const u32x4& w, const u32x4& b, const f32x16& start)
+{
+    if constexpr (std::is_same<V, bf16x8>::value)
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(acc) : "a"(w), "v"(b), "v"(start));
+    else
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(acc) : "a"(w), "v"(b), "v"(start));
+}
+
 template <typename V, int SLOT>
-__global__ __launch_bounds__(kWideThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void encode_wide_kernel(
+__global__ __launch_bounds__(kWideThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void encode_wide_kernel(
     EncArgs a, int64_t ntiles, int nstreams, int col)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[];
     constexpr int K = kWideK, KS = K / 16;
-    constexpr int kLoads = 4 + (SLOT ? 1 : 0);  // load instructions per wave and tile
+    constexpr int kLoads = 8 + (SLOT ? 1 : 0);  // load instructions per wave and tile
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 31, kb = lane >> 5;
-    const int stream = blockIdx.x;  // rows stream, stream + nstreams, ...; hash columns 256 col .. 256 col + 255
+    const int stream = blockIdx.x;
     uint8_t* const codes = wide_lds + (size_t)kWideRing * kWideSlotBytes;
     constexpr uint32_t kMapOff = (uint32_t)(kWideRing * kWideSlotBytes + 3 * kWideCodeBytes);
 
-    // ---- this wave's 32 columns of W as MFMA A operands, for the kernel's lifetime ----
+    // ---- this wave's 2 x 32 columns of W as MFMA A operands, for the kernel's lifetime ----
     // 8 x 8 patches (eight 16-byte rows each) are transposed in registers and written as 32 LDS
-    // rows of K values, then every lane reads its K / 16 operands.  A staged tile fills a ring
-    // slot, so the waves go in two shifts of four.
-    V wreg[KS];
+    // rows of K values into the wave's own ring slot, then every lane reads its K / 16 operands:
+    // 32 columns at a time.  The empty statements pin what was read to the accumulation registers.
+    u32x4 wreg[2][KS];
     {
         constexpr int KP = K + kPad;
-        const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)weight_index(a, 0) * K * a.N + col * 256 + wave * 32;
-        uint16_t* wt = reinterpret_cast<uint16_t*>(wide_lds + (size_t)(wave & 3) * kWideSlotBytes);
+        uint16_t* wt = reinterpret_cast<uint16_t*>(wide_lds + (size_t)wave * kWideSlotBytes);
 #pragma unroll
-        for (int shift = 0; shift < 2; ++shift) {
-            if ((wave >> 2) == shift) {
+        for (int g = 0; g < 2; ++g) {
+            const uint16_t* wsrc =
+                (const uint16_t*)a.w + (int64_t)weight_index(a, 0) * K * a.N + col * 256 + wave * 64 + g * 32;
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {  // 256 patches, four per lane, two at a time
-                    u32x4 row[2][8];
+            for (int half = 0; half < 2; ++half) {  // 256 patches, four per lane, two at a time
+                u32x4 row[2][8];
 #pragma unroll
-                    for (int it = 0; it < 2; ++it) {
-                        const int idx = (half * 2 + it) * 64 + lane;
-                        const uint16_t* src = wsrc + (int64_t)((idx >> 2) * 8) * a.N + 8 * (idx & 3);
+                for (int it = 0; it < 2; ++it) {
+                    const int idx = (half * 2 + it) * 64 + lane;
+                    const uint16_t* src = wsrc + (int64_t)((idx >> 2) * 8) * a.N + 8 * (idx & 3);
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) row[it][i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * a.N);
-                    }
+                    for (int i = 0; i < 8; ++i) row[it][i] = *reinterpret_cast<const u32x4*>(src + (int64_t)i * a.N);
+                }
 #pragma unroll
-                    for (int it = 0; it < 2; ++it) {
-                        const int idx = (half * 2 + it) * 64 + lane;
-                        const int kq = idx >> 2, j = idx & 3;
+                for (int it = 0; it < 2; ++it) {
+                    const int idx = (half * 2 + it) * 64 + lane;
+                    const int kq = idx >> 2, j = idx & 3;
 #pragma unroll
-                        for (int c = 0; c < 8; ++c) {
-                            const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-                            u32x4 o;
-                            o.x = __builtin_amdgcn_perm(row[it][1][c >> 1], row[it][0][c >> 1], sel);
-                            o.y = __builtin_amdgcn_perm(row[it][3][c >> 1], row[it][2][c >> 1], sel);
-                            o.z = __builtin_amdgcn_perm(row[it][5][c >> 1], row[it][4][c >> 1], sel);
-                            o.w = __builtin_amdgcn_perm(row[it][7][c >> 1], row[it][6][c >> 1], sel);
-                            *reinterpret_cast<u32x4*>(wt + (8 * j + c) * KP + kq * 8) = o;
-                        }
+                    for (int c = 0; c < 8; ++c) {
+                        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                        u32x4 o;
+                        o.x = __builtin_amdgcn_perm(row[it][1][c >> 1], row[it][0][c >> 1], sel);
+                        o.y = __builtin_amdgcn_perm(row[it][3][c >> 1], row[it][2][c >> 1], sel);
+                        o.z = __builtin_amdgcn_perm(row[it][5][c >> 1], row[it][4][c >> 1], sel);
+                        o.w = __builtin_amdgcn_perm(row[it][7][c >> 1], row[it][6][c >> 1], sel);
+                        *reinterpret_cast<u32x4*>(wt + (8 * j + c) * KP + kq * 8) = o;
                     }
                 }
-                __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    wreg[ks] = *reinterpret_cast<const V*>(wt + r * KP + ks * 16 + kb * 8);
             }
-            __syncthreads();  // the staging area becomes the next shift's, then the row ring
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                wreg[g][ks] = *reinterpret_cast<const u32x4*>(wt + r * KP + ks * 16 + kb * 8);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(wreg[g][ks]));
         }
+        __syncthreads();  // the staging areas become the row ring
     }
 
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(
@@ -1090,133 +1132,215 @@ __global__ __launch_bounds__(kWideThreads) __attribute__((amdgpu_waves_per_eu(2,
     const uint32_t row_bytes = (uint32_t)(a.x_stride_t * 2);
     constexpr int slot_sz = SLOT == 2 ? 8 : 4;
     const uint32_t slot_e = SLOT == 2 ? (uint32_t)lane >> 1 : (uint32_t)lane & 31;
-    // A wave's share of a tile's loads: rows 4 * wave + j (j = 0..3), lane l fetching piece
-    // l ^ (row & 7); rows past the end of the input re-read its last row.  Every wave also fetches
-    // the tile's 32 slot-mapping entries into a ring of their own (all eight write the same values):
-    // one more instruction, so that every wave counts the same loads per tile.
-    uint32_t off_full[4];
+    // A wave's share of a tile's loads: rows 8 * wave + j (j = 0..7), lane l fetching piece l ^ j;
+    // rows past the end of the input re-read its last row.  Every wave also fetches the tile's 32
+    // slot-mapping entries (all four write the same values): every wave counts the same loads.
+    // The load instructions of a tile are issued one at a time, between matrix instructions.
+    uint32_t off_full[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t q = 4 * (uint32_t)wave + j;
-        off_full[j] = q * row_bytes + (((uint32_t)lane ^ (q & 7)) << 4);
-    }
+    for (int j = 0; j < 8; ++j) off_full[j] = (8 * (uint32_t)wave + j) * row_bytes + (((uint32_t)lane ^ j) << 4);
     const uint32_t slot_full = slot_e * slot_sz + (SLOT == 2 ? ((uint32_t)lane & 1) * 4 : 0);
-    auto issue = [&](int64_t tile, int local) {
+    // part p of the loads of `tile` (ring position `local`): p = 0..7 a row, p = 8 the slot mapping
+    auto issue_part = [&](int64_t tile, int local, int p) {
         const int64_t t0 = tile * kRowsPerWave;
         const int64_t left64 = a.T - 1 - t0;
-        const uint64_t base = (uint64_t)(uintptr_t)((const uint16_t*)a.x + t0 * a.x_stride_t);
-        const uint32_t lds = lds0 + (local % kWideRing) * kWideSlotBytes;
-        uint32_t so = slot_full;
-        if (left64 >= 31) {
-            stream_issue_rows<1>(lds + wave * 4096, base, off_full);
-        } else {
-            const uint32_t left = (uint32_t)left64;
-            uint32_t off[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t q = 4 * (uint32_t)wave + j;
-                const uint32_t qq = q > left ? left : q;
-                off[j] = qq * row_bytes + (((uint32_t)lane ^ (q & 7)) << 4);
+        if (p < 8) {
+            const uint64_t base = (uint64_t)(uintptr_t)((const uint16_t*)a.x + t0 * a.x_stride_t);
+            const uint32_t lds = lds0 + (local % kWideRing) * kWideSlotBytes + wave * 8192 + p * 1024;
+            uint32_t off = off_full[p];
+            if (left64 < 31) {
+                const uint32_t left = (uint32_t)left64;
+                const uint32_t q = 8 * (uint32_t)wave + p;
+                off = (q > left ? left : q) * row_bytes + (((uint32_t)lane ^ p) << 4);
             }
-            stream_issue_rows<1>(lds + wave * 4096, base, off);
-            const uint32_t ee = slot_e > left ? left : slot_e;
-            so = ee * slot_sz + (SLOT == 2 ? ((uint32_t)lane & 1) * 4 : 0);
-        }
-        if constexpr (SLOT != 0)
+            uint32_t keep;
+            asm volatile("s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[lds]\n\ts_nop 0\n\t"
+                         "global_load_lds_dwordx4 %[o], %[base] nt\n\ts_mov_b32 m0, %[keep]\n\t"
+                         : [keep] "=&s"(keep)
+                         : [lds] "s"(lds), [base] "s"(base), [o] "v"(off)
+                         : "memory");
+        } else if constexpr (SLOT != 0) {
+            uint32_t so = slot_full;
+            if (left64 < 31) {
+                const uint32_t left = (uint32_t)left64;
+                const uint32_t ee = slot_e > left ? left : slot_e;
+                so = ee * slot_sz + (SLOT == 2 ? ((uint32_t)lane & 1) * 4 : 0);
+            }
             stream_issue_slots(lds0 + kMapOff + (local % kWideMapRing) * 256,
                                (uint64_t)(uintptr_t)((const char*)a.slot + t0 * slot_sz), so);
+        }
+    };
+    auto issue = [&](int64_t tile, int local) {
+#pragma unroll
+        for (int p = 0; p < 9; ++p) issue_part(tile, local, p);
     };
 
-    // operand read offset of k-step ks: row r, piece (2 ks + kb) ^ (r & 7)
     const uint32_t r_base = (uint32_t)r * 1024;
     const uint32_t r_swz = (uint32_t)r & 7;
     const int64_t n_slots = a.NB << a.bs_shift;
     const uint32_t csb = (uint32_t)a.cs_block, cst = (uint32_t)a.cs_token;
     uint32_t* const cache_c = a.cache + col * 8;
 
-    // Storing a tile's 32 code rows (lane l: half l & 1 of row l >> 1) takes two steps one tile apart:
-    // the slot-mapping entries are picked up first, the store follows when the last words have arrived.
-    int64_t held = -1;
-    auto pick_slots = [&](int64_t tile, int local) {
+    // Every wave picks up every tile's slot-mapping entries and reads its code rows; the wave whose
+    // turn it is stores them (lane l: half l & 1 of row l >> 1).  No branch around the LDS reads (a
+    // join would make the compiler wait for every operand read in flight), and what they return is
+    // used a few k-steps later, when younger operand reads are counted behind them.
+    int64_t held = -1, sv_raw = 0;
+    u32x4 code_raw = {0, 0, 0, 0};
+    auto pick_read = [&](int local) {
         const uint8_t* slot_base = wide_lds + kMapOff + (local % kWideMapRing) * 256;
         const int row = lane >> 1;
-        const int64_t t = tile * kRowsPerWave + row;
-        int64_t sv = t;
-        if constexpr (SLOT == 2) sv = *reinterpret_cast<const int64_t*>(slot_base + row * 8);
-        if constexpr (SLOT == 1) sv = *reinterpret_cast<const int32_t*>(slot_base + row * 4);
-        held = (t < a.T && sv >= 0 && sv < n_slots) ? sv : -1;
+        if constexpr (SLOT == 2) sv_raw = *reinterpret_cast<const int64_t*>(slot_base + row * 8);
+        if constexpr (SLOT == 1) sv_raw = *reinterpret_cast<const int32_t*>(slot_base + row * 4);
+        asm volatile("" ::: "memory");  // the read stays here
     };
-    auto store_tile = [&](int local) {
+    auto pick_use = [&](int64_t tile) {
+        const int64_t t = tile * kRowsPerWave + (lane >> 1);
+        const int64_t sv = SLOT == 0 ? t : sv_raw;
+        held = (tile >= 0 && t < a.T && sv >= 0 && sv < n_slots) ? sv : -1;
+    };
+    auto store_read = [&](int local) {
         const int row = lane >> 1, half = lane & 1;
-        const u32x4 code = *reinterpret_cast<const u32x4*>(codes + (local % 3) * kWideCodeBytes + row * 32 + half * 16);
-        if (held >= 0) {
+        code_raw = *reinterpret_cast<const u32x4*>(codes + (local % 3) * kWideCodeBytes + row * 32 + half * 16);
+        asm volatile("" ::: "memory");
+    };
+    auto store_use = [&](bool mine) {
+        if (held >= 0 && mine) {
             const uint32_t svl = (uint32_t)held;
-            uint32_t* dst = cache_c + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) + half * 4;
-            *reinterpret_cast<u32x4_a4*>(dst) = code;
+            uint32_t* dst = cache_c + ((svl >> a.bs_shift) * csb + (svl & (uint32_t)(a.BS - 1)) * cst) + (lane & 1) * 4;
+            *reinterpret_cast<u32x4_a4*>(dst) = code_raw;
         }
     };
-    // a wave's 32 x 32 signs of a tile -> its word of each of the tile's 32 code rows
-    auto hand_in = [&](f32x16& acc0, const f32x16& acc1, int local) {
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc0[q] += acc1[q];
-        const uint32_t half = pack_half(acc0);
-        const uint32_t word = join_halves(kb ? half << 4 : half);
-        if (lane < 32) *reinterpret_cast<uint32_t*>(codes + (local % 3) * kWideCodeBytes + r * 32 + wave * 4) = word;
+    auto hand_in = [&](uint32_t w0, uint32_t w1, int local) {
+        w0 = join_halves(kb ? w0 << 4 : w0);
+        w1 = join_halves(kb ? w1 << 4 : w1);
+        if (lane < 32) *reinterpret_cast<uint2*>(codes + (local % 3) * kWideCodeBytes + r * 32 + wave * 8) = uint2{w0, w1};
     };
 
-    // The two waves of a SIMD (w and w + 4) take the work between two barriers in opposite order, so
-    // that one of them always has products for the matrix cores: waves 0..3 multiply tile i and hand
-    // its words in before the next barrier; waves 4..7 first hand in tile i - 1, then multiply tile i.
-    // A tile's words are therefore complete one barrier later, and its rows are stored after that.
-    const bool late = wave >= 4;
-    f32x16 acc0 = acc_start(), acc1;
-#pragma unroll
-    for (int q = 0; q < 16; ++q) acc1[q] = 0.0f;
-
-    // tiles stream, stream + nstreams, ... : n of them
+    // tiles stream, stream + nstreams, ... : n of them, tile j in ring slot j % 4
     const int64_t n = stream < ntiles ? (ntiles - 1 - stream) / nstreams + 1 : 0;
-    int64_t tile = stream;
-    if (n > 0) issue(tile, 0);
-    if (n > 1) issue(tile + nstreams, 1);
-    if (n > 2) issue(tile + 2 * (int64_t)nstreams, 2);
-    for (int64_t i = 0; i < n + 2; ++i) {
-        const int local = (int)i;
-        if (i < n) {
-            // this wave's loads of tile i have landed (those of tiles i + 1 and i + 2 may be in flight)
-            if (i + 2 < n) stream_wait_loads<2 * kLoads>();
-            else if (i + 1 < n) stream_wait_loads<kLoads>();
-            else stream_wait_loads<0>();
+    const int64_t tile0 = stream;
+    constexpr int kAhead = kWideAhead;
+    u32x4 b[kAhead];
+    f32x16 cstart = acc_start();  // what every sum starts from
+    asm volatile("" : "+v"(cstart));
+    auto read_b = [&](int j, int ks) {
+        const uint8_t* buf = wide_lds + (size_t)(j % kWideRing) * kWideSlotBytes;
+        b[ks % kAhead] = *reinterpret_cast<const u32x4*>(buf + r_base + ((((uint32_t)(2 * ks) + kb) ^ r_swz) << 4));
+    };
+    // Tile j: its products go into (n0, n1) while the signs of tile j - 1 leave (p0, p1).  One
+    // barrier, in the middle of the tile: behind it tile j + 1 is complete in LDS (its operand
+    // reads start with the second half of tile j's matrix instructions, so the stream of matrix
+    // instructions runs on from tile to tile), everybody is done reading tile j - 1 (its ring
+    // slot takes tile j + 3), and the words of tile j - 2 are complete.  Tiles -1, -2 (before the
+    // first) and n (behind the last) are handled like any other - their words go nowhere, the
+    // reads of tile n find whatever the ring slot holds - so that the body has no branches but
+    // the one around the loads of tile j + 3 (STEADY: taken for granted).
+    auto tile_body = [&](auto steady, int64_t j64, f32x16& n0, f32x16& n1, f32x16& p0, f32x16& p1) {
+        constexpr bool STEADY = decltype(steady)::value;
+        const int j = (int)j64;
+        // The signs of tile j - 1 leave (p0, p1) four instructions per k-step: a wave can issue
+        // about seven vector instructions between two pairs of matrix instructions without
+        // keeping the matrix cores waiting, and its address arithmetic takes some of them.
+        uint32_t hi0 = 0, lo0 = 0, hi1 = 0, lo1 = 0, w0 = 0, w1 = 0;
+#pragma unroll
+        for (int ks = 0; ks < KS / 2; ++ks) {
+            if (ks == 0) {
+                wide_mfma_first<V>(n0, wreg[0][ks], b[ks % kAhead], cstart);
+                wide_mfma_first<V>(n1, wreg[1][ks], b[ks % kAhead], cstart);
+            } else {
+                wide_mfma<V>(n0, wreg[0][ks], b[ks % kAhead]);
+                wide_mfma<V>(n1, wreg[1][ks], b[ks % kAhead]);
+            }
+            if (ks + kAhead < KS) read_b(j, ks + kAhead);
+            if (ks >= 1 && ks <= 8) {
+                // pack_half, one step of its two chains per k-step
+                const int st = ks - 1, g = 1 - st / 4, jj = 3 - st % 4;
+                __builtin_amdgcn_sched_barrier(0);
+                if (st == 4) {
+                    hi0 <<= 4;
+                    lo0 <<= 4;
+                    hi1 <<= 4;
+                    lo1 <<= 4;
+                }
+                hi0 = __builtin_amdgcn_alignbit(hi0, __float_as_uint(p0[4 * (g + 2) + jj]), 31);
+                lo0 = __builtin_amdgcn_alignbit(lo0, __float_as_uint(p0[4 * g + jj]), 31);
+                hi1 = __builtin_amdgcn_alignbit(hi1, __float_as_uint(p1[4 * (g + 2) + jj]), 31);
+                lo1 = __builtin_amdgcn_alignbit(lo1, __float_as_uint(p1[4 * g + jj]), 31);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (ks == 9) {
+                __builtin_amdgcn_sched_barrier(0);
+                w0 = ((hi0 << 16) | lo0) ^ 0x0F0F0F0Fu;
+                w1 = ((hi1 << 16) | lo1) ^ 0x0F0F0F0Fu;
+                w0 = p0[0] != p0[0] ? 0u : w0;  // a row with a NaN: no bit set
+                w1 = p1[0] != p1[0] ? 0u : w1;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (ks == 10) {
+                __builtin_amdgcn_sched_barrier(0);
+                hand_in(w0, w1, j + 2);  // tile j - 1's place in the ring of three
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        // every wave's part of tile i is in LDS, and every wave is done reading tile i - 1: its ring
-        // slot takes tile i + 3
+        // this wave's loads of tile j + 1 have landed (those of tile j + 2 may be in flight)
+        if (STEADY || j64 + 2 < n) stream_wait_loads<kLoads>();
+        else stream_wait_loads<0>();
+        asm volatile("s_barrier" ::: "memory");
+        const bool more = STEADY || j64 + 3 < n;
+        const int64_t tile3 = tile0 + (j64 + 3) * nstreams;
+        const bool mine = ((j + 2) % kWideWaves) == wave && j >= 2;  // tile j - 2 is this wave's to store
+#pragma unroll
+        for (int ks = KS / 2; ks < KS; ++ks) {
+            wide_mfma<V>(n0, wreg[0][ks], b[ks % kAhead]);
+            wide_mfma<V>(n1, wreg[1][ks], b[ks % kAhead]);
+            if (ks + kAhead < KS) read_b(j, ks + kAhead);
+            else read_b(j + 1, ks + kAhead - KS);
+            const int part = ks - KS / 2;
+            if (part < 9 && more) issue_part(tile3, j + 3, part);
+            if (part == 10) store_read(j + 1);  // tile j - 2's place in the ring of three
+            if (part == 11) pick_read(j + 7);   // tile j - 1's entries
+            if (part == 14) store_use(mine);
+            if (part == 15) pick_use(tile0 + (j64 - 1) * nstreams);
+        }
+    };
+
+    f32x16 accA0 = acc_start(), accA1 = acc_start(), accB0 = acc_start(), accB1 = acc_start();
+    if (n > 0) issue(tile0, 0);
+    if (n > 1) issue(tile0 + nstreams, 1);
+    if (n > 2) issue(tile0 + 2 * (int64_t)nstreams, 2);
+    if (n > 0) {
+        if (n > 2) stream_wait_loads<2 * kLoads>();
+        else if (n > 1) stream_wait_loads<kLoads>();
+        else stream_wait_loads<0>();
+        asm volatile("s_barrier" ::: "memory");  // tile 0 is complete
+#pragma unroll
+        for (int ks = 0; ks < kAhead; ++ks) read_b(0, ks);
+        int64_t j = 0;
+        for (; j + 4 < n; j += 2) {
+            tile_body(std::true_type{}, j, accA0, accA1, accB0, accB1);
+            tile_body(std::true_type{}, j + 1, accB0, accB1, accA0, accA1);
+        }
+        for (; j < n; j += 2) {
+            tile_body(std::false_type{}, j, accA0, accA1, accB0, accB1);
+            if (j + 1 < n) tile_body(std::false_type{}, j + 1, accB0, accB1, accA0, accA1);
+        }
+        // the last tile's products: out of the matrix cores, packed, handed in; then the last two
+        // tiles' rows are stored
+        const int last = (int)(n - 1);
+        // nothing reads an accumulator before the matrix cores are done with it (choosing between
+        // the two sets is already such a read)
+        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(accA0), "+v"(accA1), "+v"(accB0), "+v"(accB1));
+        const f32x16& l0 = (last & 1) ? accB0 : accA0;
+        const f32x16& l1 = (last & 1) ? accB1 : accA1;
+        hand_in(pack_half(l0), pack_half(l1), last);
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        if (i + 3 < n) issue(tile + 3 * (int64_t)nstreams, local + 3);
-        if (late && i >= 1 && i <= n) {
-            hand_in(acc0, acc1, local - 1);
-            acc0 = acc_start();
-#pragma unroll
-            for (int q = 0; q < 16; ++q) acc1[q] = 0.0f;
-        }
-        if (i >= 2 && ((local - 2) % kWideWaves) == wave) store_tile(local - 2);
-        if (i >= 1 && i <= n && ((local - 1) % kWideWaves) == wave) pick_slots(tile - nstreams, local - 1);
-        if (i < n) {
-            const uint8_t* buf = wide_lds + (size_t)(local % kWideRing) * kWideSlotBytes;
-            // two accumulator chains in flight: the even and the odd k-steps, added at the end
-#pragma unroll
-            for (int ks = 0; ks < KS; ks += 2) {
-                const V b0 = *reinterpret_cast<const V*>(buf + r_base + ((((uint32_t)(2 * ks) + kb) ^ r_swz) << 4));
-                const V b1 = *reinterpret_cast<const V*>(buf + r_base + ((((uint32_t)(2 * ks + 2) + kb) ^ r_swz) << 4));
-                acc0 = Mfma<V>::run(wreg[ks], b0, acc0);
-                acc1 = Mfma<V>::run(wreg[ks + 1], b1, acc1);
-            }
-            if (!late) {
-                hand_in(acc0, acc1, local);
-                acc0 = acc_start();
-#pragma unroll
-                for (int q = 0; q < 16; ++q) acc1[q] = 0.0f;
-            }
-        }
-        tile += nstreams;
+        store_read(last + 2);
+        store_use(last >= 1 && ((last - 1) % kWideWaves) == wave);
+        pick_read(last);
+        pick_use(tile0 + (int64_t)last * nstreams);
+        store_read(last);
+        store_use((last % kWideWaves) == wave);
     }
     // no load may still be writing into this workgroup's LDS when the wave ends
     stream_wait_loads<0>();
