@@ -410,8 +410,12 @@ def encoder_latent_cache_build(torch, gen, launches=7):
         cache = torch.empty((NB5, BS5, 1, cwords), dtype=torch.int32, device="cuda")
         view = cache[..., : n_bits // 32]
         res = {}
+        # the clock the wide kernel runs at, from its own counters (first workgroup: shader cycles and 100 MHz
+        # ticks of its lifetime; the last timed launch's values remain): a launch time can only be judged beside it
+        probe = torch.zeros(2, dtype=torch.int64, device="cuda")
         for kernel, thr in (("encode_wide_kernel", 0), ("encode_mfma_kernel (tiled)", 1 << 62)):
             _lib.lib().ucm_hash_encode_set_stream_threshold(thr)
+            _lib.check(_lib.lib().ucm_hash_encode_set_clock_probe(probe.data_ptr() if thr == 0 else None))
             for i in range(2):
                 enc.compute_hash_and_cache(lat[i][:, :K].unsqueeze(1), slots, view, BS5)
             ev = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
@@ -428,6 +432,14 @@ def encoder_latent_cache_build(torch, gen, launches=7):
                            "hbm_frac": alg / ms / 1e6 / HBM_PEAK_GBPS, "TFLOPs": flops / ms / 1e9,
                            "mfma_frac_of_2500_TFLOPs": flops / ms / 1e9 / 2500.0}
         _lib.lib().ucm_hash_encode_set_stream_threshold(0)
+        _lib.check(_lib.lib().ucm_hash_encode_set_clock_probe(None))
+        cyc, ticks = (int(v) for v in probe.cpu().tolist())
+        res["encode_wide_kernel"]["shader_cycles_last_timed_launch"] = cyc
+        res["encode_wide_kernel"]["shader_clock_GHz_last_timed_launch"] = cyc / (ticks * 10.0) if ticks else None
+        # one launch = one slice of 256 hash columns: its v_mfma_32x32x16 count x 32 cycles over 1,024 SIMDs
+        res["encode_wide_kernel"]["mfma_cycles_per_launch"] = T * 256 * K // (32 * 32 * 16) * 32 // 1024
+        res["encode_wide_kernel"]["mfma_cycles_over_shader_cycles"] = (
+            res["encode_wide_kernel"]["mfma_cycles_per_launch"] / cyc if cyc else None)
         alg = T * K * 2 + T * n_bits // 8 + K * n_bits * 2 + T * 8
         flops = 2.0 * T * K * n_bits
         floor_ms = max(alg / (HBM_PEAK_GBPS * 1e6), flops / 2500e9)

@@ -95,6 +95,18 @@ int ucm_hash_encode_cache(const void* x, int x_dtype, int64_t T, int32_t H, int3
 int ucm_hash_encode_set_stream_threshold(int64_t rows);
 
 /*
+ * Measurement aid, no counterpart in the reference.  While a non-null address is set, every launch
+ * of the persistent kernel for 512 input dimensions (encode_wide_kernel) issued by the calling thread
+ * has its first workgroup write two 64-bit numbers there when it ends: the shader cycles and the
+ * ticks of the constant 100 MHz counter between its first and its last instruction.  Their ratio is
+ * the clock the workgroup ran at (cycles / ticks * 0.1 GHz); the part's clock under a matrix-heavy
+ * load is well below its data-sheet maximum, and a launch time can only be judged beside it.  The
+ * address must be 8-byte aligned device memory of at least 16 bytes that outlives the launches; pass
+ * null to switch the probe off (the default).  Other kernels ignore it.
+ */
+int ucm_hash_encode_set_clock_probe(void* two_u64_in_device_memory);
+
+/*
  * The streaming kernel's time-out contract, no counterpart in the reference.  With 2, 4 or 8 heads
  * of 128-bit codes side by side in a cache row the streaming kernel's waves exchange their codes
  * through LDS and wait for one another with a bounded number of polls; a wave that reaches the bound

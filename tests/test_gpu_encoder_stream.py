@@ -255,6 +255,35 @@ def test_wide_streaming_kernel_dense_output(stream_everything, T):
     _check_against_oracle(o[:T].reshape(T, 1, 1, N // 32), x, W, np.arange(T), 1, 0, rows)
 
 
+def test_wide_streaming_kernel_clock_probe(stream_everything):
+    """The measurement aid: with a probe address set the wide kernel's first workgroup reports its
+    lifetime in shader cycles and in 100 MHz ticks; the codes are the same with and without it."""
+    from ucm_amd import _lib
+
+    L = stream_everything
+    rng = rng_for(43)
+    T, K, N = 40000, 512, 256
+    x = torch.from_numpy(rng.standard_normal((T, 1, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    W = torch.from_numpy(rng.standard_normal((1, K, N)).astype(np.float32)).to(torch.bfloat16).cuda()
+    outs = []
+    probe = torch.zeros(2, dtype=torch.int64, device="cuda")
+    for ptr in (probe.data_ptr(), None):
+        _lib.check(L.ucm_hash_encode_set_clock_probe(ptr))
+        out = torch.zeros((T, 1, N // 32), dtype=torch.int32, device="cuda")
+        _lib.check(L.ucm_hash_encode(x.data_ptr(), 0, T, 1, K, x.stride(0), x.stride(1), W.data_ptr(), 0, 1, 0, N,
+                                     out.data_ptr(), out.stride(0), out.stride(1),
+                                     torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    cycles, ticks = (int(v) for v in probe.cpu().tolist())
+    assert cycles > 10000 and ticks > 100
+    ghz = cycles / (ticks * 10.0)
+    assert 0.3 < ghz < 3.0, ghz
+    assert torch.equal(outs[0], outs[1])
+    assert L.ucm_hash_encode_set_clock_probe(probe.data_ptr() + 4) == _lib.UCM_EPARAM  # not 8-byte aligned
+    _lib.check(L.ucm_hash_encode_set_clock_probe(None))
+
+
 def test_no_exchange_wait_reached_its_bound():
     """The waves of the streaming kernel wait for one another with bounded polls (a launch always
     ends); after the encoder tests of this process no wait may have reached the bound."""

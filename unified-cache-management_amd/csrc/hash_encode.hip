@@ -1065,11 +1065,18 @@ __device__ __forceinline__ void wide_mfma_first(f32x16& acc, const u32x4& w, con
 
 template <typename V, int SLOT>
 __global__ __launch_bounds__(kWideThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void encode_wide_kernel(
-    EncArgs a, int64_t ntiles, int nstreams, int col)
+    EncArgs a, int64_t ntiles, int nstreams, int col, unsigned long long* clock_probe)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[];
     constexpr int K = kWideK, KS = K / 16;
     constexpr int kLoads = 8 + (SLOT ? 1 : 0);  // load instructions per wave and tile
+    // measurement aid (null in normal use): the first workgroup reports its own lifetime in shader
+    // cycles and in ticks of the constant 100 MHz counter - their ratio is the clock it ran at
+    unsigned long long probe_c0 = 0, probe_r0 = 0;
+    if (clock_probe) {
+        probe_c0 = __builtin_readcyclecounter();
+        probe_r0 = __builtin_amdgcn_s_memrealtime();
+    }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 31, kb = lane >> 5;
@@ -1344,6 +1351,10 @@ __global__ __launch_bounds__(kWideThreads) __attribute__((amdgpu_waves_per_eu(1,
     }
     // no load may still be writing into this workgroup's LDS when the wave ends
     stream_wait_loads<0>();
+    if (clock_probe && blockIdx.x == 0 && threadIdx.x == 0) {
+        clock_probe[0] = __builtin_readcyclecounter() - probe_c0;
+        clock_probe[1] = __builtin_amdgcn_s_memrealtime() - probe_r0;
+    }
 }
 
 // Latency path for a handful of rows (decode): one wave per (job, head, 32 hash columns,
@@ -1657,6 +1668,7 @@ constexpr int64_t kWideMinRows256 = (int64_t)1 << 14;
 constexpr int64_t kWideMinRows512 = (int64_t)1 << 16;
 // 0 = the defaults above; set per calling thread (a test hook must not move other threads' encodes)
 thread_local int64_t t_stream_min_rows = 0;
+thread_local unsigned long long* t_clock_probe = nullptr;  // see ucm_hash_encode_set_clock_probe()
 
 int stream_workgroups()
 {
@@ -1787,7 +1799,7 @@ int launch_wide_s(const EncArgs& a, hipStream_t st)
     // over the rows (two slices side by side, meeting in L2, measured the same)
     for (int c = 0; c < ncol; ++c)
         hipLaunchKernelGGL((encode_wide_kernel<V, SLOT>), dim3((unsigned)wgs), dim3(kWideThreads), kWideLds, st, a,
-                           ntiles, wgs, c);
+                           ntiles, wgs, c, t_clock_probe);
     return ucm::launch_status("encode_wide_kernel");
 }
 
@@ -2130,6 +2142,14 @@ extern "C" int ucm_hash_encode_set_stream_threshold(int64_t rows)
 {
     ucm::clear_error();
     t_stream_min_rows = rows > 0 ? rows : 0;
+    return UCM_OK;
+}
+
+extern "C" int ucm_hash_encode_set_clock_probe(void* two_u64_in_device_memory)
+{
+    ucm::clear_error();
+    if ((uintptr_t)two_u64_in_device_memory & 7) return ucm::fail(UCM_EPARAM, "ucm_hash_encode_set_clock_probe: the address is not 8-byte aligned");
+    t_clock_probe = static_cast<unsigned long long*>(two_u64_in_device_memory);
     return UCM_OK;
 }
 

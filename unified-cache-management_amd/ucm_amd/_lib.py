@@ -30,6 +30,7 @@ _SIGNATURES = {
     "ucm_hash_encode_cache": (ci, [vp, ci, i64, i32, i32, i64, i64, vp, ci, i32, i32, i32, vp, ci,
                                    vp, i64, i32, i64, i64, i64, vp]),
     "ucm_hash_encode_set_stream_threshold": (ci, [i64]),
+    "ucm_hash_encode_set_clock_probe": (ci, [vp]),
     "ucm_hash_encode_stream_timeouts": (i64, []),
     "ucm_hash_encode_clear_stream_timeouts": (ci, []),
     "ucm_hash_encode_debug_trip_stream_latch": (ci, []),
