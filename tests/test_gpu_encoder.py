@@ -106,6 +106,40 @@ def test_per_head_weights_gqa_queries():
         assert_codes_match(c[:, h], x[:, h].float().numpy(), W[h // 4].float().numpy())
 
 
+@pytest.mark.parametrize("B,H,K,N,n_w", [
+    (16, 64, 512, 512, 1),   # the latent-attention step's queries: 32 tiles of (token, head) pairs instead of 64 half-empty ones
+    (3, 5, 128, 128, 1),     # 15 pairs: one partial tile
+    (33, 3, 64, 64, 1),      # 99 pairs in 4 tiles against 2 x 3 by head
+    (7, 6, 256, 256, 1),
+    (40, 4, 128, 128, 1),    # 2 x 4 tiles by head, 5 by pair
+    (7, 6, 128, 128, 2),     # two projections (3 heads each): tiles stay with one head
+])
+def test_few_tokens_many_heads_one_projection(B, H, K, N, n_w):
+    """Rows of the small-row kernel's tiles are (token, head) pairs when one projection serves every
+    head and that needs fewer tiles; the codes, and where they go (dense and through a slot mapping),
+    are the same as head by head."""
+    rng = rng_for(80 + B + H)
+    x = bf16_round(rng.standard_normal((B, H, K)))
+    W = bf16_round(rng.standard_normal((n_w, K, N)))
+    hpw = H // n_w
+    enc = make_encoder(K, N, torch.bfloat16, W, n_w=n_w, hpw=hpw)
+    c = enc.compute_hash(x.cuda(), per_head=True).cpu().numpy()
+    assert c.shape == (B, H, N // 8)
+    for h in range(H):
+        assert_codes_match(c[:, h], x[:, h].float().numpy(), W[h // hpw].float().numpy())
+    # the same rows through the paged store, two dropped
+    NB, BS = 5, 16
+    slots = rng.permutation(NB * BS)[:B].astype(np.int64)
+    slots[0] = -1
+    if B > 2:
+        slots[2] = NB * BS + 3
+    cache = torch.full((NB, BS, H, N // 8), 0xAB, dtype=torch.uint8, device="cuda")
+    enc.compute_hash_and_cache(x.cuda(), torch.from_numpy(slots).cuda(), cache, block_size=BS)
+    expect = np.full((NB, BS, H, N // 32), 0xABABABAB, np.uint32)
+    c_api.code_scatter(np.ascontiguousarray(c).view(np.uint32), slots, expect, BS)
+    assert np.array_equal(cache.cpu().numpy().view(np.uint32), expect)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("slot_dtype", [torch.int32, torch.int64])
 def test_compute_hash_and_cache(dtype, slot_dtype):

@@ -1367,7 +1367,20 @@ struct EncJobs {
     int waves0;  // waves of job 0; waves >= waves0 belong to job 1
 };
 
-// One wave's tile of job `a`: wave index wv counts (row tile, head, 32-column tile), columns fastest.
+// With one projection for all heads and fewer than 32 tokens (a decode step's queries: 16 tokens x
+// 64 heads), a tile of 32 consecutive tokens of ONE head is mostly empty and every head's waves
+// fetch the same columns of W again.  The rows of a tile are then 32 consecutive (token, head)
+// pairs instead: half the waves, full tiles.
+__host__ __device__ __forceinline__ bool small_rows_are_pairs(const EncArgs& a)
+{
+    if (a.H <= 1 || !(a.n_w == 1 || a.heads_per_w <= 0 || a.heads_per_w >= a.H)) return false;
+    const int64_t by_head = ((a.T + kRowsPerWave - 1) / kRowsPerWave) * a.H;
+    const int64_t by_pair = (a.T * a.H + kRowsPerWave - 1) / kRowsPerWave;
+    return by_pair < by_head;
+}
+
+// One wave's tile of job `a`: wave index wv counts (row tile, head, 32-column tile), columns fastest
+// (row tiles of (token, head) pairs: (row tile, 32-column tile)).
 template <typename V, int KS>
 __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
 {
@@ -1375,16 +1388,27 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
     const int ntiles = a.N / 32;
     const int nt = wv % ntiles;
     wv /= ntiles;
-    const int h = wv % a.H;
-    const int64_t row0 = (int64_t)(wv / a.H) * kRowsPerWave;
-
     const int lane = threadIdx.x;
     const int r = lane & 31, kb = lane >> 5;
-    const uint16_t* wsrc =
-        (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N + nt * 32 + r;
-    int64_t t = row0 + r;
-    const bool row_ok = t < a.T;
-    if (!row_ok) t = a.T - 1;
+    const bool pairs = small_rows_are_pairs(a);
+    int h;          // the lane's head (the wave's, unless the rows are pairs)
+    int64_t t;      // the lane's token
+    bool row_ok;
+    if (pairs) {
+        const int64_t rows = a.T * a.H;
+        int64_t p = (int64_t)wv * kRowsPerWave + r;
+        row_ok = p < rows;
+        if (!row_ok) p = rows - 1;
+        t = p / a.H;
+        h = (int)(p - t * a.H);
+    } else {
+        h = wv % a.H;
+        t = (int64_t)(wv / a.H) * kRowsPerWave + r;
+        row_ok = t < a.T;
+        if (!row_ok) t = a.T - 1;
+    }
+    const int wi = pairs ? weight_index(a, 0) : weight_index(a, h);  // wave-uniform either way
+    const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)wi * K * a.N + nt * 32 + r;
     const uint16_t* xr = (const uint16_t*)a.x + src_offset(a, t, h) + kb * 8;
     // where the row's word goes (a read of the slot mapping): asked for with the operands and
     // looked at after the matrix product - behind it, it is a round trip to memory of its own
@@ -1426,7 +1450,7 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
     if ((reinterpret_cast<uintptr_t>(a.w) & 15) == 0) {
         constexpr int kPatches = (K / 8) * 4;
         constexpr int kIters = (kPatches + 63) / 64;
-        const uint16_t* wslice = (const uint16_t*)a.w + (int64_t)weight_index(a, h) * K * a.N + nt * 32;
+        const uint16_t* wslice = (const uint16_t*)a.w + (int64_t)wi * K * a.N + nt * 32;
         u32x4 row[kIters][8];
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {
@@ -1812,6 +1836,7 @@ int launch_wide(const EncArgs& a, hipStream_t st)
 
 int64_t small_waves(const EncArgs& a)
 {
+    if (small_rows_are_pairs(a)) return ucm::ceil_div(a.T * a.H, kRowsPerWave) * (a.N / 32);
     return ucm::ceil_div(a.T, kRowsPerWave) * a.H * (a.N / 32);
 }
 
