@@ -1369,7 +1369,7 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
     const int j0 = (blockIdx.x * kDotWaves + wid) * RUN;
-    // round 1: the reads that need the kernel arguments only
+    // first round of reads: those that need the kernel arguments only
     const int len = a.lens[b];
     int my_entry;  // lane i: table entry of block j0 + i
     {
@@ -1412,7 +1412,7 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    // round 2: the codes.  A wave stands at its load instructions until the unit's queue has room
+    // second round of reads: the codes.  A wave stands at its load instructions until the unit's queue has room
     // (a unit takes one 1 KiB instruction per 16 cycles and answers at its share of the memory
     // rate), for microseconds when 16 waves ask for 8 KiB each.  Nobody may wait for that: the
     // building wave builds first and requests its codes afterwards, and the weights are handed over
@@ -1657,7 +1657,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
     const int j0 = (blockIdx.x * kStripWaves + wid) * RUN;
-    // round 1: the reads that need the kernel arguments only
+    // first round of reads: those that need the kernel arguments only
     const int len = a.lens[b];
     int my_entry;  // lane i: table entry of block j0 + i
     {
