@@ -998,10 +998,15 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
 // matrix instructions (128 KiB of LDS reads per tile; eight waves of 32 columns read 256 KiB).
 //
 // A wave has its SIMD to itself, so nothing hides what it waits for: the stream of matrix
-// instructions must never stop.  Operand reads run eight k-steps ahead in a ring of registers -
-// never more than 15 LDS operations in flight: the counter the waits are written against has
-// four bits, and with 16 reads ahead the first of a pair of matrix instructions now and then
-// read its operand before it had arrived.  Four tiles are in the ring.  One bare barrier per
+// instructions must never stop.  Operand reads run eight k-steps ahead in a ring of registers
+// (sixteen measured the same).  No operand of a written-out matrix instruction is written by a
+// vector instruction anywhere near it: the compiler inserts the wait states between the two only
+// for matrix instructions it knows.  An earlier form gave the accumulators their start value
+// with 16 v_mov each - which the compiler is free to move down to the first matrix instruction
+// of the next tile - and with sixteen reads ahead that instruction, never the second of its
+// pair, now and then produced wrong sums for a row or two of a tile (426 of 560,000 words);
+// the v_mov are the suspect, the LDS wait counter is not (waits counted against up to 48 reads
+// in flight release exactly when they should).  Four tiles are in the ring.  One bare barrier per
 // tile, in its middle: behind it the next tile is complete in LDS (its reads start with the
 // second half of this tile's matrix instructions, so the stream runs on from tile to tile),
 // everybody is done with the previous tile (its slot takes the tile three ahead, one load
@@ -1039,7 +1044,7 @@ constexpr int kWideAhead = 8;                      // operand reads ahead of the
 constexpr size_t kWideLds = (size_t)kWideRing * kWideSlotBytes + 3 * kWideCodeBytes + kWideMapRing * 256;
 static_assert(kWideSlotBytes % 16 == 0 && kWideTileBytes <= kWideSlotBytes, "ring slot layout");
 static_assert(kWideLds <= 160 * 1024, "ring exceeds the LDS");
-static_assert(kWideAhead + 4 <= 15 && (kWideK / 16) % kWideAhead == 0, "LDS operations in flight; ring index");
+static_assert((kWideK / 16) % kWideAhead == 0, "a tile's k-steps are whole turns of the operand ring");
 
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 
