@@ -1004,9 +1004,11 @@ __global__ __launch_bounds__(kStreamThreads) __attribute__((amdgpu_waves_per_eu(
 // for matrix instructions it knows.  An earlier form gave the accumulators their start value
 // with 16 v_mov each - which the compiler is free to move down to the first matrix instruction
 // of the next tile - and with sixteen reads ahead that instruction, never the second of its
-// pair, now and then produced wrong sums for a row or two of a tile (426 of 560,000 words);
-// the v_mov are the suspect, the LDS wait counter is not (waits counted against up to 48 reads
-// in flight release exactly when they should).  Four tiles are in the ring.  One bare barrier per
+// pair, now and then produced wrong sums for a row or two of a tile (426 of 560,000 words, the
+// same ones in every run); the same form with sixteen idle cycles in front of a tile's first
+// matrix instruction is right.  (The LDS wait counter, the first suspect, is exact: waits
+// counted against up to 48 reads in flight release when they should.)  Four tiles are in the
+// ring.  One bare barrier per
 // tile, in its middle: behind it the next tile is complete in LDS (its reads start with the
 // second half of this tile's matrix instructions, so the stream runs on from tile to tile),
 // everybody is done with the previous tile (its slot takes the tile three ahead, one load
