@@ -299,6 +299,18 @@ def graph_ms(torch, fn, reps=20, replays=5):
     return e0.elapsed_time(e1) / (reps * replays)
 
 
+def rotating(items):
+    """f() -> items[0], items[1], ... in turn: a benchmark call takes a different code cache every time, so
+    that no call finds its codes in the 256 MB last-level cache (the sets rotated over exceed 512 MB)."""
+    state = {"i": 0}
+
+    def nxt():
+        it = items[state["i"] % len(items)]
+        state["i"] += 1
+        return it
+    return nxt
+
+
 def scorer_kernel_us(torch, fn, n=30, with_call=False):
     """Mean duration in microseconds of the block-score dispatch inside fn(): the library attaches
     the two events to that dispatch as its start / stop events (eager launches).  with_call: also
@@ -555,7 +567,7 @@ def plugin_surface_mla(torch, gen):
         "vllm_hash_attention_topk": topk * bs5, "seed": 4}}}
     plugin = GSAOnDevice(cfg, UcmSparseRole.WORKER)
     nb = b5 * ctx5 // bs5
-    R = 4  # 4 x 75 MB of codes: beyond the last-level cache
+    R = 8  # 8 x 75 MB of codes: more than twice the last-level cache
     caches = [torch.randint(-2**31, 2**31 - 1, (nb, bs5, 18), dtype=torch.int32, device="cuda", generator=gen)
               for _ in range(R)]
     tables = [torch.randperm(nb, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1) for _ in range(R)]
@@ -729,7 +741,9 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         ws = torch.empty(_esa_ws(2, 8000), dtype=torch.uint8, device="cuda")
         ms = graph_ms(torch, lambda i: dot_topk(vecs, qv, cand, 3000, ws))
         out["esa_dot_topk"] = {"candidates": 2 * 8000, "dim": 1024, "topk": 3000, "ms": ms,
-                               "gather_GBps": 2 * 8000 * 4096 / ms / 1e6}
+                               "gather_GBps": 2 * 8000 * 4096 / ms / 1e6,
+                               "note": "the same 105 MB of block vectors queried every call, as in the reference's driver "
+                                       "loop: they stay in the 256 MB last-level cache between calls"}
         del vecs
 
         # --- float retrieval (KVStar) ---
@@ -754,7 +768,8 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         lens3 = torch.randint(16384, 131072 + 1, (8,), generator=gen, device="cuda").to(torch.int32)
         nblk3 = (lens3.long() + BS - 1) // BS
         nb3 = int(nblk3.sum())
-        cache3 = codes((nb3, BS, HKV, WD))
+        cache3 = [codes((nb3, BS, HKV, WD)) for _ in range(8)]  # rotated: 8 x 74 MB
+        next3 = rotating(cache3)
         table3 = torch.zeros((8, int(nblk3.max())), dtype=torch.int32, device="cuda")
         perm3 = torch.randperm(nb3, generator=gen, device="cuda").to(torch.int32)
         o = 0
@@ -762,11 +777,11 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
             table3[b, : int(nblk3[b])] = perm3[o:o + int(nblk3[b])]
             o += int(nblk3[b])
         q3 = codes((8, HQ, WD))
-        ms = graph_ms(torch, lambda i: hamming_topk(q3, cache3, table3, lens3, 128))
+        ms = graph_ms(torch, lambda i: hamming_topk(q3, cache3[i % 8], table3, lens3, 128), reps=24)
         tok3 = int(lens3.sum())
         out["config3_ragged_topk128"] = {"tokens": tok3, "ms": ms, "tokens_per_s": tok3 / ms * 1e3,
-                                         "code_GBps": tok3 * HKV * WD * 4 / ms / 1e6,
-                                         **topk_split(torch, lambda: hamming_topk(q3, cache3, table3, lens3, 128), ms,
+                                         "code_GBps": tok3 * HKV * WD * 4 / ms / 1e6, "cache_rotation": 8,
+                                         **topk_split(torch, lambda: hamming_topk(q3, next3(), table3, lens3, 128), ms,
                                                       tok3 * HKV * WD * 4)}
         del cache3, table3
         # config 2's cache with more query heads per KV head (64 / 8- and 128 / 8-head models): bit planes,
@@ -785,25 +800,30 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         del cache2, table2
         # config 5: MLA, one latent head, 128 q heads, 256-bit codes, 16 x 65536 tokens, 64-token blocks, top-128
         b5, ctx5, bs5, wd5 = 16, 65536, 64, 8
-        cache5 = codes((b5 * ctx5 // bs5, bs5, 1, wd5))
+        cache5 = [codes((b5 * ctx5 // bs5, bs5, 1, wd5)) for _ in range(16)]  # rotated: 16 x 33.5 MB
+        next5 = rotating(cache5)
         table5 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
         lens5 = torch.full((b5,), ctx5, dtype=torch.int32, device="cuda")
         q5 = codes((b5, 128, wd5))
-        ms = graph_ms(torch, lambda i: hamming_topk(q5, cache5, table5, lens5, 128))
+        ms = graph_ms(torch, lambda i: hamming_topk(q5, cache5[i % 16], table5, lens5, 128), reps=32)
+        ms_warm = graph_ms(torch, lambda i: hamming_topk(q5, cache5[0], table5, lens5, 128))
         out["config5_mla_topk128"] = {"tokens": b5 * ctx5, "ms": ms, "tokens_per_s": b5 * ctx5 / ms * 1e3,
-                                      "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6,
-                                      **topk_split(torch, lambda: hamming_topk(q5, cache5, table5, lens5, 128), ms,
+                                      "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6, "cache_rotation": 16,
+                                      "ms_same_cache_every_call": ms_warm,
+                                      **topk_split(torch, lambda: hamming_topk(q5, next5(), table5, lens5, 128), ms,
                                                    b5 * ctx5 * wd5 * 4)}
         del cache5, table5
         # the reference's own latent-attention setting: 18-word codes (512 nope + 64 rope bits), 64 query
         # heads after its head reduction (128 heads, reduction 2), same 16 x 65536 tokens
         wd6 = 18
-        cache6 = codes((b5 * ctx5 // bs5, bs5, 1, wd6))
+        cache6 = [codes((b5 * ctx5 // bs5, bs5, 1, wd6)) for _ in range(8)]  # rotated: 8 x 75.5 MB
+        next6 = rotating(cache6)
         table6 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
         q6 = codes((b5, 64, wd6))
-        ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6, table6, lens5, 128))
-        split6 = topk_split(torch, lambda: hamming_topk(q6, cache6, table6, lens5, 128), ms, b5 * ctx5 * wd6 * 4)
-        ms_tok = graph_ms(torch, lambda i: hamming_score(cache6, q6, table6, lens5, ctx5, 0, 0, False), reps=5)
+        ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6[i % 8], table6, lens5, 128), reps=24)
+        ms_warm = graph_ms(torch, lambda i: hamming_topk(q6, cache6[0], table6, lens5, 128))
+        split6 = topk_split(torch, lambda: hamming_topk(q6, next6(), table6, lens5, 128), ms, b5 * ctx5 * wd6 * 4)
+        ms_tok = graph_ms(torch, lambda i: hamming_score(cache6[i % 8], q6, table6, lens5, ctx5, 0, 0, False), reps=8)
         # the whole decode step of that layout in one native call: both parts of 16 new keys into the cache,
         # both parts of the 16 x 64 query rows hashed, score, select
         from ucm_amd.sparse import SparseDecodeStepMLA
@@ -812,27 +832,28 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
                                   sink_token=bs5, recent_token=4 * bs5, return_physical=True)
         kn6, kr6, qn6, qr6 = bf(b5, 512), bf(b5, 64), bf(b5, 64, 512), bf(b5, 64, 64)
         slots6 = (table6[:, -1].to(torch.int64) * bs5 + bs5 - 1)
-        cache6v = cache6.view(cache6.shape[0], bs5, wd6)
-        ms_step = graph_ms(torch, lambda i: stm.step(kn6, kr6, slots6, qn6, qr6, cache6v, table6, lens5))
+        cache6v = [c.view(c.shape[0], bs5, wd6) for c in cache6]
+        ms_step = graph_ms(torch, lambda i: stm.step(kn6, kr6, slots6, qn6, qr6, cache6v[i % 8], table6, lens5), reps=24)
         out["mla_576bit_64heads"] = {"tokens": b5 * ctx5, "topk128_ms": ms, "token_scores_ms": ms_tok,
-                                     "decode_step_ms": ms_step,
+                                     "decode_step_ms": ms_step, "cache_rotation": 8,
+                                     "topk128_ms_same_cache_every_call": ms_warm,
                                      "tokens_per_s": b5 * ctx5 / ms * 1e3,
                                      "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6, **split6}
         del cache6, table6
     if "token_scores" in legs:
         # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
-        cache2 = codes((NB, BS, HKV, WD))
+        cache2 = [codes((NB, BS, HKV, WD)) for _ in range(4)]  # rotated: 4 x 134 MB
         table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, NBLK)
         lens2 = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
         q2 = codes((B, HQ, WD))
-        ms = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, False), reps=10)
+        ms = graph_ms(torch, lambda i: hamming_score(cache2[i % 4], q2, table2, lens2, CTX, 0, 0, False), reps=12)
         byt = B * CTX * HKV * (WD * 4 + 2)
         # the reference's own GQA call reduces over the KV heads (hamming_topk.py:33): one fp16 row per request
-        ms_red = graph_ms(torch, lambda i: hamming_score(cache2, q2, table2, lens2, CTX, 0, 0, True), reps=10)
+        ms_red = graph_ms(torch, lambda i: hamming_score(cache2[i % 4], q2, table2, lens2, CTX, 0, 0, True), reps=12)
         byt_red = B * CTX * (HKV * WD * 4 + 2)
         out["token_scores_config2"] = {"tokens": B * CTX, "ms": ms, "tokens_per_s": B * CTX / ms * 1e3,
                                        "hbm_GBps": byt / ms / 1e6, "hbm_frac": byt / ms / 1e6 / HBM_PEAK_GBPS,
-                                       "reduce_kvhead_ms": ms_red,
+                                       "reduce_kvhead_ms": ms_red, "cache_rotation": 4,
                                        "reduce_kvhead_hbm_frac": byt_red / ms_red / 1e6 / HBM_PEAK_GBPS}
         del cache2, table2
 
