@@ -683,6 +683,10 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
     from ucm_amd.trans import Device
 
     out = {}
+
+    def codes(shape):
+        return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device="cuda", generator=gen)
+
     if "encoder" in legs:
         # --- encoder: one request's keys (32768 x 8 rows of 128) per call ---
         keys = torch.randn((CTX, HKV, D), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
@@ -761,9 +765,6 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         #     timed here on random codes: top-k = score + select; the per-token scorer alone ---
         from ucm_amd.sparse import hamming_score, hamming_topk
 
-        def codes(shape):
-            return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device="cuda", generator=gen)
-
         # config 3: batch 8, lengths uniform in [16384, 131072], 128-bit codes, top-128
         lens3 = torch.randint(16384, 131072 + 1, (8,), generator=gen, device="cuda").to(torch.int32)
         nblk3 = (lens3.long() + BS - 1) // BS
@@ -841,6 +842,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
                                      "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6, **split6}
         del cache6, table6
     if "token_scores" in legs:
+        from ucm_amd.sparse import hamming_score
         # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
         cache2 = [codes((NB, BS, HKV, WD)) for _ in range(4)]  # rotated: 4 x 134 MB
         table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, NBLK)

@@ -81,7 +81,9 @@ def test_topk_shape_takes_its_kernels_and_matches_the_checker(name):
 
 # (B, Hq, Hkv, Wd, BS, lens, kernels launched)
 SCORE_SHAPES = {
-    "config2_two_requests": (2, 32, 8, 4, 128, [32768, 30000], "token_score_fast<4>"),
+    "config2_two_requests": (2, 32, 8, 4, 128, [32768, 30000], "token_score_one<4,8>"),
+    "config2_codes_in_64_token_blocks": (2, 32, 8, 4, 64, [16384, 9000], "token_score_fast<4>"),
+    "config2_codes_two_words_wider": (2, 16, 8, 8, 128, [8192, 3000], "token_score_fast<2>"),
     "one_head_6_words": (2, 2, 1, 6, 32, [2048, 700], "token_score_pairs<1,2>"),
     "one_head_6_words_16_query_heads": (2, 16, 1, 6, 32, [2048, 700], "plane_kernel+token_score_pairs<0,5>"),
     "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], "token_score_lanes<9,1,1>"),

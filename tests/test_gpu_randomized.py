@@ -258,6 +258,47 @@ def test_per_token_scores_random_configurations(seed):
             assert np.array_equal(h, expect), what
 
 
+@pytest.mark.parametrize("seed", [55, 56])
+def test_per_token_scores_16_kib_blocks_random_configurations(seed):
+    """The per-token kernel of the hot shape (128-bit codes, blocks of exactly 16 KiB, row length a multiple
+    of four) against the checker: lengths that end inside a block, unusable table entries, sink and recent
+    windows that cut blocks, rows that end before or reach past the last table entry, both output types,
+    with and without the KV-head reduction."""
+    from ucm_amd import _lib
+    from ucm_amd.sparse import hamming_score
+
+    rng = rng_for(seed)
+    for it in range(60):
+        B = int(rng.integers(1, 5))
+        Hkv, BS = (8, 128) if rng.integers(0, 2) else (4, 256)
+        G = int(rng.choice([1, 2, 4, 8]))
+        mb = int(rng.integers(1, 24))
+        NB = B * mb + 3
+        kc = rng.integers(0, 2**32, size=(NB, BS, Hkv, 4), dtype=np.uint32)
+        q = rng.integers(0, 2**32, size=(B, Hkv * G, 4), dtype=np.uint32)
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32)
+        if rng.integers(0, 3) == 0:
+            table[rng.integers(0, B), rng.integers(0, mb)] = NB + 7 if rng.integers(0, 2) else -1
+        lens = rng.integers(0, mb * BS + 1, size=B).astype(np.int32)
+        if it % 7 == 0:
+            lens[0] = mb * BS
+        msl = max(4, mb * BS - 4 * int(rng.integers(0, BS // 4)))
+        if it % 5 == 0:
+            msl = mb * BS + 4 * int(rng.integers(1, BS))  # the row reaches past the last table entry
+        sink, recent = int(rng.integers(0, 3 * BS)), int(rng.integers(0, 3 * BS))
+        red = bool(rng.integers(0, 3) == 0)
+        what = dict(B=B, Hkv=Hkv, G=G, BS=BS, mb=mb, msl=msl, sink=sink, recent=recent, red=red, lens=lens.tolist())
+        o = c_api.hamming_score(q, kc, table, lens, msl, sink, recent, red)
+        args = (torch.from_numpy(kc.view(np.int32)).cuda(), torch.from_numpy(q.view(np.int32)).cuda()[:, None],
+                torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda(), msl, sink, recent, red)
+        g = hamming_score(*args, out_int32=True).cpu().numpy()
+        assert _lib.last_dispatch() == "token_score_one<%d,%d>" % (G, Hkv), what
+        assert np.array_equal(g, o), what
+        h = hamming_score(*args).cpu().numpy()
+        expect = np.where(o == c_api.INF, np.inf, o.astype(np.float64)).astype(np.float16)
+        assert np.array_equal(h, expect), what
+
+
 @pytest.mark.parametrize("seed", [61, 62])
 def test_one_kv_head_random_configurations(seed):
     """One KV head (the latent-attention layout) with even and odd code widths and up to 255 query

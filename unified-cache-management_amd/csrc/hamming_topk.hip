@@ -3409,8 +3409,8 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t, int tb
             tt = tt < TT ? tt : TT - 1;
             const int64_t pb = tb_shift ? pbs[tt >> bs_shift] : pb0;
             const int tok = tb_shift ? (tt & (a.BS - 1)) : tt;
-            kw[u] = *reinterpret_cast<const u32x4*>(
-                a.kc + (pb < 0 ? 0 : pb) * a.ks_block + (int64_t)tok * a.ks_token + sub * 4);
+            kw[u] = code_load(reinterpret_cast<const u32x4*>(
+                a.kc + (pb < 0 ? 0 : pb) * a.ks_block + (int64_t)tok * a.ks_token + sub * 4));
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -3428,6 +3428,59 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t, int tb
     // request holds the minimum over the heads; the sums are exact here, so the minimum of
     // the integers is the minimum of the reference's half values
     const int rows_out = t.reduce_heads ? 1 : a.Hkv;
+    // Four positions per thread and one 8- or 16-byte store where the rows allow it (block size and
+    // row length multiples of four, aligned output): a quarter of the store instructions, and all
+    // threads of the workgroup take part instead of one thread per token and head in turn.
+    const bool by_four = ((a.BS | t.max_seq_len) & 3) == 0 && (reinterpret_cast<uintptr_t>(t.out) & 15) == 0;
+    if (by_four) {
+        const int TQ = TT >> 2;
+        for (int i = threadIdx.x; i < rows_out * TQ; i += kThreads) {
+            const int hh = i / TQ, tt = (i - hh * TQ) << 2;
+            const int pos = j0 * a.BS + tt;
+            if (pos >= t.max_seq_len) continue;
+            u32x4 d = *reinterpret_cast<const u32x4*>(dyn + hh * TT + tt);
+            if (t.reduce_heads)
+                for (int h2 = 1; h2 < a.Hkv; ++h2) {
+                    const u32x4 o2 = *reinterpret_cast<const u32x4*>(dyn + h2 * TT + tt);
+                    d.x = o2.x < d.x ? o2.x : d.x;
+                    d.y = o2.y < d.y ? o2.y : d.y;
+                    d.z = o2.z < d.z ? o2.z : d.z;
+                    d.w = o2.w < d.w ? o2.w : d.w;
+                }
+            const bool have = (tb_shift ? pbs[tt >> bs_shift] : pb0) >= 0;
+            const int64_t o = ((int64_t)b * rows_out + hh) * t.max_seq_len + pos;
+            const uint32_t dv[4] = {d.x, d.y, d.z, d.w};
+            if (t.out_is_f16) {
+                uint16_t hv[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int pe = pos + e;
+                    const bool is_inf = pe >= len;
+                    const bool keep = (pe < a.sink) || (pe >= len - a.recent && pe < len);
+                    const _Float16 v = is_inf ? (_Float16)__builtin_inff()
+                                              : (keep ? (_Float16)0.0f : (have ? (_Float16)(float)(int)dv[e] : (_Float16)__builtin_inff()));
+                    __builtin_memcpy(&hv[e], &v, 2);
+                }
+                u32x2 w;
+                w.x = hv[0] | ((uint32_t)hv[1] << 16);
+                w.y = hv[2] | ((uint32_t)hv[3] << 16);
+                *reinterpret_cast<u32x2*>((uint16_t*)t.out + o) = w;
+            } else {
+                u32x4 w;
+                uint32_t iv[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int pe = pos + e;
+                    const bool is_inf = pe >= len;
+                    const bool keep = (pe < a.sink) || (pe >= len - a.recent && pe < len);
+                    iv[e] = (uint32_t)(is_inf ? kInf : (keep ? 0 : (have ? (int)dv[e] : kInf)));
+                }
+                w.x = iv[0]; w.y = iv[1]; w.z = iv[2]; w.w = iv[3];
+                *reinterpret_cast<u32x4*>((int32_t*)t.out + o) = w;
+            }
+        }
+        return;
+    }
     for (int hh = 0; hh < rows_out; ++hh) {
         for (int tt = threadIdx.x; tt < TT; tt += kThreads) {
             const int pos = j0 * a.BS + tt;
@@ -3453,6 +3506,133 @@ __global__ __launch_bounds__(kThreads) void token_score_fast(TokenArgs t, int tb
             }
         }
     }
+}
+
+// Per-token scores of the hot shape: 128-bit codes, HKV heads, a block of exactly 16 KiB
+// (1024 / HKV tokens), row length a multiple of four.  One workgroup per (request, logical block),
+// laid out as block_score_one: lane l of wave w reads pieces (w + 4u) * 64 + l, u = 0..3 - 1 KiB
+// per wave and instruction, all four before anything waits - and owns head l % HKV, whose G query
+// codes stay in registers.  The request's scalars are read together at the top, without branches
+// between them.  A distance goes to LDS once (row stride padded so that the 64 lanes of a store
+// fall into 64 banks) and leaves as four positions per thread in one 8- or 16-byte store.  Every
+// sum is an integer that fp16 holds exactly (G * 128 <= 2048), so the piecewise half-precision
+// accumulation of paged_ham_dist_mla.cu:204-241 equals the exact sum.
+template <int G, int HKV>
+__global__ __launch_bounds__(kThreads) void token_score_one(TokenArgs t)
+{
+    constexpr int BSC = 1024 / HKV;               // tokens of a block
+    constexpr int PAD = 64 / HKV < 4 ? 4 : 64 / HKV;
+    constexpr int STRIDE = BSC + PAD;             // words between the rows of two heads
+    constexpr int TQ = BSC / 4;                   // groups of four positions per head
+    __shared__ __attribute__((aligned(16))) uint32_t dist[HKV * STRIDE];
+    const ScoreArgs& a = t.s;
+    const int b = blockIdx.y, j = blockIdx.x;
+    const int lane = lane_id();
+    const int wid = wave_id();
+    const int h = lane % HKV;
+
+    // the grid covers max_seq_len, which may reach past the table's row: such a block reads the
+    // row's last entry and does not use it
+    const int jt = j < a.max_blocks ? j : a.max_blocks - 1;
+    const uintptr_t has_table = a.table ? ~(uintptr_t)0 : 0;
+    const uintptr_t ea = (reinterpret_cast<uintptr_t>(a.table + ((int64_t)b * a.table_stride + jt)) & has_table) |
+                         (reinterpret_cast<uintptr_t>(a.lens + b) & ~has_table);
+    int entry = *reinterpret_cast<const int32_t*>(ea);
+    int len = a.lens[b];
+    int64_t ks_block0 = a.ks_block, nb0 = a.NB, q_stride_b0 = a.q_stride_b;
+    asm volatile("" : "+s"(entry), "+s"(len), "+s"(ks_block0), "+s"(nb0), "+s"(q_stride_b0));
+
+    uint32_t qr[G][4];
+    {
+        const uint32_t* qp = a.q + b * q_stride_b0 + (int64_t)h * G * a.q_stride_h;
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qr[g][w] = qp[g * a.q_stride_h + w];
+    }
+    int64_t pb = ((int64_t)entry & (int64_t)has_table) | (((int64_t)b * a.max_blocks + j) & ~(int64_t)has_table);
+    if (j >= a.max_blocks || pb < 0 || pb >= nb0) pb = -1;
+    const int pos0 = j * BSC;
+    const bool reads = pb >= 0 && pos0 < len;
+    if (reads) {
+        const u32x4* base = reinterpret_cast<const u32x4*>(a.kc + pb * ks_block0) + lane;
+        u32x4 kv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) kv[u] = code_load(base + ((wid + 4 * u) << 6));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            int d = __popc(kv[u].x ^ qr[0][0]);
+            d = popc_add(kv[u].y ^ qr[0][1], d);
+            d = popc_add(kv[u].z ^ qr[0][2], d);
+            d = popc_add(kv[u].w ^ qr[0][3], d);
+#pragma unroll
+            for (int g = 1; g < G; ++g) {
+                d = popc_add(kv[u].x ^ qr[g][0], d);
+                d = popc_add(kv[u].y ^ qr[g][1], d);
+                d = popc_add(kv[u].z ^ qr[g][2], d);
+                d = popc_add(kv[u].w ^ qr[g][3], d);
+            }
+            const int tok = (((wid + 4 * u) << 6) + lane) / HKV;
+            dist[h * STRIDE + tok] = (uint32_t)d;
+        }
+    }
+    __syncthreads();
+    // with the KV-head reduction (the reference's GQA call, hamming_topk.py:33) one row per request
+    // holds the minimum over the heads
+    const int rows_out = t.reduce_heads ? 1 : HKV;
+    // a block between the sink and the recent window, all of it below the length: plain distances
+    const bool interior = reads && pos0 >= a.sink && pos0 + BSC <= len - a.recent;
+    for (int i = threadIdx.x; i < rows_out * TQ; i += kThreads) {
+        const int hh = i / TQ, tt = (i % TQ) << 2;
+        const int pos = pos0 + tt;
+        if (pos >= t.max_seq_len) continue;
+        u32x4 d = (u32x4)(0u);
+        if (reads) {
+            d = *reinterpret_cast<const u32x4*>(dist + hh * STRIDE + tt);
+            if (t.reduce_heads) {
+#pragma unroll
+                for (int h2 = 1; h2 < HKV; ++h2) {
+                    const u32x4 o2 = *reinterpret_cast<const u32x4*>(dist + h2 * STRIDE + tt);
+                    d.x = o2.x < d.x ? o2.x : d.x;
+                    d.y = o2.y < d.y ? o2.y : d.y;
+                    d.z = o2.z < d.z ? o2.z : d.z;
+                    d.w = o2.w < d.w ? o2.w : d.w;
+                }
+            }
+        }
+        const uint32_t dv[4] = {d.x, d.y, d.z, d.w};
+        const int64_t o = ((int64_t)b * rows_out + hh) * t.max_seq_len + pos;
+        if (t.out_is_f16) {
+            uint16_t hv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int pe = pos + e;
+                const bool none = !interior && (pe >= len || (!reads && !(pe < a.sink) && !(pe >= len - a.recent)));
+                const bool keep = !interior && ((pe < a.sink) || (pe >= len - a.recent));
+                const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : (_Float16)(float)(int)dv[e]);
+                __builtin_memcpy(&hv[e], &v, 2);
+            }
+            u32x2 w;
+            w.x = hv[0] | ((uint32_t)hv[1] << 16);
+            w.y = hv[2] | ((uint32_t)hv[3] << 16);
+            *reinterpret_cast<u32x2*>((uint16_t*)t.out + o) = w;
+        } else {
+            uint32_t iv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int pe = pos + e;
+                const bool none = !interior && (pe >= len || (!reads && !(pe < a.sink) && !(pe >= len - a.recent)));
+                const bool keep = !interior && ((pe < a.sink) || (pe >= len - a.recent));
+                iv[e] = (uint32_t)(none ? kInf : (keep ? 0 : (int)dv[e]));
+            }
+            u32x4 w;
+            w.x = iv[0]; w.y = iv[1]; w.z = iv[2]; w.w = iv[3];
+            *reinterpret_cast<u32x4*>((int32_t*)t.out + o) = w;
+        }
+    }
+    // (Streaming stores measured against these plain ones at 32 x 32,768 tokens: 0.4 us less with all
+    // heads written, 16.8 MB, and 1.5 us more with the one reduced row; plain stores also leave the
+    // scores in the cache for the selection that reads them next.)
 }
 
 // Per-token scores for the 8-byte-piece layout (one KV head, even code width).  A lane's piece
@@ -3729,6 +3909,23 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
                       ks_block % 4 == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 &&
                       (G == 1 || G == 2 || G == 4 || G == 8) && (int64_t)G * Wd * 32 <= 2048 &&
                       (int64_t)BS * Hkv * 4 <= 48 * 1024 && ucm::ceil_div(max_seq_len, BS) <= 0x7fffffff;
+    if (fast && Wd == 4 && (Hkv == 4 || Hkv == 8) && (int64_t)BS * Hkv == 1024 && max_seq_len % 4 == 0 &&
+        (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        const dim3 ogrid((unsigned)ucm::ceil_div(max_seq_len, BS), (unsigned)B);
+        hipStream_t st = (hipStream_t)stream;
+        note_score("token_score_one", G, Hkv);
+#define UCM_TOKEN_ONE(GG)                                                                      \
+    do {                                                                                       \
+        if (Hkv == 8) hipLaunchKernelGGL((token_score_one<GG, 8>), ogrid, dim3(kThreads), 0, st, t); \
+        else hipLaunchKernelGGL((token_score_one<GG, 4>), ogrid, dim3(kThreads), 0, st, t);      \
+    } while (0)
+        if (G == 1) UCM_TOKEN_ONE(1);
+        else if (G == 2) UCM_TOKEN_ONE(2);
+        else if (G == 4) UCM_TOKEN_ONE(4);
+        else UCM_TOKEN_ONE(8);
+#undef UCM_TOKEN_ONE
+        return ucm::launch_status("token_score_one");
+    }
     if (fast) {
         // small blocks (power-of-two sizes): several per workgroup, until it has at least 128
         // tokens and 16 KiB of codes to read
