@@ -684,7 +684,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
 
     out = {}
 
-    def codes(shape):
+    def rand_codes(shape):
         return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device="cuda", generator=gen)
 
     if "encoder" in legs:
@@ -769,7 +769,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         lens3 = torch.randint(16384, 131072 + 1, (8,), generator=gen, device="cuda").to(torch.int32)
         nblk3 = (lens3.long() + BS - 1) // BS
         nb3 = int(nblk3.sum())
-        cache3 = [codes((nb3, BS, HKV, WD)) for _ in range(8)]  # rotated: 8 x 74 MB
+        cache3 = [rand_codes((nb3, BS, HKV, WD)) for _ in range(8)]  # rotated: 8 x 74 MB
         next3 = rotating(cache3)
         table3 = torch.zeros((8, int(nblk3.max())), dtype=torch.int32, device="cuda")
         perm3 = torch.randperm(nb3, generator=gen, device="cuda").to(torch.int32)
@@ -777,7 +777,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         for b in range(8):
             table3[b, : int(nblk3[b])] = perm3[o:o + int(nblk3[b])]
             o += int(nblk3[b])
-        q3 = codes((8, HQ, WD))
+        q3 = rand_codes((8, HQ, WD))
         ms = graph_ms(torch, lambda i: hamming_topk(q3, cache3[i % 8], table3, lens3, 128), reps=24)
         tok3 = int(lens3.sum())
         out["config3_ragged_topk128"] = {"tokens": tok3, "ms": ms, "tokens_per_s": tok3 / ms * 1e3,
@@ -787,12 +787,12 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         del cache3, table3
         # config 2's cache with more query heads per KV head (64 / 8- and 128 / 8-head models): bit planes,
         # four of them up to 15 query heads per KV head, five up to 31
-        cache2 = [codes((NB, BS, HKV, WD)) for _ in range(3)]  # rotated: 3 x 128 MiB exceed the last-level cache
+        cache2 = [rand_codes((NB, BS, HKV, WD)) for _ in range(3)]  # rotated: 3 x 128 MiB exceed the last-level cache
         table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, -1)
         lens2 = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
         more = {}
         for hq in (64, 128):
-            q2 = codes((B, hq, WD))
+            q2 = rand_codes((B, hq, WD))
             ms2 = graph_ms(torch, lambda i: hamming_topk(q2, cache2[i % 3], table2, lens2, 64), reps=18)
             more["%d_query_heads" % hq] = {"ms": ms2, "tokens_per_s": B * CTX / ms2 * 1e3,
                                            "hbm_frac_operator": B * CTX * HKV * WD * 4 / ms2 / 1e6 / HBM_PEAK_GBPS,
@@ -801,11 +801,11 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         del cache2, table2
         # config 5: MLA, one latent head, 128 q heads, 256-bit codes, 16 x 65536 tokens, 64-token blocks, top-128
         b5, ctx5, bs5, wd5 = 16, 65536, 64, 8
-        cache5 = [codes((b5 * ctx5 // bs5, bs5, 1, wd5)) for _ in range(16)]  # rotated: 16 x 33.5 MB
+        cache5 = [rand_codes((b5 * ctx5 // bs5, bs5, 1, wd5)) for _ in range(16)]  # rotated: 16 x 33.5 MB
         next5 = rotating(cache5)
         table5 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
         lens5 = torch.full((b5,), ctx5, dtype=torch.int32, device="cuda")
-        q5 = codes((b5, 128, wd5))
+        q5 = rand_codes((b5, 128, wd5))
         ms = graph_ms(torch, lambda i: hamming_topk(q5, cache5[i % 16], table5, lens5, 128), reps=32)
         ms_warm = graph_ms(torch, lambda i: hamming_topk(q5, cache5[0], table5, lens5, 128))
         out["config5_mla_topk128"] = {"tokens": b5 * ctx5, "ms": ms, "tokens_per_s": b5 * ctx5 / ms * 1e3,
@@ -817,10 +817,10 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         # the reference's own latent-attention setting: 18-word codes (512 nope + 64 rope bits), 64 query
         # heads after its head reduction (128 heads, reduction 2), same 16 x 65536 tokens
         wd6 = 18
-        cache6 = [codes((b5 * ctx5 // bs5, bs5, 1, wd6)) for _ in range(8)]  # rotated: 8 x 75.5 MB
+        cache6 = [rand_codes((b5 * ctx5 // bs5, bs5, 1, wd6)) for _ in range(8)]  # rotated: 8 x 75.5 MB
         next6 = rotating(cache6)
         table6 = torch.randperm(b5 * ctx5 // bs5, generator=gen, device="cuda").to(torch.int32).reshape(b5, -1)
-        q6 = codes((b5, 64, wd6))
+        q6 = rand_codes((b5, 64, wd6))
         ms = graph_ms(torch, lambda i: hamming_topk(q6, cache6[i % 8], table6, lens5, 128), reps=24)
         ms_warm = graph_ms(torch, lambda i: hamming_topk(q6, cache6[0], table6, lens5, 128))
         split6 = topk_split(torch, lambda: hamming_topk(q6, next6(), table6, lens5, 128), ms, b5 * ctx5 * wd6 * 4)
@@ -844,10 +844,10 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
     if "token_scores" in legs:
         from ucm_amd.sparse import hamming_score
         # per-token scorer (the reference kernel's own output: fp16 distance per token and KV head), config 2 shape
-        cache2 = [codes((NB, BS, HKV, WD)) for _ in range(4)]  # rotated: 4 x 134 MB
+        cache2 = [rand_codes((NB, BS, HKV, WD)) for _ in range(4)]  # rotated: 4 x 134 MB
         table2 = torch.randperm(NB, generator=gen, device="cuda").to(torch.int32).reshape(B, NBLK)
         lens2 = torch.full((B,), CTX, dtype=torch.int32, device="cuda")
-        q2 = codes((B, HQ, WD))
+        q2 = rand_codes((B, HQ, WD))
         ms = graph_ms(torch, lambda i: hamming_score(cache2[i % 4], q2, table2, lens2, CTX, 0, 0, False), reps=12)
         byt = B * CTX * HKV * (WD * 4 + 2)
         # the reference's own GQA call reduces over the KV heads (hamming_topk.py:33): one fp16 row per request
