@@ -1386,16 +1386,25 @@ __host__ __device__ __forceinline__ bool small_rows_are_pairs(const EncArgs& a)
     return by_pair < by_head;
 }
 
-// One wave's tile of job `a`: wave index wv counts (row tile, head, 32-column tile), columns fastest
-// (row tiles of (token, head) pairs: (row tile, 32-column tile)).
-template <typename V, int KS>
+// One tile of job `a`: tile index wv counts (row tile, head, 32-column tile), columns fastest
+// (row tiles of (token, head) pairs: (row tile, 32-column tile)).  SPLIT = 1: one wave per tile.
+// SPLIT = 4 (rows of 256 and 512 values): the four waves of a workgroup take a quarter of the
+// row's k-steps each and the partial sums meet in LDS - everything a wave does before its first
+// matrix instruction (32 + 32 loads of 16 bytes per lane, 128 permutes, the LDS transpose at
+// K = 512) is one chain, and a quarter of it per wave is a quarter of the chain.
+template <typename V, int KS, int SPLIT = 1>
 __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
 {
-    constexpr int K = KS * 16;
+    static_assert(KS % SPLIT == 0, "the row's k-steps divide evenly over the waves of a tile");
+    constexpr int K = KS * 16;        // the row's width: what separates two projection matrices
+    constexpr int KSL = KS / SPLIT;   // k-steps of this wave's slice
+    constexpr int KL = KSL * 16;
+    const int slice = SPLIT > 1 ? (int)(threadIdx.x >> 6) : 0;
+    const int k0 = slice * KL;
     const int ntiles = a.N / 32;
     const int nt = wv % ntiles;
     wv /= ntiles;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63;
     const int r = lane & 31, kb = lane >> 5;
     const bool pairs = small_rows_are_pairs(a);
     int h;          // the lane's head (the wave's, unless the rows are pairs)
@@ -1415,16 +1424,18 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
         if (!row_ok) t = a.T - 1;
     }
     const int wi = pairs ? weight_index(a, 0) : weight_index(a, h);  // wave-uniform either way
-    const uint16_t* wsrc = (const uint16_t*)a.w + (int64_t)wi * K * a.N + nt * 32 + r;
-    const uint16_t* xr = (const uint16_t*)a.x + src_offset(a, t, h) + kb * 8;
+    const uint16_t* wsrc = (const uint16_t*)a.w + ((int64_t)wi * K + k0) * a.N + nt * 32 + r;
+    const uint16_t* xr = (const uint16_t*)a.x + src_offset(a, t, h) + k0 + kb * 8;
     // where the row's word goes (a read of the slot mapping): asked for with the operands and
     // looked at after the matrix product - behind it, it is a round trip to memory of its own
     const RawSlot raw = fetch_slot_flat(a, t);
 
-    // K = 512 holds 128 + 256 operand registers: one wave per SIMD, which is all a launch of
-    // this kernel has anyway
-    V av[KS];
-    uint16_t bw[KS][8];
+    // A wave holds its slice's operands in registers (K = 512 split four ways: 32 + 32, with the
+    // patches on their way 125 in all, so that four workgroups fit a compute unit: with two, the
+    // 594 tiles of a latent-attention step ran as 512 and then 82, and the launch took twice a
+    // tile's time).
+    V av[KSL];
+    uint16_t bw[KSL][8];
     if (a.gmean > 1) {
         // fp32 sum of the group's rows in order, times 1/G, rounded to the input type.  Groups of
         // 2, 4 and 8 rows are written out: a load inside a loop of run-time length is waited for
@@ -1433,9 +1444,10 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
         const float inv = 1.0f / (float)a.gmean;
         auto mean_rows = [&](auto gc) __attribute__((always_inline)) {
             constexpr int G = decltype(gc)::value;
-            constexpr int CH = KS * G > 64 ? 64 / G : KS;  // k-steps whose loads go out together
+            constexpr int kInFlight = SPLIT > 1 ? 16 : 64;  // a split tile's waves keep within a third of the registers
+            constexpr int CH = KSL * G > kInFlight ? kInFlight / G : KSL;  // k-steps whose loads go out together
 #pragma unroll
-            for (int ks0 = 0; ks0 < KS; ks0 += CH) {
+            for (int ks0 = 0; ks0 < KSL; ks0 += CH) {
                 V v[CH][G];
 #pragma unroll
                 for (int c = 0; c < CH; ++c)
@@ -1463,7 +1475,7 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
         else if (a.gmean == 8) mean_rows(std::integral_constant<int, 8>{});
         else {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
+            for (int ks = 0; ks < KSL; ++ks) {
                 float sum[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) sum[i] = 0.0f;
@@ -1480,19 +1492,20 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
         }
     } else {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
+        for (int ks = 0; ks < KSL; ++ks) av[ks] = *reinterpret_cast<const V*>(xr + ks * 16);
     }
     // The wave's 32 columns of W in operand layout (8 consecutive k of one column per lane and
     // k-step).  16-byte aligned weights: lanes fetch 8 x 8 patches (eight 16-byte rows each),
     // transpose them in registers and pass them through LDS - K / 16 loads per lane; fetching the
     // operands directly takes eight 2-byte loads per k-step (K / 2 per lane: 256 at K = 512).
-    constexpr int KP = K + kPad;
-    __shared__ __align__(16) uint16_t wt[32 * KP];
-    V bv[KS];
+    constexpr int KP = KL + kPad;
+    __shared__ __align__(16) uint16_t wt_all[SPLIT][32 * KP];
+    uint16_t* wt = wt_all[slice];
+    V bv[KSL];
     if ((reinterpret_cast<uintptr_t>(a.w) & 15) == 0) {
-        constexpr int kPatches = (K / 8) * 4;
+        constexpr int kPatches = (KL / 8) * 4;
         constexpr int kIters = (kPatches + 63) / 64;
-        const uint16_t* wslice = (const uint16_t*)a.w + (int64_t)wi * K * a.N + nt * 32;
+        const uint16_t* wslice = (const uint16_t*)a.w + ((int64_t)wi * K + k0) * a.N + nt * 32;
         u32x4 row[kIters][8];
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {
@@ -1518,10 +1531,10 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
         }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) bv[ks] = *reinterpret_cast<const V*>(wt + r * KP + ks * 16 + kb * 8);
+        for (int ks = 0; ks < KSL; ++ks) bv[ks] = *reinterpret_cast<const V*>(wt + r * KP + ks * 16 + kb * 8);
     } else {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
+        for (int ks = 0; ks < KSL; ++ks) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) bw[ks][i] = wsrc[(int64_t)(ks * 16 + kb * 8 + i) * a.N];
             __builtin_memcpy(&bv[ks], bw[ks], 16);
@@ -1530,7 +1543,30 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
 
     f32x16 acc = acc_start();
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) acc = Mfma<V>::run(bv[ks], av[ks], acc);
+    for (int ks = 0; ks < KSL; ++ks) acc = Mfma<V>::run(bv[ks], av[ks], acc);
+
+    if (SPLIT > 1) {
+        // the slices' sums meet in wave 0 in slice order.  Every slice starts from the same small
+        // negative number, which vanishes in any sum that is not exactly zero and keeps a row of
+        // zeros negative; NaN passes through the additions.
+        // A wave's partial sums go where its slice of W was: its own reads of that region are
+        // behind it (LDS operations of a wave complete in order), and nobody else touches it
+        // before the barrier.
+        static_assert(sizeof(wt_all[0]) >= 16 * 64 * sizeof(float), "a slice of W makes room for one wave's sums");
+        float* part = reinterpret_cast<float*>(wt);
+        if (slice > 0) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) part[i * 64 + lane] = acc[i];
+        }
+        __syncthreads();
+        if (slice > 0) return;
+#pragma unroll
+        for (int sl = 1; sl < SPLIT; ++sl) {
+            const float* other = reinterpret_cast<const float*>(wt_all[sl]);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[i] += other[i * 64 + lane];
+        }
+    }
     const uint32_t half = pack_half(acc);
     const uint32_t word = join_halves(kb ? half << 4 : half);
     if (row_ok && lane < 32) {
@@ -1555,13 +1591,16 @@ __device__ __forceinline__ void warm_args(const T& args)
     asm volatile("" ::"s"(t));
 }
 
+// waves that share a tile: rows of 256 values and more are split four ways
+constexpr int small_split(int KS) { return KS >= 16 ? 4 : 1; }
+
 template <typename V, int KS>
-__global__ __launch_bounds__(64) void encode_small_kernel(EncJobs js)
+__global__ __launch_bounds__(64 * small_split(KS)) __attribute__((amdgpu_waves_per_eu(small_split(KS) > 1 ? 3 : 1, 8))) void encode_small_kernel(EncJobs js)
 {
     warm_args(js);
     const bool second = (int)blockIdx.x >= js.waves0;
-    encode_small_body<V, KS>(second ? js.job[1] : js.job[0],
-                             second ? blockIdx.x - js.waves0 : blockIdx.x);
+    encode_small_body<V, KS, small_split(KS)>(second ? js.job[1] : js.job[0],
+                                              second ? blockIdx.x - js.waves0 : blockIdx.x);
 }
 
 // Four jobs in one launch, two of input width 16 * KSA and two of 16 * KSB (the two parts of a
@@ -1572,14 +1611,16 @@ struct EncJobs4 {
 };
 
 template <typename V, int KSA, int KSB>
-__global__ __launch_bounds__(64) void encode_small_mixed_kernel(EncJobs4 js)
+__global__ __launch_bounds__(64 * small_split(KSA)) __attribute__((amdgpu_waves_per_eu(3, 8))) void encode_small_mixed_kernel(EncJobs4 js)
 {
+    static_assert(small_split(KSB) == 1, "the narrow jobs' tiles take one wave of the workgroup");
     warm_args(js);
     const int w = blockIdx.x;
     if (w < js.end[1]) {
         const int j = w >= js.end[0] ? 1 : 0;
-        encode_small_body<V, KSA>(js.job[j], j ? w - js.end[0] : w);
+        encode_small_body<V, KSA, small_split(KSA)>(js.job[j], j ? w - js.end[0] : w);
     } else {
+        if (threadIdx.x >= 64) return;  // a narrow tile is one wave's work
         const int j = w >= js.end[2] ? 3 : 2;
         encode_small_body<V, KSB>(js.job[j], w - js.end[j - 1]);
     }
@@ -1889,8 +1930,8 @@ int launch_small(const EncJobs& js, int64_t waves, int K, hipStream_t st)
     switch (K) {
         case 64: hipLaunchKernelGGL((encode_small_kernel<V, 4>), grid, dim3(64), 0, st, js); break;
         case 128: hipLaunchKernelGGL((encode_small_kernel<V, 8>), grid, dim3(64), 0, st, js); break;
-        case 256: hipLaunchKernelGGL((encode_small_kernel<V, 16>), grid, dim3(64), 0, st, js); break;
-        case 512: hipLaunchKernelGGL((encode_small_kernel<V, 32>), grid, dim3(64), 0, st, js); break;
+        case 256: hipLaunchKernelGGL((encode_small_kernel<V, 16>), grid, dim3(64 * small_split(16)), 0, st, js); break;
+        case 512: hipLaunchKernelGGL((encode_small_kernel<V, 32>), grid, dim3(64 * small_split(32)), 0, st, js); break;
         default: return ucm::fail(UCM_ERROR, "internal: K %d has no small-row kernel", K);
     }
     return ucm::launch_status("encode_small_kernel");
@@ -2412,9 +2453,9 @@ int encode_two_pairs(const PairSpec& pa, const PairSpec& pb, hipStream_t st)
         }
         if (end <= 0x7fffffff) {
             if (pa.x_dtype == UCM_DT_BF16)
-                hipLaunchKernelGGL((encode_small_mixed_kernel<bf16x8, 32, 4>), dim3((unsigned)end), dim3(64), 0, st, js);
+                hipLaunchKernelGGL((encode_small_mixed_kernel<bf16x8, 32, 4>), dim3((unsigned)end), dim3(64 * small_split(32)), 0, st, js);
             else
-                hipLaunchKernelGGL((encode_small_mixed_kernel<f16x8, 32, 4>), dim3((unsigned)end), dim3(64), 0, st, js);
+                hipLaunchKernelGGL((encode_small_mixed_kernel<f16x8, 32, 4>), dim3((unsigned)end), dim3(64 * small_split(32)), 0, st, js);
             return ucm::launch_status("encode_small_mixed_kernel");
         }
     }
