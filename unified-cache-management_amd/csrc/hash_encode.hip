@@ -70,6 +70,10 @@ struct EncArgs {
     int gmean;
     int64_t x_stride_g;
     int bs_shift;  // log2(BS) when BS is a power of two, else -1
+    // log2 of N / 32, of H and of heads_per_w where these are powers of two, else -1: the small-row
+    // kernels decode a tile index with shifts then (an integer division is some forty instructions,
+    // and a tile runs five of them, one wave to a SIMD, in front of its first load)
+    int nt_shift, h_shift, hpw_shift;
     // streaming kernel: a word in pinned host memory that a wave sets when one of its bounded waits
     // gives up; the host reads it without touching the device (see stream_latch_tripped())
     unsigned int* timeout_flag;
@@ -1402,8 +1406,14 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
     const int slice = SPLIT > 1 ? (int)(threadIdx.x >> 6) : 0;
     const int k0 = slice * KL;
     const int ntiles = a.N / 32;
-    const int nt = wv % ntiles;
-    wv /= ntiles;
+    int nt;
+    if (a.nt_shift >= 0) {
+        nt = wv & (ntiles - 1);
+        wv >>= a.nt_shift;
+    } else {
+        nt = wv % ntiles;
+        wv /= ntiles;
+    }
     const int lane = threadIdx.x & 63;
     const int r = lane & 31, kb = lane >> 5;
     const bool pairs = small_rows_are_pairs(a);
@@ -1415,15 +1425,30 @@ __device__ __forceinline__ void encode_small_body(const EncArgs& a, int wv)
         int64_t p = (int64_t)wv * kRowsPerWave + r;
         row_ok = p < rows;
         if (!row_ok) p = rows - 1;
-        t = p / a.H;
-        h = (int)(p - t * a.H);
+        if (a.h_shift >= 0) {
+            t = p >> a.h_shift;
+            h = (int)(p & (a.H - 1));
+        } else {
+            t = p / a.H;
+            h = (int)(p - t * a.H);
+        }
     } else {
-        h = wv % a.H;
-        t = (int64_t)(wv / a.H) * kRowsPerWave + r;
+        int row_tile;
+        if (a.h_shift >= 0) {
+            h = wv & (a.H - 1);
+            row_tile = wv >> a.h_shift;
+        } else {
+            h = wv % a.H;
+            row_tile = wv / a.H;
+        }
+        t = (int64_t)row_tile * kRowsPerWave + r;
         row_ok = t < a.T;
         if (!row_ok) t = a.T - 1;
     }
-    const int wi = pairs ? weight_index(a, 0) : weight_index(a, h);  // wave-uniform either way
+    // wave-uniform either way
+    int wi = 0;
+    if (!pairs && a.heads_per_w > 0) wi = a.hpw_shift >= 0 ? h >> a.hpw_shift : h / a.heads_per_w;
+    wi = wi < a.n_w ? wi : a.n_w - 1;
     const uint16_t* wsrc = (const uint16_t*)a.w + ((int64_t)wi * K + k0) * a.N + nt * 32 + r;
     const uint16_t* xr = (const uint16_t*)a.x + src_offset(a, t, h) + k0 + kb * 8;
     // where the row's word goes (a read of the slot mapping): asked for with the operands and
@@ -1956,6 +1981,10 @@ void set_block_shift(EncArgs& a)
     normalize_output(a);
     a.bs_shift = -1;
     if (a.BS > 0 && (a.BS & (a.BS - 1)) == 0) a.bs_shift = __builtin_ctz((unsigned)a.BS);
+    auto log2_or_minus1 = [](int v) { return v > 0 && (v & (v - 1)) == 0 ? __builtin_ctz((unsigned)v) : -1; };
+    a.nt_shift = log2_or_minus1(a.N / 32);
+    a.h_shift = log2_or_minus1(a.H);
+    a.hpw_shift = log2_or_minus1(a.heads_per_w);
 }
 
 int check_shape(const EncArgs& a, int x_dtype, int w_dtype)
