@@ -346,6 +346,50 @@ def test_one_kv_head_random_configurations(seed):
             assert np.array_equal(h, half_piece_sums(q, kc, table, lens, msl)), what
 
 
+@pytest.mark.parametrize("seed", [65, 66])
+def test_latent_18_word_per_token_scores_planes_built_in_the_scorer(seed):
+    """18-word codes in 64-token blocks with 3 to 128 query heads: the per-token kernel that builds its bit
+    planes itself (no plane kernel, with and without a workspace), exact int32 distances against the checker
+    and the half-precision output against the reference's piecewise accumulation (paged_ham_dist_mla.cu:235-241);
+    lengths that end inside a block, unusable table entries, sink and recent windows, rows that end inside a
+    block or reach past the table."""
+    from helpers import half_piece_sums
+    from ucm_amd import _lib
+    from ucm_amd.sparse import hamming_score
+
+    rng = rng_for(seed)
+    for it in range(40):
+        B = int(rng.integers(1, 5))
+        G = int(rng.choice([3, 5, 7, 8, 15, 16, 31, 33, 64, 100, 127, 128]))
+        mb = int(rng.integers(1, 40))
+        NB = B * mb + 3
+        kc = rng.integers(0, 2**32, size=(NB, 64, 1, 18), dtype=np.uint32)
+        q = rng.integers(0, 2**32, size=(B, G, 18), dtype=np.uint32)
+        if it % 6 == 0:
+            q[:] = q[:, :1]                      # all heads equal: the counts reach G
+        if it % 9 == 0:
+            kc[:] = 0xFFFFFFFF
+        table = np.stack([rng.permutation(NB)[:mb] for _ in range(B)]).astype(np.int32)
+        if rng.integers(0, 3) == 0:
+            table[rng.integers(0, B), rng.integers(0, mb)] = NB + 7 if rng.integers(0, 2) else -1
+        lens = rng.integers(0, mb * 64 + 1, size=B).astype(np.int32)
+        if it % 4 == 0:
+            lens[0] = mb * 64
+        msl = max(mb * 64 - int(rng.integers(0, 64)), 1)
+        if it % 5 == 0:
+            msl = mb * 64 + int(rng.integers(1, 200))  # the row reaches past the last table entry
+        sink, recent = int(rng.integers(0, 130)), int(rng.integers(0, 130))
+        what = dict(B=B, G=G, mb=mb, msl=msl, sink=sink, recent=recent, lens=lens.tolist())
+        dq, dk = torch.from_numpy(q.view(np.int32)).cuda(), torch.from_numpy(kc.view(np.int32)).cuda()
+        dt, dl = torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda()
+        o = c_api.hamming_score(q, kc, table, lens, msl, sink, recent, False)
+        g = hamming_score(dk, dq[:, None], dt, dl, msl, sink, recent, False, out_int32=True).cpu().numpy()
+        assert _lib.last_dispatch().startswith("token_score_lanes_run<9,"), (_lib.last_dispatch(), what)
+        assert np.array_equal(g, o), what
+        h = hamming_score(dk, dq[:, None], dt, dl, msl, 0, 0, False).cpu().numpy()
+        assert np.array_equal(h, half_piece_sums(q, kc, table, lens, msl)), what
+
+
 @pytest.mark.parametrize("seed", [71, 72])
 def test_topk_rows_of_257_to_4096_blocks(seed):
     """Rows of 257 to 4096 blocks take the workgroup-per-row selection: ragged lengths, ties

@@ -3826,6 +3826,185 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     }
 }
 
+// Per-token scores for 64-token blocks of whole-code-per-lane layouts above four query heads:
+// block_score_lanes_run's walk (a run of kTokenRunBlocks consecutive blocks per wave, the bit planes
+// built by wave 0 of the workgroup while the first codes are in flight, up to 128 query heads) with
+// token_score_lanes' arithmetic and output (piece sums added in half precision in the reference's
+// order, paged_ham_dist_mla.cu:204-210,235-241).  No plane kernel runs and no workspace is needed.
+// (At 16 x 65,536 tokens and 64 query heads: 22.0 us per call with runs of four blocks, 24.3 us with runs
+// of eight; the plane kernel followed by token_score_lanes takes 21.7 to 21.9 us and needs the workspace.)
+constexpr int kTokenRunBlocks = 4;  // token_score_lanes_run
+
+template <int LC, int GP, bool F16>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void token_score_lanes_run(TokenArgs t)
+{
+    using LCd = LaneCode<LC, false, GP>;
+    constexpr int kRun = kTokenRunBlocks;
+    constexpr int WD = LCd::WD;
+    constexpr int NG = kWave / WD;                        // lane groups (3 for 18 words)
+    constexpr int NCH = (128 + 16 * NG - 1) / (16 * NG);  // rounds of 16 heads per lane
+    __shared__ __align__(16) uint32_t strip[kThreads / kWave][LCd::kRoundWords];
+    __shared__ __align__(16) uint32_t pl[WD * 8];
+    __shared__ __align__(16) uint32_t ptmp[(NG - 1) * WD * 8];
+    __shared__ int ctot[LC];
+    const ScoreArgs& a = t.s;
+    const int b = blockIdx.y;
+    const int lane = lane_id(), wid = wave_id();
+    const int j0 = (blockIdx.x * (kThreads / kWave) + wid) * kRun;
+    // the run's table entries: lane i holds block j0 + i (-1 past the table's row)
+    int my_entry = -1;
+    {
+        const int j = j0 + (lane < kRun ? lane : 0);
+        const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
+        const int e = a.table ? a.table[(int64_t)b * a.table_stride + jc] : b * a.max_blocks + jc;
+        my_entry = (j < a.max_blocks && e >= 0 && e < a.NB) ? e : -1;
+    }
+    const bool builder = wid == 0;
+    const int pw = lane % WD, pg = lane / WD;
+    uint32_t qx[NCH][16];
+    if (builder) {
+        const uint32_t* qb = a.q + b * a.q_stride_b + pw;
+        const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (c * 16 * NG < a.G) {
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const int h = (c * 16 + u) * NG + pg;  // heads past the group re-read the last one
+                    qx[c][u] = qb[(h < a.G ? h : a.G - 1) * qs];
+                }
+            }
+        }
+    }
+    const int len = a.lens[b];
+    auto block_src = [&](int i) -> const u32x4* {
+        const int e = __shfl(my_entry, i);
+        return reinterpret_cast<const u32x4*>(a.kc + (int64_t)(e < 0 ? 0 : e) * a.ks_block);  // block 0: never used
+    };
+    u32x4* mine = reinterpret_cast<u32x4*>(strip[wid]);
+    const uint32_t* row = strip[wid] + lane * WD;
+    // the first block's codes go out before anything waits for the planes
+    u32x4 cur[LCd::kLoads], nxt[LCd::kLoads];
+    LCd::load_round(block_src(0), 0, lane, cur);
+#pragma unroll
+    for (int u = 0; u < LCd::kLoads; ++u) nxt[u] = cur[u];
+    if (builder) {
+        uint32_t acc[8];
+#pragma unroll
+        for (int p = 0; p < 8; ++p) acc[p] = 0;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (c * 16 * NG < a.G) {
+                uint32_t n[5], cy = 0;
+#pragma unroll
+                for (int u = 0; u < 16; ++u)
+                    qx[c][u] = ((c * 16 + u) * NG + pg < a.G && pg < NG) ? qx[c][u] : 0u;
+                count16(qx[c], n);
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    uint32_t sum, c2;
+                    if (p < 5) full_add(acc[p], n[p], cy, sum, c2);
+                    else half_add(acc[p], cy, sum, c2);
+                    acc[p] = sum;
+                    cy = c2;
+                }
+            }
+        }
+        if (pg > 0 && pg < NG) {
+            u32x4* dst = reinterpret_cast<u32x4*>(ptmp + ((pg - 1) * WD + pw) * 8);
+            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
+            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
+        }
+        // the same wave reads what it has just written: LDS operations of a wave complete in order
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (pg == 0) {
+#pragma unroll
+            for (int g = 1; g < NG; ++g) {
+                const u32x4* o4 = reinterpret_cast<const u32x4*>(ptmp + ((g - 1) * WD + pw) * 8);
+                const u32x4 lo = o4[0], hi = o4[1];
+                uint32_t cy = 0;
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    uint32_t sum, c2;
+                    full_add(acc[p], p < 4 ? lo[p & 3] : hi[p & 3], cy, sum, c2);
+                    acc[p] = sum;
+                    cy = c2;
+                }
+            }
+            u32x4* dst = reinterpret_cast<u32x4*>(pl + pw * 8);
+            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
+            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // per 8-byte piece: the sum over its two words and all planes of popc(plane word) << plane
+        if (lane < LC) {
+            const u32x4* w4 = reinterpret_cast<const u32x4*>(pl + (2 * lane) * 8);
+            const u32x4 x0 = w4[0], x1 = w4[1], y0 = w4[2], y1 = w4[3];
+            int c = 0;
+#pragma unroll
+            for (int p = 0; p < GP; ++p)
+                c += (__popc(p < 4 ? x0[p & 3] : x1[p & 3]) + __popc(p < 4 ? y0[p & 3] : y1[p & 3])) << p;
+            ctot[lane] = c;
+        }
+    }
+    // a bare barrier: __syncthreads() would make every wave wait for its codes in flight
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    for (int r = 0; r < kRun; ++r) {
+        const int pos0 = (j0 + r) << 6;
+        if (pos0 >= t.max_seq_len) break;
+        const bool usable = __shfl(my_entry, r) >= 0;
+        const int nout = (64 < t.max_seq_len - pos0) ? 64 : t.max_seq_len - pos0;
+        int ntok = len - pos0;  // tokens whose codes are read
+        ntok = !usable ? 0 : (ntok < 0 ? 0 : (ntok > nout ? nout : ntok));
+        if (r + 1 < kRun) LCd::load_round(block_src(r + 1), 0, lane, nxt);
+        int di = 0;
+        _Float16 dh = (_Float16)0.0f;
+        if (ntok > 0) {
+            LCd::store_round(mine, lane, cur);
+            asm volatile("" ::: "memory");  // the planes are re-read from LDS for every block
+#pragma unroll
+            for (int i = 0; i < LC; ++i) {
+                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
+                const u32x4* pw4 = reinterpret_cast<const u32x4*>(pl + (2 * i) * 8);
+                const u32x4 x0 = pw4[0], x1 = pw4[1], y0 = pw4[2], y1 = pw4[3];
+                int x = 0;
+#pragma unroll
+                for (int p = 0; p < GP; ++p)
+                    x += (__popc(k.x & (p < 4 ? x0[p & 3] : x1[p & 3])) + __popc(k.y & (p < 4 ? y0[p & 3] : y1[p & 3]))) << p;
+                const int part = ctot[i] + a.G * (__popc(k.x) + __popc(k.y)) - 2 * x;
+                di += part;
+                if (F16) dh = dh + (_Float16)(float)part;
+            }
+            asm volatile("" ::: "memory");  // the strip is rewritten by the next block
+        }
+        if (lane < nout) {
+            const int pos = pos0 + lane;
+            const bool keep = (pos < a.sink) || (pos >= len - a.recent && pos < len);
+            const bool none = pos >= len || (!keep && !usable);
+            const int64_t o = (int64_t)b * t.max_seq_len + pos;
+            if (F16) {
+                const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : dh);
+                uint16_t bits;
+                __builtin_memcpy(&bits, &v, 2);
+                ((uint16_t*)t.out)[o] = bits;
+            } else {
+                ((int32_t*)t.out)[o] = none ? kInf : (keep ? 0 : di);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < LCd::kLoads; ++u) cur[u] = nxt[u];
+    }
+}
+
+template <int LC, int GP>
+void launch_token_lanes_run(const TokenArgs& t, dim3 grid, hipStream_t st)
+{
+    if (t.out_is_f16)
+        hipLaunchKernelGGL((token_score_lanes_run<LC, GP, true>), grid, dim3(kThreads), 0, st, t);
+    else
+        hipLaunchKernelGGL((token_score_lanes_run<LC, GP, false>), grid, dim3(kThreads), 0, st, t);
+}
+
 template <int LC, bool DIRECT, int GP>
 void launch_token_lanes(const TokenArgs& t, dim3 grid, hipStream_t st)
 {
@@ -3946,7 +4125,9 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
     const bool direct = G == 1 || G == 2 || G == 4 || G == 8;
     const bool have_planes = workspace && workspace_bytes >= score_plane_bytes(B, Wd) &&
                              (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
-    if (pairs_layout(a, k_cache) && (direct || have_planes)) {
+    // 18-word codes in 64-token blocks above four query heads (or three): the planes are built inside the scorer
+    const bool run18 = Wd == 18 && BS == 64 && G <= 128 && !(G <= 4 && direct) && lanes_layout(a, k_cache, false);
+    if (pairs_layout(a, k_cache) && (direct || have_planes || run18)) {
         hipStream_t st = (hipStream_t)stream;
         const int L = Wd / 2, TP = kWave / L;
         const int nblk = ucm::ceil_div(max_seq_len, BS);
@@ -3959,6 +4140,19 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
             else if (G == 2) launch_token_lanes<9, true, 2>(t, pgrid, st);
             else launch_token_lanes<9, true, 4>(t, pgrid, st);
             return ucm::launch_status("token_score_lanes");
+        }
+        if (run18) {
+            const int pmax = exact_planes(G);
+            const dim3 rgrid((unsigned)ucm::ceil_div(nblk, (kThreads / kWave) * kTokenRunBlocks), (unsigned)B);
+            note_score("token_score_lanes_run", 9, pmax > 8 ? 8 : pmax);
+            switch (pmax) {
+                case 4: launch_token_lanes_run<9, 4>(t, rgrid, st); break;
+                case 5: launch_token_lanes_run<9, 5>(t, rgrid, st); break;
+                case 6: launch_token_lanes_run<9, 6>(t, rgrid, st); break;
+                case 7: launch_token_lanes_run<9, 7>(t, rgrid, st); break;
+                default: launch_token_lanes_run<9, 8>(t, rgrid, st); break;
+            }
+            return ucm::launch_status("token_score_lanes_run");
         }
         // 8 query heads: bit planes when the caller brought the workspace for them
         if (direct && !(lanes && have_planes)) {
