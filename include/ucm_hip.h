@@ -252,7 +252,9 @@ int ucm_hamming_topk_static(const uint32_t* q_codes, int64_t q_stride_b, int64_t
  *             bytes, 16-byte aligned, contents need no initialisation.  It holds the bit
  *             planes of the query counts, which the kernel for one KV head and more than 8
  *             query heads (the latent-attention layout) reads; with NULL that case runs on
- *             the slower general kernel, with the same results.
+ *             the slower general kernel, with the same results.  18-word codes in 64-token
+ *             blocks with up to 128 query heads never need it: their kernel builds the planes
+ *             itself.
  */
 size_t ucm_hamming_score_workspace_bytes(int32_t B, int32_t Hq, int32_t Wd);
 int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
