@@ -1592,8 +1592,8 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 //
 // Codes.  A block goes from memory straight into the wave's LDS strip (load-to-LDS, five
 // instructions of 1 KiB, the last one half masked): no register holds a code on its way, no LDS
-// store instruction is issued.  The strip holds four blocks; a wave scores a run of eight and
-// requests block i + 4 the moment block i's reads are back.  Lane l reads token l's row (72 bytes
+// store instruction is issued.  The strip holds two blocks; a wave scores a run of four and
+// requests block i + 2 the moment block i's reads are back.  Lane l reads token l's row (72 bytes
 // apart: 16 consecutive lanes cover all banks) as nine 8-byte reads.  The 18 x 4 operand words of
 // the weights stay in registers for the whole run.
 //
@@ -1602,17 +1602,23 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 // twice the sum from G (ten bit-sliced bits), take the magnitude, and lanes g < 4 assemble the
 // four operand words of base-4 digit g: a wave takes its words from the query to the operands
 // without LDS and without meeting another wave; waves 0 and 1 build eight words each, wave 2
-// two, wave 3 none.  (Before: three steps by all four waves with LDS and a barrier between
-// them, 14.8 to 15.4 us; one wave doing all of it held the workgroup for 2.4 to 5 us.)  The
-// building waves request three of their first four blocks before the build and the fourth after
-// it, wave 3 all four at once: 14.3 to 14.6 us.  None before the build: 15.3 to 15.6 us; all
-// four: 15.0 to 15.5 us - a compute unit takes one 1 KiB load instruction per 16 cycles, and the
-// eight resident waves' first four blocks each keep every wave at its load instructions for a
-// microsecond before the build starts.
-constexpr int kStripWaves = 4;  // waves per workgroup
-constexpr int kStripRun = 8;    // blocks per wave
-constexpr int kStripSlots = 4;  // blocks of a wave in LDS
-constexpr int kStripFirst = 3;  // of those, a building wave requests before the weight build
+// two, the others none.  (Before: three steps by all four waves with LDS and a barrier between
+// them, 14.8 to 15.4 us; one wave doing all of it held the workgroup for 2.4 to 5 us.)
+//
+// Shape.  Eight waves per workgroup, a run of four blocks per wave, two blocks of a wave in LDS: two
+// workgroups (147 KB of strips) and 16 waves on a compute unit, four to a SIMD.  A block costs its
+// wave some 215 vector and 18 matrix instructions, about 1,150 issue cycles; at the clock this part
+// sustains that is most of the time the codes take to arrive, and with two waves to a SIMD (four
+// waves per workgroup, runs of eight, four blocks in LDS - the same 147 KB in flight) a SIMD stood
+// idle whenever both of its waves waited: 17.1 to 17.5 us with the codes from HBM against 15.4 us
+// now (the whole call with the codes in the last-level cache: 18.0 to 19.8 against 16.4 to 17.5 us).
+// The three building waves
+// request their first blocks after the build - the five others' requests keep memory busy
+// meanwhile (one block before the build: the same; two: 16.3 us).
+constexpr int kStripWaves = 8;  // waves per workgroup
+constexpr int kStripRun = 4;    // blocks per wave
+constexpr int kStripSlots = 2;  // blocks of a wave in LDS
+constexpr int kStripFirst = 0;  // of those, a building wave requests before the weight build (at most kStripSlots)
 
 // One block of NL KiB (+ half a KiB when TAIL) from `base` into LDS at byte address `lds`.
 template <int NL, bool TAIL>
@@ -1644,7 +1650,7 @@ __device__ __forceinline__ void strip_issue_block(uint32_t lds, uint64_t base, u
 typedef int i32x8s __attribute__((ext_vector_type(8)));
 typedef float f32x4s __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void block_score_strip18(ScoreArgs a)
+__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) void block_score_strip18(ScoreArgs a)
 {
 
     constexpr int WD = 18, RUN = kStripRun, kSlots = kStripSlots, kFirst = kStripFirst;
