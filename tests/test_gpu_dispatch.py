@@ -28,7 +28,9 @@ TOPK_SHAPES = {
     "config3_one_long_request": (1, 32, 8, 4, 128, [70001], 128, {},
                                  "block_score_one<1,8,1,4,1>+select_group_kernel<4>"),
     "config5_two_requests": (2, 128, 1, 8, 64, [65536, 700], 128, {},
-                             "block_score_dot64<2>+select_group_kernel<4>"),
+                             "block_score_strip8+select_group_kernel<4>"),
+    "config5_shape_255_query_heads": (2, 255, 1, 8, 64, [4096, 700], 16, {},
+                                      "block_score_dot64<2>+select_wave_kernel<4>"),
     "plugin_reduced_physical": (2, 8, 8, 4, 128, [4096, 3000], 8,
                                 {"reduce_heads": True, "return_physical": True},
                                 "block_score_one<1,8,1,1,1>+select_wave_kernel<4>"),
@@ -113,9 +115,10 @@ def test_per_token_scorer_takes_its_kernels_and_matches_the_checker(name):
 @pytest.mark.parametrize("G", [3, 5, 8, 15, 16, 31, 33, 48, 49, 64, 100, 127, 128, 200])
 def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
     """One KV head: the scorer reduces the G query heads to per-bit counts itself (no plane kernel)
-    when the blocks hold 64 tokens - for every G with 8-word codes (counts as nibble digits for the
-    4-bit dot product), up to 128 heads with 18-word codes (signed base-4 digits of G - 2 * count as
-    FP4 operands of the matrix instruction) and with 16-word codes (bit planes); larger blocks keep
+    when the blocks hold 64 tokens - for every G with 8-word codes (16 to 128 heads: signed base-4
+    digits of G - 2 * count as FP4 operands of the matrix instruction; fewer or more: counts as nibble
+    digits for the 4-bit dot product), up to 128 heads with 18-word codes (the matrix instruction
+    again) and with 16-word codes (bit planes); larger blocks keep
     the plane kernel.  Ragged lengths (an empty request, a length that ends inside a block, runs
     that end inside a workgroup), table entries out of range, forced blocks."""
     from ucm_amd import _lib
@@ -136,7 +139,10 @@ def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
         idx, sc = hamming_topk(_dev(q), _dev(kc), _dev(table), _dev(lens), k, sink, recent)
         got = _lib.last_dispatch()
         if (Wd, BS) == (8, 64):
-            assert got.startswith("block_score_dot64<%d>+" % (1 if G <= 15 else 2))
+            if 16 <= G <= 128:
+                assert got.startswith("block_score_strip8+")
+            else:
+                assert got.startswith("block_score_dot64<%d>+" % (1 if G <= 15 else 2))
         elif (Wd, BS) == (18, 64) and G <= 128:
             assert got.startswith("block_score_strip18+")
         elif BS == 64 and G <= 128:

@@ -1120,7 +1120,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     }
 }
 
-// 64-token blocks of 16-word codes with bit planes (18-word codes have block_score_strip18; the
+// 64-token blocks of 16-word codes with bit planes (18-word codes have block_score_strip<18>; the
 // figures below were taken with them): block_score_lanes' walk (a round of 64
 // tokens through the wave's LDS strip, planes re-read from LDS) over a run of kLaneRun consecutive
 // blocks per wave - the next block's codes are requested before the current one is computed - with
@@ -1296,7 +1296,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
 }
 
 // 64-token blocks of 8-word codes against one KV head whose G query heads enter as per-bit counts
-// (16 requests x 65,536 tokens, 128 query heads: 33 MB of codes in 16,384 blocks of 2 KiB).
+// (16 requests x 65,536 tokens, 128 query heads: 33 MB of codes in 16,384 blocks of 2 KiB).  Serves up
+// to 15 and more than 128 query heads; 16 to 128 heads take block_score_strip<8>, whose weighted bit
+// sums run on the matrix unit (9.5 against 10.8 us at 128 heads: at the clock the part sustains, this
+// kernel's 2.8 million vector instructions are 7 of its microseconds).
 //
 // Arithmetic.  With c_b the number of query heads whose bit b is set, the group-summed distance
 // of a cached code k is  sum_b c_b + G * popc(k) - 2 * sum_b k_b * c_b.  The last sum is a dot
@@ -1605,7 +1608,7 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 // two, the others none.  (Before: three steps by all four waves with LDS and a barrier between
 // them, 14.8 to 15.4 us; one wave doing all of it held the workgroup for 2.4 to 5 us.)
 //
-// Shape.  Eight waves per workgroup, a run of four blocks per wave, two blocks of a wave in LDS: two
+// Shape (18-word codes).  Eight waves per workgroup, a run of four blocks per wave, two blocks of a wave in LDS: two
 // workgroups (147 KB of strips) and 16 waves on a compute unit, four to a SIMD.  A block costs its
 // wave some 215 vector and 18 matrix instructions, about 1,150 issue cycles; at the clock this part
 // sustains that is most of the time the codes take to arrive, and with two waves to a SIMD (four
@@ -1618,23 +1621,34 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 constexpr int kStripWaves = 8;  // waves per workgroup
 constexpr int kStripRun = 4;    // blocks per wave
 constexpr int kStripSlots = 2;  // blocks of a wave in LDS
+constexpr int strip_run(int wd) { return wd == 18 ? kStripRun : 4; }  // blocks per wave
 constexpr int kStripFirst = 0;  // of those, a building wave requests before the weight build (at most kStripSlots)
 
 // One block of NL KiB (+ half a KiB when TAIL) from `base` into LDS at byte address `lds`.
 template <int NL, bool TAIL>
 __device__ __forceinline__ void strip_issue_block(uint32_t lds, uint64_t base, uint32_t off, bool low_half)
 {
-    static_assert(NL == 4, "a block of 64 codes of 16 or 18 words");
+    static_assert(NL == 4 || NL == 2, "a block of 64 codes of 8, 16 or 18 words");
     uint32_t keep;
-    asm volatile("s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[lds]\n\ts_nop 0\n\t"
-                 "global_load_lds_dwordx4 %[o], %[base] nt\n\t"
-                 "global_load_lds_dwordx4 %[o], %[base] offset:1024 nt\n\t"
-                 "global_load_lds_dwordx4 %[o], %[base] offset:2048 nt\n\t"
-                 "global_load_lds_dwordx4 %[o], %[base] offset:3072 nt\n\t"
-                 "s_mov_b32 m0, %[keep]\n\t"
-                 : [keep] "=&s"(keep)
-                 : [lds] "s"(lds), [base] "s"(base), [o] "v"(off)
-                 : "memory");
+    if (NL == 4) {
+        asm volatile("s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[lds]\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %[o], %[base] nt\n\t"
+                     "global_load_lds_dwordx4 %[o], %[base] offset:1024 nt\n\t"
+                     "global_load_lds_dwordx4 %[o], %[base] offset:2048 nt\n\t"
+                     "global_load_lds_dwordx4 %[o], %[base] offset:3072 nt\n\t"
+                     "s_mov_b32 m0, %[keep]\n\t"
+                     : [keep] "=&s"(keep)
+                     : [lds] "s"(lds), [base] "s"(base), [o] "v"(off)
+                     : "memory");
+    } else {
+        asm volatile("s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[lds]\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %[o], %[base] nt\n\t"
+                     "global_load_lds_dwordx4 %[o], %[base] offset:1024 nt\n\t"
+                     "s_mov_b32 m0, %[keep]\n\t"
+                     : [keep] "=&s"(keep)
+                     : [lds] "s"(lds), [base] "s"(base), [o] "v"(off)
+                     : "memory");
+    }
     if (TAIL) {
         if (low_half) {
             asm volatile("s_mov_b32 %[keep], m0\n\ts_add_u32 m0, %[lds], 4096\n\ts_nop 0\n\t"
@@ -1650,12 +1664,17 @@ __device__ __forceinline__ void strip_issue_block(uint32_t lds, uint64_t base, u
 typedef int i32x8s __attribute__((ext_vector_type(8)));
 typedef float f32x4s __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) void block_score_strip18(ScoreArgs a)
+template <int WD>
+__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 8))) void block_score_strip(ScoreArgs a)
 {
-
-    constexpr int WD = 18, RUN = kStripRun, kSlots = kStripSlots, kFirst = kStripFirst;
+    static_assert(WD == 18 || WD == 8, "64-token blocks of 18-word or 8-word codes");
+    // 8-word codes: blocks of 2 KiB, three of a wave in LDS (48 KB per workgroup).  Measured at 16 x 65,536
+    // tokens and 128 query heads, codes from HBM: 9.5 to 9.6 us (runs of two blocks with two in LDS, eight
+    // waves to a SIMD: 10.2 us; the 4-bit dot products of block_score_dot64 on the vector unit: 10.8 to 11.0 us)
+    constexpr int RUN = strip_run(WD), kSlots = WD == 18 ? kStripSlots : 3, kFirst = kStripFirst;
+    constexpr int kBuilders = (WD + 7) / 8;  // waves that build weights, eight code words each
     constexpr int kBlockWords = 64 * WD;
-    constexpr int kLoadsPerBlock = 5;
+    constexpr int kLoadsPerBlock = WD == 18 ? 5 : 2;
     __shared__ __align__(16) uint32_t strip[kStripWaves][kSlots * kBlockWords];
     __shared__ __align__(16) uint32_t wB[WD * 4 * 4];    // operand words [w][digit][j]
     __shared__ __align__(16) uint32_t wzero[4];
@@ -1682,7 +1701,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     const bool has_word = word < WD;
     const int G = a.G;
     uint32_t qx[16];
-    if (wid < 3) {
+    if (wid < kBuilders) {
         const uint32_t* qb = a.q + b * a.q_stride_b + (has_word ? word : 0);
         const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
 #pragma unroll
@@ -1715,10 +1734,10 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     auto issue = [&](int i) __attribute__((always_inline)) {
         int64_t pb = entry[i];
         if (pb < 0 || pb >= NB) pb = 0;  // scored as -1 below
-        strip_issue_block<4, true>(lds0 + (uint32_t)(i % kSlots) * (kBlockWords * 4),
-                                   reinterpret_cast<uint64_t>(kc + pb * ks_block), off, lane < 32);
+        strip_issue_block<(WD == 18 ? 4 : 2), (WD == 18)>(lds0 + (uint32_t)(i % kSlots) * (kBlockWords * 4),
+                                                           reinterpret_cast<uint64_t>(kc + pb * ks_block), off, lane < 32);
     };
-    if (wid < 3) {
+    if (wid < kBuilders) {
         {
             uint32_t o = 0;
 #pragma unroll
@@ -1808,7 +1827,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
             if (i < run) issue(i);
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    const int first = wid < 3 ? kFirst : kSlots;
+    const int first = wid < kBuilders ? kFirst : kSlots;
 #pragma unroll
     for (int i = 0; i < kSlots; ++i)
         if (i >= first && i < run) issue(i);
@@ -1846,11 +1865,23 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
         }
         const uint32_t* row = strip[wid] + (i % kSlots) * kBlockWords + lane * WD;
         uint32_t k[WD];
+        if (WD % 4 == 0) {
+            // rows of 32 bytes: 16-byte reads (two lanes to a bank; 8-byte reads would put four there)
 #pragma unroll
-        for (int w = 0; w < WD / 2; ++w) {
-            const u32x2 kk = *reinterpret_cast<const u32x2*>(row + 2 * w);
-            k[2 * w] = kk.x;
-            k[2 * w + 1] = kk.y;
+            for (int w = 0; w < WD / 4; ++w) {
+                const u32x4 kk = *reinterpret_cast<const u32x4*>(row + 4 * w);
+                k[4 * w] = kk.x;
+                k[4 * w + 1] = kk.y;
+                k[4 * w + 2] = kk.z;
+                k[4 * w + 3] = kk.w;
+            }
+        } else {
+#pragma unroll
+            for (int w = 0; w < WD / 2; ++w) {
+                const u32x2 kk = *reinterpret_cast<const u32x2*>(row + 2 * w);
+                k[2 * w] = kk.x;
+                k[2 * w + 1] = kk.y;
+            }
         }
         f32x4s c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -3024,7 +3055,12 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         const dim3 pgrid((unsigned)ucm::ceil_div(max_blocks, kThreads / kWave), (unsigned)B);
         // 18-word codes (and 8- or 16-word codes with bit planes) in blocks of 64, 128, ...
         // tokens: a whole code per lane
-        if (planes_inside) {
+        if (planes_inside && a.G >= 16 && a.G <= 128) {
+            // the weighted bit sums on the matrix unit, as for 18-word codes
+            note_score("block_score_strip8");
+            const dim3 g64((unsigned)ucm::ceil_div(max_blocks, kStripWaves * strip_run(8)), (unsigned)B);
+            launch_score_threads(block_score_strip<8>, g64, kStripWaves * kWave, 0, st, a);
+        } else if (planes_inside) {
             // one nibble digit of the per-bit counts up to 15 query heads, two up to 255
             const int nd = a.G <= 15 ? 1 : 2;
             note_score("block_score_dot64", nd);
@@ -3041,7 +3077,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
         } else if (planes_in_lanes && Wd == 18) {
             note_score("block_score_strip18");
             const dim3 g64((unsigned)ucm::ceil_div(max_blocks, kStripWaves * kStripRun), (unsigned)B);
-            launch_score_threads(block_score_strip18, g64, kStripWaves * kWave, 0, st, a);
+            launch_score_threads(block_score_strip<18>, g64, kStripWaves * kWave, 0, st, a);
         } else if (planes_in_lanes) {
             note_score("block_score_lanes_run", Wd / 2, pmax);
             const dim3 g64((unsigned)ucm::ceil_div(max_blocks, (kThreads / kWave) * kLanesRunBlocks), (unsigned)B);
