@@ -1298,8 +1298,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
 // 64-token blocks of 8-word codes against one KV head whose G query heads enter as per-bit counts
 // (16 requests x 65,536 tokens, 128 query heads: 33 MB of codes in 16,384 blocks of 2 KiB).  Serves up
 // to 15 and more than 128 query heads; 16 to 128 heads take block_score_strip<8>, whose weighted bit
-// sums run on the matrix unit (9.5 against 10.8 us at 128 heads: at the clock the part sustains, this
-// kernel's 2.8 million vector instructions are 7 of its microseconds).
+// sums run on the matrix unit (9.5 against 10.8 us at 128 heads: this kernel's 2.8 million vector
+// instructions are 11,000 issue cycles per SIMD, 5 of its microseconds at the 2.2 GHz measured inside
+// these scorers).
 //
 // Arithmetic.  With c_b the number of query heads whose bit b is set, the group-summed distance
 // of a cached code k is  sum_b c_b + G * popc(k) - 2 * sum_b k_b * c_b.  The last sum is a dot
@@ -1610,8 +1611,9 @@ __global__ __launch_bounds__(kDotWaves * kWave) void block_score_dot64(ScoreArgs
 //
 // Shape (18-word codes).  Eight waves per workgroup, a run of four blocks per wave, two blocks of a wave in LDS: two
 // workgroups (147 KB of strips) and 16 waves on a compute unit, four to a SIMD.  A block costs its
-// wave some 215 vector and 18 matrix instructions, about 1,150 issue cycles; at the clock this part
-// sustains that is most of the time the codes take to arrive, and with two waves to a SIMD (four
+// wave some 215 vector and 18 matrix instructions, about 1,150 issue cycles - 9 to 10 us per SIMD for
+// its 16 blocks at the 2.1 to 2.3 GHz measured inside this kernel, most of the time the codes take to
+// arrive - and with two waves to a SIMD (four
 // waves per workgroup, runs of eight, four blocks in LDS - the same 147 KB in flight) a SIMD stood
 // idle whenever both of its waves waited: 17.1 to 17.5 us with the codes from HBM against 15.4 us
 // now (the whole call with the codes in the last-level cache: 18.0 to 19.8 against 16.4 to 17.5 us).
