@@ -89,7 +89,8 @@ SCORE_SHAPES = {
     "one_head_6_words": (2, 2, 1, 6, 32, [2048, 700], "token_score_pairs<1,2>"),
     "one_head_6_words_16_query_heads": (2, 16, 1, 6, 32, [2048, 700], "plane_kernel+token_score_pairs<0,5>"),
     "latent_18_words": (2, 1, 1, 18, 64, [4096, 700], "token_score_lanes<9,1,1>"),
-    "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], "token_score_lanes_run<9,7>"),
+    "latent_18_words_64_query_heads": (2, 64, 1, 18, 64, [4096, 700], "token_score_strip<18,0>"),
+    "latent_8_words_128_query_heads": (2, 128, 1, 8, 64, [4096, 700], "token_score_strip<8,0>"),
     "latent_18_words_64_query_heads_128_token_blocks": (2, 64, 1, 18, 128, [4096, 700],
                                                         "plane_kernel+token_score_lanes<9,0,7>"),
     "odd_code_width": (2, 6, 2, 3, 16, [1024, 300], "token_score_kernel"),

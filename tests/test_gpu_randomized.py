@@ -347,12 +347,13 @@ def test_one_kv_head_random_configurations(seed):
 
 
 @pytest.mark.parametrize("seed", [65, 66])
-def test_latent_18_word_per_token_scores_planes_built_in_the_scorer(seed):
-    """18-word codes in 64-token blocks with 3 to 128 query heads: the per-token kernel that builds its bit
-    planes itself (no plane kernel, with and without a workspace), exact int32 distances against the checker
-    and the half-precision output against the reference's piecewise accumulation (paged_ham_dist_mla.cu:235-241);
-    lengths that end inside a block, unusable table entries, sink and recent windows, rows that end inside a
-    block or reach past the table."""
+def test_latent_per_token_scores_weights_built_in_the_scorer(seed):
+    """18-word codes in 64-token blocks with 3 to 128 query heads and 8-word codes with 16 to 128: the per-token
+    kernel that builds its weights itself and sums every 8-byte piece on the matrix unit (no plane kernel, no
+    workspace), exact int32 distances against the checker and the half-precision output against the
+    reference's piecewise accumulation (paged_ham_dist_mla.cu:235-241); lengths that end inside a block,
+    unusable table entries, sink and recent windows, rows that end inside a block or reach past the table,
+    row lengths that are and are not multiples of four."""
     from helpers import half_piece_sums
     from ucm_amd import _lib
     from ucm_amd.sparse import hamming_score
@@ -360,11 +361,12 @@ def test_latent_18_word_per_token_scores_planes_built_in_the_scorer(seed):
     rng = rng_for(seed)
     for it in range(40):
         B = int(rng.integers(1, 5))
-        G = int(rng.choice([3, 5, 7, 8, 15, 16, 31, 33, 64, 100, 127, 128]))
+        Wd = 18 if it % 3 else 8
+        G = int(rng.choice([3, 5, 7, 8, 15, 16, 31, 33, 64, 100, 127, 128] if Wd == 18 else [16, 31, 33, 64, 100, 127, 128]))
         mb = int(rng.integers(1, 40))
         NB = B * mb + 3
-        kc = rng.integers(0, 2**32, size=(NB, 64, 1, 18), dtype=np.uint32)
-        q = rng.integers(0, 2**32, size=(B, G, 18), dtype=np.uint32)
+        kc = rng.integers(0, 2**32, size=(NB, 64, 1, Wd), dtype=np.uint32)
+        q = rng.integers(0, 2**32, size=(B, G, Wd), dtype=np.uint32)
         if it % 6 == 0:
             q[:] = q[:, :1]                      # all heads equal: the counts reach G
         if it % 9 == 0:
@@ -378,13 +380,15 @@ def test_latent_18_word_per_token_scores_planes_built_in_the_scorer(seed):
         msl = max(mb * 64 - int(rng.integers(0, 64)), 1)
         if it % 5 == 0:
             msl = mb * 64 + int(rng.integers(1, 200))  # the row reaches past the last table entry
+        if it % 2 == 0:
+            msl = max(4, msl & ~3)                      # whole groups of four positions: the 8- and 16-byte stores
         sink, recent = int(rng.integers(0, 130)), int(rng.integers(0, 130))
-        what = dict(B=B, G=G, mb=mb, msl=msl, sink=sink, recent=recent, lens=lens.tolist())
+        what = dict(B=B, G=G, Wd=Wd, mb=mb, msl=msl, sink=sink, recent=recent, lens=lens.tolist())
         dq, dk = torch.from_numpy(q.view(np.int32)).cuda(), torch.from_numpy(kc.view(np.int32)).cuda()
         dt, dl = torch.from_numpy(table).cuda(), torch.from_numpy(lens).cuda()
         o = c_api.hamming_score(q, kc, table, lens, msl, sink, recent, False)
         g = hamming_score(dk, dq[:, None], dt, dl, msl, sink, recent, False, out_int32=True).cpu().numpy()
-        assert _lib.last_dispatch().startswith("token_score_lanes_run<9,"), (_lib.last_dispatch(), what)
+        assert _lib.last_dispatch() == "token_score_strip<%d,0>" % Wd, (_lib.last_dispatch(), what)
         assert np.array_equal(g, o), what
         h = hamming_score(dk, dq[:, None], dt, dl, msl, 0, 0, False).cpu().numpy()
         assert np.array_equal(h, half_piece_sums(q, kc, table, lens, msl)), what

@@ -1666,10 +1666,32 @@ __device__ __forceinline__ void strip_issue_block(uint32_t lds, uint64_t base, u
 typedef int i32x8s __attribute__((ext_vector_type(8)));
 typedef float f32x4s __attribute__((ext_vector_type(4)));
 
-template <int WD>
-__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 8))) void block_score_strip(ScoreArgs a)
+// Four values, each replaced by its sum over the four lanes of a quad (two v_add_f32 with a DPP
+// operand per value; a DPP operand needs two idle cycles after the instruction that wrote it, which
+// the other three values' additions provide after the first).
+__device__ __forceinline__ void quad_sum4(float& v0, float& v1, float& v2, float& v3)
+{
+    asm volatile("s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+                 "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+                 "v_add_f32_dpp %2, %2, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+                 "v_add_f32_dpp %3, %3, %3 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+                 "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+                 "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+                 "v_add_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+                 "v_add_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf"
+                 : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3));
+}
+
+// MODE 0: block scores.  MODE 1 / 2: the distance of every token as int32 / as fp16 - the reference scorer's
+// own output (paged_ham_dist_mla.cu:204-210,235-241): an 8-byte piece is two code words, two matrix
+// instructions into an accumulator of their own, and the piece sums are added in half precision in
+// the reference's order; a quad's four lanes hold the same four tokens, its first lane writes them.
+template <int WD, int MODE>
+__device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, void* out)
 {
     static_assert(WD == 18 || WD == 8, "64-token blocks of 18-word or 8-word codes");
+    constexpr bool TOKENS = MODE != 0;
     // 8-word codes: blocks of 2 KiB, three of a wave in LDS (48 KB per workgroup).  Measured at 16 x 65,536
     // tokens and 128 query heads, codes from HBM: 9.5 to 9.6 us (runs of two blocks with two in LDS, eight
     // waves to a SIMD: 10.2 us; the 4-bit dot products of block_score_dot64 on the vector unit: 10.8 to 11.0 us)
@@ -1681,6 +1703,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     __shared__ __align__(16) uint32_t wB[WD * 4 * 4];    // operand words [w][digit][j]
     __shared__ __align__(16) uint32_t wzero[4];
     __shared__ int base_s;
+    __shared__ int cpiece[WD / 2];  // per 8-byte piece: the sum over its bits of the per-bit counts
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
     const int j0 = (blockIdx.x * kStripWaves + wid) * RUN;
@@ -1714,6 +1737,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     }
     if (threadIdx.x == 0) base_s = 0;
     if (threadIdx.x < 4) wzero[threadIdx.x] = 0;
+    if (TOKENS && threadIdx.x < WD / 2) cpiece[threadIdx.x] = 0;
     // everything the rest of the kernel takes from its arguments, now
     const int64_t NB = a.NB, ks_block = a.ks_block;
     const uint32_t* kc = a.kc;
@@ -1722,7 +1746,60 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
     asm volatile("" ::"s"(sink), "s"(recent), "s"(scores), "s"(NB), "s"(G), "s"(max_blocks));
     int nblk = len > 0 ? (len + 63) >> 6 : 0;
     if (nblk > max_blocks) nblk = max_blocks;
-    if ((int)blockIdx.x * kStripWaves * RUN >= nblk) return;  // the whole workgroup
+    // per-token output: lane (column c, quarter q) holds tokens 16 (c / 4) + 4 q + r, r = 0..3, of a block;
+    // the first lane of a quad writes them.  A block that is not read still gets its row: infinity,
+    // or zero inside the sink and recent windows.
+    const int tok0 = 16 * ((lane & 15) >> 2) + 4 * (lane >> 4);
+    const bool by_four = TOKENS && (max_seq_len & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    auto emit = [&](int i, bool usable, const float (&df)[4], const _Float16 (&dh)[4]) __attribute__((always_inline)) {
+        const int pos0 = (j0 + i) << 6;
+        if ((lane & 3) != 0 || pos0 + tok0 >= max_seq_len) return;
+        const int64_t o = (int64_t)b * max_seq_len + pos0 + tok0;
+        uint32_t iv[4];
+        uint16_t hv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int pos = pos0 + tok0 + r;
+            const bool keep = (pos < sink) || (pos >= len - recent && pos < len);
+            const bool none = pos >= len || (!keep && !usable);
+            iv[r] = (uint32_t)(none ? kInf : (keep ? 0 : (int)df[r]));  // exact: an integer below 2^24
+            const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : dh[r]);
+            __builtin_memcpy(&hv[r], &v, 2);
+        }
+        if (MODE == 2) {
+            if (by_four) {
+                u32x2 w;
+                w.x = hv[0] | ((uint32_t)hv[1] << 16);
+                w.y = hv[2] | ((uint32_t)hv[3] << 16);
+                *reinterpret_cast<u32x2*>((uint16_t*)out + o) = w;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (pos0 + tok0 + r < max_seq_len) ((uint16_t*)out)[o + r] = hv[r];
+            }
+        } else {
+            if (by_four) {
+                u32x4 w;
+                w.x = iv[0]; w.y = iv[1]; w.z = iv[2]; w.w = iv[3];
+                *reinterpret_cast<u32x4*>((int32_t*)out + o) = w;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (pos0 + tok0 + r < max_seq_len) ((int32_t*)out)[o + r] = (int32_t)iv[r];
+            }
+        }
+    };
+    auto emit_unread = [&](int first_i) __attribute__((always_inline)) {
+        const float none_i[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const _Float16 none_h[4] = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
+#pragma unroll
+        for (int i = 0; i < RUN; ++i)
+            if (i >= first_i) emit(i, false, none_i, none_h);
+    };
+    if ((int)blockIdx.x * kStripWaves * RUN >= nblk) {  // the whole workgroup
+        if (TOKENS) emit_unread(0);
+        return;
+    }
     const int run = nblk - j0 < RUN ? nblk - j0 : RUN;  // <= 0: nothing to score
     int entry[RUN];
 #pragma unroll
@@ -1822,6 +1899,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
 #pragma unroll
             for (int i = 0; i < 8; ++i) c += __popc(acc[i]) << i;
             atomicAdd(&base_s, c);  // sum over all code bits of the per-bit counts
+            if (TOKENS) atomicAdd(&cpiece[word >> 1], c);
         }
     } else {
 #pragma unroll
@@ -1833,7 +1911,10 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
 #pragma unroll
     for (int i = 0; i < kSlots; ++i)
         if (i >= first && i < run) issue(i);
-    if (run <= 0) return;
+    if (run <= 0) {
+        if (TOKENS) emit_unread(0);
+        return;
+    }
     const int base = base_s;
     const int full = G * 32 * WD;
     // v_mfma_f32_16x16x128 with FP4 operands, one per code word: 16 rows x 128 values of A times
@@ -1851,7 +1932,7 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
         for (int w = 0; w < WD; ++w) Bw[w] = *reinterpret_cast<const u32x4*>(src + w * stride);
     }
     const float dscale = (col & 3) == 0 ? 1.0f : (col & 3) == 1 ? 4.0f : (col & 3) == 2 ? 16.0f : 64.0f;
-    const int tok0 = 16 * (col >> 2) + 4 * quarter;  // + r: the token of result register r
+    // tok0 + r: the token of result register r
     int result = 0;  // lane i: score of block j0 + i
 #pragma unroll
     for (int i = 0; i < RUN; ++i) {
@@ -1886,17 +1967,42 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
             }
         }
         f32x4s c = {0.0f, 0.0f, 0.0f, 0.0f};
+        float df[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        _Float16 dh[4] = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
 #pragma unroll
         for (int w = 0; w < WD; ++w) {
             const i32x8s A = {(int)(k[w] & 0x11111111u), (int)(k[w] & 0x22222222u), (int)(k[w] & 0x44444444u),
                               (int)((k[w] >> 1) & 0x44444444u), 0, 0, 0, 0};
             const i32x8s B = {(int)Bw[w].x, (int)Bw[w].y, (int)Bw[w].z, (int)Bw[w].w, 0, 0, 0, 0};
+            if (TOKENS && (w & 1) == 0) c = f32x4s{0.0f, 0.0f, 0.0f, 0.0f};
             c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, c, 4, 4, 0, 0, 0, 0);  // FP4 x FP4, scales off
+            if (TOKENS && (w & 1) == 1) {
+                // the piece's sum per token: scale by 4^digit, the piece's constant in one lane of the
+                // quad, the sum over the quad.  Small integers: every step is exact in fp32.
+                const float cpf = (lane & 3) == 0 ? (float)cpiece[w >> 1] : 0.0f;
+                float v0 = c[0] * dscale + cpf, v1 = c[1] * dscale + cpf, v2 = c[2] * dscale + cpf, v3 = c[3] * dscale + cpf;
+                quad_sum4(v0, v1, v2, v3);
+                if (MODE == 2) {
+                    dh[0] = dh[0] + (_Float16)v0;
+                    dh[1] = dh[1] + (_Float16)v1;
+                    dh[2] = dh[2] + (_Float16)v2;
+                    dh[3] = dh[3] + (_Float16)v3;
+                } else {
+                    df[0] += v0;
+                    df[1] += v1;
+                    df[2] += v2;
+                    df[3] += v3;
+                }
+            }
         }
         if (i + kSlots < run) {
             // this strip slot is free once its last reads are back
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             issue(i + kSlots);
+        }
+        if (TOKENS) {
+            emit(i, entry[i] >= 0 && entry[i] < NB, df, dh);
+            continue;
         }
         // sum_b k_b t_b of a token = sum over its four digit columns of 4^digit * column: scale, add
         // across the four lanes of a quad, then the minimum over this lane's four tokens
@@ -1917,7 +2023,23 @@ __global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_pe
         const int sc = (entry[i] < 0 || entry[i] >= NB) ? -1 : (forced ? full : full - m);
         if (lane == i) result = sc;
     }
+    if (TOKENS) {
+        emit_unread(run);
+        return;
+    }
     if (lane < run) scores[(int64_t)b * max_blocks + j0 + lane] = result;
+}
+
+template <int WD>
+__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 8))) void block_score_strip(ScoreArgs a)
+{
+    strip_body<WD, 0>(a, 0, nullptr);
+}
+
+template <int WD, bool F16>
+__global__ __launch_bounds__(kStripWaves * kWave) __attribute__((amdgpu_waves_per_eu(4, 8))) void token_score_strip(ScoreArgs a, int max_seq_len, void* out)
+{
+    strip_body<WD, F16 ? 2 : 1>(a, max_seq_len, out);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -3870,185 +3992,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))
     }
 }
 
-// Per-token scores for 64-token blocks of whole-code-per-lane layouts above four query heads:
-// block_score_lanes_run's walk (a run of kTokenRunBlocks consecutive blocks per wave, the bit planes
-// built by wave 0 of the workgroup while the first codes are in flight, up to 128 query heads) with
-// token_score_lanes' arithmetic and output (piece sums added in half precision in the reference's
-// order, paged_ham_dist_mla.cu:204-210,235-241).  No plane kernel runs and no workspace is needed.
-// (At 16 x 65,536 tokens and 64 query heads: 22.0 us per call with runs of four blocks, 24.3 us with runs
-// of eight; the plane kernel followed by token_score_lanes takes 21.7 to 21.9 us and needs the workspace.)
-constexpr int kTokenRunBlocks = 4;  // token_score_lanes_run
-
-template <int LC, int GP, bool F16>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void token_score_lanes_run(TokenArgs t)
-{
-    using LCd = LaneCode<LC, false, GP>;
-    constexpr int kRun = kTokenRunBlocks;
-    constexpr int WD = LCd::WD;
-    constexpr int NG = kWave / WD;                        // lane groups (3 for 18 words)
-    constexpr int NCH = (128 + 16 * NG - 1) / (16 * NG);  // rounds of 16 heads per lane
-    __shared__ __align__(16) uint32_t strip[kThreads / kWave][LCd::kRoundWords];
-    __shared__ __align__(16) uint32_t pl[WD * 8];
-    __shared__ __align__(16) uint32_t ptmp[(NG - 1) * WD * 8];
-    __shared__ int ctot[LC];
-    const ScoreArgs& a = t.s;
-    const int b = blockIdx.y;
-    const int lane = lane_id(), wid = wave_id();
-    const int j0 = (blockIdx.x * (kThreads / kWave) + wid) * kRun;
-    // the run's table entries: lane i holds block j0 + i (-1 past the table's row)
-    int my_entry = -1;
-    {
-        const int j = j0 + (lane < kRun ? lane : 0);
-        const int jc = j < a.max_blocks ? j : a.max_blocks - 1;
-        const int e = a.table ? a.table[(int64_t)b * a.table_stride + jc] : b * a.max_blocks + jc;
-        my_entry = (j < a.max_blocks && e >= 0 && e < a.NB) ? e : -1;
-    }
-    const bool builder = wid == 0;
-    const int pw = lane % WD, pg = lane / WD;
-    uint32_t qx[NCH][16];
-    if (builder) {
-        const uint32_t* qb = a.q + b * a.q_stride_b + pw;
-        const int qs = (int)a.q_stride_h;  // a request's query codes span far less than 2^31 words
-#pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-            if (c * 16 * NG < a.G) {
-#pragma unroll
-                for (int u = 0; u < 16; ++u) {
-                    const int h = (c * 16 + u) * NG + pg;  // heads past the group re-read the last one
-                    qx[c][u] = qb[(h < a.G ? h : a.G - 1) * qs];
-                }
-            }
-        }
-    }
-    const int len = a.lens[b];
-    auto block_src = [&](int i) -> const u32x4* {
-        const int e = __shfl(my_entry, i);
-        return reinterpret_cast<const u32x4*>(a.kc + (int64_t)(e < 0 ? 0 : e) * a.ks_block);  // block 0: never used
-    };
-    u32x4* mine = reinterpret_cast<u32x4*>(strip[wid]);
-    const uint32_t* row = strip[wid] + lane * WD;
-    // the first block's codes go out before anything waits for the planes
-    u32x4 cur[LCd::kLoads], nxt[LCd::kLoads];
-    LCd::load_round(block_src(0), 0, lane, cur);
-#pragma unroll
-    for (int u = 0; u < LCd::kLoads; ++u) nxt[u] = cur[u];
-    if (builder) {
-        uint32_t acc[8];
-#pragma unroll
-        for (int p = 0; p < 8; ++p) acc[p] = 0;
-#pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-            if (c * 16 * NG < a.G) {
-                uint32_t n[5], cy = 0;
-#pragma unroll
-                for (int u = 0; u < 16; ++u)
-                    qx[c][u] = ((c * 16 + u) * NG + pg < a.G && pg < NG) ? qx[c][u] : 0u;
-                count16(qx[c], n);
-#pragma unroll
-                for (int p = 0; p < 8; ++p) {
-                    uint32_t sum, c2;
-                    if (p < 5) full_add(acc[p], n[p], cy, sum, c2);
-                    else half_add(acc[p], cy, sum, c2);
-                    acc[p] = sum;
-                    cy = c2;
-                }
-            }
-        }
-        if (pg > 0 && pg < NG) {
-            u32x4* dst = reinterpret_cast<u32x4*>(ptmp + ((pg - 1) * WD + pw) * 8);
-            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
-            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
-        }
-        // the same wave reads what it has just written: LDS operations of a wave complete in order
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (pg == 0) {
-#pragma unroll
-            for (int g = 1; g < NG; ++g) {
-                const u32x4* o4 = reinterpret_cast<const u32x4*>(ptmp + ((g - 1) * WD + pw) * 8);
-                const u32x4 lo = o4[0], hi = o4[1];
-                uint32_t cy = 0;
-#pragma unroll
-                for (int p = 0; p < 8; ++p) {
-                    uint32_t sum, c2;
-                    full_add(acc[p], p < 4 ? lo[p & 3] : hi[p & 3], cy, sum, c2);
-                    acc[p] = sum;
-                    cy = c2;
-                }
-            }
-            u32x4* dst = reinterpret_cast<u32x4*>(pl + pw * 8);
-            dst[0] = u32x4{acc[0], acc[1], acc[2], acc[3]};
-            dst[1] = u32x4{acc[4], acc[5], acc[6], acc[7]};
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        // per 8-byte piece: the sum over its two words and all planes of popc(plane word) << plane
-        if (lane < LC) {
-            const u32x4* w4 = reinterpret_cast<const u32x4*>(pl + (2 * lane) * 8);
-            const u32x4 x0 = w4[0], x1 = w4[1], y0 = w4[2], y1 = w4[3];
-            int c = 0;
-#pragma unroll
-            for (int p = 0; p < GP; ++p)
-                c += (__popc(p < 4 ? x0[p & 3] : x1[p & 3]) + __popc(p < 4 ? y0[p & 3] : y1[p & 3])) << p;
-            ctot[lane] = c;
-        }
-    }
-    // a bare barrier: __syncthreads() would make every wave wait for its codes in flight
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    for (int r = 0; r < kRun; ++r) {
-        const int pos0 = (j0 + r) << 6;
-        if (pos0 >= t.max_seq_len) break;
-        const bool usable = __shfl(my_entry, r) >= 0;
-        const int nout = (64 < t.max_seq_len - pos0) ? 64 : t.max_seq_len - pos0;
-        int ntok = len - pos0;  // tokens whose codes are read
-        ntok = !usable ? 0 : (ntok < 0 ? 0 : (ntok > nout ? nout : ntok));
-        if (r + 1 < kRun) LCd::load_round(block_src(r + 1), 0, lane, nxt);
-        int di = 0;
-        _Float16 dh = (_Float16)0.0f;
-        if (ntok > 0) {
-            LCd::store_round(mine, lane, cur);
-            asm volatile("" ::: "memory");  // the planes are re-read from LDS for every block
-#pragma unroll
-            for (int i = 0; i < LC; ++i) {
-                const u32x2 k = *reinterpret_cast<const u32x2*>(row + 2 * i);
-                const u32x4* pw4 = reinterpret_cast<const u32x4*>(pl + (2 * i) * 8);
-                const u32x4 x0 = pw4[0], x1 = pw4[1], y0 = pw4[2], y1 = pw4[3];
-                int x = 0;
-#pragma unroll
-                for (int p = 0; p < GP; ++p)
-                    x += (__popc(k.x & (p < 4 ? x0[p & 3] : x1[p & 3])) + __popc(k.y & (p < 4 ? y0[p & 3] : y1[p & 3]))) << p;
-                const int part = ctot[i] + a.G * (__popc(k.x) + __popc(k.y)) - 2 * x;
-                di += part;
-                if (F16) dh = dh + (_Float16)(float)part;
-            }
-            asm volatile("" ::: "memory");  // the strip is rewritten by the next block
-        }
-        if (lane < nout) {
-            const int pos = pos0 + lane;
-            const bool keep = (pos < a.sink) || (pos >= len - a.recent && pos < len);
-            const bool none = pos >= len || (!keep && !usable);
-            const int64_t o = (int64_t)b * t.max_seq_len + pos;
-            if (F16) {
-                const _Float16 v = none ? (_Float16)__builtin_inff() : (keep ? (_Float16)0.0f : dh);
-                uint16_t bits;
-                __builtin_memcpy(&bits, &v, 2);
-                ((uint16_t*)t.out)[o] = bits;
-            } else {
-                ((int32_t*)t.out)[o] = none ? kInf : (keep ? 0 : di);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < LCd::kLoads; ++u) cur[u] = nxt[u];
-    }
-}
-
-template <int LC, int GP>
-void launch_token_lanes_run(const TokenArgs& t, dim3 grid, hipStream_t st)
-{
-    if (t.out_is_f16)
-        hipLaunchKernelGGL((token_score_lanes_run<LC, GP, true>), grid, dim3(kThreads), 0, st, t);
-    else
-        hipLaunchKernelGGL((token_score_lanes_run<LC, GP, false>), grid, dim3(kThreads), 0, st, t);
-}
-
 template <int LC, bool DIRECT, int GP>
 void launch_token_lanes(const TokenArgs& t, dim3 grid, hipStream_t st)
 {
@@ -4169,9 +4112,11 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
     const bool direct = G == 1 || G == 2 || G == 4 || G == 8;
     const bool have_planes = workspace && workspace_bytes >= score_plane_bytes(B, Wd) &&
                              (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
-    // 18-word codes in 64-token blocks above four query heads (or three): the planes are built inside the scorer
+    // 64-token blocks of 18-word codes above four query heads (or three) and of 8-word codes with 16 to 128:
+    // the scorer builds its weights itself
     const bool run18 = Wd == 18 && BS == 64 && G <= 128 && !(G <= 4 && direct) && lanes_layout(a, k_cache, false);
-    if (pairs_layout(a, k_cache) && (direct || have_planes || run18)) {
+    const bool run8 = Wd == 8 && BS == 64 && G >= 16 && G <= 128 && lanes_layout(a, k_cache, false);
+    if (pairs_layout(a, k_cache) && (direct || have_planes || run18 || run8)) {
         hipStream_t st = (hipStream_t)stream;
         const int L = Wd / 2, TP = kWave / L;
         const int nblk = ucm::ceil_div(max_seq_len, BS);
@@ -4185,18 +4130,19 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
             else launch_token_lanes<9, true, 4>(t, pgrid, st);
             return ucm::launch_status("token_score_lanes");
         }
-        if (run18) {
-            const int pmax = exact_planes(G);
-            const dim3 rgrid((unsigned)ucm::ceil_div(nblk, (kThreads / kWave) * kTokenRunBlocks), (unsigned)B);
-            note_score("token_score_lanes_run", 9, pmax > 8 ? 8 : pmax);
-            switch (pmax) {
-                case 4: launch_token_lanes_run<9, 4>(t, rgrid, st); break;
-                case 5: launch_token_lanes_run<9, 5>(t, rgrid, st); break;
-                case 6: launch_token_lanes_run<9, 6>(t, rgrid, st); break;
-                case 7: launch_token_lanes_run<9, 7>(t, rgrid, st); break;
-                default: launch_token_lanes_run<9, 8>(t, rgrid, st); break;
+        if (run18 || run8) {
+            // the weighted bit sums of every 8-byte piece on the matrix unit; no plane kernel, no workspace
+            const dim3 rgrid((unsigned)ucm::ceil_div(nblk, kStripWaves * strip_run(Wd)), (unsigned)B);
+            const dim3 threads(kStripWaves * kWave);
+            note_score("token_score_strip", Wd, out_is_f16 ? 1 : 0);
+            if (Wd == 18) {
+                if (out_is_f16) hipLaunchKernelGGL((token_score_strip<18, true>), rgrid, threads, 0, st, a, max_seq_len, out);
+                else hipLaunchKernelGGL((token_score_strip<18, false>), rgrid, threads, 0, st, a, max_seq_len, out);
+            } else {
+                if (out_is_f16) hipLaunchKernelGGL((token_score_strip<8, true>), rgrid, threads, 0, st, a, max_seq_len, out);
+                else hipLaunchKernelGGL((token_score_strip<8, false>), rgrid, threads, 0, st, a, max_seq_len, out);
             }
-            return ucm::launch_status("token_score_lanes_run");
+            return ucm::launch_status("token_score_strip");
         }
         // 8 query heads: bit planes when the caller brought the workspace for them
         if (direct && !(lanes && have_planes)) {
