@@ -253,8 +253,8 @@ int ucm_hamming_topk_static(const uint32_t* q_codes, int64_t q_stride_b, int64_t
  *             planes of the query counts, which the kernel for one KV head and more than 8
  *             query heads (the latent-attention layout) reads; with NULL that case runs on
  *             the slower general kernel, with the same results.  18-word codes in 64-token
- *             blocks with up to 128 query heads never need it: their kernel builds the planes
- *             itself.
+ *             blocks with up to 128 query heads (and 8-word codes with 16 to 128) never need
+ *             it: their kernel builds its weights itself.
  */
 size_t ucm_hamming_score_workspace_bytes(int32_t B, int32_t Hq, int32_t Wd);
 int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stride_h,
