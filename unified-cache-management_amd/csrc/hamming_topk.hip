@@ -2009,13 +2009,14 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
         const int pos0 = (j0 + i) << 6;
         const int ntok = (64 < len - pos0) ? 64 : len - pos0;
         float mn = 3.0e38f;
+        {
+            float v[4] = {c[0] * dscale, c[1] * dscale, c[2] * dscale, c[3] * dscale};
+            quad_sum4(v[0], v[1], v[2], v[3]);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float v = c[r] * dscale;
-            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
-            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
-            if (tok0 + r >= ntok) v = 3.0e38f;  // the last block of a request
-            mn = v < mn ? v : mn;
+            for (int r = 0; r < 4; ++r) {
+                if (tok0 + r >= ntok) v[r] = 3.0e38f;  // the last block of a request
+                mn = v[r] < mn ? v[r] : mn;
+            }
         }
         const int d = (int)mn;  // exact: every term is an integer below 2^24 (all masked: saturates)
         const int m = __builtin_amdgcn_readlane(wave_min_lane63(d), 63) + base;
