@@ -1665,6 +1665,7 @@ __device__ __forceinline__ void strip_issue_block(uint32_t lds, uint64_t base, u
 
 typedef int i32x8s __attribute__((ext_vector_type(8)));
 typedef float f32x4s __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2s __attribute__((ext_vector_type(2)));
 
 // Four values, each replaced by its sum over the four lanes of a quad (two v_add_f32 with a DPP
 // operand per value; a DPP operand needs two idle cycles after the instruction that wrote it, which
@@ -1703,7 +1704,9 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
     __shared__ __align__(16) uint32_t wB[WD * 4 * 4];    // operand words [w][digit][j]
     __shared__ __align__(16) uint32_t wzero[4];
     __shared__ int base_s;
-    __shared__ int cpiece[WD / 2];  // per 8-byte piece: the sum over its bits of the per-bit counts
+    // per 8-byte piece: the sum over its bits of the per-bit counts, and a row of zeros for the lanes
+    // that do not carry it
+    __shared__ int cpiece[2 * (WD / 2)];
     const int b = blockIdx.y;
     const int lane = lane_id(), wid = wave_id();
     const int j0 = (blockIdx.x * kStripWaves + wid) * RUN;
@@ -1737,7 +1740,7 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
     }
     if (threadIdx.x == 0) base_s = 0;
     if (threadIdx.x < 4) wzero[threadIdx.x] = 0;
-    if (TOKENS && threadIdx.x < WD / 2) cpiece[threadIdx.x] = 0;
+    if (TOKENS && threadIdx.x < 2 * (WD / 2)) cpiece[threadIdx.x] = 0;
     // everything the rest of the kernel takes from its arguments, now
     const int64_t NB = a.NB, ks_block = a.ks_block;
     const uint32_t* kc = a.kc;
@@ -1916,6 +1919,8 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
         return;
     }
     const int base = base_s;
+    // the first lane of a quad adds the piece's constant: it reads the row of constants, the others the zeros
+    const int* cp_row = cpiece + ((lane & 3) == 0 ? 0 : WD / 2);
     const int full = G * 32 * WD;
     // v_mfma_f32_16x16x128 with FP4 operands, one per code word: 16 rows x 128 values of A times
     // 128 x 16 of B.  Lane l supplies row l % 16 of A / column l % 16 of B for the K quarter l / 16,
@@ -1968,7 +1973,7 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
         }
         f32x4s c = {0.0f, 0.0f, 0.0f, 0.0f};
         float df[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        _Float16 dh[4] = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
+        f16x2s dh01 = {(_Float16)0.0f, (_Float16)0.0f}, dh23 = dh01;
 #pragma unroll
         for (int w = 0; w < WD; ++w) {
             const i32x8s A = {(int)(k[w] & 0x11111111u), (int)(k[w] & 0x22222222u), (int)(k[w] & 0x44444444u),
@@ -1979,14 +1984,13 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
             if (TOKENS && (w & 1) == 1) {
                 // the piece's sum per token: scale by 4^digit, the piece's constant in one lane of the
                 // quad, the sum over the quad.  Small integers: every step is exact in fp32.
-                const float cpf = (lane & 3) == 0 ? (float)cpiece[w >> 1] : 0.0f;
+                const float cpf = (float)cp_row[w >> 1];
                 float v0 = c[0] * dscale + cpf, v1 = c[1] * dscale + cpf, v2 = c[2] * dscale + cpf, v3 = c[3] * dscale + cpf;
                 quad_sum4(v0, v1, v2, v3);
                 if (MODE == 2) {
-                    dh[0] = dh[0] + (_Float16)v0;
-                    dh[1] = dh[1] + (_Float16)v1;
-                    dh[2] = dh[2] + (_Float16)v2;
-                    dh[3] = dh[3] + (_Float16)v3;
+                    // two tokens to an instruction: packed conversion (round to nearest even) and packed addition
+                    dh01 = dh01 + f16x2s{(_Float16)v0, (_Float16)v1};
+                    dh23 = dh23 + f16x2s{(_Float16)v2, (_Float16)v3};
                 } else {
                     df[0] += v0;
                     df[1] += v1;
@@ -2001,6 +2005,7 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
             issue(i + kSlots);
         }
         if (TOKENS) {
+            const _Float16 dh[4] = {dh01.x, dh01.y, dh23.x, dh23.y};
             emit(i, entry[i] >= 0 && entry[i] < NB, df, dh);
             continue;
         }
