@@ -717,6 +717,7 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
         codes = torch.empty((NBK, BS, HKV, WD), dtype=torch.int32, device="cuda")
         perms = [torch.randperm(NBK, generator=gen, device="cuda")[:NBLK].to(torch.int32) for _ in range(4)]
         tok = torch.arange(CTX, device="cuda")
+        rows = CTX * HKV
 
         def fused(i):
             enc_k.compute_hash_from_paged_cache(kcache, perms[i % 4], CTX, codes, BS)
