@@ -359,6 +359,25 @@ def topk_split(torch, fn, ms, code_bytes):
                              "hold both)"}
 
 
+def scorer_clock(torch, fn, n=40):
+    """Shader clock inside the latent scorer of fn(): the library's probe has the last wave of the first
+    workgroup write the shader cycles and the 100 MHz ticks of its life (ucm_hamming_topk_set_clock_probe);
+    the figures are those of the last of n back-to-back calls."""
+    L = _lib_mod().lib()
+    probe = torch.zeros(2, dtype=torch.int64, device="cuda")
+    _lib_mod().check(L.ucm_hamming_topk_set_clock_probe(probe.data_ptr()))
+    try:
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+    finally:
+        _lib_mod().check(L.ucm_hamming_topk_set_clock_probe(None))
+    cycles, ticks = (int(v) for v in probe.cpu().tolist())
+    if ticks <= 0:
+        return {}
+    return {"scorer_shader_clock_GHz": cycles / (ticks * 10.0), "scorer_wave_life_us": ticks / 100.0}
+
+
 OP_FLOOR_US = 25.3  # measured with stand-alone probes of the same traffic shape (see the design notes)
 NO_GRAPH = False  # set by --no-graph: no HIP graph is captured anywhere and no hold kernel is queued
 
@@ -813,7 +832,8 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
                                       "code_GBps": b5 * ctx5 * wd5 * 4 / ms / 1e6, "cache_rotation": 16,
                                       "ms_same_cache_every_call": ms_warm,
                                       **topk_split(torch, lambda: hamming_topk(q5, next5(), table5, lens5, 128), ms,
-                                                   b5 * ctx5 * wd5 * 4)}
+                                                   b5 * ctx5 * wd5 * 4),
+                                      **scorer_clock(torch, lambda: hamming_topk(q5, next5(), table5, lens5, 128))}
         del cache5, table5
         # the reference's own latent-attention setting: 18-word codes (512 nope + 64 rope bits), 64 query
         # heads after its head reduction (128 heads, reduction 2), same 16 x 65536 tokens
@@ -840,7 +860,8 @@ def extras(torch, enc_k, gen, legs=ALL_LEGS):
                                      "decode_step_ms": ms_step, "cache_rotation": 8,
                                      "topk128_ms_same_cache_every_call": ms_warm,
                                      "tokens_per_s": b5 * ctx5 / ms * 1e3,
-                                     "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6, **split6}
+                                     "code_GBps": b5 * ctx5 * wd6 * 4 / ms / 1e6, **split6,
+                                     **scorer_clock(torch, lambda: hamming_topk(q6, next6(), table6, lens5, 128))}
         del cache6, table6
     if "token_scores" in legs:
         from ucm_amd.sparse import hamming_score

@@ -278,6 +278,19 @@ int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_str
 int ucm_hamming_topk_set_profile_events(void* before, void* after);
 
 /*
+ * Measurement aid, no counterpart in the reference.  While a non-null address is set, every launch of
+ * the scorer for 64-token blocks of latent-attention codes (block_score_strip / token_score_strip: one
+ * KV head, 18-word codes with up to 128 query heads, 8-word codes with 16 to 128) issued by the
+ * calling thread through ucm_hamming_topk, ucm_hamming_score or a decode-step call has the last wave
+ * of its first workgroup write two 64-bit numbers there when it ends: the shader cycles and the ticks
+ * of the constant 100 MHz counter of its life.  cycles / ticks * 0.1 is the clock in GHz that the wave
+ * ran at; the kernel's instruction counts can only be priced at that clock.  The address must be
+ * 8-byte aligned device memory of at least 16 bytes that outlives the launches; pass null to switch
+ * the probe off (the default).  Other kernels ignore it.
+ */
+int ucm_hamming_topk_set_clock_probe(void* two_u64_in_device_memory);
+
+/*
  * Test hook, no counterpart in the reference.  Writes the names of the kernels that the last
  * ucm_hamming_topk / ucm_hamming_topk_static / ucm_sparse_decode_step* / ucm_gsa_decode_step /
  * ucm_hamming_score call on the calling thread launched, e.g.

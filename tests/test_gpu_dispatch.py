@@ -185,3 +185,39 @@ def test_latent_18_word_scorer_extreme_weights(G):
         oi, os_ = c_api.hamming_topk(q, kc, table, lens, 12, sink, recent, 0)
         assert np.array_equal(sc.cpu().numpy(), os_)
         assert np.array_equal(idx.cpu().numpy(), oi)
+
+
+@pytest.mark.parametrize("Wd,G", [(18, 64), (8, 128)])
+def test_latent_scorer_clock_probe(Wd, G):
+    """The measurement aid of the latent scorers: with a probe address set, the last wave of the first
+    workgroup reports the shader cycles and the 100 MHz ticks of its life (a plausible clock), in the block
+    scorer and in its per-token mode; results are the same with and without it; a misaligned address is
+    refused."""
+    from ucm_amd import _lib
+    from ucm_amd.sparse import hamming_score, hamming_topk
+
+    L = _lib.lib()
+    q, kc, table, lens = make_paged_case(99 + Wd, 2, G, 1, Wd, 64, [8192, 700])
+    args = (_dev(q), _dev(kc), _dev(table), _dev(lens), 16)
+    ref_idx, ref_sc = hamming_topk(*args)
+    ref_tok = hamming_score(_dev(kc), _dev(q), _dev(table), _dev(lens), 8192, 0, 0, False)
+    probe = torch.zeros(2, dtype=torch.int64, device="cuda")
+    _lib.check(L.ucm_hamming_topk_set_clock_probe(probe.data_ptr()))
+    try:
+        for mode in ("blocks", "tokens"):
+            probe.zero_()
+            if mode == "blocks":
+                idx, sc = hamming_topk(*args)
+                assert _lib.last_dispatch().startswith("block_score_strip%d+" % Wd)
+                assert torch.equal(idx, ref_idx) and torch.equal(sc, ref_sc)
+            else:
+                tok = hamming_score(_dev(kc), _dev(q), _dev(table), _dev(lens), 8192, 0, 0, False)
+                assert _lib.last_dispatch() == "token_score_strip<%d,1>" % Wd
+                assert torch.equal(tok, ref_tok)
+            torch.cuda.synchronize()
+            cycles, ticks = (int(v) for v in probe.cpu().tolist())
+            assert cycles > 1000 and ticks > 10, (mode, cycles, ticks)
+            assert 0.3 < cycles / (ticks * 10.0) < 3.5, (mode, cycles, ticks)
+        assert L.ucm_hamming_topk_set_clock_probe(probe.data_ptr() + 4) == _lib.UCM_EPARAM
+    finally:
+        _lib.check(L.ucm_hamming_topk_set_clock_probe(None))

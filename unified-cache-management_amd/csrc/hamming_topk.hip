@@ -56,6 +56,7 @@ struct ScoreArgs {
                              // wave-per-row selection follows: the 8 scores of a block are then
                              // one 32-byte store instead of eight 4-byte stores into lines that
                              // other workgroups write too
+    unsigned long long* clock_probe;  // strip scorers: see ucm_hamming_topk_set_clock_probe(); else null
 };
 
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
@@ -1698,6 +1699,14 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
     // waves to a SIMD: 10.2 us; the 4-bit dot products of block_score_dot64 on the vector unit: 10.8 to 11.0 us)
     constexpr int RUN = strip_run(WD), kSlots = WD == 18 ? kStripSlots : 3, kFirst = kStripFirst;
     constexpr int kBuilders = (WD + 7) / 8;  // waves that build weights, eight code words each
+    // (fetched with the other arguments at the top: nothing is requested of the arguments once the codes flow)
+    unsigned long long* const probe =
+        (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x >= (kStripWaves - 1) * kWave) ? a.clock_probe : nullptr;
+    unsigned long long probe_c0 = 0, probe_r0 = 0;
+    if (probe) {
+        probe_c0 = __builtin_readcyclecounter();
+        probe_r0 = __builtin_amdgcn_s_memrealtime();
+    }
     constexpr int kBlockWords = 64 * WD;
     constexpr int kLoadsPerBlock = WD == 18 ? 5 : 2;
     __shared__ __align__(16) uint32_t strip[kStripWaves][kSlots * kBlockWords];
@@ -2029,11 +2038,13 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
         const int sc = (entry[i] < 0 || entry[i] >= NB) ? -1 : (forced ? full : full - m);
         if (lane == i) result = sc;
     }
-    if (TOKENS) {
-        emit_unread(run);
-        return;
+    if (TOKENS) emit_unread(run);
+    else if (lane < run) scores[(int64_t)b * max_blocks + j0 + lane] = result;
+    // the last wave of the first workgroup: shader cycles and 100 MHz ticks of its life
+    if (probe && threadIdx.x == kStripWaves * kWave - 1) {
+        probe[0] = __builtin_readcyclecounter() - probe_c0;
+        probe[1] = __builtin_amdgcn_s_memrealtime() - probe_r0;
     }
-    if (lane < run) scores[(int64_t)b * max_blocks + j0 + lane] = result;
 }
 
 template <int WD>
@@ -2744,6 +2755,7 @@ Workspace carve(void* base, int B, int Hkv, int max_blocks)
 // Profiling hook: when set, the block-score launch carries these events as the kernel's own
 // start/stop markers (timestamps of the dispatch itself, without the launch latency an event
 // recorded on the stream would add).
+thread_local unsigned long long* g_clock_probe = nullptr;  // see ucm_hamming_topk_set_clock_probe()
 thread_local hipEvent_t g_prof_before = nullptr;
 thread_local hipEvent_t g_prof_after = nullptr;
 
@@ -3056,7 +3068,7 @@ int hamming_topk_run(const uint32_t* q_codes, int64_t q_stride_b, int64_t q_stri
     a.table = block_table; a.table_stride = table_stride; a.max_blocks = max_blocks;
     a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
     a.recent = recent_tok; a.planes = ws.planes; a.scores = ws.scores; a.reduce_out = 0;
-    a.sc_h = max_blocks; a.sc_j = 1;
+    a.sc_h = max_blocks; a.sc_j = 1; a.clock_probe = g_clock_probe;
     // the wave-per-row selection (same test as at its launch below) reads either layout
     const bool wave_select = !(flags & UCM_TOPK_SCORE_ORDER) && max_blocks <= 256;
     bool reduced_scores = false;  // the score kernel already took the maximum over the heads
@@ -3518,6 +3530,14 @@ extern "C" int64_t ucm_hamming_last_dispatch(char* buf, size_t cap)
         snprintf(buf, cap, "%s", tmp);
     }
     return n;
+}
+
+extern "C" int ucm_hamming_topk_set_clock_probe(void* two_u64_in_device_memory)
+{
+    ucm::clear_error();
+    UCM_REQUIRE((reinterpret_cast<uintptr_t>(two_u64_in_device_memory) & 7) == 0, "the address is not 8-byte aligned");
+    g_clock_probe = static_cast<unsigned long long*>(two_u64_in_device_memory);
+    return UCM_OK;
 }
 
 extern "C" int ucm_hamming_topk_set_profile_events(void* before, void* after)
@@ -4073,6 +4093,7 @@ extern "C" int ucm_hamming_score(const uint32_t* q_codes, int64_t q_stride_b, in
     a.table = block_table; a.table_stride = table_stride; a.max_blocks = max_blocks;
     a.lens = seq_lens; a.B = B; a.Hq = Hq; a.G = Hq / Hkv; a.sink = sink_tok;
     a.recent = recent_tok; a.TB = 1; a.reduce_out = 0; a.planes = nullptr; a.scores = nullptr;
+    a.clock_probe = g_clock_probe;
     t.max_seq_len = max_seq_len; t.reduce_heads = reduce_heads; t.out_is_f16 = out_is_f16;
     t.out = out;
     const int G = a.G;

@@ -43,6 +43,7 @@ _SIGNATURES = {
     "ucm_hamming_topk_static": (ci, [vp, i64, i64, vp, i64, i32, i32, i32, i64, i64, i64, vp, i32, i32,
                                      vp, i32, i32, i32, i32, i32, u32, vp, vp, vp]),
     "ucm_hamming_topk_set_profile_events": (ci, [vp, vp]),
+    "ucm_hamming_topk_set_clock_probe": (ci, [vp]),
     "ucm_hamming_last_dispatch": (i64, [C.c_char_p, sz]),
     "ucm_sparse_decode_step": (ci, [vp, i64, i64, i64, vp, ci, vp, i64, i64, ci, i32, vp, ci, i32, i32,
                                     vp, i64, i32, i32, i64, i64, i64, vp, i32, i32, vp, i32, i32, i32,
