@@ -156,22 +156,26 @@ def test_planes_built_inside_the_scorer_for_every_group_size(G, Wd, BS):
         assert np.array_equal(idx.cpu().numpy(), oi)
 
 
-@pytest.mark.parametrize("G", [3, 63, 64, 112, 127, 128])
-def test_latent_18_word_scorer_extreme_weights(G):
-    """The 18-word scorer multiplies code bits with signed weights G - 2 * count on the matrix unit
-    (FP4 operands, float accumulation) and must stay exact at the ends of its range: every query
-    head equal (all counts 0 or G, weights of magnitude G, up to 128), all-ones and all-zero cached
-    codes (the largest sums), one bit set per word, and a run of blocks that ends inside a
-    workgroup's run with a last block of a single token."""
+@pytest.mark.parametrize("Wd,G", [(18, 3), (18, 63), (18, 64), (18, 112), (18, 127), (18, 128),
+                                  (8, 16), (8, 63), (8, 64), (8, 127), (8, 128)])
+def test_latent_18_word_scorer_extreme_weights(Wd, G):
+    """The latent scorers (18-word and 8-word codes) multiply code bits with signed weights G - 2 * count
+    on the matrix unit (FP4 operands, float accumulation) and must stay exact at the ends of their range:
+    every query head equal (all counts 0 or G, weights of magnitude G, up to 128), all-ones and all-zero
+    cached codes (the largest sums), one bit set per word, and a run of blocks that ends inside a
+    workgroup's run with a last block of a single token - block scores, and the per-token mode's int32
+    distances and half-precision sums (paged_ham_dist_mla.cu:235-241)."""
+    from helpers import half_piece_sums
     from ucm_amd import _lib
-    from ucm_amd.sparse import hamming_topk
+    from ucm_amd.sparse import hamming_score, hamming_topk
 
     lens = [64 * 9 + 1, 64 * 40, 17]
-    q, kc, table, lens = make_paged_case(900 + G, len(lens), G, 1, 18, 64, lens)
+    q, kc, table, lens = make_paged_case(900 + G + Wd, len(lens), G, 1, Wd, 64, lens)
+    half = Wd // 2
     q[0, :, :] = q[0, :1, :]              # request 0: all heads equal
     q[1, : G // 2, :] = 0xFFFFFFFF        # request 1: counts of G // 2 or G everywhere
-    q[1, G // 2:, :9] = 0
-    q[1, G // 2:, 9:] = 0xFFFFFFFF
+    q[1, G // 2:, :half] = 0
+    q[1, G // 2:, half:] = 0xFFFFFFFF
     nb = kc.shape[0]
     kc[0::5] = 0xFFFFFFFF                 # whole blocks of all-ones / all-zero codes
     kc[1::5] = 0
@@ -180,11 +184,17 @@ def test_latent_18_word_scorer_extreme_weights(G):
     assert nb >= 5
     for sink, recent in ((0, 0), (64, 64)):
         idx, sc = hamming_topk(_dev(q), _dev(kc), _dev(table), _dev(lens), 12, sink, recent)
-        assert _lib.last_dispatch().startswith("block_score_strip18+")
+        assert _lib.last_dispatch().startswith("block_score_strip%d+" % Wd)
         torch.cuda.synchronize()
         oi, os_ = c_api.hamming_topk(q, kc, table, lens, 12, sink, recent, 0)
         assert np.array_equal(sc.cpu().numpy(), os_)
         assert np.array_equal(idx.cpu().numpy(), oi)
+        msl = 64 * 40
+        tok = hamming_score(_dev(kc), _dev(q), _dev(table), _dev(lens), msl, sink, recent, False, out_int32=True)
+        assert _lib.last_dispatch() == "token_score_strip<%d,0>" % Wd
+        assert np.array_equal(tok.cpu().numpy(), c_api.hamming_score(q, kc, table, lens, msl, sink, recent, False))
+    h = hamming_score(_dev(kc), _dev(q), _dev(table), _dev(lens), 64 * 40, 0, 0, False).cpu().numpy()
+    assert np.array_equal(h, half_piece_sums(q, kc, table, lens, 64 * 40))
 
 
 @pytest.mark.parametrize("Wd,G", [(18, 64), (8, 128)])
