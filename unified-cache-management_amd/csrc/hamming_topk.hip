@@ -1696,7 +1696,8 @@ __device__ __forceinline__ void strip_body(const ScoreArgs& a, int max_seq_len, 
     constexpr bool TOKENS = MODE != 0;
     // 8-word codes: blocks of 2 KiB, three of a wave in LDS (48 KB per workgroup).  Measured at 16 x 65,536
     // tokens and 128 query heads, codes from HBM: 9.5 to 9.6 us (runs of two blocks with two in LDS, eight
-    // waves to a SIMD: 10.2 us; sixteen waves per workgroup, one workgroup and one build per compute unit: 10.1 us;
+    // waves to a SIMD: 10.2 us; sixteen waves per workgroup, one workgroup and one build per compute unit: 10.1 us; four waves
+    // per workgroup, four workgroups and builds per compute unit: 10.2 us;
     // the 4-bit dot products of block_score_dot64 on the vector unit: 10.8 to 11.0 us)
     constexpr int RUN = strip_run(WD), kSlots = WD == 18 ? kStripSlots : 3, kFirst = kStripFirst;
     constexpr int kBuilders = (WD + 7) / 8;  // waves that build weights, eight code words each
